@@ -1,0 +1,37 @@
+// kx_common.h -- error plumbing shared by the translation units of libkx.
+// The reference wraps every CUDA call in ck() and exits (src/kimi_exec.cu:500-502);
+// here the same checks set a thread-local message and return a code.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include "../../include/kx.h"
+
+#define KX_OK 0
+#define KX_ERR_ARG 1
+#define KX_ERR_HIP 2
+#define KX_ERR_STATE 3
+
+void kx_set_error(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
+
+#define KX_HIP(call)                                                                      \
+  do {                                                                                    \
+    hipError_t kx_e_ = (call);                                                            \
+    if (kx_e_ != hipSuccess) {                                                            \
+      kx_set_error("%s: %s (%s:%d)", #call, hipGetErrorString(kx_e_), __FILE__, __LINE__); \
+      return KX_ERR_HIP;                                                                  \
+    }                                                                                     \
+  } while (0)
+
+#define KX_REQUIRE(cond, ...)    \
+  do {                           \
+    if (!(cond)) {               \
+      kx_set_error(__VA_ARGS__); \
+      return KX_ERR_ARG;         \
+    }                            \
+  } while (0)
+
+#define KX_LAUNCH_CHECK() KX_HIP(hipGetLastError())
+
+static inline hipStream_t kx_stream(void *s) { return (hipStream_t)s; }
+static inline int kx_cdiv(int a, int b) { return (a + b - 1) / b; }

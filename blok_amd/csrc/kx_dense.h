@@ -1,0 +1,49 @@
+// kx_dense.h -- internal launch interface of the bf16 GEMV family (kx_dense.hip).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+enum {
+  KX_EPI_BF16 = 0,        // y = bf(sum)                           matvec_bf16_k
+  KX_EPI_F32 = 1,         // y = sum (router logits)               matvec_bf16_f32_k
+  KX_EPI_SWIGLU = 2,      // two matrices: bf(bf(silu(bf(g)))*bf(u)) silu_mul_k
+  KX_EPI_RESID = 3,       // x = bf(x + bf(sum))                   add_k
+  KX_EPI_MOE_COMBINE = 4, // shared down + routed combine + residual
+  KX_EPI_ARGMAX = 5       // bf16-rounded logits as f32 for the argmax reduction
+};
+
+#define KX_GEMV_RI 4
+
+struct KxGemvArgs {
+  const uint16_t *w0;  // bf16 [rows, cols]
+  const uint16_t *w1;  // second matrix for KX_EPI_SWIGLU
+  const uint16_t *x;   // bf16 activations, row stride x_stride
+  int x_stride;
+  void *out;
+  int out_stride;
+  int rows, cols, tokens;
+  int nw, rs;  // set by kx_gemv_launch
+  // KX_EPI_MOE_COMBINE
+  const uint16_t *expert_out;  // bf16 [tokens*topk, rows]
+  const float *route_w;        // f32 [tokens, topk]
+  int topk;
+  uint32_t flags;
+};
+
+int kx_gemv_launch(int epi, KxGemvArgs a, hipStream_t st);
+int kx_rmsnorm_launch(const uint16_t *x, const uint16_t *w, uint16_t *y, int tokens, int n, int x_stride,
+                      int y_stride, float eps, hipStream_t st);
+int kx_argmax_launch(const float *logits, int tokens, int n, int stride, uint32_t *out, hipStream_t st);
+
+// kx_i4.hip
+int kx_i4_launch(bool dual, const uint32_t *packed0, const uint16_t *scale0, const uint32_t *packed1,
+                 const uint16_t *scale1, const uint16_t *x, uint16_t *out, const int *active,
+                 const int *n_active, const int *offsets, const int *pairs, int n_pairs, int rows,
+                 int cols, int x_div, size_t expert_words, size_t expert_scales, int tt, int grid,
+                 hipStream_t st);
+
+// kx_router.hip
+int kx_router_topk_launch(const float *logits, const float *bias, uint16_t *ids, float *weights, int tokens,
+                          int experts, int topk, float routed_scale, hipStream_t st);
+int kx_bucket_launch(const uint16_t *ids, int tokens, int experts, int topk, int *counts, int *offsets,
+                     int *pairs, int *active, int *n_active, hipStream_t st);

@@ -1,0 +1,176 @@
+// kx_moe.hip -- one routed-MoE decode layer for T tokens.
+//
+// Reference: the MoE branch of run(), src/kimi_exec.cu:835-877 -- router gate
+// matvec (fp32 logits), sigmoid + bias + top-8, a blocking copy of the 8 ids to
+// the host, then per slot 32+112 tile launches each preceded by NVMe reads,
+// expert_accum_k per tile, round_bf16_k, the shared expert through bf16_mlp and
+// the residual add.  Here: six launches, no host round trip.
+//   1 router logits  (bf16 GEMV, fp32 out)
+//   2 sigmoid/bias/top-k
+//   3 bucketing (pairs sorted by expert, list of active experts)
+//   4 routed gate+up INT4 GEMV with the SwiGLU epilogue   -> mid  [T*topk, moe_inter]
+//   5 routed down INT4 GEMV                               -> eout [T*topk, hidden]
+//   6 shared gate+up bf16 GEMV with SwiGLU                -> smid [T, shared_inter]
+//   7 shared down bf16 GEMV; epilogue combines the topk routed outputs in slot
+//     order, adds the shared output and the residual.
+#include "kx_common.h"
+#include "kx_dense.h"
+
+struct kx_moe_workspace {
+  int max_tokens;
+  kx_config cfg;
+  float *logits;      // [T, E]
+  uint16_t *ids;      // [T, topk]
+  float *weights;     // [T, topk]
+  int *counts;        // [E]
+  int *offsets;       // [E+1]
+  int *pairs;         // [T*topk]
+  int *active;        // [E]
+  int *n_active;      // [1]
+  uint16_t *mid;      // [T*topk, moe_inter]
+  uint16_t *eout;     // [T*topk, hidden]
+  uint16_t *smid;     // [T, shared_inter]
+  hipEvent_t ev[6];
+};
+
+static int check_cfg(const kx_config *c) {
+  KX_REQUIRE(c, "kx_moe: null config");
+  KX_REQUIRE(c->hidden > 0 && c->hidden % 1024 == 0, "kx_moe: hidden=%d must be a multiple of 1024", c->hidden);
+  KX_REQUIRE(c->moe_inter > 0 && c->moe_inter % 1024 == 0, "kx_moe: moe_inter=%d must be a multiple of 1024", c->moe_inter);
+  KX_REQUIRE(c->shared_inter > 0 && c->shared_inter % 512 == 0, "kx_moe: shared_inter=%d must be a multiple of 512", c->shared_inter);
+  KX_REQUIRE(c->experts > 0 && c->experts <= 1024, "kx_moe: experts=%d outside [1, 1024]", c->experts);
+  KX_REQUIRE(c->topk > 0 && c->topk <= c->experts && c->topk <= 64, "kx_moe: topk=%d outside [1, min(64, experts)]", c->topk);
+  return KX_OK;
+}
+
+extern "C" int kx_moe_workspace_create(const kx_config *cfg, int32_t max_tokens, kx_moe_workspace **out) {
+  KX_REQUIRE(out, "kx_moe_workspace_create: null out pointer");
+  *out = nullptr;
+  int rc = check_cfg(cfg);
+  if (rc) return rc;
+  KX_REQUIRE(max_tokens > 0, "kx_moe_workspace_create: max_tokens=%d must be positive", max_tokens);
+  kx_moe_workspace *ws = new kx_moe_workspace();
+  ws->max_tokens = max_tokens;
+  ws->cfg = *cfg;
+  const size_t T = (size_t)max_tokens, E = (size_t)cfg->experts, K = (size_t)cfg->topk;
+  struct { void **p; size_t bytes; } allocs[] = {
+      {(void **)&ws->logits, T * E * 4}, {(void **)&ws->ids, T * K * 2}, {(void **)&ws->weights, T * K * 4},
+      {(void **)&ws->counts, E * 4}, {(void **)&ws->offsets, (E + 1) * 4}, {(void **)&ws->pairs, T * K * 4},
+      {(void **)&ws->active, E * 4}, {(void **)&ws->n_active, 4},
+      {(void **)&ws->mid, T * K * (size_t)cfg->moe_inter * 2}, {(void **)&ws->eout, T * K * (size_t)cfg->hidden * 2},
+      {(void **)&ws->smid, T * (size_t)cfg->shared_inter * 2}};
+  for (auto &al : allocs) {
+    hipError_t e = hipMalloc(al.p, al.bytes);
+    if (e != hipSuccess) {
+      kx_set_error("kx_moe_workspace_create: hipMalloc(%zu): %s", al.bytes, hipGetErrorString(e));
+      kx_moe_workspace_destroy(ws);
+      return KX_ERR_HIP;
+    }
+  }
+  for (auto &e : ws->ev) KX_HIP(hipEventCreate(&e));
+  *out = ws;
+  return KX_OK;
+}
+
+extern "C" int kx_moe_workspace_destroy(kx_moe_workspace *ws) {
+  if (!ws) return KX_OK;
+  void *ptrs[] = {ws->logits, ws->ids, ws->weights, ws->counts, ws->offsets, ws->pairs,
+                  ws->active, ws->n_active, ws->mid, ws->eout, ws->smid};
+  for (void *p : ptrs)
+    if (p) (void)hipFree(p);
+  for (auto &e : ws->ev)
+    if (e) (void)hipEventDestroy(e);
+  delete ws;
+  return KX_OK;
+}
+
+extern "C" int kx_moe_workspace_views(kx_moe_workspace *ws, void **d_logits, void **d_ids, void **d_weights,
+                                      void **d_counts, void **d_offsets, void **d_pairs, void **d_mid,
+                                      void **d_expert_out) {
+  KX_REQUIRE(ws, "kx_moe_workspace_views: null workspace");
+  if (d_logits) *d_logits = ws->logits;
+  if (d_ids) *d_ids = ws->ids;
+  if (d_weights) *d_weights = ws->weights;
+  if (d_counts) *d_counts = ws->counts;
+  if (d_offsets) *d_offsets = ws->offsets;
+  if (d_pairs) *d_pairs = ws->pairs;
+  if (d_mid) *d_mid = ws->mid;
+  if (d_expert_out) *d_expert_out = ws->eout;
+  return KX_OK;
+}
+
+// tokens per pass of the routed kernels: with T tokens and topk of E experts the
+// expected tokens per active expert stays near 1 until T*topk approaches E.
+static int routed_tt(int tokens, int topk, int experts) {
+  long pairs = (long)tokens * topk;
+  if (pairs <= experts) return 1;
+  if (pairs <= 4L * experts) return 2;
+  return 4;
+}
+
+static int moe_layer(const kx_config *c, const kx_moe_weights *w, kx_moe_workspace *ws, const void *d_n, void *d_x,
+                     int tokens, uint32_t flags, hipStream_t st, bool timed) {
+  int rc = check_cfg(c);
+  if (rc) return rc;
+  KX_REQUIRE(w && ws && d_n && d_x, "kx_moe_decode_layer: null argument");
+  KX_REQUIRE(tokens > 0 && tokens <= ws->max_tokens, "kx_moe_decode_layer: tokens=%d outside [1, %d]", tokens, ws->max_tokens);
+  KX_REQUIRE(c->hidden == ws->cfg.hidden && c->moe_inter == ws->cfg.moe_inter && c->experts == ws->cfg.experts &&
+                 c->topk == ws->cfg.topk && c->shared_inter == ws->cfg.shared_inter,
+             "kx_moe_decode_layer: workspace was created for another shape");
+  const int H = c->hidden, I = c->moe_inter, E = c->experts, K = c->topk;
+  const uint16_t *n = (const uint16_t *)d_n;
+  if (timed) KX_HIP(hipEventRecord(ws->ev[0], st));
+  // 1-3 router
+  KxGemvArgs g = {};
+  g.w0 = (const uint16_t *)w->d_router_gate; g.x = n; g.x_stride = H; g.out = ws->logits; g.out_stride = E;
+  g.rows = E; g.cols = H; g.tokens = tokens;
+  if ((rc = kx_gemv_launch(KX_EPI_F32, g, st))) return rc;
+  if ((rc = kx_router_topk_launch(ws->logits, (const float *)w->d_router_bias, ws->ids, ws->weights, tokens, E, K,
+                                  c->routed_scale, st))) return rc;
+  if ((rc = kx_bucket_launch(ws->ids, tokens, E, K, ws->counts, ws->offsets, ws->pairs, ws->active, ws->n_active, st)))
+    return rc;
+  if (timed) KX_HIP(hipEventRecord(ws->ev[1], st));
+  // 4 routed gate/up + SwiGLU
+  const int tt = routed_tt(tokens, K, E);
+  const int grid = 1024;
+  if ((rc = kx_i4_launch(true, (const uint32_t *)w->d_gate_packed, (const uint16_t *)w->d_gate_scale,
+                         (const uint32_t *)w->d_up_packed, (const uint16_t *)w->d_up_scale, n, ws->mid, ws->active,
+                         ws->n_active, ws->offsets, ws->pairs, 0, I, H, K, (size_t)I * (H / 8), (size_t)I * (H / 32),
+                         tt, grid, st))) return rc;
+  if (timed) KX_HIP(hipEventRecord(ws->ev[2], st));
+  // 5 routed down
+  if ((rc = kx_i4_launch(false, (const uint32_t *)w->d_down_packed, (const uint16_t *)w->d_down_scale, nullptr, nullptr,
+                         ws->mid, ws->eout, ws->active, ws->n_active, ws->offsets, ws->pairs, 0, H, I, 1,
+                         (size_t)H * (I / 8), (size_t)H * (I / 32), tt, grid, st))) return rc;
+  if (timed) KX_HIP(hipEventRecord(ws->ev[3], st));
+  // 6 shared gate/up + SwiGLU
+  KxGemvArgs s = {};
+  s.w0 = (const uint16_t *)w->d_shared_gate; s.w1 = (const uint16_t *)w->d_shared_up; s.x = n; s.x_stride = H;
+  s.out = ws->smid; s.out_stride = c->shared_inter; s.rows = c->shared_inter; s.cols = H; s.tokens = tokens;
+  if ((rc = kx_gemv_launch(KX_EPI_SWIGLU, s, st))) return rc;
+  if (timed) KX_HIP(hipEventRecord(ws->ev[4], st));
+  // 7 shared down + combine + residual
+  KxGemvArgs d = {};
+  d.w0 = (const uint16_t *)w->d_shared_down; d.x = ws->smid; d.x_stride = c->shared_inter; d.out = d_x;
+  d.out_stride = H; d.rows = H; d.cols = c->shared_inter; d.tokens = tokens; d.expert_out = ws->eout;
+  d.route_w = ws->weights; d.topk = K; d.flags = flags;
+  if ((rc = kx_gemv_launch(KX_EPI_MOE_COMBINE, d, st))) return rc;
+  if (timed) KX_HIP(hipEventRecord(ws->ev[5], st));
+  return KX_OK;
+}
+
+extern "C" int kx_moe_decode_layer(const kx_config *cfg, const kx_moe_weights *w, kx_moe_workspace *ws, const void *d_n,
+                                   void *d_x, int32_t tokens, uint32_t flags, void *stream) {
+  return moe_layer(cfg, w, ws, d_n, d_x, tokens, flags, kx_stream(stream), false);
+}
+
+extern "C" int kx_moe_decode_layer_timed(const kx_config *cfg, const kx_moe_weights *w, kx_moe_workspace *ws,
+                                         const void *d_n, void *d_x, int32_t tokens, uint32_t flags, void *stream,
+                                         float *ms5) {
+  KX_REQUIRE(ms5, "kx_moe_decode_layer_timed: null output");
+  int rc = moe_layer(cfg, w, ws, d_n, d_x, tokens, flags, kx_stream(stream), true);
+  if (rc) return rc;
+  KX_HIP(hipEventSynchronize(ws->ev[5]));
+  for (int i = 0; i < 5; ++i) KX_HIP(hipEventElapsedTime(&ms5[i], ws->ev[i], ws->ev[i + 1]));
+  return KX_OK;
+}

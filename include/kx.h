@@ -1,0 +1,168 @@
+/* kx.h -- C ABI of the MI355X (gfx950) implementation of blok's kimi_exec
+ * forward hot path.
+ *
+ * The reference (akhilnairCSE110/blok) has no plugin or FFI surface: its hot
+ * path is the body of one CUDA executable, src/kimi_exec.cu.  Each entry point
+ * below replaces the host function or kernel of that file named in its
+ * comment, with the same operand meaning; shapes default to the constants at
+ * src/kimi_exec.cu:176-186.
+ *
+ * Conventions
+ *  - every function returns 0 on success and a non-zero code on failure;
+ *    kx_last_error() then returns a message (thread local).  The reference
+ *    prints and exits (die(), src/kimi_exec.cu:495-498); a library cannot.
+ *  - pointers named d_* are device (HBM) addresses, h_* are host addresses.
+ *  - bf16 tensors are arrays of uint16_t bit patterns, row-major.
+ *  - `stream` is a hipStream_t passed as void*; NULL is the default stream.
+ *    Operator calls only enqueue work; they do not synchronise.
+ *  - INT4 weights use the compressed-tensors pack_quantized layout the
+ *    reference validates at src/kimi_exec.cu:599-606: packed int32 [N, K/8],
+ *    nibble j of a word is column 8*word+j, stored value = q + 8; scales
+ *    bf16 [N, K/32].
+ */
+#ifndef KX_H
+#define KX_H
+#include <stddef.h>
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Model shape and numeric constants (src/kimi_exec.cu:176-186). */
+typedef struct kx_config {
+  int32_t n_layers;      /* decoder layers in the stack (reference: 61)            */
+  int32_t first_dense;   /* layers [0, first_dense) use the dense MLP (reference 1) */
+  int32_t hidden;        /* 7168 */
+  int32_t heads;         /* 64   */
+  int32_t qk_nope;       /* 128  */
+  int32_t qk_rope;       /* 64   */
+  int32_t v_head;        /* 128  */
+  int32_t q_rank;        /* 1536 */
+  int32_t kv_rank;       /* 512  */
+  int32_t experts;       /* 384  */
+  int32_t topk;          /* 8    */
+  int32_t moe_inter;     /* 2048 */
+  int32_t shared_inter;  /* 2048 */
+  int32_t dense_inter;   /* 18432 */
+  int32_t vocab;         /* 163840 */
+  int32_t max_batch;     /* sequences decoded together                           */
+  int32_t max_context;   /* positions of latent KV cache per sequence            */
+  uint32_t eos_id;       /* 163586: generation stops before emitting it          */
+  float rms_eps;         /* 1e-5 */
+  float rope_theta;      /* 50000 */
+  float routed_scale;    /* 2.827 */
+  float yarn_factor;     /* 32 here; the reference pins 64 (:184)                 */
+  float yarn_beta_fast;  /* 32 */
+  float yarn_beta_slow;  /* 1  */
+  float yarn_orig_ctx;   /* 4096 */
+  float yarn_mscale_all_dim; /* 1 */
+  float init_sigma;      /* std of the random-init bf16 weights (0.02)            */
+  uint64_t seed;         /* seed of every synthetic tensor                        */
+} kx_config;
+
+/* Kimi-K2 shapes, 24 layers (1 dense + 23 MoE), batch 1, context 4096. */
+int kx_config_default(kx_config *cfg);
+const char *kx_last_error(void);
+
+/* ---- device plumbing (reference: Buf / DeviceTensor, :137-174) ---------- */
+int kx_device_info(char *name, size_t name_len, int32_t *compute_units, uint64_t *hbm_bytes);
+int kx_dev_malloc(void **d_ptr, size_t bytes);
+int kx_dev_free(void *d_ptr);
+int kx_dev_memset(void *d_ptr, int value, size_t bytes, void *stream);
+int kx_h2d(void *d_dst, const void *h_src, size_t bytes);
+int kx_d2h(void *h_dst, const void *d_src, size_t bytes);
+int kx_sync(void *stream);
+/* hipEvent timing on `stream` */
+int kx_event_create(void **event);
+int kx_event_destroy(void *event);
+int kx_event_record(void *event, void *stream);
+int kx_event_elapsed_ms(void *start, void *stop, float *ms); /* waits for stop */
+
+/* ---- synthetic tensors: value = f(seed, tensor_id, index) --------------- */
+int kx_fill_normal_bf16(void *d_out, uint64_t n, uint64_t seed, uint64_t tensor_id, float sigma,
+                        int absval, void *stream);
+int kx_fill_normal_f32(void *d_out, uint64_t n, uint64_t seed, uint64_t tensor_id, float sigma,
+                       void *stream);
+int kx_fill_words_u32(void *d_out, uint64_t n, uint64_t seed, uint64_t tensor_id, void *stream);
+
+/* ---- INT4 operators ------------------------------------------------------
+ * kx_i4_unpack : nibble extraction of matvec_i4_bf16_scale_k (:309-311);
+ *                d_q int8 [rows, cols] in [-8, 7].
+ * kx_i4_dequant: the dequantized weight bf((float)q * scale) of :306,:312;
+ *                d_w bf16 [rows, cols].
+ * kx_i4_gemv   : matvec_i4_slice (:688-690) / matvec_i4_bf16_scale_k
+ *                (:300-323) for T activation rows at once:
+ *                y[t, r] = bf(sum_k x[t, k] * w[r, k]), x bf16 [T, cols],
+ *                y bf16 [T, rows].  cols must be a multiple of 1024.         */
+int kx_i4_unpack(const void *d_packed, void *d_q, int32_t rows, int32_t cols, void *stream);
+int kx_i4_dequant(const void *d_packed, const void *d_scale, void *d_w, int32_t rows, int32_t cols,
+                  void *stream);
+int kx_i4_gemv(const void *d_packed, const void *d_scale, const void *d_x, void *d_y, int32_t rows,
+               int32_t cols, int32_t tokens, void *stream);
+
+/* ---- dense operators -----------------------------------------------------
+ * kx_rmsnorm  : rmsnorm_k (:258-270); x, y bf16 [T, n], w bf16 [n].
+ * kx_gemv_bf16: matvec_bf16_k (:272-284) when out_f32 == 0 (y bf16 [T, rows],
+ *               rounded) and matvec_bf16_f32_k (:286-298) when out_f32 != 0
+ *               (y f32 [T, rows], unrounded).  cols multiple of 512.         */
+int kx_rmsnorm(const void *d_x, const void *d_w, void *d_y, int32_t tokens, int32_t n, float eps,
+               void *stream);
+int kx_gemv_bf16(const void *d_w, const void *d_x, void *d_y, int32_t rows, int32_t cols,
+                 int32_t tokens, int out_f32, void *stream);
+
+/* ---- router --------------------------------------------------------------
+ * kx_router_topk: sigmoid_k + add_bf16_k + router_topk_k (:372-397) on fp32
+ *                 logits [T, E]: ids u16 [T, topk] in descending select
+ *                 score, lowest index on ties; weights f32 [T, topk].
+ * kx_bucket     : token -> expert bucketing (the reference's host loop at
+ *                 :845 for batch 1).  counts i32 [E], offsets i32 [E+1],
+ *                 pairs i32 [T*topk] holding token*topk+slot sorted by
+ *                 (expert, token, slot); active i32 [E] lists the experts
+ *                 with at least one pair in ascending order, n_active i32 [1]. */
+int kx_router_topk(const void *d_logits, const void *d_bias, void *d_ids, void *d_weights,
+                   int32_t tokens, int32_t experts, int32_t topk, float routed_scale, void *stream);
+int kx_bucket(const void *d_ids, int32_t tokens, int32_t experts, int32_t topk, void *d_counts,
+              void *d_offsets, void *d_pairs, void *d_active, void *d_n_active, void *stream);
+
+/* ---- one routed-MoE decode layer (the `else` branch of run(), :835-877) ---
+ * Weights of one layer.  Expert tensors hold all E experts back to back.    */
+typedef struct kx_moe_weights {
+  const void *d_router_gate;   /* bf16 [E, hidden]                      */
+  const void *d_router_bias;   /* f32  [E]                              */
+  const void *d_gate_packed;   /* i32  [E, moe_inter, hidden/8]         */
+  const void *d_gate_scale;    /* bf16 [E, moe_inter, hidden/32]        */
+  const void *d_up_packed;     /* i32  [E, moe_inter, hidden/8]         */
+  const void *d_up_scale;      /* bf16 [E, moe_inter, hidden/32]        */
+  const void *d_down_packed;   /* i32  [E, hidden, moe_inter/8]         */
+  const void *d_down_scale;    /* bf16 [E, hidden, moe_inter/32]        */
+  const void *d_shared_gate;   /* bf16 [shared_inter, hidden]           */
+  const void *d_shared_up;     /* bf16 [shared_inter, hidden]           */
+  const void *d_shared_down;   /* bf16 [hidden, shared_inter]           */
+} kx_moe_weights;
+
+/* Scratch for kx_moe_decode_layer; sized for `max_tokens`. */
+typedef struct kx_moe_workspace kx_moe_workspace;
+int kx_moe_workspace_create(const kx_config *cfg, int32_t max_tokens, kx_moe_workspace **ws);
+int kx_moe_workspace_destroy(kx_moe_workspace *ws);
+/* device views of the last call's routing results (for parity checks) */
+int kx_moe_workspace_views(kx_moe_workspace *ws, void **d_logits, void **d_ids, void **d_weights,
+                           void **d_counts, void **d_offsets, void **d_pairs, void **d_mid,
+                           void **d_expert_out);
+
+/* d_n   bf16 [T, hidden]: the post-attention RMSNorm output (input of the FFN)
+ * d_x   bf16 [T, hidden]: the residual stream; on return x = bf(x + down)
+ *       with down = bf(bf(sum_slot y_slot * w_slot) + bf(shared)) (:868-877).
+ * flags bit0: skip the residual add and write `down` to d_x instead.        */
+int kx_moe_decode_layer(const kx_config *cfg, const kx_moe_weights *w, kx_moe_workspace *ws,
+                        const void *d_n, void *d_x, int32_t tokens, uint32_t flags, void *stream);
+/* per-phase kernel time of the most recent kx_moe_decode_layer_timed call, ms:
+ * [0] router+bucket [1] routed gate/up [2] routed down [3] shared gate/up
+ * [4] shared down + combine.  Synchronises.                                 */
+int kx_moe_decode_layer_timed(const kx_config *cfg, const kx_moe_weights *w, kx_moe_workspace *ws,
+                              const void *d_n, void *d_x, int32_t tokens, uint32_t flags,
+                              void *stream, float *ms5);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KX_H */

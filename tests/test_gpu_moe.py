@@ -1,0 +1,165 @@
+"""GPU parity of the router, the bucketing and one routed-MoE decode layer.
+
+Bars: expert ids, bucketing and (kx schedule) every tensor of the layer are
+bit-exact; against the reference schedule the layer output is within max-rel 1e-2.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle as O
+from kxt import (check, dev, moe_case, moe_cfg, moe_device_weights, moe_oracle_weights, say)
+from oracle import ptr
+
+pytestmark = pytest.mark.gpu
+from blok_amd.lib import DevBuf  # noqa: E402
+
+
+def _router(kxlib, logits, bias, topk, scale=2.827):
+    T, E = logits.shape
+    dl, db = dev(logits), dev(bias)
+    di, dw = DevBuf(T * topk * 2), DevBuf(T * topk * 4)
+    check(kxlib.kx_router_topk(dl.ptr, db.ptr, di.ptr, dw.ptr, T, E, topk, scale, None))
+    check(kxlib.kx_sync(None))
+    return di.to_numpy(np.uint16, (T, topk)), dw.to_numpy(np.float32, (T, topk))
+
+
+@pytest.mark.parametrize("T,E,topk", [(1, 384, 8), (64, 384, 8), (5, 16, 4), (3, 1000, 8), (2, 8, 8)])
+def test_router_topk_bit_exact(kxlib, ox, T, E, topk):
+    say(f"router T={T} E={E} topk={topk}")
+    logits = O.normal_f32(T * E, 5, 1, 1.0).reshape(T, E)
+    bias = O.normal_f32(E, 5, 2, 0.01)
+    ids, w = _router(kxlib, logits, bias, topk)
+    ids1, w1 = np.empty_like(ids), np.empty_like(w)
+    ox.ox_router_topk(ptr(logits), ptr(bias), ptr(ids1), ptr(w1), T, E, topk, 2.827, 1)
+    assert (ids == ids1).all()
+    assert (w.view(np.uint32) == w1.view(np.uint32)).all()
+    ids0, w0 = np.empty_like(ids), np.empty_like(w)
+    ox.ox_router_topk(ptr(logits), ptr(bias), ptr(ids0), ptr(w0), T, E, topk, 2.827, 0)
+    assert (ids == ids0).all()
+    assert np.allclose(w, w0, rtol=1e-5)
+
+
+def test_router_ties_take_lowest_index(kxlib, ox):
+    E, topk = 384, 8
+    logits = np.zeros((3, E), dtype=np.float32)          # every score equal
+    logits[1, 100:110] = 2.0                              # ten equal winners, eight slots
+    logits[2, ::7] = 1.0
+    bias = np.zeros(E, dtype=np.float32)
+    ids, w = _router(kxlib, logits, bias, topk)
+    assert ids[0].tolist() == list(range(8))
+    assert ids[1].tolist() == list(range(100, 108))
+    assert ids[2].tolist() == [0, 7, 14, 21, 28, 35, 42, 49]
+    ids1, w1 = np.empty_like(ids), np.empty_like(w)
+    ox.ox_router_topk(ptr(logits), ptr(bias), ptr(ids1), ptr(w1), 3, E, topk, 2.827, 1)
+    assert (ids == ids1).all() and (w.view(np.uint32) == w1.view(np.uint32)).all()
+
+
+@pytest.mark.parametrize("T,E,topk", [(1, 384, 8), (8, 384, 8), (64, 384, 8), (2048, 384, 8), (7, 16, 4)])
+def test_bucket_bit_exact(kxlib, ox, T, E, topk):
+    say(f"bucket T={T} E={E} topk={topk}")
+    logits = O.normal_f32(T * E, 6, 1, 1.0).reshape(T, E)
+    bias = O.normal_f32(E, 6, 2, 0.01)
+    ids = np.empty((T, topk), dtype=np.uint16)
+    wts = np.empty((T, topk), dtype=np.float32)
+    ox.ox_router_topk(ptr(logits), ptr(bias), ptr(ids), ptr(wts), T, E, topk, 2.827, 1)
+    di = dev(ids)
+    dc, do, dp, da, dn = DevBuf(E * 4), DevBuf((E + 1) * 4), DevBuf(T * topk * 4), DevBuf(E * 4), DevBuf(4)
+    check(kxlib.kx_bucket(di.ptr, T, E, topk, dc.ptr, do.ptr, dp.ptr, da.ptr, dn.ptr, None))
+    check(kxlib.kx_sync(None))
+    counts = np.empty(E, dtype=np.int32)
+    offsets = np.empty(E + 1, dtype=np.int32)
+    pairs = np.empty(T * topk, dtype=np.int32)
+    active = np.empty(E, dtype=np.int32)
+    na = ox.ox_bucket(ptr(ids), T, E, topk, ptr(counts), ptr(offsets), ptr(pairs), ptr(active))
+    assert (dc.to_numpy(np.int32, (E,)) == counts).all()
+    assert (do.to_numpy(np.int32, (E + 1,)) == offsets).all()
+    assert (dp.to_numpy(np.int32, (T * topk,)) == pairs).all()
+    assert dn.to_numpy(np.int32, (1,))[0] == na
+    assert (da.to_numpy(np.int32, (E,))[:na] == active[:na]).all()
+
+
+def _run_layer(kxlib, ox, H, I, SI, E, K, T, seed, flags=0):
+    host, n, x = moe_case(kxlib, H, I, SI, E, K, T, seed)
+    cfg = moe_cfg(H, I, SI, E, K)
+    w, bufs = moe_device_weights(host)
+    ws = C.c_void_p()
+    check(kxlib.kx_moe_workspace_create(C.byref(cfg), T, C.byref(ws)))
+    dn, dx = dev(n), dev(x)
+    check(kxlib.kx_moe_decode_layer(C.byref(cfg), C.byref(w), ws, dn.ptr, dx.ptr, T, flags, None))
+    check(kxlib.kx_sync(None))
+    views = [C.c_void_p() for _ in range(8)]
+    check(kxlib.kx_moe_workspace_views(ws, *[C.byref(v) for v in views]))
+    got = {"x": dx.to_numpy(np.uint16, (T, H))}
+    tmp = DevBuf.__new__(DevBuf)
+    def grab(v, dtype, shape):
+        tmp.ptr, tmp.nbytes = v.value, int(np.prod(shape)) * np.dtype(dtype).itemsize
+        return tmp.to_numpy(dtype, shape)
+    got["logits"] = grab(views[0], np.float32, (T, E))
+    got["ids"] = grab(views[1], np.uint16, (T, K))
+    got["weights"] = grab(views[2], np.float32, (T, K))
+    got["mid"] = grab(views[6], np.uint16, (T * K, I))
+    got["eout"] = grab(views[7], np.uint16, (T * K, H))
+    tmp.ptr = None
+    check(kxlib.kx_moe_workspace_destroy(ws))
+    exp = {}
+    for mode in (1, 0):
+        xo = x.copy()
+        o = {"logits": np.empty((T, E), np.float32), "ids": np.empty((T, K), np.uint16),
+             "weights": np.empty((T, K), np.float32), "mid": np.empty((T * K, I), np.uint16),
+             "eout": np.empty((T * K, H), np.uint16)}
+        wo = moe_oracle_weights(host)
+        ox.ox_moe_layer(C.byref(wo), ptr(n), ptr(xo), T, H, I, SI, E, K, 2.827, flags, mode,
+                        ptr(o["logits"]), ptr(o["ids"]), ptr(o["weights"]), ptr(o["mid"]), ptr(o["eout"]))
+        o["x"] = xo
+        exp[mode] = o
+    return got, exp
+
+
+def _assert_layer(got, exp):
+    e1, e0 = exp[1], exp[0]
+    assert (got["logits"].view(np.uint32) == e1["logits"].view(np.uint32)).all(), "router logits differ (kx schedule)"
+    assert (got["ids"] == e1["ids"]).all(), "expert ids differ"
+    assert (got["weights"].view(np.uint32) == e1["weights"].view(np.uint32)).all()
+    assert (got["mid"] == e1["mid"]).all(), f"{np.count_nonzero(got['mid'] != e1['mid'])} mid values differ"
+    assert (got["eout"] == e1["eout"]).all()
+    assert (got["x"] == e1["x"]).all()
+    if (e0["ids"] == e1["ids"]).all():   # same experts under both schedules: compare values
+        assert O.max_rel(O.bf16_to_f32(got["x"]), O.bf16_to_f32(e0["x"])) < 1e-2
+        assert O.max_rel(O.bf16_to_f32(got["mid"]), O.bf16_to_f32(e0["mid"])) < 1e-2
+
+
+@pytest.mark.parametrize("T", [1, 8, 64])
+def test_moe_layer_small_shape(kxlib, ox, T):
+    say(f"moe layer small T={T}")
+    got, exp = _run_layer(kxlib, ox, 1024, 1024, 512, 32, 4, T, 7)
+    _assert_layer(got, exp)
+
+
+def test_moe_layer_flags_write_down_only(kxlib, ox):
+    got, exp = _run_layer(kxlib, ox, 1024, 1024, 512, 16, 8, 3, 8, flags=1)
+    _assert_layer(got, exp)
+
+
+@pytest.mark.parametrize("T", [1, 8])
+def test_moe_layer_kimi_shape(kxlib, ox, T):
+    # BASELINE config 2: hidden 7168, 384 experts top-8, moe_inter 2048, shared 2048
+    say(f"moe layer kimi shape T={T}")
+    got, exp = _run_layer(kxlib, ox, 7168, 2048, 2048, 384, 8, T, 9)
+    _assert_layer(got, exp)
+
+
+def test_moe_errors(kxlib):
+    cfg = moe_cfg(1000, 1024, 512, 16, 4)
+    ws = C.c_void_p()
+    assert kxlib.kx_moe_workspace_create(C.byref(cfg), 4, C.byref(ws)) != 0
+    assert b"hidden" in kxlib.kx_last_error()
+    cfg = moe_cfg(1024, 1024, 512, 16, 4)
+    check(kxlib.kx_moe_workspace_create(C.byref(cfg), 4, C.byref(ws)))
+    from blok_amd.lib import KxMoeWeights
+    w = KxMoeWeights()
+    b = DevBuf(64)
+    assert kxlib.kx_moe_decode_layer(C.byref(cfg), C.byref(w), ws, b.ptr, b.ptr, 5, 0, None) != 0
+    assert b"tokens" in kxlib.kx_last_error()
+    check(kxlib.kx_moe_workspace_destroy(ws))
