@@ -1,0 +1,238 @@
+#!/usr/bin/env python3
+"""bench.py -- throughput of the kimi_exec forward hot path on one MI355X.
+
+One "step" is one pass of the hot path over one batch of synthetic input that is
+already resident in HBM.  Workloads (BASELINE.json configs):
+  moe_layer : config 2, one routed-MoE decode layer at Kimi-K2 shape for T tokens.
+              Weights of several independent layers are cycled so that neither L2
+              nor the 256 MB Infinity Cache can serve them.
+Prints ONE JSON line with the fields the driver reads plus `roofline` (dominant
+kernel: the fused INT4 gate/up GEMV) and `cpu_baseline` (the scalar oracle timed
+on this box's host cores).
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0
+
+
+def build_if_missing():
+    from blok_amd.lib import lib_path
+    if not os.path.exists(lib_path()):
+        import __graft_entry__
+        __graft_entry__.build()
+
+
+def moe_layer_bytes(cfg, tokens, distinct):
+    """Algorithmic HBM bytes of one MoE decode layer (unique bytes that must cross once)."""
+    H, I, SI, E = cfg.hidden, cfg.moe_inter, cfg.shared_inter, cfg.experts
+    per_matrix = I * H // 2 + I * H // 32 * 2              # packed + scales (gate, up and down alike)
+    expert = 3 * per_matrix
+    shared = 3 * SI * H * 2
+    router = E * H * 2
+    io = tokens * H * 2 * 2
+    return {"expert": expert, "gate_up": 2 * per_matrix, "down": per_matrix,
+            "routed": distinct * expert, "shared": shared, "router": router,
+            "layer": distinct * expert + shared + router + io}
+
+
+class MoeLayerSet:
+    """n_layers independent MoE layers generated in place on the device."""
+
+    TENSORS = ("router_gate", "router_bias", "gate_packed", "gate_scale", "up_packed", "up_scale",
+               "down_packed", "down_scale", "shared_gate", "shared_up", "shared_down")
+
+    def __init__(self, lib, cfg, n_layers, seed):
+        from blok_amd.lib import DevBuf, KxMoeWeights, check
+        H, I, SI, E = cfg.hidden, cfg.moe_inter, cfg.shared_inter, cfg.experts
+        self.spec = {  # name: (kind, elements, sigma, tensor id)
+            "router_gate": ("bf16", E * H, float(H) ** -0.5, 10), "router_bias": ("f32", E, 0.01, 11),
+            "gate_packed": ("u32", E * I * H // 8, 0, 12), "gate_scale": ("abs", E * I * H // 32, 0.02, 13),
+            "up_packed": ("u32", E * I * H // 8, 0, 14), "up_scale": ("abs", E * I * H // 32, 0.02, 15),
+            "down_packed": ("u32", E * H * I // 8, 0, 16), "down_scale": ("abs", E * H * I // 32, 0.02, 17),
+            "shared_gate": ("bf16", SI * H, 0.02, 18), "shared_up": ("bf16", SI * H, 0.02, 19),
+            "shared_down": ("bf16", H * SI, 0.02, 20)}
+        self.layers, self.bufs, self.seed = [], [], seed
+        for layer in range(n_layers):
+            w = KxMoeWeights()
+            for name in self.TENSORS:
+                kind, n, sigma, tid = self.spec[name]
+                b = DevBuf(n * (2 if kind in ("bf16", "abs") else 4))
+                s = seed + 1000 * layer
+                if kind == "u32":
+                    check(lib.kx_fill_words_u32(b.ptr, n, s, tid, None))
+                elif kind == "f32":
+                    check(lib.kx_fill_normal_f32(b.ptr, n, s, tid, sigma, None))
+                else:
+                    check(lib.kx_fill_normal_bf16(b.ptr, n, s, tid, sigma, 1 if kind == "abs" else 0, None))
+                setattr(w, "d_" + name, b.ptr)
+                self.bufs.append(b)
+            self.layers.append(w)
+        check(lib.kx_sync(None))
+
+    def host_layer(self, layer):
+        """The same tensors regenerated on the host by the oracle's generator."""
+        import oracle as O
+        out = {}
+        s = self.seed + 1000 * layer
+        for name in self.TENSORS:
+            kind, n, sigma, tid = self.spec[name]
+            if kind == "u32":
+                out[name] = O.words_u32(n, s, tid)
+            elif kind == "f32":
+                out[name] = O.normal_f32(n, s, tid, sigma)
+            else:
+                out[name] = O.normal_bf16(n, s, tid, sigma, 1 if kind == "abs" else 0)
+        return out
+
+
+def run_moe_layer(args):
+    import oracle as O
+    from blok_amd.lib import DevBuf, check, default_config, kx
+    lib = kx()
+    cfg = default_config()
+    T = args.tokens
+    name = C.create_string_buffer(256)
+    cus, hbm = C.c_int32(), C.c_uint64()
+    check(lib.kx_device_info(name, 256, C.byref(cus), C.byref(hbm)))
+    n_layers = args.layers
+    layers = MoeLayerSet(lib, cfg, n_layers, args.seed)
+    ws = C.c_void_p()
+    check(lib.kx_moe_workspace_create(C.byref(cfg), T, C.byref(ws)))
+    n_host = O.normal_bf16(T * cfg.hidden, args.seed, 30, 1.0).reshape(T, cfg.hidden)
+    x_host = O.normal_bf16(T * cfg.hidden, args.seed, 31, 1.0).reshape(T, cfg.hidden)
+    dn, dx = DevBuf.from_numpy(n_host), DevBuf.from_numpy(x_host)
+    views = [C.c_void_p() for _ in range(8)]
+    check(lib.kx_moe_workspace_views(ws, *[C.byref(v) for v in views]))
+
+    def step(i, timed=None):
+        w = layers.layers[i % n_layers]
+        if timed is None:
+            check(lib.kx_moe_decode_layer(C.byref(cfg), C.byref(w), ws, dn.ptr, dx.ptr, T, 0, None))
+        else:
+            check(lib.kx_moe_decode_layer_timed(C.byref(cfg), C.byref(w), ws, dn.ptr, dx.ptr, T, 0, None, timed))
+
+    for i in range(args.warmup):
+        step(i)
+    check(lib.kx_sync(None))
+    # timed region: K steps, events on the launch stream
+    e0, e1 = C.c_void_p(), C.c_void_p()
+    check(lib.kx_event_create(C.byref(e0)))
+    check(lib.kx_event_create(C.byref(e1)))
+    check(lib.kx_sync(None))
+    t0 = time.perf_counter()
+    check(lib.kx_event_record(e0, None))
+    for i in range(args.steps):
+        step(args.warmup + i)
+    check(lib.kx_event_record(e1, None))
+    check(lib.kx_sync(None))
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ms = C.c_float()
+    check(lib.kx_event_elapsed_ms(e0, e1, C.byref(ms)))
+    ms_per_step = ms.value / args.steps
+
+    # per-kernel durations (events around each launch) and distinct experts, same steps
+    phases = np.zeros(5)
+    distinct = []
+    ms5 = (C.c_float * 5)()
+    counts = np.empty(cfg.experts, dtype=np.int32)
+    for i in range(args.steps):
+        step(args.warmup + i, ms5)
+        phases += np.array(list(ms5))
+        check(lib.kx_d2h(counts.ctypes.data, views[3].value, counts.nbytes))
+        distinct.append(int(np.count_nonzero(counts)))
+    phases /= args.steps
+    U = float(np.mean(distinct))
+    by = moe_layer_bytes(cfg, T, U)
+    gate_up_gbs = U * by["gate_up"] / (phases[1] * 1e-3) / 1e9
+    down_gbs = U * by["down"] / (phases[2] * 1e-3) / 1e9
+    routed_gbs = by["routed"] / ((phases[1] + phases[2]) * 1e-3) / 1e9
+    layer_gbs = by["layer"] / (ms_per_step * 1e-3) / 1e9
+
+    # CPU baseline: the oracle's reference schedule on the same layer-0 weights, bounded sample
+    cpu = None
+    if not args.no_cpu:
+        from kxt import moe_oracle_weights
+        ox = O.load()
+        host = layers.host_layer(0)
+        wo = moe_oracle_weights(host)
+        tc = min(T, args.cpu_tokens)
+        xo = x_host[:tc].copy()
+        t0 = time.perf_counter()
+        reps = 0
+        while True:
+            ox.ox_moe_layer(C.byref(wo), n_host[:tc].ctypes.data, xo.ctypes.data, tc, cfg.hidden, cfg.moe_inter,
+                            cfg.shared_inter, cfg.experts, cfg.topk, cfg.routed_scale, 1, 0,
+                            None, None, None, None, None)
+            reps += 1
+            if time.perf_counter() - t0 > args.cpu_seconds or reps >= 64:
+                break
+        dt = time.perf_counter() - t0
+        cpu = {"value": round(tc * reps / dt, 3), "unit": "tok/s", "cores": ox.ox_num_threads(), "kind": "port",
+               "sample": f"{reps} x one MoE decode layer, {tc} token(s), layer-0 weights, reference schedule "
+                         f"(oracle mode 0), OpenMP over output rows, {dt:.1f} s"}
+    check(lib.kx_moe_workspace_destroy(ws))
+
+    out = {
+        "metric": "decode tok/s + INT4 expert GEMV HBM GB/s (% of peak), Kimi-K2 shapes, 1 GPU",
+        "value": round(T / (ms_per_step * 1e-3), 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "int4 weights x bf16 activations, f32 accumulate",
+        "data": "synthetic",
+        "config": {"workload": f"moe_decode_layer (BASELINE config 2), T={T}, hidden 7168, 384 experts top-8, "
+                               f"moe_inter 2048, shared 2048; {n_layers} independent layers cycled (cold weights)",
+                   "tokens": T, "distinct_experts_per_step": round(U, 2), "device": name.value.decode(),
+                   "compute_units": cus.value},
+        "roofline": {"bound": "hbm", "achieved": round(gate_up_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gate_up_gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "i4_gemv_k<dual> (routed gate+up + SwiGLU)",
+                     "algorithmic_bytes_per_launch": int(U * by["gate_up"]),
+                     "avg_launch_ms": round(float(phases[1]), 5)},
+        "int4_expert_gemv": {"routed_gbs": round(routed_gbs, 1), "routed_frac_of_peak": round(routed_gbs / HBM_PEAK_GBS, 4),
+                             "gate_up_gbs": round(gate_up_gbs, 1), "down_gbs": round(down_gbs, 1),
+                             "layer_gbs": round(layer_gbs, 1)},
+        "phase_ms": {"router_bucket": round(float(phases[0]), 5), "routed_gate_up": round(float(phases[1]), 5),
+                     "routed_down": round(float(phases[2]), 5), "shared_gate_up": round(float(phases[3]), 5),
+                     "shared_down_combine": round(float(phases[4]), 5)},
+        "wall_ms_per_step": round(wall_ms / args.steps, 5),
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(out), flush=True)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=40)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--workload", default="moe_layer")
+    ap.add_argument("--tokens", type=int, default=1)
+    ap.add_argument("--layers", type=int, default=4, help="independent layers cycled to keep weights cold")
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--cpu-tokens", type=int, default=4)
+    ap.add_argument("--cpu-seconds", type=float, default=10.0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    build_if_missing()
+    if args.workload == "moe_layer":
+        run_moe_layer(args)
+    else:
+        print(f"unknown workload {args.workload}", file=sys.stderr)
+        sys.exit(2)
+
+
+if __name__ == "__main__":
+    main()
