@@ -37,8 +37,8 @@ int kx_argmax_launch(const float *logits, int tokens, int n, int stride, uint32_
 
 // kx_i4.hip
 int kx_i4_launch(bool dual, const uint32_t *packed0, const uint16_t *scale0, const uint32_t *packed1,
-                 const uint16_t *scale1, const uint16_t *x, uint16_t *out, const int *active,
-                 const int *n_active, const int *offsets, const int *pairs, int n_pairs, int rows,
+                 const uint16_t *scale1, const uint16_t *x, uint16_t *out, const int4 *work,
+                 const int *pairs, int n_pairs, int rows,
                  int cols, int x_div, size_t expert_words, size_t expert_scales, int tt, int grid,
                  hipStream_t st);
 
@@ -46,4 +46,4 @@ int kx_i4_launch(bool dual, const uint32_t *packed0, const uint16_t *scale0, con
 int kx_router_topk_launch(const float *logits, const float *bias, uint16_t *ids, float *weights, int tokens,
                           int experts, int topk, float routed_scale, hipStream_t st);
 int kx_bucket_launch(const uint16_t *ids, int tokens, int experts, int topk, int *counts, int *offsets,
-                     int *pairs, int *active, int *n_active, hipStream_t st);
+                     int *pairs, int4 *work, int *n_active, hipStream_t st);

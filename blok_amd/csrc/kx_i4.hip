@@ -83,11 +83,10 @@ struct XGroup {
 __device__ __forceinline__ float bf_lo(uint32_t u) { return kx_bits_f32(u << 16); }
 __device__ __forceinline__ float bf_hi(uint32_t u) { return kx_bits_f32(u & 0xffff0000u); }
 
-__device__ __forceinline__ void load_xgroup(XGroup &g, const uint16_t *x /* 32 bf16, 64 B aligned */) {
-  const uint4 *p = (const uint4 *)x;
+__device__ __forceinline__ void prep_xgroup(XGroup &g, const uint4 (&raw)[4] /* 32 bf16 of the group */) {
 #pragma unroll
   for (int w = 0; w < 4; ++w) {
-    uint4 u = p[w];  // x[8w .. 8w+7]
+    const uint4 u = raw[w];  // x[8w .. 8w+7]
     g.v[w * 8 + 0] = bf_lo(u.x);             // k = 8w+0
     g.v[w * 8 + 1] = bf_lo(u.z);             // k = 8w+4
     g.v[w * 8 + 2] = bf_hi(u.x) * 0.0625f;   // k = 8w+1
@@ -129,13 +128,62 @@ __device__ __forceinline__ float group_dot(const I4Dec &d, const XGroup &g) {
   return acc;
 }
 
-__device__ __forceinline__ float half_wave_sum(float v) {
-  v += __shfl_xor(v, 16);
-  v += __shfl_xor(v, 8);
-  v += __shfl_xor(v, 4);
-  v += __shfl_xor(v, 2);
-  v += __shfl_xor(v, 1);
-  return v;
+// ---- half-wave (32 lane) reduction ---------------------------------------------------
+// Sums NV per-lane values over the 32 lanes of a half-wave with the xor-butterfly tree
+// (16, 8, 4, 2, 1).  Level 16 swaps rows between two registers (v_permlane16_swap), so
+// each lane keeps half of the values; level 8 does the same with a rotate-by-8 inside the
+// 16-lane row; levels 4, 2, 1 are DPP row shifts, valid in lanes that are multiples of 8.
+// The sums have the bits of a full butterfly because fp32 addition commutes.
+// On return, in lanes with (l & 7) == 0, v[0] is the total of value index
+//   (l >> 4) * NV/2 + ((l >> 3) & 1) * NV/4 + j   for the j-th survivor (j < NV/4, or the
+// single value when NV <= 2) -- see half_wave_index().
+__device__ __forceinline__ void swap_rows16(float &a, float &b) {
+  // rows 1,3 of a <-> rows 0,2 of b
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+constexpr int DPP_ROW_SHL1 = 0x101, DPP_ROW_SHL2 = 0x102, DPP_ROW_SHL4 = 0x104, DPP_ROW_ROR8 = 0x128;
+
+// NV in {2, 4, 8, 16}: after the call v[0 .. NV/4-1] (NV >= 4) or v[0] (NV == 2) hold totals
+template <int NV>
+__device__ __forceinline__ void half_wave_reduce(float (&v)[NV], int l) {
+  static_assert(NV == 2 || NV == 4 || NV == 8 || NV == 16, "values per reduction");
+  // level 16: value i pairs with value i + NV/2
+#pragma unroll
+  for (int i = 0; i < NV / 2; ++i) {
+    swap_rows16(v[i], v[i + NV / 2]);
+    v[i] = v[i] + v[i + NV / 2];  // rows 0,2: value i; rows 1,3: value i + NV/2
+  }
+  if constexpr (NV >= 4) {
+    // level 8: value i pairs with value i + NV/4 (within the NV/2 this lane kept)
+    const bool hi = (l & 8) != 0;
+#pragma unroll
+    for (int i = 0; i < NV / 4; ++i) {
+      float send = hi ? v[i] : v[i + NV / 4];
+      float mine = hi ? v[i + NV / 4] : v[i];
+      v[i] = mine + dpp_f<DPP_ROW_ROR8>(send);
+    }
+#pragma unroll
+    for (int i = 0; i < NV / 4; ++i) {
+      v[i] = v[i] + dpp_f<DPP_ROW_SHL4>(v[i]);
+      v[i] = v[i] + dpp_f<DPP_ROW_SHL2>(v[i]);
+      v[i] = v[i] + dpp_f<DPP_ROW_SHL1>(v[i]);
+    }
+  } else {
+    v[0] = v[0] + dpp_f<DPP_ROW_ROR8>(v[0]);
+    v[0] = v[0] + dpp_f<DPP_ROW_SHL4>(v[0]);
+    v[0] = v[0] + dpp_f<DPP_ROW_SHL2>(v[0]);
+    v[0] = v[0] + dpp_f<DPP_ROW_SHL1>(v[0]);
+  }
+}
+// value index held in v[j] of lane l after half_wave_reduce<NV>
+template <int NV>
+__device__ __forceinline__ int half_wave_index(int l, int j) {
+  if constexpr (NV >= 4) return ((l >> 4) & 1) * (NV / 2) + ((l >> 3) & 1) * (NV / 4) + j;
+  else return (l >> 4) & 1;
 }
 
 struct I4Args {
@@ -145,173 +193,234 @@ struct I4Args {
   const uint16_t *scale1;
   const uint16_t *x;  // bf16 rows of `cols`
   uint16_t *out;      // bf16 rows of `rows`, indexed by pair
-  const int *active;  // expert ids with work; nullptr: one matrix, pairs 0..n_pairs-1
-  const int *n_active;
-  const int *offsets;  // [E+1] exclusive offsets into pairs
-  const int *pairs;    // pair ids sorted by expert
-  int n_pairs;         // used when active == nullptr
+  const int4 *work;   // {expert, first, last, pairs[first]} per expert with work, then {-1,..};
+                      // nullptr: one matrix, pairs 0..n_pairs-1
+  const int *pairs;   // pair ids sorted by expert
+  int n_pairs;        // used when work == nullptr
+  int n_slots;        // records in `work`
   int rows, cols;
-  int x_div;  // activation row = pair / x_div
+  int x_div;   // activation row = pair / x_div
   int ks, rs;  // 1024-column slices, row sets; ks*rs waves per workgroup
+  int nt;      // tiles per chunk
   size_t expert_words, expert_scales;
 };
 
-// RI rows per half-wave per item, TT tokens per pass
-template <bool DUAL, int RI, int TT>
-__global__ void __launch_bounds__(1024) i4_gemv_k(I4Args a) {
-  extern __shared__ float lds[];  // [mats][RT][TT][ks] partials, then scale tiles
+constexpr int I4_RI = 2;  // rows per half-wave per tile
+
+// A workgroup of ks*rs waves takes chunks of nt tiles of RT = rs*4 rows of one expert.
+// Wave (s, rset): slice s of rows rset*4 .. rset*4+3 of each tile; its half-waves take
+// alternate rows.  Per chunk: the group scales of all its rows are staged in LDS once,
+// the packed words stream through two register buffers (tile i+1 is in flight while
+// tile i is computed), partial sums go to LDS and are summed over the slices at the end
+// of the chunk.  A last chunk that would run past the matrix is moved back to end at
+// the last row (the overlap is computed twice, with identical results).
+// KS_T > 0 fixes ks (and rs, nt) at compile time; 0 reads them from the arguments.
+template <bool DUAL, int TT, int KS_T, int MAXT, int WPE>
+__global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) i4_gemv_k(I4Args a) {
+  extern __shared__ float lds[];
+  constexpr int MATS = DUAL ? 2 : 1;
+  constexpr int RI = I4_RI;
+  constexpr int NV = RI * MATS * TT;
+  constexpr int NOUT = NV >= 4 ? NV / 4 : 1;
+  constexpr int SC_ITERS = 4;  // scale staging: 16-byte pieces per thread and matrix
+  const int ks = KS_T ? KS_T : a.ks;
+  const int rs = KS_T ? (KS_T >= 5 ? 1 : 8 / KS_T) : a.rs;
+  const int RT = rs * 2 * RI;
+  const int nt = KS_T ? (DUAL ? 32 : 64) / (KS_T >= 5 ? 4 : 32 / KS_T) : a.nt;
+  const int CR = RT * nt;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int l = lane & 31, h = lane >> 5;
-  const int s = wave % a.ks, rset = wave / a.ks;
-  const int RT = a.rs * 2 * RI;  // rows per item
-  const int MATS = DUAL ? 2 : 1;
-  const int groups = a.cols >> 5;
-  float *part = lds;
-  uint16_t *sc_lds = (uint16_t *)(lds + MATS * RT * TT * a.ks);  // [mats][RT][groups]
-  const int tiles = (a.rows + RT - 1) / RT;
-  const int n_active = a.active ? *a.n_active : 1;
-  const int n_items = n_active * tiles;
+  const int s = wave % ks, rset = wave / ks;
+  const int groups = ks * 32, row_words = ks * 128;
+  float *part = lds;                                              // [mats][CR][TT][ks]
+  uint16_t *sc_lds = (uint16_t *)(lds + MATS * CR * TT * ks);     // [mats][CR][groups]
+  const int cpe = (a.rows + CR - 1) / CR;                         // chunks per expert
+  const int n_chunks = (a.work ? a.n_slots : 1) * cpe;
+  const int row_lane = rset * RI * 2 + h;                         // row of this lane in tile 0, i = 0
+  const uint32_t w_off = (uint32_t)row_lane * (uint32_t)row_words + (uint32_t)(s * 32 + l) * 4;
+  const uint16_t *sc_lane = sc_lds + row_lane * groups + s * 32 + l;
   uint32_t magic;
   asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(magic));
 
-  for (int item = blockIdx.x; item < n_items; item += gridDim.x) {
-    const int ai = item / tiles, tile = item - ai * tiles;
-    const int e = a.active ? a.active[ai] : 0;
-    const int p_begin = a.active ? a.offsets[e] : 0;
-    const int p_end = a.active ? a.offsets[e + 1] : a.n_pairs;
-    const int r0 = tile * RT;
-    const uint32_t *pk[2] = {a.packed0 + (size_t)e * a.expert_words,
-                             DUAL ? a.packed1 + (size_t)e * a.expert_words : nullptr};
-    const uint16_t *scg[2] = {a.scale0 + (size_t)e * a.expert_scales,
-                              DUAL ? a.scale1 + (size_t)e * a.expert_scales : nullptr};
+  for (int chunk = blockIdx.x; chunk < n_chunks; chunk += gridDim.x) {
+    const int ai = chunk / cpe;
+    int c0 = (chunk - ai * cpe) * CR;
+    c0 = c0 + CR <= a.rows ? c0 : a.rows - CR;  // host guarantees rows >= CR
+    int4 wk = a.work ? a.work[ai] : make_int4(0, 0, a.n_pairs, 0);
+    const int e = __builtin_amdgcn_readfirstlane(wk.x);
+    if (e < 0) break;  // records with work come first
+    const int p_begin = __builtin_amdgcn_readfirstlane(wk.y), p_end = __builtin_amdgcn_readfirstlane(wk.z);
+    const int first_pair = __builtin_amdgcn_readfirstlane(wk.w);
+    const uint32_t *pk[2] = {a.packed0 + (size_t)e * a.expert_words + (size_t)c0 * row_words,
+                             DUAL ? a.packed1 + (size_t)e * a.expert_words + (size_t)c0 * row_words : nullptr};
 
-    // issue the weight loads of this item first
-    uint4 wv[MATS][RI];
-    int rows_i[RI];
-#pragma unroll
-    for (int i = 0; i < RI; ++i) {
-      int row = r0 + (rset * RI + i) * 2 + h;
-      rows_i[i] = row;
-      int row_c = row < a.rows ? row : a.rows - 1;
-#pragma unroll
-      for (int m = 0; m < MATS; ++m)
-        wv[m][i] = ld_stream(pk[m] + (size_t)row_c * (a.cols >> 3) + (size_t)(s * 32 + l) * 4);
-    }
-    // stage the scale rows of the tile in LDS (contiguous in memory)
-    {
-      const int rows_here = min(RT, a.rows - r0);
-      const int n16 = rows_here * groups / 8;  // uint4 chunks (groups is a multiple of 32)
-      for (int m = 0; m < MATS; ++m) {
-        const uint4 *src = (const uint4 *)(scg[m] + (size_t)r0 * groups);
-        uint4 *dst = (uint4 *)(sc_lds + (size_t)m * RT * groups);
-        for (int i = threadIdx.x; i < n16; i += blockDim.x) dst[i] = src[i];
-      }
-    }
-    __syncthreads();
-    float scf[MATS][RI];
-#pragma unroll
-    for (int i = 0; i < RI; ++i)
-#pragma unroll
-      for (int m = 0; m < MATS; ++m) {
-        int rt = min(rows_i[i], a.rows - 1) - r0;
-        scf[m][i] = kx_bf16_f32(sc_lds[((size_t)m * RT + rt) * groups + s * 32 + l]);
-      }
-
-    for (int pc = p_begin; pc < p_end; pc += TT) {
-      XGroup xg[TT];
-#pragma unroll
-      for (int t = 0; t < TT; ++t) {
-        int pi = min(pc + t, p_end - 1);
-        int pair = a.active ? a.pairs[pi] : pi;
-        load_xgroup(xg[t], a.x + (size_t)(pair / a.x_div) * a.cols + (size_t)(s * 32 + l) * 32);
-      }
+    auto load_tile = [&](uint4 (&buf)[MATS][RI], int tile) {
 #pragma unroll
       for (int i = 0; i < RI; ++i)
 #pragma unroll
-        for (int m = 0; m < MATS; ++m) {
-          I4Dec dec;
-          decode_words(dec, wv[m][i], magic);
+        for (int m = 0; m < MATS; ++m)
+          buf[m][i] = ld_stream(pk[m] + (size_t)((tile * RT + i * 2) * row_words) + w_off);
+    };
+
+    for (int pc = p_begin; pc < p_end; pc += TT) {
+      uint4 bufA[MATS][RI], bufB[MATS][RI];
+      load_tile(bufA, 0);
+      XGroup xg[TT];
+      uint4 xraw[TT][4];
 #pragma unroll
-          for (int t = 0; t < TT; ++t) {
-            float v = scf[m][i] * group_dot(dec, xg[t]);
-            v = half_wave_sum(v);
-            if (l == 0) part[((m * RT + (rset * RI + i) * 2 + h) * TT + t) * a.ks + s] = v;
-          }
+      for (int t = 0; t < TT; ++t) {
+        const int pi = min(pc + t, p_end - 1);
+        const int pair = !a.work ? pi : (pi == p_begin ? first_pair : a.pairs[pi]);
+        const uint4 *xp = (const uint4 *)(a.x + (size_t)(pair / a.x_div) * a.cols) + (s * 32 + l) * 4;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) xraw[t][w] = xp[w];
+      }
+      if (pc == p_begin) {
+        // group scales of the chunk: CR*groups contiguous bf16 per matrix; every load is
+        // issued before the first LDS write
+        const int n16 = CR * groups / 8;
+        uint4 stg[MATS][SC_ITERS];
+#pragma unroll
+        for (int m = 0; m < MATS; ++m) {
+          const uint4 *sg = (const uint4 *)((m ? a.scale1 : a.scale0) + (size_t)e * a.expert_scales + (size_t)c0 * groups);
+#pragma unroll
+          for (int it = 0; it < SC_ITERS; ++it) stg[m][it] = sg[min((int)(threadIdx.x + it * blockDim.x), n16 - 1)];
         }
-      __syncthreads();
-      // sequential sum over the slices, rounding and epilogue
-      for (int idx = threadIdx.x; idx < RT * TT; idx += blockDim.x) {
-        int rt = idx % RT, t = idx / RT;
-        int row = r0 + rt;
-        if (row < a.rows && pc + t < p_end) {
-          int pair = a.active ? a.pairs[pc + t] : pc + t;
-          const float *p0 = part + ((0 * RT + rt) * TT + t) * a.ks;
-          float y0 = p0[0];
-          for (int q = 1; q < a.ks; ++q) y0 += p0[q];
-          float res;
-          if (DUAL) {
-            const float *p1 = part + ((1 * RT + rt) * TT + t) * a.ks;
-            float y1 = p1[0];
-            for (int q = 1; q < a.ks; ++q) y1 += p1[q];
-            res = kx_swiglu(kx_bfround(y0), kx_bfround(y1));
-          } else {
-            res = y0;
+#pragma unroll
+        for (int m = 0; m < MATS; ++m) {
+          uint4 *dst = (uint4 *)(sc_lds + (size_t)m * CR * groups);
+#pragma unroll
+          for (int it = 0; it < SC_ITERS; ++it) {
+            const int i = threadIdx.x + it * blockDim.x;
+            if (i < n16) dst[i] = stg[m][it];
           }
-          a.out[(size_t)pair * a.rows + row] = kx_bf16_rne(res);
         }
       }
+#pragma unroll
+      for (int t = 0; t < TT; ++t) prep_xgroup(xg[t], xraw[t]);
+      __syncthreads();  // scales visible; previous pass has consumed `part`
+
+      auto compute_tile = [&](uint4 (&buf)[MATS][RI], int tile) {
+        float v[NV];
+#pragma unroll
+        for (int i = 0; i < RI; ++i)
+#pragma unroll
+          for (int m = 0; m < MATS; ++m) {
+            I4Dec dec;
+            decode_words(dec, buf[m][i], magic);
+            const float sc = kx_bf16_f32(sc_lane[(m * CR + tile * RT + i * 2) * groups]);
+#pragma unroll
+            for (int t = 0; t < TT; ++t) v[(i * MATS + m) * TT + t] = sc * group_dot(dec, xg[t]);
+          }
+        half_wave_reduce<NV>(v, l);
+        if ((l & 7) == 0) {
+#pragma unroll
+          for (int j = 0; j < NOUT; ++j) {
+            const int idx = half_wave_index<NV>(l, j);  // (i*MATS + m)*TT + t
+            const int t = idx % TT, m = (idx / TT) % MATS, i = idx / (TT * MATS);
+            const int rc = tile * RT + row_lane + i * 2;
+            if (NV >= 4 || (l & 8) == 0) part[((m * CR + rc) * TT + t) * ks + s] = v[j];
+          }
+        }
+      };
+
+      for (int tile = 0; tile < nt; tile += 2) {
+        if (tile + 1 < nt) load_tile(bufB, tile + 1);
+        compute_tile(bufA, tile);
+        if (tile + 2 < nt) load_tile(bufA, tile + 2);
+        if (tile + 1 < nt) compute_tile(bufB, tile + 1);
+      }
       __syncthreads();
+      // sequential sum over the slices, rounding and epilogue
+      for (int idx = threadIdx.x; idx < CR * TT; idx += blockDim.x) {
+        const int rc = idx % CR, t = idx / CR;
+        if (pc + t < p_end) {
+          const int pair = !a.work ? pc + t : a.pairs[pc + t];
+          const float *p0 = part + ((0 * CR + rc) * TT + t) * ks;
+          float y0 = p0[0];
+          for (int q = 1; q < ks; ++q) y0 += p0[q];
+          float res = y0;
+          if (DUAL) {
+            const float *p1 = part + ((1 * CR + rc) * TT + t) * ks;
+            float y1 = p1[0];
+            for (int q = 1; q < ks; ++q) y1 += p1[q];
+            res = kx_swiglu(kx_bfround(y0), kx_bfround(y1));
+          }
+          a.out[(size_t)pair * a.rows + c0 + rc] = kx_bf16_rne(res);
+        }
+      }
     }
+    __syncthreads();  // the next chunk overwrites the staged scales
   }
 }
 
 struct I4Launch {
-  int ks, rs, threads, rt;
+  int ks, rs, nt, threads, cr;
   size_t lds;
 };
 
-template <int RI>
 int plan(int cols, int rows, int mats, int tt, I4Launch &pl) {
   KX_REQUIRE(cols > 0 && cols % 1024 == 0, "kx_i4: cols=%d must be a positive multiple of 1024", cols);
-  KX_REQUIRE(rows > 0, "kx_i4: rows=%d must be positive", rows);
+  KX_REQUIRE(rows >= 4, "kx_i4: rows=%d must be at least 4", rows);
   pl.ks = cols / 1024;
   KX_REQUIRE(pl.ks <= 16, "kx_i4: cols=%d exceeds 16384", cols);
-  pl.rs = pl.ks >= 7 ? 1 : (8 / pl.ks);
+  pl.rs = pl.ks >= 5 ? 1 : (8 / pl.ks);
+  while (pl.rs > 1 && pl.rs * 4 > rows) pl.rs >>= 1;  // a tile must fit in the matrix
   pl.threads = pl.ks * pl.rs * 64;
-  pl.rt = pl.rs * 2 * RI;
-  pl.lds = (size_t)mats * pl.rt * tt * pl.ks * sizeof(float) + (size_t)mats * pl.rt * (cols / 32) * 2;
+  const int rt = pl.rs * 2 * I4_RI;
+  // chunk: 32 rows of both matrices (gate/up) or 64 rows of one
+  int nt = (mats == 2 ? 32 : 64) / rt;
+  nt = nt < 1 ? 1 : nt;
+  while (nt > 1 && rt * nt > rows) --nt;
+  pl.nt = nt;
+  pl.cr = rt * nt;
+  pl.lds = (size_t)mats * pl.cr * tt * pl.ks * sizeof(float) + (size_t)mats * pl.cr * (cols / 32) * 2;
+  KX_REQUIRE(pl.lds <= 160 * 1024, "kx_i4: cols=%d needs %zu bytes of LDS", cols, pl.lds);
+  // scale staging moves cr*groups/8 16-byte pieces per matrix with at most 4 per thread
+  KX_REQUIRE(pl.cr * (cols / 32) / 8 <= 4 * pl.threads, "kx_i4: chunk of %d rows x %d columns exceeds the scale staging", pl.cr, cols);
   return KX_OK;
+}
+
+template <bool DUAL, int KS_T, int MAXT>
+void launch_tt(const I4Args &a, int tt, dim3 g, dim3 b, size_t lds, hipStream_t st) {
+  // waves per SIMD the register budget is held to: two 7- or 8-wave workgroups per CU
+  // for one token per pass, fewer when more activations live in registers
+  if (tt == 1) hipLaunchKernelGGL((i4_gemv_k<DUAL, 1, KS_T, MAXT, 4>), g, b, lds, st, a);
+  else if (tt == 2) hipLaunchKernelGGL((i4_gemv_k<DUAL, 2, KS_T, MAXT, (MAXT > 512 ? 4 : 3)>), g, b, lds, st, a);
+  else hipLaunchKernelGGL((i4_gemv_k<DUAL, 4, KS_T, MAXT, (MAXT > 512 ? 4 : 2)>), g, b, lds, st, a);
 }
 
 }  // namespace
 
-// rows per half-wave per item
-#define KX_I4_RI 4
-
-// Launches the fused gate/up (DUAL) or single-matrix GEMV over a bucketed pair
-// list.  max_pairs_per_expert picks the tokens-per-pass variant.
+// Launches the fused gate/up (dual) or single-matrix GEMV over a bucketed pair list.
+// tt: tokens per pass (1, 2 or 4).  n_slots: records in `work`.
 int kx_i4_launch(bool dual, const uint32_t *packed0, const uint16_t *scale0, const uint32_t *packed1,
-                 const uint16_t *scale1, const uint16_t *x, uint16_t *out, const int *active,
-                 const int *n_active, const int *offsets, const int *pairs, int n_pairs, int rows,
-                 int cols, int x_div, size_t expert_words, size_t expert_scales, int tt, int grid,
-                 hipStream_t st) {
+                 const uint16_t *scale1, const uint16_t *x, uint16_t *out, const int4 *work,
+                 const int *pairs, int n_pairs, int rows, int cols, int x_div, size_t expert_words,
+                 size_t expert_scales, int tt, int n_slots, hipStream_t st) {
   I4Launch pl;
-  int rc = plan<KX_I4_RI>(cols, rows, dual ? 2 : 1, tt, pl);
+  int rc = plan(cols, rows, dual ? 2 : 1, tt, pl);
   if (rc) return rc;
   I4Args a;
   a.packed0 = packed0; a.scale0 = scale0; a.packed1 = packed1; a.scale1 = scale1;
-  a.x = x; a.out = out; a.active = active; a.n_active = n_active; a.offsets = offsets; a.pairs = pairs;
-  a.n_pairs = n_pairs; a.rows = rows; a.cols = cols; a.x_div = x_div; a.ks = pl.ks; a.rs = pl.rs;
+  a.x = x; a.out = out; a.work = work; a.pairs = pairs; a.n_pairs = n_pairs; a.n_slots = n_slots;
+  a.rows = rows; a.cols = cols; a.x_div = x_div; a.ks = pl.ks; a.rs = pl.rs; a.nt = pl.nt;
   a.expert_words = expert_words; a.expert_scales = expert_scales;
-  dim3 g(grid), b(pl.threads);
-  if (dual) {
-    if (tt == 1) hipLaunchKernelGGL((i4_gemv_k<true, KX_I4_RI, 1>), g, b, pl.lds, st, a);
-    else if (tt == 2) hipLaunchKernelGGL((i4_gemv_k<true, KX_I4_RI, 2>), g, b, pl.lds, st, a);
-    else hipLaunchKernelGGL((i4_gemv_k<true, KX_I4_RI, 4>), g, b, pl.lds, st, a);
+  long chunks = (long)n_slots * kx_cdiv(rows, pl.cr);
+  dim3 g((unsigned)(chunks < 4096 ? chunks : 4096)), b(pl.threads);
+  const bool full = pl.rs == (pl.ks >= 5 ? 1 : 8 / pl.ks) && pl.nt == (dual ? 32 : 64) / (pl.rs * 4);
+  if (full && pl.ks == 7) {        // Kimi-K2 gate/up: K = 7168
+    if (dual) launch_tt<true, 7, 448>(a, tt, g, b, pl.lds, st);
+    else launch_tt<false, 7, 448>(a, tt, g, b, pl.lds, st);
+  } else if (full && pl.ks == 2) {  // Kimi-K2 down: K = 2048
+    if (dual) launch_tt<true, 2, 512>(a, tt, g, b, pl.lds, st);
+    else launch_tt<false, 2, 512>(a, tt, g, b, pl.lds, st);
+  } else if (pl.threads <= 512) {
+    if (dual) launch_tt<true, 0, 512>(a, tt, g, b, pl.lds, st);
+    else launch_tt<false, 0, 512>(a, tt, g, b, pl.lds, st);
   } else {
-    if (tt == 1) hipLaunchKernelGGL((i4_gemv_k<false, KX_I4_RI, 1>), g, b, pl.lds, st, a);
-    else if (tt == 2) hipLaunchKernelGGL((i4_gemv_k<false, KX_I4_RI, 2>), g, b, pl.lds, st, a);
-    else hipLaunchKernelGGL((i4_gemv_k<false, KX_I4_RI, 4>), g, b, pl.lds, st, a);
+    if (dual) launch_tt<true, 0, 1024>(a, tt, g, b, pl.lds, st);
+    else launch_tt<false, 0, 1024>(a, tt, g, b, pl.lds, st);
   }
   KX_LAUNCH_CHECK();
   return KX_OK;
@@ -343,12 +452,7 @@ extern "C" int kx_i4_gemv(const void *d_packed, const void *d_scale, const void 
   KX_REQUIRE(d_packed && d_scale && d_x && d_y, "kx_i4_gemv: null pointer");
   KX_REQUIRE(tokens > 0, "kx_i4_gemv: tokens=%d must be positive", tokens);
   int tt = tokens >= 4 ? 4 : tokens >= 2 ? 2 : 1;
-  I4Launch pl;
-  int rc = plan<KX_I4_RI>(cols, rows, 1, tt, pl);
-  if (rc) return rc;
-  int tiles = kx_cdiv(rows, pl.rt);
-  int grid = tiles < 1024 ? tiles : 1024;
   return kx_i4_launch(false, (const uint32_t *)d_packed, (const uint16_t *)d_scale, nullptr, nullptr,
-                      (const uint16_t *)d_x, (uint16_t *)d_y, nullptr, nullptr, nullptr, nullptr, tokens, rows,
-                      cols, 1, 0, 0, tt, grid, kx_stream(stream));
+                      (const uint16_t *)d_x, (uint16_t *)d_y, nullptr, nullptr, tokens, rows, cols, 1, 0, 0, tt, 1,
+                      kx_stream(stream));
 }

@@ -25,7 +25,7 @@ struct kx_moe_workspace {
   int *counts;        // [E]
   int *offsets;       // [E+1]
   int *pairs;         // [T*topk]
-  int *active;        // [E]
+  int4 *work;         // [E] {expert, first, last, first pair}
   int *n_active;      // [1]
   uint16_t *mid;      // [T*topk, moe_inter]
   uint16_t *eout;     // [T*topk, hidden]
@@ -56,7 +56,7 @@ extern "C" int kx_moe_workspace_create(const kx_config *cfg, int32_t max_tokens,
   struct { void **p; size_t bytes; } allocs[] = {
       {(void **)&ws->logits, T * E * 4}, {(void **)&ws->ids, T * K * 2}, {(void **)&ws->weights, T * K * 4},
       {(void **)&ws->counts, E * 4}, {(void **)&ws->offsets, (E + 1) * 4}, {(void **)&ws->pairs, T * K * 4},
-      {(void **)&ws->active, E * 4}, {(void **)&ws->n_active, 4},
+      {(void **)&ws->work, E * 16}, {(void **)&ws->n_active, 4},
       {(void **)&ws->mid, T * K * (size_t)cfg->moe_inter * 2}, {(void **)&ws->eout, T * K * (size_t)cfg->hidden * 2},
       {(void **)&ws->smid, T * (size_t)cfg->shared_inter * 2}};
   for (auto &al : allocs) {
@@ -75,7 +75,7 @@ extern "C" int kx_moe_workspace_create(const kx_config *cfg, int32_t max_tokens,
 extern "C" int kx_moe_workspace_destroy(kx_moe_workspace *ws) {
   if (!ws) return KX_OK;
   void *ptrs[] = {ws->logits, ws->ids, ws->weights, ws->counts, ws->offsets, ws->pairs,
-                  ws->active, ws->n_active, ws->mid, ws->eout, ws->smid};
+                  ws->work, ws->n_active, ws->mid, ws->eout, ws->smid};
   for (void *p : ptrs)
     if (p) (void)hipFree(p);
   for (auto &e : ws->ev)
@@ -127,21 +127,21 @@ static int moe_layer(const kx_config *c, const kx_moe_weights *w, kx_moe_workspa
   if ((rc = kx_gemv_launch(KX_EPI_F32, g, st))) return rc;
   if ((rc = kx_router_topk_launch(ws->logits, (const float *)w->d_router_bias, ws->ids, ws->weights, tokens, E, K,
                                   c->routed_scale, st))) return rc;
-  if ((rc = kx_bucket_launch(ws->ids, tokens, E, K, ws->counts, ws->offsets, ws->pairs, ws->active, ws->n_active, st)))
+  if ((rc = kx_bucket_launch(ws->ids, tokens, E, K, ws->counts, ws->offsets, ws->pairs, ws->work, ws->n_active, st)))
     return rc;
   if (timed) KX_HIP(hipEventRecord(ws->ev[1], st));
   // 4 routed gate/up + SwiGLU
   const int tt = routed_tt(tokens, K, E);
-  const int grid = 1024;
+  const int max_active = (long)tokens * K < E ? tokens * K : E;
   if ((rc = kx_i4_launch(true, (const uint32_t *)w->d_gate_packed, (const uint16_t *)w->d_gate_scale,
-                         (const uint32_t *)w->d_up_packed, (const uint16_t *)w->d_up_scale, n, ws->mid, ws->active,
-                         ws->n_active, ws->offsets, ws->pairs, 0, I, H, K, (size_t)I * (H / 8), (size_t)I * (H / 32),
-                         tt, grid, st))) return rc;
+                         (const uint32_t *)w->d_up_packed, (const uint16_t *)w->d_up_scale, n, ws->mid, ws->work,
+                         ws->pairs, 0, I, H, K, (size_t)I * (H / 8), (size_t)I * (H / 32),
+                         tt, max_active, st))) return rc;
   if (timed) KX_HIP(hipEventRecord(ws->ev[2], st));
   // 5 routed down
   if ((rc = kx_i4_launch(false, (const uint32_t *)w->d_down_packed, (const uint16_t *)w->d_down_scale, nullptr, nullptr,
-                         ws->mid, ws->eout, ws->active, ws->n_active, ws->offsets, ws->pairs, 0, H, I, 1,
-                         (size_t)H * (I / 8), (size_t)H * (I / 32), tt, grid, st))) return rc;
+                         ws->mid, ws->eout, ws->work, ws->pairs, 0, H, I, 1,
+                         (size_t)H * (I / 8), (size_t)H * (I / 32), tt, max_active, st))) return rc;
   if (timed) KX_HIP(hipEventRecord(ws->ev[3], st));
   // 6 shared gate/up + SwiGLU
   KxGemvArgs s = {};

@@ -17,25 +17,44 @@
 
 namespace {
 
-constexpr int MAX_EPL = 16;  // experts per lane: up to 1024 experts
+// ---- wave-wide exact reductions through DPP (max / min have no rounding, any order) ----
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ int dpp_i(int v) {
+  return __builtin_amdgcn_update_dpp(v, v, CTRL, ROW_MASK, 0xf, false);
+}
+constexpr int DPP_XOR1 = 0xB1, DPP_XOR2 = 0x4E, DPP_HALF_MIRROR = 0x141, DPP_MIRROR = 0x140,
+              DPP_BCAST15 = 0x142, DPP_BCAST31 = 0x143;
 
+__device__ __forceinline__ float wave_max_f32(float v) {
+#define KX_STEP(C, M) v = fmaxf(v, __builtin_bit_cast(float, dpp_i<C, M>(__builtin_bit_cast(int, v))))
+  KX_STEP(DPP_XOR1, 0xf); KX_STEP(DPP_XOR2, 0xf); KX_STEP(DPP_HALF_MIRROR, 0xf); KX_STEP(DPP_MIRROR, 0xf);
+  KX_STEP(DPP_BCAST15, 0xa); KX_STEP(DPP_BCAST31, 0xc);
+#undef KX_STEP
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+__device__ __forceinline__ int wave_min_i32(int v) {
+#define KX_STEP(C, M) v = min(v, dpp_i<C, M>(v))
+  KX_STEP(DPP_XOR1, 0xf); KX_STEP(DPP_XOR2, 0xf); KX_STEP(DPP_HALF_MIRROR, 0xf); KX_STEP(DPP_MIRROR, 0xf);
+  KX_STEP(DPP_BCAST15, 0xa); KX_STEP(DPP_BCAST31, 0xc);
+#undef KX_STEP
+  return __builtin_amdgcn_readlane(v, 63);
+}
+
+// one wave per token; lane owns experts lane, lane+64, ... (EPL of them)
+template <int EPL>
 __global__ void __launch_bounds__(64) router_topk_k(const float *__restrict__ logits, const float *__restrict__ bias,
                                                     uint16_t *__restrict__ ids, float *__restrict__ weights, int E,
                                                     int topk, float routed_scale) {
   const int tok = blockIdx.x, lane = threadIdx.x;
   const float *lg = logits + (size_t)tok * E;
-  float sc[MAX_EPL], sel[MAX_EPL];
+  float sc[EPL], sel[EPL];
   const float NEG_INF = -__builtin_inff();
 #pragma unroll
-  for (int j = 0; j < MAX_EPL; ++j) {
+  for (int j = 0; j < EPL; ++j) {
     int e = lane + 64 * j;
-    if (e < E) {
-      sc[j] = kx_sigmoidf(lg[e]);
-      sel[j] = sc[j] + bias[e];
-    } else {
-      sc[j] = 0.0f;
-      sel[j] = NEG_INF;
-    }
+    float x = e < E ? lg[e] : 0.0f, b = e < E ? bias[e] : 0.0f;
+    sc[j] = kx_sigmoidf(x);
+    sel[j] = e < E ? sc[j] + b : NEG_INF;
   }
   float sum = 0.0f;
   float my_w = 0.0f;  // lane k keeps the k-th winner's score
@@ -43,56 +62,60 @@ __global__ void __launch_bounds__(64) router_topk_k(const float *__restrict__ lo
     float best = NEG_INF;
     int bi = 0x7fffffff;
 #pragma unroll
-    for (int j = 0; j < MAX_EPL; ++j)
+    for (int j = 0; j < EPL; ++j)
       if (sel[j] > best) { best = sel[j]; bi = lane + 64 * j; }
-    for (int m = 32; m; m >>= 1) {
-      float ov = __shfl_xor(best, m);
-      int oi = __shfl_xor(bi, m);
-      if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
-    }
-    if (bi == 0x7fffffff) bi = 0;  // every candidate was -inf: the reference keeps id 0
+    const float m = wave_max_f32(best);
+    int win = wave_min_i32(best == m ? bi : 0x7fffffff);
+    if (win == 0x7fffffff) win = 0;  // every candidate was -inf: the reference keeps id 0 (:391-393)
     float s_win = 0.0f;
 #pragma unroll
-    for (int j = 0; j < MAX_EPL; ++j)
-      if (bi == lane + 64 * j) { s_win = sc[j]; sel[j] = NEG_INF; }
-    s_win = __shfl(s_win, bi & 63);
+    for (int j = 0; j < EPL; ++j)
+      if (win == lane + 64 * j) { s_win = sc[j]; sel[j] = NEG_INF; }
+    s_win = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, s_win), win & 63));
     sum += s_win;
     if (lane == k) my_w = s_win;
-    if (lane == 0) ids[(size_t)tok * topk + k] = (uint16_t)bi;
+    if (lane == 0) ids[(size_t)tok * topk + k] = (uint16_t)win;
   }
   if (lane < topk) weights[(size_t)tok * topk + lane] = my_w / (sum + 1.0e-20f) * routed_scale;
 }
 
+// one workgroup, thread e owns expert e: count, exclusive scan, stable placement
 __global__ void __launch_bounds__(1024) bucket_k(const uint16_t *__restrict__ ids, int n_pairs, int E,
                                                  int *__restrict__ counts, int *__restrict__ offsets,
-                                                 int *__restrict__ pairs, int *__restrict__ active,
+                                                 int *__restrict__ pairs, int4 *__restrict__ work,
                                                  int *__restrict__ n_active) {
   __shared__ int s_cnt[1024];
-  __shared__ int s_off[1025];
-  const int e = threadIdx.x;
+  __shared__ int s_act[1024];
+  const int e = threadIdx.x, n = blockDim.x;
   int cnt = 0;
   if (e < E)
     for (int p = 0; p < n_pairs; ++p) cnt += (ids[p] == e) ? 1 : 0;
   s_cnt[e] = cnt;
+  s_act[e] = cnt > 0 ? 1 : 0;
   __syncthreads();
-  if (e == 0) {
-    int run = 0, na = 0;
-    for (int i = 0; i < E; ++i) {
-      s_off[i] = run;
-      if (s_cnt[i] > 0) active[na++] = i;
-      run += s_cnt[i];
-    }
-    s_off[E] = run;
-    offsets[E] = run;
-    *n_active = na;
+  for (int d = 1; d < n; d <<= 1) {  // inclusive Hillis-Steele scans of both arrays
+    int a = e >= d ? s_cnt[e - d] : 0, b = e >= d ? s_act[e - d] : 0;
+    __syncthreads();
+    s_cnt[e] += a;
+    s_act[e] += b;
+    __syncthreads();
   }
-  __syncthreads();
+  const int off = s_cnt[e] - cnt, slot = s_act[e] - (cnt > 0 ? 1 : 0), total_active = s_act[n - 1];
   if (e < E) {
     counts[e] = cnt;
-    offsets[e] = s_off[e];
-    int pos = s_off[e];
+    offsets[e] = off;
+    int pos = off, first = 0;
     for (int p = 0; p < n_pairs; ++p)
-      if (ids[p] == e) pairs[pos++] = p;
+      if (ids[p] == e) {
+        if (pos == off) first = p;
+        pairs[pos++] = p;
+      }
+    if (cnt > 0) work[slot] = make_int4(e, off, off + cnt, first);
+    if (e >= total_active) work[e] = make_int4(-1, 0, 0, 0);
+  }
+  if (e == 0) {
+    offsets[E] = s_cnt[n - 1];
+    *n_active = total_active;
   }
 }
 
@@ -101,21 +124,28 @@ __global__ void __launch_bounds__(1024) bucket_k(const uint16_t *__restrict__ id
 int kx_router_topk_launch(const float *logits, const float *bias, uint16_t *ids, float *weights, int tokens,
                           int experts, int topk, float routed_scale, hipStream_t st) {
   KX_REQUIRE(tokens > 0, "kx_router_topk: tokens=%d must be positive", tokens);
-  KX_REQUIRE(experts > 0 && experts <= 64 * MAX_EPL, "kx_router_topk: experts=%d outside [1, %d]", experts, 64 * MAX_EPL);
+  KX_REQUIRE(experts > 0 && experts <= 1024, "kx_router_topk: experts=%d outside [1, %d]", experts, 1024);
   KX_REQUIRE(topk > 0 && topk <= 64 && topk <= experts, "kx_router_topk: topk=%d outside [1, min(64, experts)]", topk);
-  hipLaunchKernelGGL(router_topk_k, dim3(tokens), dim3(64), 0, st, logits, bias, ids, weights, experts, topk,
-                     routed_scale);
+  const int epl = kx_cdiv(experts, 64);
+#define KX_RT(N) hipLaunchKernelGGL(router_topk_k<N>, dim3(tokens), dim3(64), 0, st, logits, bias, ids, weights, experts, topk, routed_scale)
+  if (epl <= 1) KX_RT(1);
+  else if (epl <= 2) KX_RT(2);
+  else if (epl <= 4) KX_RT(4);
+  else if (epl <= 6) KX_RT(6);
+  else if (epl <= 8) KX_RT(8);
+  else KX_RT(16);
+#undef KX_RT
   KX_LAUNCH_CHECK();
   return KX_OK;
 }
 
 int kx_bucket_launch(const uint16_t *ids, int tokens, int experts, int topk, int *counts, int *offsets, int *pairs,
-                     int *active, int *n_active, hipStream_t st) {
+                     int4 *work, int *n_active, hipStream_t st) {
   KX_REQUIRE(tokens > 0 && topk > 0, "kx_bucket: tokens=%d topk=%d must be positive", tokens, topk);
   KX_REQUIRE(experts > 0 && experts <= 1024, "kx_bucket: experts=%d outside [1, 1024]", experts);
   int threads = kx_cdiv(experts, 64) * 64;
   hipLaunchKernelGGL(bucket_k, dim3(1), dim3(threads), 0, st, ids, tokens * topk, experts, counts, offsets, pairs,
-                     active, n_active);
+                     work, n_active);
   KX_LAUNCH_CHECK();
   return KX_OK;
 }
@@ -128,8 +158,8 @@ extern "C" int kx_router_topk(const void *d_logits, const void *d_bias, void *d_
 }
 
 extern "C" int kx_bucket(const void *d_ids, int32_t tokens, int32_t experts, int32_t topk, void *d_counts,
-                         void *d_offsets, void *d_pairs, void *d_active, void *d_n_active, void *stream) {
-  KX_REQUIRE(d_ids && d_counts && d_offsets && d_pairs && d_active && d_n_active, "kx_bucket: null pointer");
+                         void *d_offsets, void *d_pairs, void *d_work, void *d_n_active, void *stream) {
+  KX_REQUIRE(d_ids && d_counts && d_offsets && d_pairs && d_work && d_n_active, "kx_bucket: null pointer");
   return kx_bucket_launch((const uint16_t *)d_ids, tokens, experts, topk, (int *)d_counts, (int *)d_offsets,
-                          (int *)d_pairs, (int *)d_active, (int *)d_n_active, kx_stream(stream));
+                          (int *)d_pairs, (int4 *)d_work, (int *)d_n_active, kx_stream(stream));
 }

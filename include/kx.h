@@ -117,12 +117,14 @@ int kx_gemv_bf16(const void *d_w, const void *d_x, void *d_y, int32_t rows, int3
  * kx_bucket     : token -> expert bucketing (the reference's host loop at
  *                 :845 for batch 1).  counts i32 [E], offsets i32 [E+1],
  *                 pairs i32 [T*topk] holding token*topk+slot sorted by
- *                 (expert, token, slot); active i32 [E] lists the experts
- *                 with at least one pair in ascending order, n_active i32 [1]. */
+ *                 (expert, token, slot); work i32 [E, 4] holds one record
+ *                 {expert, first, last, pairs[first]} per expert with at
+ *                 least one pair, in ascending expert order, followed by
+ *                 {-1, 0, 0, 0} records; n_active i32 [1] counts the former. */
 int kx_router_topk(const void *d_logits, const void *d_bias, void *d_ids, void *d_weights,
                    int32_t tokens, int32_t experts, int32_t topk, float routed_scale, void *stream);
 int kx_bucket(const void *d_ids, int32_t tokens, int32_t experts, int32_t topk, void *d_counts,
-              void *d_offsets, void *d_pairs, void *d_active, void *d_n_active, void *stream);
+              void *d_offsets, void *d_pairs, void *d_work, void *d_n_active, void *stream);
 
 /* ---- one routed-MoE decode layer (the `else` branch of run(), :835-877) ---
  * Weights of one layer.  Expert tensors hold all E experts back to back.    */

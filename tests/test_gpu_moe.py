@@ -65,7 +65,7 @@ def test_bucket_bit_exact(kxlib, ox, T, E, topk):
     wts = np.empty((T, topk), dtype=np.float32)
     ox.ox_router_topk(ptr(logits), ptr(bias), ptr(ids), ptr(wts), T, E, topk, 2.827, 1)
     di = dev(ids)
-    dc, do, dp, da, dn = DevBuf(E * 4), DevBuf((E + 1) * 4), DevBuf(T * topk * 4), DevBuf(E * 4), DevBuf(4)
+    dc, do, dp, da, dn = DevBuf(E * 4), DevBuf((E + 1) * 4), DevBuf(T * topk * 4), DevBuf(E * 16), DevBuf(4)
     check(kxlib.kx_bucket(di.ptr, T, E, topk, dc.ptr, do.ptr, dp.ptr, da.ptr, dn.ptr, None))
     check(kxlib.kx_sync(None))
     counts = np.empty(E, dtype=np.int32)
@@ -77,7 +77,12 @@ def test_bucket_bit_exact(kxlib, ox, T, E, topk):
     assert (do.to_numpy(np.int32, (E + 1,)) == offsets).all()
     assert (dp.to_numpy(np.int32, (T * topk,)) == pairs).all()
     assert dn.to_numpy(np.int32, (1,))[0] == na
-    assert (da.to_numpy(np.int32, (E,))[:na] == active[:na]).all()
+    work = da.to_numpy(np.int32, (E, 4))
+    act = active[:na]
+    assert (work[:na, 0] == act).all()
+    assert (work[:na, 1] == offsets[act]).all() and (work[:na, 2] == offsets[act + 1]).all()
+    assert (work[:na, 3] == pairs[offsets[act]]).all()
+    assert (work[na:] == np.array([-1, 0, 0, 0])).all()
 
 
 def _run_layer(kxlib, ox, H, I, SI, E, K, T, seed, flags=0):
