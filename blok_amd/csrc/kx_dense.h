@@ -12,7 +12,6 @@ enum {
   KX_EPI_ARGMAX = 5       // bf16-rounded logits as f32 for the argmax reduction
 };
 
-#define KX_GEMV_RI 4
 
 struct KxGemvArgs {
   const uint16_t *w0;  // bf16 [rows, cols]
@@ -22,7 +21,7 @@ struct KxGemvArgs {
   void *out;
   int out_stride;
   int rows, cols, tokens;
-  int nw, rs;  // set by kx_gemv_launch
+  int nw, rs, nt, epi;  // set by kx_gemv_launch
   // KX_EPI_MOE_COMBINE
   const uint16_t *expert_out;  // bf16 [tokens*topk, rows]
   const float *route_w;        // f32 [tokens, topk]

@@ -16,6 +16,7 @@
 #include "kx_common.h"
 #include "kx_dense.h"
 #include "kx_math.h"
+#include "kx_wave.h"
 
 namespace {
 
@@ -27,16 +28,6 @@ __device__ __forceinline__ uint4 ld_stream16(const uint16_t *p) {
 }
 __device__ __forceinline__ float bf_lo(uint32_t u) { return kx_bits_f32(u << 16); }
 __device__ __forceinline__ float bf_hi(uint32_t u) { return kx_bits_f32(u & 0xffff0000u); }
-
-__device__ __forceinline__ float wave_sum(float v) {
-  v += __shfl_xor(v, 32);
-  v += __shfl_xor(v, 16);
-  v += __shfl_xor(v, 8);
-  v += __shfl_xor(v, 4);
-  v += __shfl_xor(v, 2);
-  v += __shfl_xor(v, 1);
-  return v;
-}
 
 __device__ __forceinline__ void unpack8(float (&f)[8], uint4 u) {
   f[0] = bf_lo(u.x); f[1] = bf_hi(u.x); f[2] = bf_lo(u.y); f[3] = bf_hi(u.y);
@@ -59,8 +50,9 @@ __global__ void __launch_bounds__(256) rmsnorm_k(const uint16_t *__restrict__ x,
 #pragma unroll
     for (int e = 0; e < 8; ++e) v = __builtin_fmaf(f[e], f[e], v);
   }
-  v = wave_sum(v);
-  if ((threadIdx.x & 63) == 0) ws[threadIdx.x >> 6] = v;
+  float vv[1] = {v};
+  kxw::reduce<1, 64>(vv, threadIdx.x & 63);
+  if ((threadIdx.x & 63) == 0) ws[threadIdx.x >> 6] = vv[0];
   __syncthreads();
   float total = ((ws[0] + ws[1]) + ws[2]) + ws[3];
   float scale = kx_rsqrtf(total / (float)n + eps);
@@ -80,105 +72,133 @@ __global__ void __launch_bounds__(256) rmsnorm_k(const uint16_t *__restrict__ x,
 }
 
 // ---- GEMV -------------------------------------------------------------------------
-// RI rows per wave per item, TT tokens per pass, SPW slices per wave.
-template <int EPI, int RI, int TT, int SPW>
+// A workgroup of nw*rs waves takes chunks of nt tiles of RT = rs*RI rows.  Wave
+// (wslot, rset) owns the 512-column slices wslot, wslot+nw, ... of rows rset*RI ..
+// rset*RI+RI-1 of each tile, one slice per pass over the chunk.  The 16-byte weight
+// loads of tile i+1 are in flight while tile i is computed; partial sums per (row,
+// token, slice) go to LDS and are summed left to right over the slices at the end of
+// the chunk, where the epilogue runs.  A last chunk that would run past the matrix is
+// moved back to end at the last row (the overlap is computed twice, identically).
+template <int MATS, int RI, int TT>
 __global__ void __launch_bounds__(1024) gemv_bf16_k(KxGemvArgs a) {
-  extern __shared__ float part[];  // [mats][RT][TT][S]
-  constexpr int MATS = (EPI == KX_EPI_SWIGLU) ? 2 : 1;
+  extern __shared__ float part[];  // [mats][CR][tokens][S]
+  constexpr int NV = RI * MATS * TT;
+  constexpr int NOUT = kxw::reduce_out<NV, 64>();
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int S = a.cols >> 9;
-  const int wslot = wave % a.nw, rset = wave / a.nw;  // wave owns slices wslot*SPW .. +SPW-1
-  const int RT = a.rs * RI;
-  const int tiles = (a.rows + RT - 1) / RT;
-  const uint16_t *wm[2] = {a.w0, a.w1};
+  const int S = a.cols >> 9, T = a.tokens;
+  const int wslot = wave % a.nw, rset = wave / a.nw;
+  const int RT = a.rs * RI, CR = RT * a.nt;
+  const int n_chunks = (a.rows + CR - 1) / CR;
+  const bool x_once = T <= TT;  // activations stay in registers for the whole chunk
+  const uint16_t *wm[2] = {a.w0, MATS == 2 ? a.w1 : a.w0};
 
-  for (int tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
-    const int r0 = tile * RT;
-    uint4 wv[MATS][RI][SPW];
+  for (int chunk = blockIdx.x; chunk < n_chunks; chunk += gridDim.x) {
+    int c0 = chunk * CR;
+    c0 = c0 + CR <= a.rows ? c0 : a.rows - CR;  // host guarantees rows >= CR
+    for (int s = wslot; s < S; s += a.nw) {
+      const uint32_t col = (uint32_t)s * 512u + (uint32_t)lane * 8u;
+      const uint16_t *wb[2] = {wm[0] + (size_t)(c0 + rset * RI) * a.cols, wm[1] + (size_t)(c0 + rset * RI) * a.cols};
+      auto load_tile = [&](uint4 (&buf)[MATS][RI], int tile) {
 #pragma unroll
-    for (int i = 0; i < RI; ++i) {
-      int row = r0 + rset * RI + i;
-      int row_c = row < a.rows ? row : a.rows - 1;
+        for (int i = 0; i < RI; ++i)
 #pragma unroll
-      for (int m = 0; m < MATS; ++m)
+          for (int m = 0; m < MATS; ++m)
+            buf[m][i] = ld_stream16(wb[m] + (size_t)((tile * RT + i) * a.cols) + col);
+      };
+      float xs[TT][8];
+      auto load_x = [&](int t0) {
 #pragma unroll
-        for (int q = 0; q < SPW; ++q) {
-          int s = wslot * SPW + q;
-          int s_c = s < S ? s : S - 1;
-          wv[m][i][q] = ld_stream16(wm[m] + (size_t)row_c * a.cols + (size_t)s_c * 512 + lane * 8);
+        for (int t = 0; t < TT; ++t) {
+          const int tok = min(t0 + t, T - 1);
+          unpack8(xs[t], *(const uint4 *)(a.x + (size_t)tok * a.x_stride + col));
         }
-    }
-    for (int t0 = 0; t0 < a.tokens; t0 += TT) {
-      float xs[TT][SPW][8];
+      };
+      auto compute_tile = [&](uint4 (&buf)[MATS][RI], int tile) {
+        for (int t0 = 0; t0 < T; t0 += TT) {
+          if (!x_once) load_x(t0);
+          float v[NV];
 #pragma unroll
-      for (int t = 0; t < TT; ++t) {
-        int tok = min(t0 + t, a.tokens - 1);
+          for (int i = 0; i < RI; ++i)
 #pragma unroll
-        for (int q = 0; q < SPW; ++q) {
-          int s = wslot * SPW + q;
-          int s_c = s < S ? s : S - 1;
-          unpack8(xs[t][q], *(const uint4 *)(a.x + (size_t)tok * a.x_stride + (size_t)s_c * 512 + lane * 8));
-        }
-      }
+            for (int m = 0; m < MATS; ++m) {
+              float wf[8];
+              unpack8(wf, buf[m][i]);
 #pragma unroll
-      for (int i = 0; i < RI; ++i)
+              for (int t = 0; t < TT; ++t) {
+                float acc = 0.0f;
 #pragma unroll
-        for (int m = 0; m < MATS; ++m)
+                for (int e = 0; e < 8; ++e) acc = __builtin_fmaf(wf[e], xs[t][e], acc);
+                v[(i * MATS + m) * TT + t] = acc;
+              }
+            }
+          kxw::reduce<NV, 64>(v, lane);
+          if (kxw::reduce_writer<NV, 64>(lane)) {
 #pragma unroll
-          for (int q = 0; q < SPW; ++q) {
-            float wf[8];
-            unpack8(wf, wv[m][i][q]);
-            int s = wslot * SPW + q;
-#pragma unroll
-            for (int t = 0; t < TT; ++t) {
-              float acc = 0.0f;
-#pragma unroll
-              for (int e = 0; e < 8; ++e) acc = __builtin_fmaf(wf[e], xs[t][q][e], acc);
-              acc = wave_sum(acc);
-              if (lane == 0 && s < S) part[((m * RT + rset * RI + i) * TT + t) * S + s] = acc;
+            for (int j = 0; j < NOUT; ++j) {
+              const int idx = kxw::reduce_index<NV, 64>(lane, j);  // (i*MATS + m)*TT + t
+              const int t = idx % TT, m = (idx / TT) % MATS, i = idx / (TT * MATS);
+              const int rc = tile * RT + rset * RI + i, tok = t0 + t;
+              if (tok < T) part[((m * CR + rc) * T + tok) * S + s] = v[j];
             }
           }
-      __syncthreads();
-      for (int idx = threadIdx.x; idx < RT * TT; idx += blockDim.x) {
-        int rt = idx % RT, t = idx / RT;
-        int row = r0 + rt, tok = t0 + t;
-        if (row < a.rows && tok < a.tokens) {
-          const float *p0 = part + ((0 * RT + rt) * TT + t) * S;
-          float y0 = p0[0];
-          for (int q = 1; q < S; ++q) y0 += p0[q];
-          if (EPI == KX_EPI_BF16) {
-            ((uint16_t *)a.out)[(size_t)tok * a.out_stride + row] = kx_bf16_rne(y0);
-          } else if (EPI == KX_EPI_F32) {
-            ((float *)a.out)[(size_t)tok * a.out_stride + row] = y0;
-          } else if (EPI == KX_EPI_SWIGLU) {
-            const float *p1 = part + ((1 * RT + rt) * TT + t) * S;
-            float y1 = p1[0];
-            for (int q = 1; q < S; ++q) y1 += p1[q];
-            ((uint16_t *)a.out)[(size_t)tok * a.out_stride + row] =
-                kx_bf16_rne(kx_swiglu(kx_bfround(y0), kx_bfround(y1)));
-          } else if (EPI == KX_EPI_RESID) {
-            // x = bf(x + bf(y))  (add_k, :248-251)
-            uint16_t *xr = (uint16_t *)a.out + (size_t)tok * a.out_stride + row;
-            *xr = kx_bf16_rne(kx_bf16_f32(*xr) + kx_bfround(y0));
-          } else if (EPI == KX_EPI_MOE_COMBINE) {
-            // down = bf(sum_slot y_slot * w_slot) in slot order (:868,:871), then
-            // down = bf(down + bf(shared)) (:684), then x = bf(x + down) (:877)
-            float acc = 0.0f;
-            for (int k = 0; k < a.topk; ++k)
-              acc = __builtin_fmaf(kx_bf16_f32(a.expert_out[((size_t)tok * a.topk + k) * a.rows + row]),
-                                   a.route_w[(size_t)tok * a.topk + k], acc);
-            float down = kx_bfround(kx_bfround(acc) + kx_bfround(y0));
-            uint16_t *xr = (uint16_t *)a.out + (size_t)tok * a.out_stride + row;
-            if (a.flags & 1u) *xr = kx_bf16_rne(down);
-            else *xr = kx_bf16_rne(kx_bf16_f32(*xr) + down);
-          } else if (EPI == KX_EPI_ARGMAX) {
-            // bf16-rounded logits; the per-tile argmax is reduced by a second kernel
-            ((float *)a.out)[(size_t)tok * a.out_stride + row] = kx_bfround(y0);
-          }
         }
+      };
+      uint4 bufA[MATS][RI], bufB[MATS][RI];
+      load_tile(bufA, 0);
+      if (x_once) load_x(0);
+      for (int tile = 0; tile < a.nt; tile += 2) {
+        if (tile + 1 < a.nt) load_tile(bufB, tile + 1);
+        compute_tile(bufA, tile);
+        if (tile + 2 < a.nt) load_tile(bufA, tile + 2);
+        if (tile + 1 < a.nt) compute_tile(bufB, tile + 1);
       }
-      __syncthreads();
     }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < CR * T; idx += blockDim.x) {
+      const int rc = idx % CR, tok = idx / CR;
+      const int row = c0 + rc;
+      const float *p0 = part + ((0 * CR + rc) * T + tok) * S;
+      float y0 = p0[0];
+      for (int q = 1; q < S; ++q) y0 += p0[q];
+      float y1 = 0.0f;
+      if (MATS == 2) {
+        const float *p1 = part + ((1 * CR + rc) * T + tok) * S;
+        y1 = p1[0];
+        for (int q = 1; q < S; ++q) y1 += p1[q];
+      }
+      switch (a.epi) {
+        case KX_EPI_BF16:
+          ((uint16_t *)a.out)[(size_t)tok * a.out_stride + row] = kx_bf16_rne(y0);
+          break;
+        case KX_EPI_F32:
+          ((float *)a.out)[(size_t)tok * a.out_stride + row] = y0;
+          break;
+        case KX_EPI_SWIGLU:
+          ((uint16_t *)a.out)[(size_t)tok * a.out_stride + row] = kx_bf16_rne(kx_swiglu(kx_bfround(y0), kx_bfround(y1)));
+          break;
+        case KX_EPI_RESID: {  // x = bf(x + bf(y))  (add_k, :248-251)
+          uint16_t *xr = (uint16_t *)a.out + (size_t)tok * a.out_stride + row;
+          *xr = kx_bf16_rne(kx_bf16_f32(*xr) + kx_bfround(y0));
+          break;
+        }
+        case KX_EPI_MOE_COMBINE: {
+          // down = bf(sum_slot y_slot * w_slot) in slot order (:868,:871), then
+          // down = bf(down + bf(shared)) (:684), then x = bf(x + down) (:877)
+          float acc = 0.0f;
+          for (int k = 0; k < a.topk; ++k)
+            acc = __builtin_fmaf(kx_bf16_f32(a.expert_out[((size_t)tok * a.topk + k) * a.rows + row]),
+                                 a.route_w[(size_t)tok * a.topk + k], acc);
+          const float down = kx_bfround(kx_bfround(acc) + kx_bfround(y0));
+          uint16_t *xr = (uint16_t *)a.out + (size_t)tok * a.out_stride + row;
+          *xr = (a.flags & 1u) ? kx_bf16_rne(down) : kx_bf16_rne(kx_bf16_f32(*xr) + down);
+          break;
+        }
+        case KX_EPI_ARGMAX:  // bf16-rounded logits; a second kernel reduces them
+          ((float *)a.out)[(size_t)tok * a.out_stride + row] = kx_bfround(y0);
+          break;
+      }
+    }
+    __syncthreads();
   }
 }
 
@@ -208,46 +228,74 @@ __global__ void __launch_bounds__(1024) argmax_rows_k(const float *__restrict__ 
   }
 }
 
-template <int EPI, int RI, int TT>
-void launch_spw(const KxGemvArgs &a, int spw, dim3 g, dim3 b, size_t lds, hipStream_t st) {
-  if (spw == 1) hipLaunchKernelGGL((gemv_bf16_k<EPI, RI, TT, 1>), g, b, lds, st, a);
-  else if (spw == 2) hipLaunchKernelGGL((gemv_bf16_k<EPI, RI, TT, 2>), g, b, lds, st, a);
-  else hipLaunchKernelGGL((gemv_bf16_k<EPI, RI, TT, 3>), g, b, lds, st, a);
+template <int MATS, int RI>
+void launch_tt(const KxGemvArgs &a, int tt, dim3 g, dim3 b, size_t lds, hipStream_t st) {
+  if constexpr (RI * MATS * 4 <= 16) {
+    if (tt >= 4) { hipLaunchKernelGGL((gemv_bf16_k<MATS, RI, 4>), g, b, lds, st, a); return; }
+  }
+  if constexpr (RI * MATS * 2 <= 16) {
+    if (tt >= 2) { hipLaunchKernelGGL((gemv_bf16_k<MATS, RI, 2>), g, b, lds, st, a); return; }
+  }
+  hipLaunchKernelGGL((gemv_bf16_k<MATS, RI, 1>), g, b, lds, st, a);
 }
 
-template <int EPI>
-void launch_tt(const KxGemvArgs &a, int tt, int spw, dim3 g, dim3 b, size_t lds, hipStream_t st) {
-  if (tt == 1) launch_spw<EPI, KX_GEMV_RI, 1>(a, spw, g, b, lds, st);
-  else if (tt == 2) launch_spw<EPI, KX_GEMV_RI, 2>(a, spw, g, b, lds, st);
-  else launch_spw<EPI, KX_GEMV_RI, 4>(a, spw, g, b, lds, st);
+template <int MATS>
+void launch_ri(const KxGemvArgs &a, int ri, int tt, dim3 g, dim3 b, size_t lds, hipStream_t st) {
+  if constexpr (MATS == 1) {
+    if (ri == 4) { launch_tt<MATS, 4>(a, tt, g, b, lds, st); return; }
+  }
+  if (ri >= 2) launch_tt<MATS, 2>(a, tt, g, b, lds, st);
+  else launch_tt<MATS, 1>(a, tt, g, b, lds, st);
 }
 
 }  // namespace
 
+// Tokens are taken in blocks of at most 32 (LDS holds a partial per token and slice).
 int kx_gemv_launch(int epi, KxGemvArgs a, hipStream_t st) {
   KX_REQUIRE(a.cols > 0 && a.cols % 512 == 0, "kx_gemv: cols=%d must be a positive multiple of 512", a.cols);
   KX_REQUIRE(a.rows > 0 && a.tokens > 0, "kx_gemv: rows=%d tokens=%d must be positive", a.rows, a.tokens);
+  KX_REQUIRE(epi >= KX_EPI_BF16 && epi <= KX_EPI_ARGMAX, "kx_gemv: unknown epilogue %d", epi);
   const int S = a.cols / 512;
-  const int spw = (S + 15) / 16;
-  KX_REQUIRE(spw <= 3, "kx_gemv: cols=%d exceeds 24576", a.cols);
-  a.nw = (S + spw - 1) / spw;
-  a.rs = a.nw >= 8 ? 1 : 8 / a.nw;
-  const int tt = a.tokens >= 4 ? 4 : a.tokens >= 2 ? 2 : 1;
   const int mats = epi == KX_EPI_SWIGLU ? 2 : 1;
-  const int RT = a.rs * KX_GEMV_RI;
-  const size_t lds = (size_t)mats * RT * tt * S * sizeof(float);
-  const int tiles = kx_cdiv(a.rows, RT);
-  dim3 g(tiles < 2048 ? tiles : 2048), b(a.nw * a.rs * 64);
-  switch (epi) {
-    case KX_EPI_BF16: launch_tt<KX_EPI_BF16>(a, tt, spw, g, b, lds, st); break;
-    case KX_EPI_F32: launch_tt<KX_EPI_F32>(a, tt, spw, g, b, lds, st); break;
-    case KX_EPI_SWIGLU: launch_tt<KX_EPI_SWIGLU>(a, tt, spw, g, b, lds, st); break;
-    case KX_EPI_RESID: launch_tt<KX_EPI_RESID>(a, tt, spw, g, b, lds, st); break;
-    case KX_EPI_MOE_COMBINE: launch_tt<KX_EPI_MOE_COMBINE>(a, tt, spw, g, b, lds, st); break;
-    case KX_EPI_ARGMAX: launch_tt<KX_EPI_ARGMAX>(a, tt, spw, g, b, lds, st); break;
-    default: kx_set_error("kx_gemv: unknown epilogue %d", epi); return KX_ERR_ARG;
+  a.epi = epi;
+  // waves per workgroup: the largest divisor of S up to 8 (even slice counts per wave),
+  // times row sets to reach 8 waves
+  a.nw = 1;
+  for (int d = 2; d <= 8; ++d)
+    if (S % d == 0) a.nw = d;
+  a.rs = 8 / a.nw;
+  while (a.rs > 1 && a.rs > a.rows) a.rs >>= 1;
+  // rows per wave and tile, tiles per chunk: a few hundred chunks when the matrix allows
+  int ri = a.rows >= 2048 * a.rs ? 4 : a.rows >= 768 * a.rs ? 2 : 1;
+  while (ri > 1 && ri * a.rs > a.rows) ri >>= 1;
+  if (ri * mats > 4) ri = 4 / mats;
+  const int rt = a.rs * ri;
+  int nt = a.rows / (rt * 256);
+  nt = nt < 1 ? 1 : nt > 8 ? 8 : nt;
+  a.nt = nt;
+  const int CR = rt * nt;
+  const int all_tokens = a.tokens;
+  const uint16_t *x0 = a.x;
+  char *out0 = (char *)a.out;
+  const size_t out_elem = (epi == KX_EPI_F32 || epi == KX_EPI_ARGMAX) ? 4 : 2;
+  for (int t0 = 0; t0 < all_tokens; t0 += 32) {
+    a.tokens = all_tokens - t0 < 32 ? all_tokens - t0 : 32;
+    a.x = x0 + (size_t)t0 * a.x_stride;
+    a.out = out0 + (size_t)t0 * a.out_stride * out_elem;
+    KxGemvArgs b = a;
+    if (epi == KX_EPI_MOE_COMBINE) {
+      b.expert_out = a.expert_out + (size_t)t0 * a.topk * a.rows;
+      b.route_w = a.route_w + (size_t)t0 * a.topk;
+    }
+    const int tt = b.tokens >= 4 ? 4 : b.tokens >= 2 ? 2 : 1;
+    const size_t lds = (size_t)mats * CR * b.tokens * S * sizeof(float);
+    KX_REQUIRE(lds <= 160 * 1024, "kx_gemv: %zu bytes of LDS needed", lds);
+    const int chunks = kx_cdiv(a.rows, CR);
+    dim3 g(chunks < 4096 ? chunks : 4096), blk(a.nw * a.rs * 64);
+    if (mats == 2) launch_ri<2>(b, ri, tt, g, blk, lds, st);
+    else launch_ri<1>(b, ri, tt, g, blk, lds, st);
+    KX_LAUNCH_CHECK();
   }
-  KX_LAUNCH_CHECK();
   return KX_OK;
 }
 

@@ -22,12 +22,13 @@
 //    nibbles 0,2,4,6 and 1152 for nibbles 1,3,5,7 (x' = x/16 there);
 //  * the group scale is applied once per group: part = scale * acc;
 //  * reductions: xor-butterfly over the 32 lanes of the half-wave
-//    (16,8,4,2,1), then a sequential sum over the 1024-column slices.
+//    (16,8,4,2,1; see kx_wave.h), then a sequential sum over the 1024-column slices.
 //
 // All arithmetic is IEEE binary32 (fma, mul, add), so a scalar host program
 // that follows the same order reproduces the result bit for bit.
 #include "kx_common.h"
 #include "kx_math.h"
+#include "kx_wave.h"
 
 namespace {
 
@@ -128,64 +129,6 @@ __device__ __forceinline__ float group_dot(const I4Dec &d, const XGroup &g) {
   return acc;
 }
 
-// ---- half-wave (32 lane) reduction ---------------------------------------------------
-// Sums NV per-lane values over the 32 lanes of a half-wave with the xor-butterfly tree
-// (16, 8, 4, 2, 1).  Level 16 swaps rows between two registers (v_permlane16_swap), so
-// each lane keeps half of the values; level 8 does the same with a rotate-by-8 inside the
-// 16-lane row; levels 4, 2, 1 are DPP row shifts, valid in lanes that are multiples of 8.
-// The sums have the bits of a full butterfly because fp32 addition commutes.
-// On return, in lanes with (l & 7) == 0, v[0] is the total of value index
-//   (l >> 4) * NV/2 + ((l >> 3) & 1) * NV/4 + j   for the j-th survivor (j < NV/4, or the
-// single value when NV <= 2) -- see half_wave_index().
-__device__ __forceinline__ void swap_rows16(float &a, float &b) {
-  // rows 1,3 of a <-> rows 0,2 of b
-  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
-}
-template <int CTRL>
-__device__ __forceinline__ float dpp_f(float v) {
-  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
-}
-constexpr int DPP_ROW_SHL1 = 0x101, DPP_ROW_SHL2 = 0x102, DPP_ROW_SHL4 = 0x104, DPP_ROW_ROR8 = 0x128;
-
-// NV in {2, 4, 8, 16}: after the call v[0 .. NV/4-1] (NV >= 4) or v[0] (NV == 2) hold totals
-template <int NV>
-__device__ __forceinline__ void half_wave_reduce(float (&v)[NV], int l) {
-  static_assert(NV == 2 || NV == 4 || NV == 8 || NV == 16, "values per reduction");
-  // level 16: value i pairs with value i + NV/2
-#pragma unroll
-  for (int i = 0; i < NV / 2; ++i) {
-    swap_rows16(v[i], v[i + NV / 2]);
-    v[i] = v[i] + v[i + NV / 2];  // rows 0,2: value i; rows 1,3: value i + NV/2
-  }
-  if constexpr (NV >= 4) {
-    // level 8: value i pairs with value i + NV/4 (within the NV/2 this lane kept)
-    const bool hi = (l & 8) != 0;
-#pragma unroll
-    for (int i = 0; i < NV / 4; ++i) {
-      float send = hi ? v[i] : v[i + NV / 4];
-      float mine = hi ? v[i + NV / 4] : v[i];
-      v[i] = mine + dpp_f<DPP_ROW_ROR8>(send);
-    }
-#pragma unroll
-    for (int i = 0; i < NV / 4; ++i) {
-      v[i] = v[i] + dpp_f<DPP_ROW_SHL4>(v[i]);
-      v[i] = v[i] + dpp_f<DPP_ROW_SHL2>(v[i]);
-      v[i] = v[i] + dpp_f<DPP_ROW_SHL1>(v[i]);
-    }
-  } else {
-    v[0] = v[0] + dpp_f<DPP_ROW_ROR8>(v[0]);
-    v[0] = v[0] + dpp_f<DPP_ROW_SHL4>(v[0]);
-    v[0] = v[0] + dpp_f<DPP_ROW_SHL2>(v[0]);
-    v[0] = v[0] + dpp_f<DPP_ROW_SHL1>(v[0]);
-  }
-}
-// value index held in v[j] of lane l after half_wave_reduce<NV>
-template <int NV>
-__device__ __forceinline__ int half_wave_index(int l, int j) {
-  if constexpr (NV >= 4) return ((l >> 4) & 1) * (NV / 2) + ((l >> 3) & 1) * (NV / 4) + j;
-  else return (l >> 4) & 1;
-}
-
 struct I4Args {
   const uint32_t *packed0;
   const uint16_t *scale0;
@@ -221,7 +164,7 @@ __global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(WPE, 
   constexpr int MATS = DUAL ? 2 : 1;
   constexpr int RI = I4_RI;
   constexpr int NV = RI * MATS * TT;
-  constexpr int NOUT = NV >= 4 ? NV / 4 : 1;
+  constexpr int NOUT = kxw::reduce_out<NV, 32>();
   constexpr int SC_ITERS = 4;  // scale staging: 16-byte pieces per thread and matrix
   const int ks = KS_T ? KS_T : a.ks;
   const int rs = KS_T ? (KS_T >= 5 ? 1 : 8 / KS_T) : a.rs;
@@ -312,14 +255,14 @@ __global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(WPE, 
 #pragma unroll
             for (int t = 0; t < TT; ++t) v[(i * MATS + m) * TT + t] = sc * group_dot(dec, xg[t]);
           }
-        half_wave_reduce<NV>(v, l);
-        if ((l & 7) == 0) {
+        kxw::reduce<NV, 32>(v, lane);
+        if (kxw::reduce_writer<NV, 32>(lane)) {
 #pragma unroll
           for (int j = 0; j < NOUT; ++j) {
-            const int idx = half_wave_index<NV>(l, j);  // (i*MATS + m)*TT + t
+            const int idx = kxw::reduce_index<NV, 32>(lane, j);  // (i*MATS + m)*TT + t
             const int t = idx % TT, m = (idx / TT) % MATS, i = idx / (TT * MATS);
             const int rc = tile * RT + row_lane + i * 2;
-            if (NV >= 4 || (l & 8) == 0) part[((m * CR + rc) * TT + t) * ks + s] = v[j];
+            part[((m * CR + rc) * TT + t) * ks + s] = v[j];
           }
         }
       };

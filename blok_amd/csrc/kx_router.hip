@@ -14,31 +14,12 @@
 #include "kx_common.h"
 #include "kx_dense.h"
 #include "kx_math.h"
+#include "kx_wave.h"
 
 namespace {
 
-// ---- wave-wide exact reductions through DPP (max / min have no rounding, any order) ----
-template <int CTRL, int ROW_MASK = 0xf>
-__device__ __forceinline__ int dpp_i(int v) {
-  return __builtin_amdgcn_update_dpp(v, v, CTRL, ROW_MASK, 0xf, false);
-}
-constexpr int DPP_XOR1 = 0xB1, DPP_XOR2 = 0x4E, DPP_HALF_MIRROR = 0x141, DPP_MIRROR = 0x140,
-              DPP_BCAST15 = 0x142, DPP_BCAST31 = 0x143;
-
-__device__ __forceinline__ float wave_max_f32(float v) {
-#define KX_STEP(C, M) v = fmaxf(v, __builtin_bit_cast(float, dpp_i<C, M>(__builtin_bit_cast(int, v))))
-  KX_STEP(DPP_XOR1, 0xf); KX_STEP(DPP_XOR2, 0xf); KX_STEP(DPP_HALF_MIRROR, 0xf); KX_STEP(DPP_MIRROR, 0xf);
-  KX_STEP(DPP_BCAST15, 0xa); KX_STEP(DPP_BCAST31, 0xc);
-#undef KX_STEP
-  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
-}
-__device__ __forceinline__ int wave_min_i32(int v) {
-#define KX_STEP(C, M) v = min(v, dpp_i<C, M>(v))
-  KX_STEP(DPP_XOR1, 0xf); KX_STEP(DPP_XOR2, 0xf); KX_STEP(DPP_HALF_MIRROR, 0xf); KX_STEP(DPP_MIRROR, 0xf);
-  KX_STEP(DPP_BCAST15, 0xa); KX_STEP(DPP_BCAST31, 0xc);
-#undef KX_STEP
-  return __builtin_amdgcn_readlane(v, 63);
-}
+using kxw::wave_max_f32;
+using kxw::wave_min_i32;
 
 // one wave per token; lane owns experts lane, lane+64, ... (EPL of them)
 template <int EPL>
