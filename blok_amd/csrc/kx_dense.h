@@ -22,6 +22,10 @@ struct KxGemvArgs {
   int out_stride;
   int rows, cols, tokens;
   int nw, rs, nt, epi;  // set by kx_gemv_launch
+  // optional block structure (absorbed W_UV: one 128-row block per head inside kv_b):
+  // output rows [k*row_block, (k+1)*row_block) use weight rows k*w_block_stride + w_block_off + r
+  // and the activation row at x + k*x_block_stride.  row_block == 0: plain matrix.
+  int row_block, w_block_stride, w_block_off, x_block_stride;
   // KX_EPI_MOE_COMBINE
   const uint16_t *expert_out;  // bf16 [tokens*topk, rows]
   const float *route_w;        // f32 [tokens, topk]

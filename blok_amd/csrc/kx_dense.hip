@@ -78,7 +78,8 @@ __global__ void __launch_bounds__(256) rmsnorm_k(const uint16_t *__restrict__ x,
 // loads of tile i+1 are in flight while tile i is computed; partial sums per (row,
 // token, slice) go to LDS and are summed left to right over the slices at the end of
 // the chunk, where the epilogue runs.  A last chunk that would run past the matrix is
-// moved back to end at the last row (the overlap is computed twice, identically).
+// moved back to end at the last row; the rows it shares with the previous chunk are
+// computed twice but written once, by the previous chunk.
 template <int MATS, int RI, int TT>
 __global__ void __launch_bounds__(1024) gemv_bf16_k(KxGemvArgs a) {
   extern __shared__ float part[];  // [mats][CR][tokens][S]
@@ -97,7 +98,10 @@ __global__ void __launch_bounds__(1024) gemv_bf16_k(KxGemvArgs a) {
     c0 = c0 + CR <= a.rows ? c0 : a.rows - CR;  // host guarantees rows >= CR
     for (int s = wslot; s < S; s += a.nw) {
       const uint32_t col = (uint32_t)s * 512u + (uint32_t)lane * 8u;
-      const uint16_t *wb[2] = {wm[0] + (size_t)(c0 + rset * RI) * a.cols, wm[1] + (size_t)(c0 + rset * RI) * a.cols};
+      const int blk = a.row_block ? c0 / a.row_block : 0;
+      const int wrow0 = a.row_block ? blk * a.w_block_stride + a.w_block_off + (c0 - blk * a.row_block) : c0;
+      const uint16_t *xb = a.x + (size_t)blk * a.x_block_stride;
+      const uint16_t *wb[2] = {wm[0] + (size_t)(wrow0 + rset * RI) * a.cols, wm[1] + (size_t)(wrow0 + rset * RI) * a.cols};
       auto load_tile = [&](uint4 (&buf)[MATS][RI], int tile) {
 #pragma unroll
         for (int i = 0; i < RI; ++i)
@@ -110,7 +114,7 @@ __global__ void __launch_bounds__(1024) gemv_bf16_k(KxGemvArgs a) {
 #pragma unroll
         for (int t = 0; t < TT; ++t) {
           const int tok = min(t0 + t, T - 1);
-          unpack8(xs[t], *(const uint4 *)(a.x + (size_t)tok * a.x_stride + col));
+          unpack8(xs[t], *(const uint4 *)(xb + (size_t)tok * a.x_stride + col));
         }
       };
       auto compute_tile = [&](uint4 (&buf)[MATS][RI], int tile) {
@@ -157,6 +161,7 @@ __global__ void __launch_bounds__(1024) gemv_bf16_k(KxGemvArgs a) {
     for (int idx = threadIdx.x; idx < CR * T; idx += blockDim.x) {
       const int rc = idx % CR, tok = idx / CR;
       const int row = c0 + rc;
+      if (row < chunk * CR) continue;  // rows of a moved-back last chunk that the previous chunk owns
       const float *p0 = part + ((0 * CR + rc) * T + tok) * S;
       float y0 = p0[0];
       for (int q = 1; q < S; ++q) y0 += p0[q];
@@ -272,6 +277,10 @@ int kx_gemv_launch(int epi, KxGemvArgs a, hipStream_t st) {
   const int rt = a.rs * ri;
   int nt = a.rows / (rt * 256);
   nt = nt < 1 ? 1 : nt > 8 ? 8 : nt;
+  if (a.row_block) {  // a chunk must not straddle blocks
+    KX_REQUIRE(a.rows % a.row_block == 0 && a.row_block % rt == 0, "kx_gemv: row_block=%d does not fit tiles of %d rows", a.row_block, rt);
+    while (a.row_block % (rt * nt)) --nt;
+  }
   a.nt = nt;
   const int CR = rt * nt;
   const int all_tokens = a.tokens;

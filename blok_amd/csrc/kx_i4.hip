@@ -277,7 +277,7 @@ __global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(WPE, 
       // sequential sum over the slices, rounding and epilogue
       for (int idx = threadIdx.x; idx < CR * TT; idx += blockDim.x) {
         const int rc = idx % CR, t = idx / CR;
-        if (pc + t < p_end) {
+        if (pc + t < p_end && c0 + rc >= (chunk - ai * cpe) * CR) {  // a moved-back chunk skips the rows it shares
           const int pair = !a.work ? pc + t : a.pairs[pc + t];
           const float *p0 = part + ((0 * CR + rc) * TT + t) * ks;
           float y0 = p0[0];

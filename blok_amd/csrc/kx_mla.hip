@@ -1,0 +1,392 @@
+// kx_mla.hip -- MLA decode attention on the absorbed latent KV cache, with the
+// RMSNorm / RoPE steps that sit on its path.
+//
+// Reference: the attention half of run(), src/kimi_exec.cu:812-827 -- q_a/q_b and
+// kv_a/kv_b projections, rope_k (:346-357) with the YaRN frequencies (:325-344),
+// an expanded fp32 K/V cache on NVMe (:192-238) and tiled_attention (:692-716),
+// a three-pass softmax that streams every K tile three times.  Here the cache
+// holds what kv_a produced: per position the RMS-normed 512-d latent and the
+// rotated 64-d rope key (bf16, 1152 B instead of 81920 B), and the kv_b
+// projection is absorbed into the query and the output:
+//   q_lat[h] = bf(W_UK[h]^T q_nope[h])            (W_UK[h] = kv_b rows h*256 .. +127)
+//   s[t,h]   = bf(bf(q_lat[h].c_t + q_rope[h].k_rope_t) * rsqrt(192) * mscale^2)
+//   o_lat[h] = softmax(s)[t] . c_t ;  o[h] = bf(W_UV[h] o_lat[h])   (rows h*256+128 ..)
+// One pass over the cache with an online softmax; the sequence is cut into spans
+// of span_tiles 64-position tiles that run in parallel and are merged afterwards.
+//
+// Summation order (fixed; span_tiles depends on the sequence length only):
+//   score      one fma chain over the 576 cache columns, ascending
+//   tile       m = max s; p = exp(s - M'); z = xor-butterfly(64) of p;
+//              running: M' = max(M, m), a = exp(M - M'), Z = fma(Z, a, z),
+//              O[c] = (O[c] * a) then fma chain over the tile's positions of bf(p) * c_t[c]
+//   merge      M = max M_j; w_j = exp(M_j - M); Z = fma(Z_j, w_j, Z), O = fma(O_j, w_j, O)
+//              over spans ascending; o_lat = bf(O / Z)
+//   q_lat      eight chains over d = j, j+8, ... then ((0+1)+(2+3))+((4+5)+(6+7))
+#include <math.h>
+#include "kx_common.h"
+#include "kx_dense.h"
+#include "kx_math.h"
+#include "kx_mla.h"
+#include "kx_wave.h"
+
+// ---- host: YaRN frequencies, rope table, score scale ---------------------------------
+static float yarn_correction_dim(const kx_config *c, float rotations, float dim) {  // :325-327
+  volatile float two_pi = 2.0f * 3.14159265358979323846f;
+  return dim * logf(c->yarn_orig_ctx / (rotations * two_pi)) / (2.0f * logf(c->rope_theta));
+}
+static float yarn_inv_freq(const kx_config *c, int pair) {  // :334-344
+  const float dim = (float)c->qk_rope;
+  const float freq_extra = powf(c->rope_theta, -2.0f * (float)pair / dim);
+  const float freq_inter = freq_extra / c->yarn_factor;
+  float low = floorf(yarn_correction_dim(c, c->yarn_beta_fast, dim));
+  float high = ceilf(yarn_correction_dim(c, c->yarn_beta_slow, dim));
+  low = fmaxf(low, 0.0f);
+  high = fminf(high, dim - 1.0f);
+  if (low == high) high += 0.001f;  // :330
+  const float ramp = fminf(1.0f, fmaxf(0.0f, ((float)pair - low) / (high - low)));
+  const float mask = 1.0f - ramp;
+  return freq_inter * (1.0f - mask) + freq_extra * mask;
+}
+
+extern "C" int kx_rope_table(const kx_config *cfg, int32_t pos0, int32_t n, uint16_t *h_out) {
+  KX_REQUIRE(cfg && h_out, "kx_rope_table: null argument");
+  KX_REQUIRE(cfg->qk_rope > 0 && cfg->qk_rope % 2 == 0 && n >= 0 && pos0 >= 0, "kx_rope_table: bad shape");
+  const int half = cfg->qk_rope / 2;
+  for (int p = 0; p < half; ++p) {
+    const float freq = yarn_inv_freq(cfg, p);
+    for (int i = 0; i < n; ++i) {
+      const float ang = (float)(pos0 + i) * freq;  // :351, int * float
+      h_out[(size_t)i * cfg->qk_rope + p] = kx_bf16_rne(cosf(ang));
+      h_out[(size_t)i * cfg->qk_rope + half + p] = kx_bf16_rne(sinf(ang));
+    }
+  }
+  return KX_OK;
+}
+
+extern "C" int kx_softmax_scale(const kx_config *cfg, float *rs, float *mscale) {
+  KX_REQUIRE(cfg && rs && mscale, "kx_softmax_scale: null argument");
+  *rs = kx_rsqrtf((float)(cfg->qk_nope + cfg->qk_rope));
+  *mscale = 0.1f * cfg->yarn_mscale_all_dim * logf(cfg->yarn_factor) + 1.0f;  // :428
+  return KX_OK;
+}
+
+int kx_mla_span_tiles(int seq) {
+  int tiles = (seq + 63) / 64, st = 1;
+  while (tiles > 64 * st) st *= 2;
+  return st;
+}
+
+namespace {
+
+__device__ __forceinline__ float bf_lo(uint32_t u) { return kx_bits_f32(u << 16); }
+__device__ __forceinline__ float bf_hi(uint32_t u) { return kx_bits_f32(u & 0xffff0000u); }
+__device__ __forceinline__ void unpack8(float (&f)[8], uint4 u) {
+  f[0] = bf_lo(u.x); f[1] = bf_hi(u.x); f[2] = bf_lo(u.y); f[3] = bf_hi(u.y);
+  f[4] = bf_lo(u.z); f[5] = bf_hi(u.z); f[6] = bf_lo(u.w); f[7] = bf_hi(u.w);
+}
+
+// RMSNorm of one row by a 256-thread workgroup; the schedule of rmsnorm_k (kx_dense.hip)
+__device__ __forceinline__ void rmsnorm_block(const uint16_t *xr, const uint16_t *w, uint16_t *yr, int n, float eps,
+                                              float *ws /* 4 floats of LDS */) {
+  const int chunks = n >> 3;
+  float v = 0.0f;
+  for (int c = threadIdx.x; c < chunks; c += 256) {
+    float f[8];
+    unpack8(f, ((const uint4 *)xr)[c]);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v = __builtin_fmaf(f[e], f[e], v);
+  }
+  float vv[1] = {v};
+  kxw::reduce<1, 64>(vv, threadIdx.x & 63);
+  __syncthreads();  // ws may still be read from a previous call
+  if ((threadIdx.x & 63) == 0) ws[threadIdx.x >> 6] = vv[0];
+  __syncthreads();
+  const float total = ((ws[0] + ws[1]) + ws[2]) + ws[3];
+  const float scale = kx_rsqrtf(total / (float)n + eps);
+  for (int c = threadIdx.x; c < chunks; c += 256) {
+    float f[8], g[8];
+    unpack8(f, ((const uint4 *)xr)[c]);
+    unpack8(g, ((const uint4 *)w)[c]);
+    uint32_t o[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      uint32_t a = kx_bf16_rne(kx_bfround(f[2 * e] * scale) * g[2 * e]);
+      uint32_t b = kx_bf16_rne(kx_bfround(f[2 * e + 1] * scale) * g[2 * e + 1]);
+      o[e] = a | (b << 16);
+    }
+    ((uint4 *)yr)[c] = make_uint4(o[0], o[1], o[2], o[3]);
+  }
+}
+
+// interleaved-pair rotation of rope_k (:352-356): reads (2p, 2p+1), writes (p, half+p)
+__device__ __forceinline__ void rope_pair(float x0, float x1, float c, float s, float &y_lo, float &y_hi) {
+  y_lo = kx_bfround(kx_bfround(x0 * c) - kx_bfround(x1 * s));
+  y_hi = kx_bfround(kx_bfround(x1 * c) + kx_bfround(x0 * s));
+}
+
+// After the fused q_a / kv_a projection: q_a RMSNorm (:814), kv_a RMSNorm on the latent
+// part only (:817), RoPE of the shared rope key (:820-823), write of the cache row (:824).
+// qkv bf16 [T][q_rank + kv_rank + rope]; one workgroup per token (= sequence).
+__global__ void __launch_bounds__(256) kv_finish_k(const uint16_t *__restrict__ qkv, const uint16_t *__restrict__ w_qa_ln,
+                                                   const uint16_t *__restrict__ w_kv_ln, const uint16_t *__restrict__ rope_row,
+                                                   uint16_t *__restrict__ qa_out, uint16_t *__restrict__ cache, int q_rank,
+                                                   int kv_rank, int rope, size_t seq_stride, int pos, float eps) {
+  __shared__ float ws[4];
+  const int t = blockIdx.x, kva = kv_rank + rope;
+  const uint16_t *row = qkv + (size_t)t * (q_rank + kva);
+  uint16_t *crow = cache + (size_t)t * seq_stride + (size_t)pos * kva;
+  rmsnorm_block(row, w_qa_ln, qa_out + (size_t)t * q_rank, q_rank, eps, ws);
+  rmsnorm_block(row + q_rank, w_kv_ln, crow, kv_rank, eps, ws);
+  const int half = rope >> 1;
+  if ((int)threadIdx.x < half) {
+    const int p = threadIdx.x;
+    const uint16_t *kr = row + q_rank + kv_rank;
+    float lo, hi;
+    rope_pair(kx_bf16_f32(kr[2 * p]), kx_bf16_f32(kr[2 * p + 1]), kx_bf16_f32(rope_row[p]), kx_bf16_f32(rope_row[half + p]),
+              lo, hi);
+    crow[kv_rank + p] = kx_bf16_rne(lo);
+    crow[kv_rank + half + p] = kx_bf16_rne(hi);
+  }
+}
+
+// q_abs[t][h] = (bf(W_UK[h]^T q_nope[h]) | rope(q_rope[h])) as f32.  Grid (heads, T), 8 waves:
+// wave j runs the chain over d = j, j+8, ...; lane owns 8 latent columns.
+__global__ void __launch_bounds__(512) q_absorb_k(const uint16_t *__restrict__ q, const uint16_t *__restrict__ kvb,
+                                                  const uint16_t *__restrict__ rope_row, float *__restrict__ qabs,
+                                                  int heads, int nope, int rope, int v_head, int kv_rank) {
+  extern __shared__ float part[];  // [8][kv_rank]
+  const int h = blockIdx.x, t = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int qk = nope + rope, kva = kv_rank + rope;
+  const uint16_t *qh = q + ((size_t)t * heads + h) * qk;
+  const uint16_t *wuk = kvb + (size_t)h * (nope + v_head) * kv_rank;
+  float *out = qabs + ((size_t)t * heads + h) * kva;
+  for (int c0 = lane * 8; c0 < kv_rank; c0 += 512) {
+    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int d = wave; d < nope; d += 8) {
+      float wf[8];
+      unpack8(wf, *(const uint4 *)(wuk + (size_t)d * kv_rank + c0));
+      const float qd = kx_bf16_f32(qh[d]);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(wf[e], qd, acc[e]);
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) part[wave * kv_rank + c0 + e] = acc[e];
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < kv_rank; c += blockDim.x) {
+    const float *p = part + c;
+    const float s = ((p[0] + p[kv_rank]) + (p[2 * kv_rank] + p[3 * kv_rank])) +
+                    ((p[4 * kv_rank] + p[5 * kv_rank]) + (p[6 * kv_rank] + p[7 * kv_rank]));
+    out[c] = kx_bfround(s);
+  }
+  const int half = rope >> 1;
+  if ((int)threadIdx.x < half) {
+    const int p = threadIdx.x;
+    float lo, hi;
+    rope_pair(kx_bf16_f32(qh[nope + 2 * p]), kx_bf16_f32(qh[nope + 2 * p + 1]), kx_bf16_f32(rope_row[p]),
+              kx_bf16_f32(rope_row[half + p]), lo, hi);
+    out[kv_rank + p] = lo;
+    out[kv_rank + half + p] = hi;
+  }
+}
+
+struct MlaArgs {
+  const uint16_t *cache;  // bf16 [B][seq_stride/kva positions][kva]
+  const float *qabs;      // f32 [B][heads][kva]
+  float *pm, *pz, *po;    // partials [B][spans][heads], same, [B][spans][heads][kv_rank]
+  int heads, seq, span_tiles, spans;
+  size_t seq_stride;      // elements between sequences in the cache
+  float rs, mscale;
+};
+
+// kv_rank 512, rope 64 (the Kimi-K2 latent layout).  HG heads per wave, 4 waves per workgroup.
+// grid (spans, heads / (4*HG), B).
+template <int HG>
+__global__ void __launch_bounds__(256) mla_partial_k(MlaArgs a) {
+  constexpr int R = 512, KVA = 576;
+  __shared__ float p_lds[4][HG][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int span = blockIdx.x, b = blockIdx.z;
+  const int h0 = (blockIdx.y * 4 + wave) * HG;
+  const uint16_t *cache = a.cache + (size_t)b * a.seq_stride;
+  const float *q = a.qabs + ((size_t)b * a.heads + h0) * KVA;
+  const int tiles = (a.seq + 63) >> 6;
+  const int tile_end = min(tiles, (span + 1) * a.span_tiles);
+  float M[HG], Z[HG], O[HG][8];
+#pragma unroll
+  for (int h = 0; h < HG; ++h) {
+    M[h] = -__builtin_inff();
+    Z[h] = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) O[h][e] = 0.0f;
+  }
+  for (int tile = span * a.span_tiles; tile < tile_end; ++tile) {
+    const int t0 = tile << 6, n = min(64, a.seq - t0);
+    // scores: lane = position, one fma chain over the 576 columns per head
+    const uint16_t *row = cache + (size_t)(t0 + min(lane, n - 1)) * KVA;
+    float acc[HG];
+#pragma unroll
+    for (int h = 0; h < HG; ++h) acc[h] = 0.0f;
+    for (int j = 0; j < KVA / 8; ++j) {
+      float cf[8];
+      unpack8(cf, ((const uint4 *)row)[j]);
+#pragma unroll
+      for (int h = 0; h < HG; ++h) {
+        const float *qh = q + h * KVA + j * 8;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[h] = __builtin_fmaf(cf[e], qh[e], acc[h]);
+      }
+    }
+    float alpha[HG];
+#pragma unroll
+    for (int h = 0; h < HG; ++h) {
+      float s = kx_bfround(kx_bfround(acc[h]) * a.rs * a.mscale * a.mscale);  // :429
+      if (lane >= n) s = -__builtin_inff();
+      const float mt = kxw::wave_max_f32(s);
+      const float Mn = fmaxf(M[h], mt);
+      alpha[h] = kx_expf(M[h] - Mn);
+      const float p = lane < n ? kx_expf(s - Mn) : 0.0f;
+      float z[1] = {p};
+      kxw::reduce<1, 64>(z, lane);
+      const float zt = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, z[0])));
+      Z[h] = __builtin_fmaf(Z[h], alpha[h], zt);
+      M[h] = Mn;
+      p_lds[wave][h][lane] = kx_bfround(p);
+    }
+    __syncthreads();
+    // PV: lane = 8 latent columns, positions in order
+#pragma unroll
+    for (int h = 0; h < HG; ++h)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) O[h][e] = O[h][e] * alpha[h];
+    const uint16_t *col = cache + (size_t)t0 * KVA + lane * 8;
+    for (int t = 0; t < n; ++t) {
+      float cf[8];
+      unpack8(cf, *(const uint4 *)(col + (size_t)t * KVA));
+#pragma unroll
+      for (int h = 0; h < HG; ++h) {
+        const float p = p_lds[wave][h][t];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) O[h][e] = __builtin_fmaf(p, cf[e], O[h][e]);
+      }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int h = 0; h < HG; ++h) {
+    const size_t idx = ((size_t)b * a.spans + span) * a.heads + h0 + h;
+    if (lane == 0) { a.pm[idx] = M[h]; a.pz[idx] = Z[h]; }
+    float4 *o = (float4 *)(a.po + idx * R + lane * 8);
+    o[0] = make_float4(O[h][0], O[h][1], O[h][2], O[h][3]);
+    o[1] = make_float4(O[h][4], O[h][5], O[h][6], O[h][7]);
+  }
+}
+
+// merge of the spans; grid (heads, B), one wave, lane = 8 latent columns
+__global__ void __launch_bounds__(64) mla_combine_k(const float *__restrict__ pm, const float *__restrict__ pz,
+                                                    const float *__restrict__ po, uint16_t *__restrict__ o_lat, int heads,
+                                                    int spans) {
+  constexpr int R = 512;
+  const int h = blockIdx.x, b = blockIdx.y, lane = threadIdx.x;
+  float M = -__builtin_inff();
+  for (int j = 0; j < spans; ++j) M = fmaxf(M, pm[((size_t)b * spans + j) * heads + h]);
+  float Z = 0.0f, O[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int j = 0; j < spans; ++j) {
+    const size_t idx = ((size_t)b * spans + j) * heads + h;
+    const float w = kx_expf(pm[idx] - M);
+    Z = __builtin_fmaf(pz[idx], w, Z);
+    const float4 *o = (const float4 *)(po + idx * R + lane * 8);
+    const float4 o0 = o[0], o1 = o[1];
+    O[0] = __builtin_fmaf(o0.x, w, O[0]); O[1] = __builtin_fmaf(o0.y, w, O[1]);
+    O[2] = __builtin_fmaf(o0.z, w, O[2]); O[3] = __builtin_fmaf(o0.w, w, O[3]);
+    O[4] = __builtin_fmaf(o1.x, w, O[4]); O[5] = __builtin_fmaf(o1.y, w, O[5]);
+    O[6] = __builtin_fmaf(o1.z, w, O[6]); O[7] = __builtin_fmaf(o1.w, w, O[7]);
+  }
+  uint32_t r[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+    r[e] = (uint32_t)kx_bf16_rne(O[2 * e] / Z) | ((uint32_t)kx_bf16_rne(O[2 * e + 1] / Z) << 16);
+  *(uint4 *)(o_lat + ((size_t)b * heads + h) * R + lane * 8) = make_uint4(r[0], r[1], r[2], r[3]);
+}
+
+}  // namespace
+
+int kx_kv_finish_launch(const uint16_t *qkv, const uint16_t *w_qa_ln, const uint16_t *w_kv_ln, const uint16_t *rope_row,
+                        uint16_t *qa_out, uint16_t *cache, int tokens, int q_rank, int kv_rank, int rope,
+                        size_t seq_stride, int pos, float eps, hipStream_t st) {
+  KX_REQUIRE(q_rank % 8 == 0 && kv_rank % 8 == 0 && rope % 2 == 0 && rope / 2 <= 256, "kx_kv_finish: bad shape");
+  hipLaunchKernelGGL(kv_finish_k, dim3(tokens), dim3(256), 0, st, qkv, w_qa_ln, w_kv_ln, rope_row, qa_out, cache, q_rank,
+                     kv_rank, rope, seq_stride, pos, eps);
+  KX_LAUNCH_CHECK();
+  return KX_OK;
+}
+
+int kx_q_absorb_launch(const uint16_t *q, const uint16_t *kvb, const uint16_t *rope_row, float *qabs, int tokens,
+                       int heads, int nope, int rope, int v_head, int kv_rank, hipStream_t st) {
+  KX_REQUIRE(kv_rank % 8 == 0 && rope % 2 == 0 && rope / 2 <= 512, "kx_q_absorb: bad shape");
+  hipLaunchKernelGGL(q_absorb_k, dim3(heads, tokens), dim3(512), (size_t)8 * kv_rank * sizeof(float), st, q, kvb, rope_row,
+                     qabs, heads, nope, rope, v_head, kv_rank);
+  KX_LAUNCH_CHECK();
+  return KX_OK;
+}
+
+size_t kx_mla_partial_floats(int batch, int heads, int kv_rank, int max_seq) {
+  const int tiles = (max_seq + 63) / 64, st = kx_mla_span_tiles(max_seq);
+  int spans = (tiles + st - 1) / st;
+  if (spans < 64) spans = tiles < 64 ? tiles : 64;  // shorter sequences use up to 64 spans
+  return (size_t)batch * spans * heads * (kv_rank + 2);
+}
+
+int kx_mla_attend_launch(const kx_config *c, const uint16_t *cache, size_t seq_stride, const float *qabs, float *partial,
+                         uint16_t *o_lat, int batch, int seq, hipStream_t st) {
+  KX_REQUIRE(c->kv_rank == 512 && c->qk_rope == 64, "kx_mla: the attention kernel is built for kv_rank 512, qk_rope 64 (got %d, %d)",
+             c->kv_rank, c->qk_rope);
+  KX_REQUIRE(c->heads % 4 == 0, "kx_mla: heads=%d must be a multiple of 4", c->heads);
+  KX_REQUIRE(batch > 0 && seq > 0, "kx_mla: batch=%d seq=%d must be positive", batch, seq);
+  MlaArgs a;
+  a.cache = cache; a.qabs = qabs; a.heads = c->heads; a.seq = seq; a.seq_stride = seq_stride;
+  a.span_tiles = kx_mla_span_tiles(seq);
+  const int tiles = (seq + 63) / 64;
+  a.spans = (tiles + a.span_tiles - 1) / a.span_tiles;
+  const size_t n = (size_t)batch * a.spans * c->heads;
+  a.pm = partial; a.pz = partial + n; a.po = partial + 2 * n;
+  float rs, ms;
+  kx_softmax_scale(c, &rs, &ms);
+  a.rs = rs; a.mscale = ms;
+  // heads per wave: enough waves to fill the chip, as few as possible otherwise
+  const long waves1 = (long)batch * a.spans * c->heads;  // waves at one head per wave
+  int hg = 1;
+  while (hg < 8 && c->heads % (4 * hg * 2) == 0 && waves1 / (hg * 2) >= 4096) hg *= 2;
+  dim3 g(a.spans, c->heads / (4 * hg), batch), b(256);
+  if (hg == 1) hipLaunchKernelGGL(mla_partial_k<1>, g, b, 0, st, a);
+  else if (hg == 2) hipLaunchKernelGGL(mla_partial_k<2>, g, b, 0, st, a);
+  else if (hg == 4) hipLaunchKernelGGL(mla_partial_k<4>, g, b, 0, st, a);
+  else hipLaunchKernelGGL(mla_partial_k<8>, g, b, 0, st, a);
+  KX_LAUNCH_CHECK();
+  hipLaunchKernelGGL(mla_combine_k, dim3(c->heads, batch), dim3(64), 0, st, a.pm, a.pz, a.po, o_lat, c->heads, a.spans);
+  KX_LAUNCH_CHECK();
+  return KX_OK;
+}
+
+// ---- C ABI: BASELINE config 3 as an operator -------------------------------------------
+extern "C" int kx_mla_workspace_bytes(const kx_config *cfg, int32_t batch, int32_t max_seq, size_t *bytes) {
+  KX_REQUIRE(cfg && bytes, "kx_mla_workspace_bytes: null argument");
+  KX_REQUIRE(batch > 0 && max_seq > 0, "kx_mla_workspace_bytes: batch=%d max_seq=%d must be positive", batch, max_seq);
+  *bytes = kx_mla_partial_floats(batch, cfg->heads, cfg->kv_rank, max_seq) * sizeof(float);
+  return KX_OK;
+}
+
+extern "C" int kx_mla_decode(const kx_config *cfg, const void *d_cache, size_t seq_stride, const void *d_qabs,
+                             void *d_workspace, void *d_o_lat, int32_t batch, int32_t seq, void *stream) {
+  KX_REQUIRE(cfg && d_cache && d_qabs && d_workspace && d_o_lat, "kx_mla_decode: null argument");
+  KX_REQUIRE(seq_stride >= (size_t)seq * (cfg->kv_rank + cfg->qk_rope), "kx_mla_decode: seq_stride shorter than the sequence");
+  return kx_mla_attend_launch(cfg, (const uint16_t *)d_cache, seq_stride, (const float *)d_qabs, (float *)d_workspace,
+                              (uint16_t *)d_o_lat, batch, seq, kx_stream(stream));
+}
+
+extern "C" int kx_q_absorb(const kx_config *cfg, const void *d_q, const void *d_kvb, const void *d_rope_row, void *d_qabs,
+                           int32_t tokens, void *stream) {
+  KX_REQUIRE(cfg && d_q && d_kvb && d_rope_row && d_qabs, "kx_q_absorb: null argument");
+  return kx_q_absorb_launch((const uint16_t *)d_q, (const uint16_t *)d_kvb, (const uint16_t *)d_rope_row, (float *)d_qabs,
+                            tokens, cfg->heads, cfg->qk_nope, cfg->qk_rope, cfg->v_head, cfg->kv_rank, kx_stream(stream));
+}

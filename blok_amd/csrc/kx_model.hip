@@ -1,0 +1,464 @@
+// kx_model.hip -- the decoder stack: prefill, decode step, greedy sample, generate.
+//
+// Reference: generate() and its run() lambda, src/kimi_exec.cu:780-893.  The
+// reference allocates 19 single-token fp32 scratch buffers (:792-799), streams
+// every weight tile from NVMe inside the layer loop and synchronises with the
+// host once per MoE layer (:844) and twice per vocabulary tile (:728-730).
+// Here one arena in HBM holds the seeded random-init weights, the latent KV
+// cache and the scratch of a step for `max_batch` sequences; a step enqueues
+// kernels on one stream and never waits for the host.
+//
+// Per layer (T = batch tokens, all at the same position):
+//   rmsnorm -> [q_a ; kv_a] GEMV -> q_a norm, kv_a norm, rope(k), cache write
+//   -> q_b GEMV -> W_UK absorb + rope(q) -> attention over the latent cache
+//   -> W_UV GEMV per head -> o_proj GEMV with the residual add
+//   rmsnorm -> dense SwiGLU MLP (layers < first_dense) or the routed MoE layer.
+#include <math.h>
+#include <string.h>
+#include <vector>
+#include "kx_common.h"
+#include "kx_dense.h"
+#include "kx_mla.h"
+
+namespace {
+
+enum {  // tensor ids: global tensors use the id itself, layer L uses (L+1)*64 + id
+  TID_EMBED = 1, TID_FINAL_NORM = 2, TID_LM_HEAD = 3,
+  TL_INPUT_LN = 0, TL_QA = 1, TL_QA_LN = 2, TL_QB = 3, TL_KVA = 4, TL_KV_LN = 5, TL_KVB = 6, TL_O = 7, TL_POST_LN = 8,
+  TL_DENSE_GATE = 9, TL_DENSE_UP = 10, TL_DENSE_DOWN = 11, TL_ROUTER = 12, TL_ROUTER_BIAS = 13,
+  TL_GATE_P = 14, TL_GATE_S = 15, TL_UP_P = 16, TL_UP_S = 17, TL_DOWN_P = 18, TL_DOWN_S = 19,
+  TL_SH_GATE = 20, TL_SH_UP = 21, TL_SH_DOWN = 22
+};
+
+struct Layer {
+  uint16_t *input_ln, *qkv_a, *qa_ln, *qb, *kv_ln, *kvb, *o, *post_ln;
+  uint16_t *dgate, *dup, *ddown;
+  kx_moe_weights moe;
+  uint16_t *cache;  // [max_batch][max_context][kv_rank + qk_rope]
+};
+
+__global__ void embed_k(const uint16_t *__restrict__ embed, const uint32_t *__restrict__ ids, uint16_t *__restrict__ x,
+                        int hidden) {
+  const uint4 *src = (const uint4 *)(embed + (size_t)ids[blockIdx.x] * hidden);
+  uint4 *dst = (uint4 *)(x + (size_t)blockIdx.x * hidden);
+  for (int i = threadIdx.x; i < hidden / 8; i += blockDim.x) dst[i] = src[i];
+}
+__global__ void copy_ids_k(const uint32_t *__restrict__ src, uint32_t *__restrict__ dst, int n) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[i] = src[i];
+}
+
+}  // namespace
+
+struct kx_model {
+  kx_config c;
+  char *arena = nullptr;
+  size_t arena_bytes = 0;
+  uint16_t *embed, *final_norm, *lm_head, *rope_tab;
+  std::vector<Layer> layers;
+  // scratch of one step
+  uint16_t *x, *n, *qkv, *qa, *q, *o_lat, *att, *dmid;
+  float *qabs, *partial, *logits;
+  uint32_t *ids, *next, *history;  // [max_context][B], [B], [max_context][B]
+  kx_moe_workspace *moe_ws = nullptr;
+  hipStream_t st = nullptr;
+  hipEvent_t ev[3] = {nullptr, nullptr, nullptr};
+  int batch = 0, pos = 0;
+  bool sampled = false;
+  float ms_prefill = 0, ms_decode = 0;
+};
+
+namespace {
+
+struct Plan {  // byte offsets of everything in the arena
+  size_t total = 0, weights = 0, cache = 0, scratch = 0;
+  size_t take(size_t bytes) {
+    size_t at = total;
+    total += (bytes + 255) & ~(size_t)255;
+    return at;
+  }
+};
+
+int check_model_cfg(const kx_config *c) {
+  KX_REQUIRE(c, "kx_model: null config");
+  KX_REQUIRE(c->n_layers > 0 && c->first_dense >= 0 && c->first_dense <= c->n_layers, "kx_model: n_layers=%d first_dense=%d", c->n_layers, c->first_dense);
+  KX_REQUIRE(c->hidden > 0 && c->hidden % 1024 == 0, "kx_model: hidden=%d must be a multiple of 1024", c->hidden);
+  KX_REQUIRE(c->q_rank > 0 && c->q_rank % 512 == 0, "kx_model: q_rank=%d must be a multiple of 512", c->q_rank);
+  KX_REQUIRE(c->kv_rank == 512 && c->qk_rope == 64, "kx_model: kv_rank=%d qk_rope=%d must be 512 and 64", c->kv_rank, c->qk_rope);
+  KX_REQUIRE(c->heads > 0 && c->heads % 4 == 0, "kx_model: heads=%d must be a multiple of 4", c->heads);
+  KX_REQUIRE(c->qk_nope > 0 && c->qk_nope % 8 == 0 && c->v_head > 0 && (c->heads * c->v_head) % 512 == 0,
+             "kx_model: qk_nope=%d v_head=%d", c->qk_nope, c->v_head);
+  KX_REQUIRE(c->first_dense == 0 || (c->dense_inter > 0 && c->dense_inter % 512 == 0), "kx_model: dense_inter=%d must be a multiple of 512", c->dense_inter);
+  KX_REQUIRE(c->vocab > 0 && c->max_batch > 0 && c->max_context > 0, "kx_model: vocab=%d max_batch=%d max_context=%d", c->vocab, c->max_batch, c->max_context);
+  if (c->first_dense < c->n_layers) {
+    KX_REQUIRE(c->moe_inter > 0 && c->moe_inter % 1024 == 0, "kx_model: moe_inter=%d must be a multiple of 1024", c->moe_inter);
+    KX_REQUIRE(c->shared_inter > 0 && c->shared_inter % 512 == 0, "kx_model: shared_inter=%d must be a multiple of 512", c->shared_inter);
+    KX_REQUIRE(c->experts > 0 && c->experts <= 1024 && c->topk > 0 && c->topk <= c->experts, "kx_model: experts=%d topk=%d", c->experts, c->topk);
+  }
+  return KX_OK;
+}
+
+// lays the model out; when m != nullptr also sets its pointers (arena must be allocated)
+int layout(const kx_config *c, Plan &p, kx_model *m) {
+  const size_t H = c->hidden, V = c->vocab, E = c->experts, I = c->moe_inter, SI = c->shared_inter, D = c->dense_inter;
+  const size_t KD = (size_t)c->heads * (c->qk_nope + c->qk_rope), VD = (size_t)c->heads * c->v_head;
+  const size_t KVA = c->kv_rank + c->qk_rope, KVB = (size_t)c->heads * (c->qk_nope + c->v_head), B = c->max_batch;
+  char *base = m ? m->arena : nullptr;
+#define KX_AT(T, bytes) ((T)(base + p.take(bytes)))
+  auto *embed = KX_AT(uint16_t *, V * H * 2);
+  auto *final_norm = KX_AT(uint16_t *, H * 2);
+  auto *lm_head = KX_AT(uint16_t *, V * H * 2);
+  auto *rope_tab = KX_AT(uint16_t *, (size_t)c->max_context * c->qk_rope * 2);
+  if (m) { m->embed = embed; m->final_norm = final_norm; m->lm_head = lm_head; m->rope_tab = rope_tab; m->layers.resize(c->n_layers); }
+  for (int l = 0; l < c->n_layers; ++l) {
+    Layer L = {};
+    L.input_ln = KX_AT(uint16_t *, H * 2);
+    L.qkv_a = KX_AT(uint16_t *, ((size_t)c->q_rank + KVA) * H * 2);
+    L.qa_ln = KX_AT(uint16_t *, (size_t)c->q_rank * 2);
+    L.qb = KX_AT(uint16_t *, KD * c->q_rank * 2);
+    L.kv_ln = KX_AT(uint16_t *, (size_t)c->kv_rank * 2);
+    L.kvb = KX_AT(uint16_t *, KVB * c->kv_rank * 2);
+    L.o = KX_AT(uint16_t *, H * VD * 2);
+    L.post_ln = KX_AT(uint16_t *, H * 2);
+    if (l < c->first_dense) {
+      L.dgate = KX_AT(uint16_t *, D * H * 2);
+      L.dup = KX_AT(uint16_t *, D * H * 2);
+      L.ddown = KX_AT(uint16_t *, H * D * 2);
+    } else {
+      L.moe.d_router_gate = KX_AT(void *, E * H * 2);
+      L.moe.d_router_bias = KX_AT(void *, E * 4);
+      L.moe.d_gate_packed = KX_AT(void *, E * I * H / 2);
+      L.moe.d_gate_scale = KX_AT(void *, E * I * H / 32 * 2);
+      L.moe.d_up_packed = KX_AT(void *, E * I * H / 2);
+      L.moe.d_up_scale = KX_AT(void *, E * I * H / 32 * 2);
+      L.moe.d_down_packed = KX_AT(void *, E * H * I / 2);
+      L.moe.d_down_scale = KX_AT(void *, E * H * I / 32 * 2);
+      L.moe.d_shared_gate = KX_AT(void *, SI * H * 2);
+      L.moe.d_shared_up = KX_AT(void *, SI * H * 2);
+      L.moe.d_shared_down = KX_AT(void *, H * SI * 2);
+    }
+    if (m) m->layers[l] = L;
+  }
+  p.weights = p.total;
+  for (int l = 0; l < c->n_layers; ++l) {
+    auto *cache = KX_AT(uint16_t *, B * c->max_context * KVA * 2);
+    if (m) m->layers[l].cache = cache;
+  }
+  p.cache = p.total - p.weights;
+  const size_t inter = D > KD ? D : KD;
+  auto *x = KX_AT(uint16_t *, B * H * 2);
+  auto *n = KX_AT(uint16_t *, B * H * 2);
+  auto *qkv = KX_AT(uint16_t *, B * ((size_t)c->q_rank + KVA) * 2);
+  auto *qa = KX_AT(uint16_t *, B * (size_t)c->q_rank * 2);
+  auto *q = KX_AT(uint16_t *, B * KD * 2);
+  auto *o_lat = KX_AT(uint16_t *, B * (size_t)c->heads * c->kv_rank * 2);
+  auto *att = KX_AT(uint16_t *, B * VD * 2);
+  auto *dmid = KX_AT(uint16_t *, B * inter * 2);
+  auto *qabs = KX_AT(float *, B * (size_t)c->heads * KVA * 4);
+  auto *partial = KX_AT(float *, kx_mla_partial_floats(c->max_batch, c->heads, c->kv_rank, c->max_context) * 4);
+  auto *logits = KX_AT(float *, B * V * 4);
+  auto *ids = KX_AT(uint32_t *, (size_t)c->max_context * B * 4);
+  auto *next = KX_AT(uint32_t *, B * 4);
+  auto *history = KX_AT(uint32_t *, (size_t)c->max_context * B * 4);
+#undef KX_AT
+  p.scratch = p.total - p.weights - p.cache;
+  if (m) {
+    m->x = x; m->n = n; m->qkv = qkv; m->qa = qa; m->q = q; m->o_lat = o_lat; m->att = att; m->dmid = dmid;
+    m->qabs = qabs; m->partial = partial; m->logits = logits; m->ids = ids; m->next = next; m->history = history;
+  }
+  return KX_OK;
+}
+
+int init_weights(kx_model *m) {
+  const kx_config &c = m->c;
+  const size_t H = c.hidden, V = c.vocab, E = c.experts, I = c.moe_inter, SI = c.shared_inter, D = c.dense_inter;
+  const size_t KD = (size_t)c.heads * (c.qk_nope + c.qk_rope), VD = (size_t)c.heads * c.v_head;
+  const size_t KVA = c.kv_rank + c.qk_rope, KVB = (size_t)c.heads * (c.qk_nope + c.v_head);
+  const float sg = c.init_sigma, es = c.expert_scale_sigma;
+  void *st = m->st;
+  int rc;
+#define KX_TRY(call) do { if ((rc = (call))) return rc; } while (0)
+  KX_TRY(kx_fill_normal_bf16(m->embed, V * H, c.seed, TID_EMBED, 1.0f, 0, st));
+  KX_TRY(kx_fill_affine_bf16(m->final_norm, H, c.seed, TID_FINAL_NORM, 1.0f, 0.02f, st));
+  KX_TRY(kx_fill_normal_bf16(m->lm_head, V * H, c.seed, TID_LM_HEAD, sg, 0, st));
+  for (int l = 0; l < c.n_layers; ++l) {
+    Layer &L = m->layers[l];
+    const uint64_t b = (uint64_t)(l + 1) * 64;
+    KX_TRY(kx_fill_affine_bf16(L.input_ln, H, c.seed, b + TL_INPUT_LN, 1.0f, 0.02f, st));
+    KX_TRY(kx_fill_normal_bf16(L.qkv_a, (size_t)c.q_rank * H, c.seed, b + TL_QA, sg, 0, st));
+    KX_TRY(kx_fill_normal_bf16(L.qkv_a + (size_t)c.q_rank * H, KVA * H, c.seed, b + TL_KVA, sg, 0, st));
+    KX_TRY(kx_fill_affine_bf16(L.qa_ln, c.q_rank, c.seed, b + TL_QA_LN, 1.0f, 0.02f, st));
+    KX_TRY(kx_fill_normal_bf16(L.qb, KD * c.q_rank, c.seed, b + TL_QB, sg, 0, st));
+    KX_TRY(kx_fill_affine_bf16(L.kv_ln, c.kv_rank, c.seed, b + TL_KV_LN, 1.0f, 0.02f, st));
+    KX_TRY(kx_fill_normal_bf16(L.kvb, KVB * c.kv_rank, c.seed, b + TL_KVB, sg, 0, st));
+    KX_TRY(kx_fill_normal_bf16(L.o, H * VD, c.seed, b + TL_O, sg, 0, st));
+    KX_TRY(kx_fill_affine_bf16(L.post_ln, H, c.seed, b + TL_POST_LN, 1.0f, 0.02f, st));
+    if (l < c.first_dense) {
+      KX_TRY(kx_fill_normal_bf16(L.dgate, D * H, c.seed, b + TL_DENSE_GATE, sg, 0, st));
+      KX_TRY(kx_fill_normal_bf16(L.dup, D * H, c.seed, b + TL_DENSE_UP, sg, 0, st));
+      KX_TRY(kx_fill_normal_bf16(L.ddown, H * D, c.seed, b + TL_DENSE_DOWN, sg, 0, st));
+    } else {
+      kx_moe_weights &w = L.moe;
+      KX_TRY(kx_fill_normal_bf16((void *)w.d_router_gate, E * H, c.seed, b + TL_ROUTER, 1.0f / sqrtf((float)H), 0, st));
+      KX_TRY(kx_fill_normal_f32((void *)w.d_router_bias, E, c.seed, b + TL_ROUTER_BIAS, 0.01f, st));
+      KX_TRY(kx_fill_words_u32((void *)w.d_gate_packed, E * I * H / 8, c.seed, b + TL_GATE_P, st));
+      KX_TRY(kx_fill_normal_bf16((void *)w.d_gate_scale, E * I * H / 32, c.seed, b + TL_GATE_S, es, 1, st));
+      KX_TRY(kx_fill_words_u32((void *)w.d_up_packed, E * I * H / 8, c.seed, b + TL_UP_P, st));
+      KX_TRY(kx_fill_normal_bf16((void *)w.d_up_scale, E * I * H / 32, c.seed, b + TL_UP_S, es, 1, st));
+      KX_TRY(kx_fill_words_u32((void *)w.d_down_packed, E * H * I / 8, c.seed, b + TL_DOWN_P, st));
+      KX_TRY(kx_fill_normal_bf16((void *)w.d_down_scale, E * H * I / 32, c.seed, b + TL_DOWN_S, es, 1, st));
+      KX_TRY(kx_fill_normal_bf16((void *)w.d_shared_gate, SI * H, c.seed, b + TL_SH_GATE, sg, 0, st));
+      KX_TRY(kx_fill_normal_bf16((void *)w.d_shared_up, SI * H, c.seed, b + TL_SH_UP, sg, 0, st));
+      KX_TRY(kx_fill_normal_bf16((void *)w.d_shared_down, H * SI, c.seed, b + TL_SH_DOWN, sg, 0, st));
+    }
+  }
+  // rope table for every position, computed on the host
+  std::vector<uint16_t> tab((size_t)c.max_context * c.qk_rope);
+  KX_TRY(kx_rope_table(&c, 0, c.max_context, tab.data()));
+  KX_HIP(hipMemcpyAsync(m->rope_tab, tab.data(), tab.size() * 2, hipMemcpyHostToDevice, m->st));
+  KX_HIP(hipStreamSynchronize(m->st));
+#undef KX_TRY
+  return KX_OK;
+}
+
+// one run() of the reference for `B` tokens at position m->pos; ids on the device
+int step(kx_model *m, const uint32_t *d_ids, bool sample) {
+  const kx_config &c = m->c;
+  const int B = m->batch, H = c.hidden, pos = m->pos;
+  const int KD = c.heads * (c.qk_nope + c.qk_rope), VD = c.heads * c.v_head, KVA = c.kv_rank + c.qk_rope;
+  const int QKV = c.q_rank + KVA;
+  hipStream_t st = m->st;
+  int rc;
+#define KX_TRY(call) do { if ((rc = (call))) return rc; } while (0)
+  hipLaunchKernelGGL(embed_k, dim3(B), dim3(256), 0, st, m->embed, d_ids, m->x, H);  // embed_token (:651-655)
+  KX_LAUNCH_CHECK();
+  const uint16_t *rope_row = m->rope_tab + (size_t)pos * c.qk_rope;
+  const size_t seq_stride = (size_t)c.max_context * KVA;
+  for (int l = 0; l < c.n_layers; ++l) {
+    Layer &L = m->layers[l];
+    KX_TRY(kx_rmsnorm_launch(m->x, L.input_ln, m->n, B, H, H, H, c.rms_eps, st));                      // :812
+    KxGemvArgs g = {};
+    g.w0 = L.qkv_a; g.x = m->n; g.x_stride = H; g.out = m->qkv; g.out_stride = QKV; g.rows = QKV; g.cols = H; g.tokens = B;
+    KX_TRY(kx_gemv_launch(KX_EPI_BF16, g, st));                                                         // :813, :816
+    KX_TRY(kx_kv_finish_launch(m->qkv, L.qa_ln, L.kv_ln, rope_row, m->qa, L.cache, B, c.q_rank, c.kv_rank, c.qk_rope,
+                               seq_stride, pos, c.rms_eps, st));                                        // :814, :817, :820-824
+    g = {};
+    g.w0 = L.qb; g.x = m->qa; g.x_stride = c.q_rank; g.out = m->q; g.out_stride = KD; g.rows = KD; g.cols = c.q_rank; g.tokens = B;
+    KX_TRY(kx_gemv_launch(KX_EPI_BF16, g, st));                                                         // :815
+    KX_TRY(kx_q_absorb_launch(m->q, L.kvb, rope_row, m->qabs, B, c.heads, c.qk_nope, c.qk_rope, c.v_head, c.kv_rank, st));
+    KX_TRY(kx_mla_attend_launch(&c, L.cache, seq_stride, m->qabs, m->partial, m->o_lat, B, pos + 1, st));  // :825
+    g = {};
+    g.w0 = L.kvb; g.x = m->o_lat; g.x_stride = c.heads * c.kv_rank; g.out = m->att; g.out_stride = VD; g.rows = VD;
+    g.cols = c.kv_rank; g.tokens = B; g.row_block = c.v_head; g.w_block_stride = c.qk_nope + c.v_head;
+    g.w_block_off = c.qk_nope; g.x_block_stride = c.kv_rank;
+    KX_TRY(kx_gemv_launch(KX_EPI_BF16, g, st));                                                         // W_UV of :818
+    g = {};
+    g.w0 = L.o; g.x = m->att; g.x_stride = VD; g.out = m->x; g.out_stride = H; g.rows = H; g.cols = VD; g.tokens = B;
+    KX_TRY(kx_gemv_launch(KX_EPI_RESID, g, st));                                                        // :826-827
+    KX_TRY(kx_rmsnorm_launch(m->x, L.post_ln, m->n, B, H, H, H, c.rms_eps, st));                       // :829
+    if (l < c.first_dense) {                                                                            // bf16_mlp (:674-686)
+      g = {};
+      g.w0 = L.dgate; g.w1 = L.dup; g.x = m->n; g.x_stride = H; g.out = m->dmid; g.out_stride = c.dense_inter;
+      g.rows = c.dense_inter; g.cols = H; g.tokens = B;
+      KX_TRY(kx_gemv_launch(KX_EPI_SWIGLU, g, st));
+      g = {};
+      g.w0 = L.ddown; g.x = m->dmid; g.x_stride = c.dense_inter; g.out = m->x; g.out_stride = H; g.rows = H;
+      g.cols = c.dense_inter; g.tokens = B;
+      KX_TRY(kx_gemv_launch(KX_EPI_RESID, g, st));                                                      // :684, :877
+    } else {
+      KX_TRY(kx_moe_decode_layer(&c, &L.moe, m->moe_ws, m->n, m->x, B, 0, st));                         // :835-877
+    }
+  }
+  if (sample) {                                                                                          // :880-881
+    KX_TRY(kx_rmsnorm_launch(m->x, m->final_norm, m->n, B, H, H, H, c.rms_eps, st));
+    KxGemvArgs g = {};
+    g.w0 = m->lm_head; g.x = m->n; g.x_stride = H; g.out = m->logits; g.out_stride = c.vocab; g.rows = c.vocab; g.cols = H;
+    g.tokens = B;
+    KX_TRY(kx_gemv_launch(KX_EPI_ARGMAX, g, st));
+    KX_TRY(kx_argmax_launch(m->logits, B, c.vocab, c.vocab, m->next, st));
+  }
+#undef KX_TRY
+  m->sampled = sample;
+  m->pos = pos + 1;
+  return KX_OK;
+}
+
+}  // namespace
+
+extern "C" int kx_model_bytes(const kx_config *cfg, uint64_t *weights, uint64_t *kv_cache, uint64_t *scratch) {
+  int rc = check_model_cfg(cfg);
+  if (rc) return rc;
+  Plan p;
+  layout(cfg, p, nullptr);
+  if (weights) *weights = p.weights;
+  if (kv_cache) *kv_cache = p.cache;
+  if (scratch) *scratch = p.scratch;
+  return KX_OK;
+}
+
+extern "C" int kx_model_create(const kx_config *cfg, kx_model **out) {
+  KX_REQUIRE(out, "kx_model_create: null out pointer");
+  *out = nullptr;
+  int rc = check_model_cfg(cfg);
+  if (rc) return rc;
+  Plan p;
+  layout(cfg, p, nullptr);
+  size_t free_b = 0, total_b = 0;
+  KX_HIP(hipMemGetInfo(&free_b, &total_b));
+  KX_REQUIRE(p.total + ((size_t)1 << 30) <= free_b, "kx_model_create: the model needs %.1f GB of HBM, %.1f GB are free",
+             p.total / 1e9, free_b / 1e9);
+  kx_model *m = new kx_model();
+  m->c = *cfg;
+  hipError_t e = hipMalloc((void **)&m->arena, p.total);
+  if (e != hipSuccess) {
+    kx_set_error("kx_model_create: hipMalloc(%zu): %s", p.total, hipGetErrorString(e));
+    delete m;
+    return KX_ERR_HIP;
+  }
+  m->arena_bytes = p.total;
+  Plan p2;
+  layout(cfg, p2, m);
+  rc = KX_OK;
+  if (hipStreamCreate(&m->st) != hipSuccess) rc = KX_ERR_HIP;
+  for (auto &ev : m->ev)
+    if (!rc && hipEventCreate(&ev) != hipSuccess) rc = KX_ERR_HIP;
+  if (!rc && cfg->first_dense < cfg->n_layers) rc = kx_moe_workspace_create(cfg, cfg->max_batch, &m->moe_ws);
+  if (!rc) rc = init_weights(m);
+  if (rc) {
+    if (rc == KX_ERR_HIP && !kx_last_error()[0]) kx_set_error("kx_model_create: HIP resource creation failed");
+    kx_model_destroy(m);
+    return rc;
+  }
+  *out = m;
+  return KX_OK;
+}
+
+extern "C" int kx_model_destroy(kx_model *m) {
+  if (!m) return KX_OK;
+  if (m->st) (void)hipStreamSynchronize(m->st);
+  if (m->moe_ws) kx_moe_workspace_destroy(m->moe_ws);
+  for (auto &ev : m->ev)
+    if (ev) (void)hipEventDestroy(ev);
+  if (m->st) (void)hipStreamDestroy(m->st);
+  if (m->arena) (void)hipFree(m->arena);
+  delete m;
+  return KX_OK;
+}
+
+static int check_ids(const kx_model *m, const uint32_t *ids, size_t n) {
+  for (size_t i = 0; i < n; ++i)
+    KX_REQUIRE(ids[i] < (uint32_t)m->c.vocab, "token id %u outside the vocabulary of %d", ids[i], m->c.vocab);  // :552, :652
+  return KX_OK;
+}
+
+extern "C" int kx_prefill(kx_model *m, const uint32_t *h_ids, int32_t batch, int32_t prompt_len) {
+  KX_REQUIRE(m && h_ids, "kx_prefill: null argument");
+  KX_REQUIRE(batch > 0 && batch <= m->c.max_batch, "kx_prefill: batch=%d outside [1, %d]", batch, m->c.max_batch);
+  KX_REQUIRE(prompt_len > 0 && prompt_len <= m->c.max_context, "kx_prefill: prompt_len=%d outside [1, %d]", prompt_len, m->c.max_context);  // :555, :784
+  int rc = check_ids(m, h_ids, (size_t)batch * prompt_len);
+  if (rc) return rc;
+  std::vector<uint32_t> pm((size_t)prompt_len * batch);  // position-major
+  for (int b = 0; b < batch; ++b)
+    for (int i = 0; i < prompt_len; ++i) pm[(size_t)i * batch + b] = h_ids[(size_t)b * prompt_len + i];
+  KX_HIP(hipMemcpyAsync(m->ids, pm.data(), pm.size() * 4, hipMemcpyHostToDevice, m->st));
+  KX_HIP(hipStreamSynchronize(m->st));  // pm goes out of scope
+  m->batch = batch;
+  m->pos = 0;
+  for (int i = 0; i < prompt_len; ++i)  // :886: one run() per prompt token, sampling on the last
+    if ((rc = step(m, m->ids + (size_t)i * batch, i + 1 == prompt_len))) return rc;
+  return KX_OK;
+}
+
+extern "C" int kx_decode_step(kx_model *m, const uint32_t *h_ids) {
+  KX_REQUIRE(m, "kx_decode_step: null model");
+  KX_REQUIRE(m->batch > 0, "kx_decode_step: no prefill has run");
+  KX_REQUIRE(m->pos < m->c.max_context, "kx_decode_step: the context of %d positions is full", m->c.max_context);  // :784
+  const uint32_t *src = m->next;
+  if (h_ids) {
+    int rc = check_ids(m, h_ids, m->batch);
+    if (rc) return rc;
+    uint32_t *slot = m->ids + (size_t)m->pos * m->batch;
+    KX_HIP(hipMemcpyAsync(slot, h_ids, (size_t)m->batch * 4, hipMemcpyHostToDevice, m->st));
+    KX_HIP(hipStreamSynchronize(m->st));
+    src = slot;
+  } else {
+    KX_REQUIRE(m->sampled, "kx_decode_step: no sampled ids to feed (pass h_ids)");
+    // the sampler overwrites `next`; feed a copy
+    uint32_t *slot = m->ids + (size_t)m->pos * m->batch;
+    hipLaunchKernelGGL(copy_ids_k, dim3(kx_cdiv(m->batch, 64)), dim3(64), 0, m->st, m->next, slot, m->batch);
+    KX_LAUNCH_CHECK();
+    src = slot;
+  }
+  return step(m, src, true);
+}
+
+extern "C" int kx_greedy_sample(kx_model *m, uint32_t *h_out) {
+  KX_REQUIRE(m && h_out, "kx_greedy_sample: null argument");
+  KX_REQUIRE(m->sampled, "kx_greedy_sample: the last step did not sample");
+  KX_HIP(hipMemcpyAsync(h_out, m->next, (size_t)m->batch * 4, hipMemcpyDeviceToHost, m->st));
+  KX_HIP(hipStreamSynchronize(m->st));
+  return KX_OK;
+}
+
+extern "C" int kx_generate(kx_model *m, const uint32_t *h_prompt, int32_t batch, int32_t prompt_len, int32_t n_tokens,
+                           int ignore_eos, uint32_t *h_out, int32_t *h_counts) {
+  KX_REQUIRE(m && h_prompt && h_out && h_counts, "kx_generate: null argument");
+  KX_REQUIRE(n_tokens > 0, "kx_generate: n_tokens=%d must be positive", n_tokens);  // :542
+  KX_REQUIRE((int64_t)prompt_len + n_tokens <= m->c.max_context, "requested sequence exceeds the context of %d positions", m->c.max_context);  // :784
+  int rc;
+  KX_HIP(hipEventRecord(m->ev[0], m->st));
+  if ((rc = kx_prefill(m, h_prompt, batch, prompt_len))) return rc;
+  KX_HIP(hipEventRecord(m->ev[1], m->st));
+  const int cp = kx_cdiv(batch, 64);
+  for (int i = 0; i < n_tokens; ++i) {  // :887-890
+    hipLaunchKernelGGL(copy_ids_k, dim3(cp), dim3(64), 0, m->st, m->next, m->history + (size_t)i * batch, batch);
+    KX_LAUNCH_CHECK();
+    if (i + 1 < n_tokens && (rc = step(m, m->history + (size_t)i * batch, true))) return rc;
+  }
+  KX_HIP(hipEventRecord(m->ev[2], m->st));
+  std::vector<uint32_t> hist((size_t)n_tokens * batch);
+  KX_HIP(hipMemcpyAsync(hist.data(), m->history, hist.size() * 4, hipMemcpyDeviceToHost, m->st));
+  KX_HIP(hipStreamSynchronize(m->st));
+  KX_HIP(hipEventElapsedTime(&m->ms_prefill, m->ev[0], m->ev[1]));
+  KX_HIP(hipEventElapsedTime(&m->ms_decode, m->ev[1], m->ev[2]));
+  for (int b = 0; b < batch; ++b) {  // generation stops before the end-of-sequence id is emitted (:887-888)
+    int n = 0;
+    for (int i = 0; i < n_tokens; ++i) {
+      const uint32_t id = hist[(size_t)i * batch + b];
+      if (!ignore_eos && id == m->c.eos_id) break;
+      h_out[(size_t)b * n_tokens + n++] = id;
+    }
+    h_counts[b] = n;
+  }
+  return KX_OK;
+}
+
+extern "C" int kx_model_timing(kx_model *m, float *ms2) {
+  KX_REQUIRE(m && ms2, "kx_model_timing: null argument");
+  ms2[0] = m->ms_prefill;
+  ms2[1] = m->ms_decode;
+  return KX_OK;
+}
+
+extern "C" int kx_model_hidden(kx_model *m, uint16_t *h_out) {
+  KX_REQUIRE(m && h_out && m->batch > 0, "kx_model_hidden: null argument or no step has run");
+  KX_HIP(hipMemcpyAsync(h_out, m->x, (size_t)m->batch * m->c.hidden * 2, hipMemcpyDeviceToHost, m->st));
+  KX_HIP(hipStreamSynchronize(m->st));
+  return KX_OK;
+}
+extern "C" int kx_model_logits(kx_model *m, float *h_out) {
+  KX_REQUIRE(m && h_out && m->sampled, "kx_model_logits: null argument or the last step did not sample");
+  KX_HIP(hipMemcpyAsync(h_out, m->logits, (size_t)m->batch * m->c.vocab * 4, hipMemcpyDeviceToHost, m->st));
+  KX_HIP(hipStreamSynchronize(m->st));
+  return KX_OK;
+}
+extern "C" int kx_model_latent(kx_model *m, int32_t layer, int32_t seq_index, int32_t pos0, int32_t n, uint16_t *h_out) {
+  KX_REQUIRE(m && h_out, "kx_model_latent: null argument");
+  KX_REQUIRE(layer >= 0 && layer < m->c.n_layers && seq_index >= 0 && seq_index < m->c.max_batch && pos0 >= 0 && n >= 0 &&
+                 pos0 + n <= m->c.max_context, "kx_model_latent: index out of range");
+  const size_t KVA = m->c.kv_rank + m->c.qk_rope;
+  KX_HIP(hipMemcpyAsync(h_out, m->layers[layer].cache + ((size_t)seq_index * m->c.max_context + pos0) * KVA, (size_t)n * KVA * 2,
+                        hipMemcpyDeviceToHost, m->st));
+  KX_HIP(hipStreamSynchronize(m->st));
+  return KX_OK;
+}

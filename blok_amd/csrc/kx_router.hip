@@ -60,17 +60,29 @@ __global__ void __launch_bounds__(64) router_topk_k(const float *__restrict__ lo
   if (lane < topk) weights[(size_t)tok * topk + lane] = my_w / (sum + 1.0e-20f) * routed_scale;
 }
 
-// one workgroup, thread e owns expert e: count, exclusive scan, stable placement
+// one workgroup, thread e owns expert e: count, exclusive scan, stable placement.
+// The ids are staged in LDS (padded with 0xffff to a multiple of 8) and scanned 8 at a time.
 __global__ void __launch_bounds__(1024) bucket_k(const uint16_t *__restrict__ ids, int n_pairs, int E,
                                                  int *__restrict__ counts, int *__restrict__ offsets,
                                                  int *__restrict__ pairs, int4 *__restrict__ work,
                                                  int *__restrict__ n_active) {
+  extern __shared__ uint4 s_ids4[];  // ceil(n_pairs / 8) pieces
   __shared__ int s_cnt[1024];
   __shared__ int s_act[1024];
   const int e = threadIdx.x, n = blockDim.x;
+  const int n8 = (n_pairs + 7) >> 3;
+  uint16_t *s_ids = (uint16_t *)s_ids4;
+  for (int p = threadIdx.x; p < n8 * 8; p += n) s_ids[p] = p < n_pairs ? ids[p] : (uint16_t)0xffff;
+  __syncthreads();
+  const uint32_t me = (uint32_t)e, me2 = me | (me << 16);
   int cnt = 0;
   if (e < E)
-    for (int p = 0; p < n_pairs; ++p) cnt += (ids[p] == e) ? 1 : 0;
+    for (int q = 0; q < n8; ++q) {
+      const uint4 u = s_ids4[q];
+      const uint32_t w[4] = {u.x ^ me2, u.y ^ me2, u.z ^ me2, u.w ^ me2};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) cnt += ((w[j] & 0xffffu) == 0) + ((w[j] >> 16) == 0);
+    }
   s_cnt[e] = cnt;
   s_act[e] = cnt > 0 ? 1 : 0;
   __syncthreads();
@@ -86,10 +98,18 @@ __global__ void __launch_bounds__(1024) bucket_k(const uint16_t *__restrict__ id
     counts[e] = cnt;
     offsets[e] = off;
     int pos = off, first = 0;
-    for (int p = 0; p < n_pairs; ++p)
-      if (ids[p] == e) {
-        if (pos == off) first = p;
-        pairs[pos++] = p;
+    if (cnt > 0)
+      for (int q = 0; q < n8 && pos < off + cnt; ++q) {
+        const uint4 u = s_ids4[q];
+        const uint32_t w[4] = {u.x ^ me2, u.y ^ me2, u.z ^ me2, u.w ^ me2};
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const uint32_t h = (j & 1) ? (w[j >> 1] >> 16) : (w[j >> 1] & 0xffffu);
+          if (h == 0) {
+            if (pos == off) first = q * 8 + j;
+            pairs[pos++] = q * 8 + j;
+          }
+        }
       }
     if (cnt > 0) work[slot] = make_int4(e, off, off + cnt, first);
     if (e >= total_active) work[e] = make_int4(-1, 0, 0, 0);
@@ -125,7 +145,9 @@ int kx_bucket_launch(const uint16_t *ids, int tokens, int experts, int topk, int
   KX_REQUIRE(tokens > 0 && topk > 0, "kx_bucket: tokens=%d topk=%d must be positive", tokens, topk);
   KX_REQUIRE(experts > 0 && experts <= 1024, "kx_bucket: experts=%d outside [1, 1024]", experts);
   int threads = kx_cdiv(experts, 64) * 64;
-  hipLaunchKernelGGL(bucket_k, dim3(1), dim3(threads), 0, st, ids, tokens * topk, experts, counts, offsets, pairs,
+  const size_t lds = (size_t)kx_cdiv(tokens * topk, 8) * 16;
+  KX_REQUIRE(lds <= 128 * 1024, "kx_bucket: %d pairs exceed the %d the bucketing kernel stages", tokens * topk, 65536);
+  hipLaunchKernelGGL(bucket_k, dim3(1), dim3(threads), lds, st, ids, tokens * topk, experts, counts, offsets, pairs,
                      work, n_active);
   KX_LAUNCH_CHECK();
   return KX_OK;

@@ -27,7 +27,7 @@ extern "C" int kx_config_default(kx_config *c) {
   c->max_batch = 1; c->max_context = 4096; c->eos_id = 163586u;
   c->rms_eps = 1.0e-5f; c->rope_theta = 50000.0f; c->routed_scale = 2.827f;
   c->yarn_factor = 32.0f; c->yarn_beta_fast = 32.0f; c->yarn_beta_slow = 1.0f;
-  c->yarn_orig_ctx = 4096.0f; c->yarn_mscale_all_dim = 1.0f; c->init_sigma = 0.02f;
+  c->yarn_orig_ctx = 4096.0f; c->yarn_mscale_all_dim = 1.0f; c->init_sigma = 0.02f; c->expert_scale_sigma = 0.02f;
   c->seed = 0;
   return KX_OK;
 }
@@ -105,6 +105,11 @@ __global__ void fill_normal_bf16_k(uint16_t *out, uint64_t n, uint64_t key, floa
   uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
   for (; i < n; i += stride) out[i] = kx_rng_normal_bf16(key, i, sigma, absval);
 }
+__global__ void fill_affine_bf16_k(uint16_t *out, uint64_t n, uint64_t key, float mean, float sigma) {
+  uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) out[i] = kx_bf16_rne(mean + kx_rng_normal_f32(key, i, sigma));
+}
 __global__ void fill_normal_f32_k(float *out, uint64_t n, uint64_t key, float sigma) {
   uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
@@ -144,6 +149,15 @@ extern "C" int kx_fill_words_u32(void *d_out, uint64_t n, uint64_t seed, uint64_
   if (!n) return KX_OK;
   hipLaunchKernelGGL(fill_words_k, dim3(fill_grid(n)), dim3(256), 0, kx_stream(stream), (uint32_t *)d_out, n,
                      kx_rng_key(seed, tensor_id));
+  KX_LAUNCH_CHECK();
+  return KX_OK;
+}
+extern "C" int kx_fill_affine_bf16(void *d_out, uint64_t n, uint64_t seed, uint64_t tensor_id, float mean, float sigma,
+                                   void *stream) {
+  KX_REQUIRE(d_out || !n, "kx_fill_affine_bf16: null pointer");
+  if (!n) return KX_OK;
+  hipLaunchKernelGGL(fill_affine_bf16_k, dim3(fill_grid(n)), dim3(256), 0, kx_stream(stream), (uint16_t *)d_out, n,
+                     kx_rng_key(seed, tensor_id), mean, sigma);
   KX_LAUNCH_CHECK();
   return KX_OK;
 }

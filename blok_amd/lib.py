@@ -27,7 +27,7 @@ class KxConfig(C.Structure):
         "kv_rank", "experts", "topk", "moe_inter", "shared_inter", "dense_inter", "vocab",
         "max_batch", "max_context")] + [("eos_id", C.c_uint32)] + [(n, C.c_float) for n in (
             "rms_eps", "rope_theta", "routed_scale", "yarn_factor", "yarn_beta_fast",
-            "yarn_beta_slow", "yarn_orig_ctx", "yarn_mscale_all_dim", "init_sigma")] + [
+            "yarn_beta_slow", "yarn_orig_ctx", "yarn_mscale_all_dim", "init_sigma", "expert_scale_sigma")] + [
                 ("seed", C.c_uint64)]
 
 
@@ -67,6 +67,23 @@ _SIGS = {
     "kx_moe_workspace_destroy": [_P],
     "kx_moe_workspace_views": [_P, _PP, _PP, _PP, _PP, _PP, _PP, _PP, _PP],
     "kx_moe_decode_layer": [C.POINTER(KxConfig), C.POINTER(KxMoeWeights), _P, _P, _P, _I, C.c_uint32, _P],
+    "kx_fill_affine_bf16": [_P, _U64, _U64, _U64, _F, _F, _P],
+    "kx_rope_table": [C.POINTER(KxConfig), _I, _I, _P],
+    "kx_softmax_scale": [C.POINTER(KxConfig), C.POINTER(C.c_float), C.POINTER(C.c_float)],
+    "kx_q_absorb": [C.POINTER(KxConfig), _P, _P, _P, _P, _I, _P],
+    "kx_mla_workspace_bytes": [C.POINTER(KxConfig), _I, _I, C.POINTER(_SZ)],
+    "kx_mla_decode": [C.POINTER(KxConfig), _P, _SZ, _P, _P, _P, _I, _I, _P],
+    "kx_model_bytes": [C.POINTER(KxConfig), C.POINTER(C.c_uint64), C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)],
+    "kx_model_create": [C.POINTER(KxConfig), _PP],
+    "kx_model_destroy": [_P],
+    "kx_prefill": [_P, _P, _I, _I],
+    "kx_decode_step": [_P, _P],
+    "kx_greedy_sample": [_P, _P],
+    "kx_generate": [_P, _P, _I, _I, _I, C.c_int, _P, _P],
+    "kx_model_hidden": [_P, _P],
+    "kx_model_logits": [_P, _P],
+    "kx_model_latent": [_P, _I, _I, _I, _I, _P],
+    "kx_model_timing": [_P, C.POINTER(C.c_float)],
     "kx_moe_decode_layer_timed": [C.POINTER(KxConfig), C.POINTER(KxMoeWeights), _P, _P, _P, _I,
                                   C.c_uint32, _P, C.POINTER(C.c_float)],
 }

@@ -57,6 +57,7 @@ typedef struct kx_config {
   float yarn_orig_ctx;   /* 4096 */
   float yarn_mscale_all_dim; /* 1 */
   float init_sigma;      /* std of the random-init bf16 weights (0.02)            */
+  float expert_scale_sigma; /* INT4 group scales are |N(0, this)| (0.02)           */
   uint64_t seed;         /* seed of every synthetic tensor                        */
 } kx_config;
 
@@ -163,6 +164,60 @@ int kx_moe_decode_layer(const kx_config *cfg, const kx_moe_weights *w, kx_moe_wo
 int kx_moe_decode_layer_timed(const kx_config *cfg, const kx_moe_weights *w, kx_moe_workspace *ws,
                               const void *d_n, void *d_x, int32_t tokens, uint32_t flags,
                               void *stream, float *ms5);
+
+/* ---- MLA decode attention (tiled_attention, :692-716, on the absorbed latent cache) ----
+ * kx_rope_table   : rope_k's cos/sin (:351) with the YaRN frequencies (:325-344) for positions
+ *                   pos0 .. pos0+n-1; h_out bf16 [n][qk_rope]: qk_rope/2 cosines, then sines.
+ * kx_softmax_scale: the two factors of the score scale (:428-429).
+ * kx_q_absorb     : d_q bf16 [T][heads][qk_nope+qk_rope] (q_b output, :815) ->
+ *                   d_qabs f32 [T][heads][kv_rank+qk_rope] = (bf(W_UK^T q_nope) | rope(q_rope));
+ *                   d_kvb bf16 [heads*(qk_nope+v_head)][kv_rank] (kv_b_proj, :751);
+ *                   d_rope_row bf16 [qk_rope] is the table row of the tokens' position.
+ * kx_mla_decode   : d_cache bf16, sequence b at d_cache + b*seq_stride (elements), rows of
+ *                   kv_rank+qk_rope = (normed latent | rotated rope key); attends the first
+ *                   `seq` positions; d_o_lat bf16 [batch][heads][kv_rank] is the softmax-weighted
+ *                   latent (W_UV is applied by the caller, kx_gemv_bf16 per head).
+ *                   d_workspace: kx_mla_workspace_bytes(cfg, batch, max seq) bytes.              */
+int kx_rope_table(const kx_config *cfg, int32_t pos0, int32_t n, uint16_t *h_out);
+int kx_softmax_scale(const kx_config *cfg, float *rsqrt_head, float *mscale);
+int kx_q_absorb(const kx_config *cfg, const void *d_q, const void *d_kvb, const void *d_rope_row,
+                void *d_qabs, int32_t tokens, void *stream);
+int kx_mla_workspace_bytes(const kx_config *cfg, int32_t batch, int32_t max_seq, size_t *bytes);
+int kx_mla_decode(const kx_config *cfg, const void *d_cache, size_t seq_stride, const void *d_qabs,
+                  void *d_workspace, void *d_o_lat, int32_t batch, int32_t seq, void *stream);
+
+/* ---- the decoder stack: generate() / run() (:780-893) ------------------------------------
+ * A kx_model owns one HBM arena: seeded random-init weights of cfg->n_layers layers (layer
+ * l < first_dense dense, the others MoE), the latent KV cache [layers][max_batch][max_context]
+ * and the scratch of one decode step.  Not re-entrant; one private stream; a decode step
+ * only enqueues work (expert ids and sampled ids stay on the device).
+ * kx_prefill     : run() over the prompt token by token as the reference does (:886), sampling
+ *                  on the last prompt token; h_ids u32 [batch][prompt_len]; restarts at position 0.
+ * kx_decode_step : one run() at the next position; h_ids u32 [batch], or NULL to feed the ids
+ *                  sampled by the previous step (no host round trip).
+ * kx_greedy_sample: sample_lm_head (:718-734): lowest-index argmax over the bf16-rounded
+ *                  logits of the last step; h_out u32 [batch]; synchronises.
+ * kx_generate    : the loops at :885-890; h_out u32 [batch][n_tokens], h_counts i32 [batch] ids
+ *                  emitted per sequence (stops before eos_id unless ignore_eos).              */
+typedef struct kx_model kx_model;
+int kx_model_bytes(const kx_config *cfg, uint64_t *weights, uint64_t *kv_cache, uint64_t *scratch);
+int kx_model_create(const kx_config *cfg, kx_model **model);
+int kx_model_destroy(kx_model *model);
+int kx_prefill(kx_model *model, const uint32_t *h_ids, int32_t batch, int32_t prompt_len);
+int kx_decode_step(kx_model *model, const uint32_t *h_ids);
+int kx_greedy_sample(kx_model *model, uint32_t *h_out);
+int kx_generate(kx_model *model, const uint32_t *h_prompt, int32_t batch, int32_t prompt_len,
+                int32_t n_tokens, int ignore_eos, uint32_t *h_out, int32_t *h_counts);
+/* views for parity checks (synchronise): residual stream bf16 [batch][hidden], logits f32
+ * [batch][vocab] of the last sampled step, latent cache rows bf16 [n][kv_rank+qk_rope]         */
+int kx_model_hidden(kx_model *model, uint16_t *h_out);
+int kx_model_logits(kx_model *model, float *h_out);
+int kx_model_latent(kx_model *model, int32_t layer, int32_t seq_index, int32_t pos0, int32_t n, uint16_t *h_out);
+/* ms of GPU time of the last kx_generate: [0] prefill, [1] decode steps                         */
+int kx_model_timing(kx_model *model, float *ms2);
+/* bf(mean + sigma*z) fill used for the norm weights */
+int kx_fill_affine_bf16(void *d_out, uint64_t n, uint64_t seed, uint64_t tensor_id, float mean,
+                        float sigma, void *stream);
 
 #ifdef __cplusplus
 }

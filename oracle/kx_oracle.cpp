@@ -136,6 +136,17 @@ void ox_fill_normal_bf16(uint16_t *out, uint64_t n, uint64_t seed, uint64_t tid,
     out[i] = absval ? (uint16_t)(h & 0x7fff) : h;
   }
 }
+// bf(mean + sigma*z): the norm weights of the random-init stack
+void ox_fill_affine_bf16(uint16_t *out, uint64_t n, uint64_t seed, uint64_t tid, float mean, float sigma) {
+  uint64_t key = rng_key(seed, tid);
+#pragma omp parallel for schedule(static)
+  for (int64_t i = 0; i < (int64_t)n; ++i) out[i] = bf16_bits(mean + rng_normal_f32(key, (uint64_t)i, sigma));
+}
+// token ids uniform in [0, vocab)
+void ox_fill_tokens_u32(uint32_t *out, uint64_t n, uint64_t seed, uint64_t tid, uint32_t vocab) {
+  uint64_t key = rng_key(seed, tid);
+  for (uint64_t i = 0; i < n; ++i) out[i] = (uint32_t)(rng_u64(key, i) % vocab);
+}
 void ox_fill_normal_f32(float *out, uint64_t n, uint64_t seed, uint64_t tid, float sigma) {
   uint64_t key = rng_key(seed, tid);
 #pragma omp parallel for schedule(static)
@@ -440,6 +451,465 @@ void ox_moe_layer(const ox_moe_weights *w, const uint16_t *n, uint16_t *x, int t
     }
   }
 }
+
+// ---------------------------------------------------------------------------------
+// RoPE / YaRN tables (:325-357) and the softmax scale (:428-429)
+// ---------------------------------------------------------------------------------
+struct ox_config {  // same layout as kx_config (include/kx.h)
+  int32_t n_layers, first_dense, hidden, heads, qk_nope, qk_rope, v_head, q_rank, kv_rank, experts, topk,
+      moe_inter, shared_inter, dense_inter, vocab, max_batch, max_context;
+  uint32_t eos_id;
+  float rms_eps, rope_theta, routed_scale, yarn_factor, yarn_beta_fast, yarn_beta_slow, yarn_orig_ctx,
+      yarn_mscale_all_dim, init_sigma, expert_scale_sigma;
+  uint64_t seed;
+};
+
+static float yarn_correction_dim(const ox_config *c, float rotations, float dim) {  // :325-327
+  volatile float two_pi = 2.0f * 3.14159265358979323846f;
+  return dim * logf(c->yarn_orig_ctx / (rotations * two_pi)) / (2.0f * logf(c->rope_theta));
+}
+static float yarn_ramp(float low, float high, float at) {  // :329-332
+  if (low == high) high += 0.001f;
+  return fminf(1.0f, fmaxf(0.0f, (at - low) / (high - low)));
+}
+float ox_yarn_inv_freq(const ox_config *c, int pair) {  // :334-344
+  float dim = (float)c->qk_rope;
+  float freq_extra = powf(c->rope_theta, -2.0f * (float)pair / dim);
+  float freq_inter = freq_extra / c->yarn_factor;
+  float low = floorf(yarn_correction_dim(c, c->yarn_beta_fast, dim));
+  float high = ceilf(yarn_correction_dim(c, c->yarn_beta_slow, dim));
+  low = fmaxf(low, 0.0f);
+  high = fminf(high, dim - 1.0f);
+  float inv_freq_mask = 1.0f - yarn_ramp(low, high, (float)pair);
+  return freq_inter * (1.0f - inv_freq_mask) + freq_extra * inv_freq_mask;
+}
+// table row of a position: qk_rope/2 cosines then qk_rope/2 sines, rounded to bf16 (:351)
+void ox_rope_table(const ox_config *c, int pos0, int n, uint16_t *out) {
+  int half = c->qk_rope / 2;
+  for (int i = 0; i < n; ++i)
+    for (int p = 0; p < half; ++p) {
+      float freq = ox_yarn_inv_freq(c, p);
+      float ang = (float)(pos0 + i) * freq;
+      out[(size_t)i * c->qk_rope + p] = bf16_bits(cosf(ang));
+      out[(size_t)i * c->qk_rope + half + p] = bf16_bits(sinf(ang));
+    }
+}
+// the two factors of the score scale: rsqrt(qk_nope+qk_rope) and mscale (:428-429)
+void ox_softmax_scale(const ox_config *c, float *rs, float *mscale) {
+  *rs = rsqrt_o((float)(c->qk_nope + c->qk_rope));
+  *mscale = 0.1f * c->yarn_mscale_all_dim * logf(c->yarn_factor) + 1.0f;
+}
+// interleaved-pair rotation: reads (2p, 2p+1), writes (p, half+p) (:352-356); x, y f32 of bf16 values
+static void rope_apply(const float *x, float *y, const uint16_t *tab, int rotary) {
+  int half = rotary / 2;
+  for (int p = 0; p < half; ++p) {
+    float c = bf16_val(tab[p]), s = bf16_val(tab[half + p]);
+    float x0 = x[2 * p], x1 = x[2 * p + 1];
+    y[p] = bf(bf(x0 * c) - bf(x1 * s));
+    y[half + p] = bf(bf(x1 * c) + bf(x0 * s));
+  }
+}
+
+// ---------------------------------------------------------------------------------
+// The decoder stack: run() / generate() (:780-893)
+// ---------------------------------------------------------------------------------
+enum {  // tensor ids: global tensors use the id itself, layer L uses (L+1)*64 + id
+  TID_EMBED = 1, TID_FINAL_NORM = 2, TID_LM_HEAD = 3, TID_PROMPT = 4,
+  TL_INPUT_LN = 0, TL_QA = 1, TL_QA_LN = 2, TL_QB = 3, TL_KVA = 4, TL_KV_LN = 5, TL_KVB = 6, TL_O = 7, TL_POST_LN = 8,
+  TL_DENSE_GATE = 9, TL_DENSE_UP = 10, TL_DENSE_DOWN = 11, TL_ROUTER = 12, TL_ROUTER_BIAS = 13,
+  TL_GATE_P = 14, TL_GATE_S = 15, TL_UP_P = 16, TL_UP_S = 17, TL_DOWN_P = 18, TL_DOWN_S = 19,
+  TL_SH_GATE = 20, TL_SH_UP = 21, TL_SH_DOWN = 22
+};
+
+struct OxLayer {
+  std::vector<uint16_t> input_ln, qa, qa_ln, qb, kva, kv_ln, kvb, o, post_ln;
+  std::vector<uint16_t> dgate, dup, ddown;
+  std::vector<uint16_t> router, gate_s, up_s, down_s, sh_gate, sh_up, sh_down;
+  std::vector<float> router_bias;
+  std::vector<uint32_t> gate_p, up_p, down_p;
+  // latent cache [B][max_context][kv_rank + qk_rope] bf16; mode 0 also keeps the expanded
+  // fp32 K [B][ctx][heads*(nope+rope)] and V [B][ctx][heads*v_head] of the reference (:192-238)
+  std::vector<uint16_t> latent;
+  std::vector<float> K, V;
+};
+
+struct ox_model {
+  ox_config c;
+  int mode;
+  float expert_scale_sigma;
+  std::vector<uint16_t> embed, final_norm, lm_head, rope_tab;
+  std::vector<OxLayer> layers;
+  std::vector<uint16_t> x;  // residual stream [B][hidden]
+  std::vector<float> last_logits;  // [B][vocab] bf16-rounded logits of the last sampled step
+};
+
+static void fill_bf16(std::vector<uint16_t> &v, size_t n, uint64_t seed, uint64_t tid, float sigma, int absval = 0) {
+  v.resize(n);
+  ox_fill_normal_bf16(v.data(), n, seed, tid, sigma, absval);
+}
+static void fill_ln(std::vector<uint16_t> &v, size_t n, uint64_t seed, uint64_t tid) {
+  v.resize(n);
+  ox_fill_affine_bf16(v.data(), n, seed, tid, 1.0f, 0.02f);
+}
+static void fill_words(std::vector<uint32_t> &v, size_t n, uint64_t seed, uint64_t tid) {
+  v.resize(n);
+  ox_fill_words_u32(v.data(), n, seed, tid);
+}
+
+ox_model *ox_model_create(const ox_config *cfg, int mode) {
+  const float expert_scale_sigma = cfg->expert_scale_sigma;
+  ox_model *m = new ox_model();
+  m->c = *cfg;
+  m->mode = mode;
+  m->expert_scale_sigma = expert_scale_sigma;
+  const ox_config &c = m->c;
+  const size_t H = c.hidden, V = c.vocab, E = c.experts, I = c.moe_inter, SI = c.shared_inter, D = c.dense_inter;
+  const size_t KD = (size_t)c.heads * (c.qk_nope + c.qk_rope), VD = (size_t)c.heads * c.v_head;
+  const size_t KVA = c.kv_rank + c.qk_rope, KVB = (size_t)c.heads * (c.qk_nope + c.v_head);
+  const float sg = c.init_sigma;
+  fill_bf16(m->embed, V * H, c.seed, TID_EMBED, 1.0f);
+  fill_ln(m->final_norm, H, c.seed, TID_FINAL_NORM);
+  fill_bf16(m->lm_head, V * H, c.seed, TID_LM_HEAD, sg);
+  m->rope_tab.resize((size_t)c.max_context * c.qk_rope);
+  ox_rope_table(&c, 0, c.max_context, m->rope_tab.data());
+  m->layers.resize(c.n_layers);
+  for (int l = 0; l < c.n_layers; ++l) {
+    OxLayer &L = m->layers[l];
+    const uint64_t b = (uint64_t)(l + 1) * 64;
+    fill_ln(L.input_ln, H, c.seed, b + TL_INPUT_LN);
+    fill_bf16(L.qa, (size_t)c.q_rank * H, c.seed, b + TL_QA, sg);
+    fill_ln(L.qa_ln, c.q_rank, c.seed, b + TL_QA_LN);
+    fill_bf16(L.qb, KD * c.q_rank, c.seed, b + TL_QB, sg);
+    fill_bf16(L.kva, KVA * H, c.seed, b + TL_KVA, sg);
+    fill_ln(L.kv_ln, c.kv_rank, c.seed, b + TL_KV_LN);
+    fill_bf16(L.kvb, KVB * c.kv_rank, c.seed, b + TL_KVB, sg);
+    fill_bf16(L.o, H * VD, c.seed, b + TL_O, sg);
+    fill_ln(L.post_ln, H, c.seed, b + TL_POST_LN);
+    if (l < c.first_dense) {
+      fill_bf16(L.dgate, D * H, c.seed, b + TL_DENSE_GATE, sg);
+      fill_bf16(L.dup, D * H, c.seed, b + TL_DENSE_UP, sg);
+      fill_bf16(L.ddown, H * D, c.seed, b + TL_DENSE_DOWN, sg);
+    } else {
+      fill_bf16(L.router, E * H, c.seed, b + TL_ROUTER, 1.0f / sqrtf((float)H));
+      L.router_bias.resize(E);
+      ox_fill_normal_f32(L.router_bias.data(), E, c.seed, b + TL_ROUTER_BIAS, 0.01f);
+      fill_words(L.gate_p, E * I * H / 8, c.seed, b + TL_GATE_P);
+      fill_bf16(L.gate_s, E * I * H / 32, c.seed, b + TL_GATE_S, expert_scale_sigma, 1);
+      fill_words(L.up_p, E * I * H / 8, c.seed, b + TL_UP_P);
+      fill_bf16(L.up_s, E * I * H / 32, c.seed, b + TL_UP_S, expert_scale_sigma, 1);
+      fill_words(L.down_p, E * H * I / 8, c.seed, b + TL_DOWN_P);
+      fill_bf16(L.down_s, E * H * I / 32, c.seed, b + TL_DOWN_S, expert_scale_sigma, 1);
+      fill_bf16(L.sh_gate, SI * H, c.seed, b + TL_SH_GATE, sg);
+      fill_bf16(L.sh_up, SI * H, c.seed, b + TL_SH_UP, sg);
+      fill_bf16(L.sh_down, H * SI, c.seed, b + TL_SH_DOWN, sg);
+    }
+    L.latent.assign((size_t)c.max_batch * c.max_context * KVA, 0);
+    if (!mode) {
+      L.K.assign((size_t)c.max_batch * c.max_context * KD, 0.0f);
+      L.V.assign((size_t)c.max_batch * c.max_context * VD, 0.0f);
+    }
+  }
+  m->x.assign((size_t)c.max_batch * H, 0);
+  m->last_logits.assign((size_t)c.max_batch * V, 0.0f);
+  return m;
+}
+void ox_model_destroy(ox_model *m) { delete m; }
+
+// y = bf(W x) for one token through the selected schedule
+static void mv(const ox_model *m, const std::vector<uint16_t> &w, const uint16_t *x, uint16_t *y, int rows, int cols) {
+  ox_gemv_bf16(w.data(), x, y, rows, cols, 1, 0, m->mode);
+}
+
+// softmax + PV of the reference over the expanded fp32 K/V of one sequence (:692-716), 64-position tiles
+static void attn_ref(const ox_model *m, const OxLayer &L, int b, int seq, const float *q_rot, uint16_t *out) {
+  const ox_config &c = m->c;
+  const int QK = c.qk_nope + c.qk_rope, KD = c.heads * QK, VD = c.heads * c.v_head;
+  float rs, ms;
+  ox_softmax_scale(&c, &rs, &ms);
+  const float *Kb = &L.K[(size_t)b * c.max_context * KD], *Vb = &L.V[(size_t)b * c.max_context * VD];
+#pragma omp parallel for schedule(static)
+  for (int h = 0; h < c.heads; ++h) {
+    std::vector<float> sc(seq);
+    for (int t = 0; t < seq; ++t) {  // attn_tile_score_k (:414-431)
+      float s[256];
+      for (int i = 0; i < 256; ++i) {
+        float v = 0;
+        for (int j = i; j < QK; j += 256) v = fmaf(q_rot[h * QK + j], Kb[(size_t)t * KD + h * QK + j], v);
+        s[i] = v;
+      }
+      sc[t] = bf(bf(tree256(s)) * rs * ms * ms);
+    }
+    float mx = -INFINITY;
+    for (int t = 0; t < seq; ++t) mx = fmaxf(mx, sc[t]);  // :433-445
+    float sum = 0;
+    for (int start = 0; start < seq; start += 64) {  // attn_tile_sum_k (:447-459), tile sums added in order
+      int n = std::min(64, seq - start);
+      float s[256];
+      for (int i = 0; i < 256; ++i) s[i] = i < n ? expf(sc[start + i] - mx) : 0.0f;
+      sum += tree256(s);
+    }
+    for (int d = 0; d < c.v_head; ++d) {  // attn_tile_accum_k (:461-470) + attn_finish_k (:472-475)
+      float o = 0;
+      for (int start = 0; start < seq; start += 64) {
+        int n = std::min(64, seq - start);
+        float acc = 0;
+        for (int t = 0; t < n; ++t) {
+          float p = bf(expf(sc[start + t] - mx) / sum);
+          acc = fmaf(p, Vb[(size_t)(start + t) * VD + h * c.v_head + d], acc);
+        }
+        o += acc;
+      }
+      out[h * c.v_head + d] = bf16_bits(o);
+    }
+  }
+}
+
+// micro-tiles per span of the kx attention schedule: a function of the sequence length only
+int ox_mla_span_tiles(int seq) {
+  int tiles = (seq + 63) / 64, st = 1;
+  while (tiles > 64 * st) st *= 2;
+  return st;
+}
+
+// absorbed attention in the kx schedule over the latent cache of one sequence.
+// cache bf16 [seq][kv_rank + qk_rope]; qabs f32 [heads][kv_rank + qk_rope] (bf16 values):
+// W_UK^T q_nope then rotated q_rope.  out: o_lat bf16 [heads][kv_rank].
+static void attn_kx_seq(const ox_config &c, const uint16_t *cache, int seq, const float *qabs, uint16_t *o_lat) {
+  const int R = c.kv_rank, KVA = c.kv_rank + c.qk_rope;
+  float rs, ms;
+  ox_softmax_scale(&c, &rs, &ms);
+  const int tiles = (seq + 63) / 64, st = ox_mla_span_tiles(seq), spans = (tiles + st - 1) / st;
+#pragma omp parallel for schedule(static)
+  for (int h = 0; h < c.heads; ++h) {
+    const float *q = qabs + (size_t)h * KVA;
+    std::vector<float> pm(spans), pz(spans), po((size_t)spans * R);
+    for (int sp = 0; sp < spans; ++sp) {
+      float M = -INFINITY, Z = 0.0f;
+      std::vector<float> O(R, 0.0f);
+      for (int tile = sp * st; tile < std::min(tiles, (sp + 1) * st); ++tile) {
+        const int t0 = tile * 64, n = std::min(64, seq - t0);
+        float s[64], p[64];
+        float mt = -INFINITY;
+        for (int l = 0; l < 64; ++l) {
+          if (l < n) {
+            const uint16_t *row = cache + (size_t)(t0 + l) * KVA;
+            float acc = 0.0f;
+            for (int i = 0; i < KVA; ++i) acc = fmaf(bf16_val(row[i]), q[i], acc);
+            s[l] = bf(bf(acc) * rs * ms * ms);
+          } else {
+            s[l] = -INFINITY;
+          }
+          mt = fmaxf(mt, s[l]);
+        }
+        const float Mn = fmaxf(M, mt);
+        const float alpha = exp_kx(M - Mn);
+        for (int l = 0; l < 64; ++l) p[l] = l < n ? exp_kx(s[l] - Mn) : 0.0f;
+        float pp[64];
+        memcpy(pp, p, sizeof pp);
+        const float zt = butterfly(pp, 64);
+        Z = fmaf(Z, alpha, zt);
+        for (int i = 0; i < R; ++i) {
+          float o = O[i] * alpha;
+          for (int l = 0; l < n; ++l) o = fmaf(bf(p[l]), bf16_val(cache[(size_t)(t0 + l) * KVA + i]), o);
+          O[i] = o;
+        }
+        M = Mn;
+      }
+      pm[sp] = M; pz[sp] = Z;
+      memcpy(&po[(size_t)sp * R], O.data(), sizeof(float) * R);
+    }
+    float M = -INFINITY;
+    for (int sp = 0; sp < spans; ++sp) M = fmaxf(M, pm[sp]);
+    float Z = 0.0f;
+    std::vector<float> O(R, 0.0f);
+    for (int sp = 0; sp < spans; ++sp) {
+      const float w = exp_kx(pm[sp] - M);
+      Z = fmaf(pz[sp], w, Z);
+      for (int i = 0; i < R; ++i) O[i] = fmaf(po[(size_t)sp * R + i], w, O[i]);
+    }
+    for (int i = 0; i < R; ++i) o_lat[(size_t)h * R + i] = bf16_bits(O[i] / Z);
+  }
+}
+// the same attention with the reference's three passes and rounding points (:414-475) applied to the
+// absorbed operands: s = bf(bf(q.k)*scale); m = max; Z = sum expf(s-m); p = bf(expf(s-m)/Z); o = bf(sum p*c)
+static void attn_ref_absorbed_seq(const ox_config &c, const uint16_t *cache, int seq, const float *qabs, uint16_t *o_lat) {
+  const int R = c.kv_rank, KVA = c.kv_rank + c.qk_rope;
+  float rs, ms;
+  ox_softmax_scale(&c, &rs, &ms);
+#pragma omp parallel for schedule(static)
+  for (int h = 0; h < c.heads; ++h) {
+    const float *q = qabs + (size_t)h * KVA;
+    std::vector<float> s(seq);
+    float m = -INFINITY;
+    for (int t = 0; t < seq; ++t) {
+      float acc = 0.0f;
+      for (int i = 0; i < KVA; ++i) acc = fmaf(bf16_val(cache[(size_t)t * KVA + i]), q[i], acc);
+      s[t] = bf(bf(acc) * rs * ms * ms);
+      m = fmaxf(m, s[t]);
+    }
+    float Z = 0.0f;
+    for (int t = 0; t < seq; ++t) Z += expf(s[t] - m);
+    std::vector<float> O(R, 0.0f);
+    for (int t = 0; t < seq; ++t) {
+      const float p = bf(expf(s[t] - m) / Z);
+      for (int i = 0; i < R; ++i) O[i] = fmaf(p, bf16_val(cache[(size_t)t * KVA + i]), O[i]);
+    }
+    for (int i = 0; i < R; ++i) o_lat[(size_t)h * R + i] = bf16_bits(O[i]);
+  }
+}
+// BASELINE config 3 as an operator: cache bf16, sequence b at cache + b*seq_stride; qabs f32
+// [batch][heads][kv_rank+qk_rope]; o_lat bf16 [batch][heads][kv_rank]
+void ox_mla_decode(const ox_config *c, const uint16_t *cache, size_t seq_stride, const float *qabs, uint16_t *o_lat,
+                   int batch, int seq, int mode) {
+  const size_t KVA = c->kv_rank + c->qk_rope;
+  for (int b = 0; b < batch; ++b) {
+    const uint16_t *cb = cache + (size_t)b * seq_stride;
+    const float *qb = qabs + (size_t)b * c->heads * KVA;
+    uint16_t *ob = o_lat + (size_t)b * c->heads * c->kv_rank;
+    if (mode) attn_kx_seq(*c, cb, seq, qb, ob);
+    else attn_ref_absorbed_seq(*c, cb, seq, qb, ob);
+  }
+}
+static void attn_kx(const ox_model *m, const OxLayer &L, int b, int seq, const float *qabs, uint16_t *o_lat) {
+  const size_t KVA = m->c.kv_rank + m->c.qk_rope;
+  attn_kx_seq(m->c, &L.latent[(size_t)b * m->c.max_context * KVA], seq, qabs, o_lat);
+}
+
+// one decode step of every sequence in the batch at position pos (:801-884); returns sampled ids if sample
+static void model_step(ox_model *m, const uint32_t *ids, int B, int pos, int sample, uint32_t *out_ids) {
+  const ox_config &c = m->c;
+  const int H = c.hidden, QK = c.qk_nope + c.qk_rope, KD = c.heads * QK, VD = c.heads * c.v_head;
+  const int KVA = c.kv_rank + c.qk_rope, R = c.kv_rank, mode = m->mode;
+  const uint16_t *tab = &m->rope_tab[(size_t)pos * c.qk_rope];
+  std::vector<uint16_t> n(H), qa(c.q_rank), q(KD), kva(KVA), att(VD), o(H), tmp;
+  for (int b = 0; b < B; ++b) {
+    uint16_t *x = &m->x[(size_t)b * H];
+    memcpy(x, &m->embed[(size_t)ids[b] * H], (size_t)H * 2);  // embed_token (:651-655)
+    for (int l = 0; l < c.n_layers; ++l) {
+      OxLayer &L = m->layers[l];
+      rmsnorm_row(x, L.input_ln.data(), n.data(), H, c.rms_eps, mode);                       // :812
+      mv(m, L.qa, n.data(), qa.data(), c.q_rank, H);                                          // :813
+      { std::vector<uint16_t> t(qa); rmsnorm_row(t.data(), L.qa_ln.data(), qa.data(), c.q_rank, c.rms_eps, mode); }  // :814
+      mv(m, L.qb, qa.data(), q.data(), KD, c.q_rank);                                         // :815
+      mv(m, L.kva, n.data(), kva.data(), KVA, H);                                             // :816
+      { std::vector<uint16_t> t(kva.begin(), kva.begin() + R);
+        rmsnorm_row(t.data(), L.kv_ln.data(), kva.data(), R, c.rms_eps, mode); }              // :817 (first kv_rank only)
+      // RoPE on the shared k_rope and on every head's q_rope (:346-357)
+      std::vector<float> kr_in(c.qk_rope), kr(c.qk_rope), qf(KD), q_rot(KD);
+      for (int i = 0; i < c.qk_rope; ++i) kr_in[i] = bf16_val(kva[R + i]);
+      rope_apply(kr_in.data(), kr.data(), tab, c.qk_rope);
+      for (int i = 0; i < KD; ++i) qf[i] = bf16_val(q[i]);
+      q_rot = qf;
+      for (int h = 0; h < c.heads; ++h) rope_apply(&qf[h * QK + c.qk_nope], &q_rot[h * QK + c.qk_nope], tab, c.qk_rope);
+      // latent cache row (both modes keep it; identical information to the reference's K/V)
+      uint16_t *lat = &L.latent[((size_t)b * c.max_context + pos) * KVA];
+      memcpy(lat, kva.data(), (size_t)R * 2);
+      for (int i = 0; i < c.qk_rope; ++i) lat[R + i] = bf16_bits(kr[i]);
+      if (!mode) {
+        // kv_b projection, split into K nope and V, K rope broadcast to every head (:818-820), stored as fp32 (:824)
+        std::vector<uint16_t> kv((size_t)c.heads * (c.qk_nope + c.v_head));
+        mv(m, L.kvb, kva.data(), kv.data(), c.heads * (c.qk_nope + c.v_head), R);
+        float *Kp = &L.K[((size_t)b * c.max_context + pos) * KD], *Vp = &L.V[((size_t)b * c.max_context + pos) * VD];
+        for (int h = 0; h < c.heads; ++h) {
+          for (int d = 0; d < c.qk_nope; ++d) Kp[h * QK + d] = bf16_val(kv[(size_t)h * (c.qk_nope + c.v_head) + d]);
+          for (int d = 0; d < c.qk_rope; ++d) Kp[h * QK + c.qk_nope + d] = kr[d];
+          for (int d = 0; d < c.v_head; ++d) Vp[h * c.v_head + d] = bf16_val(kv[(size_t)h * (c.qk_nope + c.v_head) + c.qk_nope + d]);
+        }
+        attn_ref(m, L, b, pos + 1, q_rot.data(), att.data());                                 // :825
+      } else {
+        // absorbed: q_lat[h][c] = bf(sum_d W_UK[h][d][c] q_nope[h][d]): eight chains over d = j, j+8, ...
+        // then ((0+1)+(2+3))+((4+5)+(6+7))
+        std::vector<float> qabs((size_t)c.heads * KVA);
+#pragma omp parallel for schedule(static)
+        for (int h = 0; h < c.heads; ++h) {
+          for (int cc = 0; cc < R; ++cc) {
+            float ch[8];
+            for (int j = 0; j < 8; ++j) {
+              float acc = 0.0f;
+              for (int d = j; d < c.qk_nope; d += 8)
+                acc = fmaf(bf16_val(L.kvb[((size_t)h * (c.qk_nope + c.v_head) + d) * R + cc]), qf[h * QK + d], acc);
+              ch[j] = acc;
+            }
+            qabs[(size_t)h * KVA + cc] = bf(((ch[0] + ch[1]) + (ch[2] + ch[3])) + ((ch[4] + ch[5]) + (ch[6] + ch[7])));
+          }
+          for (int i = 0; i < c.qk_rope; ++i) qabs[(size_t)h * KVA + R + i] = q_rot[h * QK + c.qk_nope + i];
+        }
+        std::vector<uint16_t> o_lat((size_t)c.heads * R);
+        attn_kx(m, L, b, pos + 1, qabs.data(), o_lat.data());
+        // o[h] = bf(W_UV[h] o_lat[h])
+        for (int h = 0; h < c.heads; ++h)
+          ox_gemv_bf16(&L.kvb[((size_t)h * (c.qk_nope + c.v_head) + c.qk_nope) * R], &o_lat[(size_t)h * R],
+                       &att[(size_t)h * c.v_head], c.v_head, R, 1, 0, 1);
+      }
+      mv(m, L.o, att.data(), o.data(), H, VD);                                                // :826
+      for (int i = 0; i < H; ++i) x[i] = bf16_bits(bf16_val(x[i]) + bf16_val(o[i]));           // :827
+      rmsnorm_row(x, L.post_ln.data(), n.data(), H, c.rms_eps, mode);                         // :829
+      if (l < c.first_dense) {  // bf16_mlp (:674-686) on down = 0
+        const int D = c.dense_inter;
+        std::vector<uint16_t> g(D), u(D), mid(D), y(H);
+        mv(m, L.dgate, n.data(), g.data(), D, H);
+        mv(m, L.dup, n.data(), u.data(), D, H);
+        for (int r = 0; r < D; ++r) mid[r] = bf16_bits(swiglu_m(bf16_val(g[r]), bf16_val(u[r]), mode));
+        mv(m, L.ddown, mid.data(), y.data(), H, D);
+        for (int i = 0; i < H; ++i) {
+          float down = bf(0.0f + bf16_val(y[i]));                                             // :684
+          x[i] = bf16_bits(bf16_val(x[i]) + down);                                            // :877
+        }
+      } else {
+        ox_moe_weights w = {L.router.data(), L.router_bias.data(), L.gate_p.data(), L.gate_s.data(), L.up_p.data(),
+                            L.up_s.data(), L.down_p.data(), L.down_s.data(), L.sh_gate.data(), L.sh_up.data(),
+                            L.sh_down.data()};
+        ox_moe_layer(&w, n.data(), x, 1, H, c.moe_inter, c.shared_inter, c.experts, c.topk, c.routed_scale, 0, mode,
+                     nullptr, nullptr, nullptr, nullptr, nullptr);
+      }
+    }
+    if (sample) {  // final norm, lm_head, lowest-index argmax over bf16-rounded logits (:880-881, :718-734)
+      rmsnorm_row(x, m->final_norm.data(), n.data(), H, c.rms_eps, mode);
+      std::vector<uint16_t> lg(c.vocab);
+      mv(m, m->lm_head, n.data(), lg.data(), c.vocab, H);
+      float best = -INFINITY;
+      uint32_t tok = 0;
+      for (int v = 0; v < c.vocab; ++v) {
+        float f = bf16_val(lg[v]);
+        m->last_logits[(size_t)b * c.vocab + v] = f;
+        if (f > best) best = f, tok = (uint32_t)v;
+      }
+      out_ids[b] = tok;
+    }
+  }
+}
+
+// generate(): prefill token by token, sampling only on the last prompt token, then decode (:885-890).
+// prompt u32 [B][P]; out u32 [B][n_tokens]; counts i32 [B] = ids emitted (generation stops before EOS
+// unless ignore_eos).  Returns 0, or 1 on a bad argument.
+int ox_generate(ox_model *m, const uint32_t *prompt, int B, int P, int n_tokens, int ignore_eos, uint32_t *out,
+                int *counts) {
+  const ox_config &c = m->c;
+  if (B < 1 || B > c.max_batch || P < 1 || n_tokens < 1 || P + n_tokens > c.max_context) return 1;
+  for (int i = 0; i < B * P; ++i)
+    if (prompt[i] >= (uint32_t)c.vocab) return 1;
+  std::vector<uint32_t> cur(B), next(B);
+  for (int i = 0; i < P; ++i) {
+    for (int b = 0; b < B; ++b) cur[b] = prompt[(size_t)b * P + i];
+    model_step(m, cur.data(), B, i, i + 1 == P, next.data());
+  }
+  std::vector<int> done(B, 0);
+  for (int b = 0; b < B; ++b) counts[b] = 0;
+  for (int i = 0; i < n_tokens; ++i) {
+    for (int b = 0; b < B; ++b) {
+      if (!done[b] && !ignore_eos && next[b] == c.eos_id) done[b] = 1;
+      if (!done[b]) out[(size_t)b * n_tokens + counts[b]++] = next[b];
+    }
+    if (i + 1 < n_tokens) {
+      cur = next;
+      model_step(m, cur.data(), B, P + i, 1, next.data());
+    }
+  }
+  return 0;
+}
+const float *ox_model_logits(ox_model *m) { return m->last_logits.data(); }
+const uint16_t *ox_model_hidden(ox_model *m) { return m->x.data(); }
+const uint16_t *ox_model_latent(ox_model *m, int layer) { return m->layers[layer].latent.data(); }
 
 int ox_num_threads(void) {
 #ifdef _OPENMP

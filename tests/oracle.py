@@ -37,6 +37,19 @@ _SIGS = {
     "ox_bucket": ([_P, _I, _I, _I, _P, _P, _P, _P], _I),
     "ox_moe_layer": ([C.POINTER(OxMoeWeights), _P, _P, _I, _I, _I, _I, _I, _I, _F, C.c_uint32, _I,
                       _P, _P, _P, _P, _P], None),
+    "ox_fill_affine_bf16": ([_P, _U64, _U64, _U64, _F, _F], None),
+    "ox_fill_tokens_u32": ([_P, _U64, _U64, _U64, C.c_uint32], None),
+    "ox_yarn_inv_freq": ([_P, _I], _F),
+    "ox_rope_table": ([_P, _I, _I, _P], None),
+    "ox_softmax_scale": ([_P, C.POINTER(C.c_float), C.POINTER(C.c_float)], None),
+    "ox_mla_span_tiles": ([_I], _I),
+    "ox_mla_decode": ([_P, _P, C.c_size_t, _P, _P, _I, _I, _I], None),
+    "ox_model_create": ([_P, _I], _P),
+    "ox_model_destroy": ([_P], None),
+    "ox_generate": ([_P, _P, _I, _I, _I, _I, _P, _P], _I),
+    "ox_model_logits": ([_P], C.POINTER(C.c_float)),
+    "ox_model_hidden": ([_P], C.POINTER(C.c_uint16)),
+    "ox_model_latent": ([_P, _I], C.POINTER(C.c_uint16)),
     "ox_num_threads": ([], _I),
     "ox_set_threads": ([_I], None),
 }
@@ -97,3 +110,59 @@ def max_rel(a, b):
     a = np.asarray(a, dtype=np.float64)
     b = np.asarray(b, dtype=np.float64)
     return float(np.max(np.abs(a - b)) / max(np.max(np.abs(b)), 1e-30))
+
+
+def tokens_u32(n, seed, tid, vocab):
+    out = np.empty(n, dtype=np.uint32)
+    load().ox_fill_tokens_u32(ptr(out), n, seed, tid, vocab)
+    return out
+
+
+def small_config(n_layers=3, first_dense=1, batch=1, context=96):
+    """A stack with every feature of the Kimi-K2 one at sizes the scalar oracle finishes in seconds.
+    kv_rank 512 / qk_rope 64 / qk_nope 128 / v_head 128 are the real ones (the attention kernel is built for them)."""
+    from blok_amd.lib import KxConfig
+    c = KxConfig()
+    c.n_layers, c.first_dense = n_layers, first_dense
+    c.hidden, c.heads, c.qk_nope, c.qk_rope, c.v_head = 1024, 8, 128, 64, 128
+    c.q_rank, c.kv_rank, c.experts, c.topk = 512, 512, 16, 4
+    c.moe_inter, c.shared_inter, c.dense_inter, c.vocab = 1024, 512, 1536, 2048
+    c.max_batch, c.max_context, c.eos_id = batch, context, 2047
+    c.rms_eps, c.rope_theta, c.routed_scale = 1e-5, 50000.0, 2.827
+    c.yarn_factor, c.yarn_beta_fast, c.yarn_beta_slow, c.yarn_orig_ctx, c.yarn_mscale_all_dim = 32.0, 32.0, 1.0, 4096.0, 1.0
+    c.init_sigma, c.expert_scale_sigma, c.seed = 0.02, 0.02, 1234
+    return c
+
+
+class OxModel:
+    def __init__(self, cfg, mode):
+        self.cfg, self.lib = cfg, load()
+        self.h = self.lib.ox_model_create(C.byref(cfg), mode)
+
+    def generate(self, prompt, n_tokens, ignore_eos=True):
+        B, P = prompt.shape
+        out = np.zeros((B, n_tokens), dtype=np.uint32)
+        counts = np.zeros(B, dtype=np.int32)
+        rc = self.lib.ox_generate(self.h, ptr(np.ascontiguousarray(prompt)), B, P, n_tokens, int(ignore_eos), ptr(out), ptr(counts))
+        return rc, out, counts
+
+    def logits(self, B):
+        p = self.lib.ox_model_logits(self.h)
+        return np.ctypeslib.as_array(p, shape=(self.cfg.max_batch, self.cfg.vocab))[:B].copy()
+
+    def hidden(self, B):
+        p = self.lib.ox_model_hidden(self.h)
+        return np.ctypeslib.as_array(p, shape=(self.cfg.max_batch, self.cfg.hidden))[:B].copy()
+
+    def latent(self, layer):
+        p = self.lib.ox_model_latent(self.h, layer)
+        kva = self.cfg.kv_rank + self.cfg.qk_rope
+        return np.ctypeslib.as_array(p, shape=(self.cfg.max_batch, self.cfg.max_context, kva)).copy()
+
+    def close(self):
+        if self.h:
+            self.lib.ox_model_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        self.close()
