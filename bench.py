@@ -3,12 +3,15 @@
 
 One "step" is one pass of the hot path over one batch of synthetic input that is
 already resident in HBM.  Workloads (BASELINE.json configs):
-  moe_layer : config 2, one routed-MoE decode layer at Kimi-K2 shape for T tokens.
-              Weights of several independent layers are cycled so that neither L2
+  stack     : (default) config 5, the truncated Kimi-K2-shaped stack: a step is one greedy
+              decode step of `--batch` sequences after a `--prompt`-token prompt.  `value` is
+              its decode tok/s.  The same run then times config 2 (one MoE decode layer,
+              T = batch, cold weights) for `roofline`, whose dominant kernel is the fused INT4
+              gate/up GEMV, and the scalar oracle on a bounded sample for `cpu_baseline`.
+  moe_layer : config 2 alone, one routed-MoE decode layer at Kimi-K2 shape for `--tokens`
+              tokens.  Weights of several independent layers are cycled so that neither L2
               nor the 256 MB Infinity Cache can serve them.
-Prints ONE JSON line with the fields the driver reads plus `roofline` (dominant
-kernel: the fused INT4 gate/up GEMV) and `cpu_baseline` (the scalar oracle timed
-on this box's host cores).
+Prints ONE JSON line.
 """
 import argparse
 import ctypes as C
@@ -96,7 +99,7 @@ class MoeLayerSet:
         return out
 
 
-def run_moe_layer(args):
+def run_moe_layer(args, emit=True):
     import oracle as O
     from blok_amd.lib import DevBuf, check, default_config, kx
     lib = kx()
@@ -207,15 +210,144 @@ def run_moe_layer(args):
         "wall_ms_per_step": round(wall_ms / args.steps, 5),
         "cpu_baseline": cpu,
     }
+    if emit:
+        print(json.dumps(out), flush=True)
+    return out
+
+
+def stack_bytes_per_token(cfg, distinct_per_layer):
+    """Algorithmic HBM bytes of one batch-1 decode step of the truncated stack (weights read once)."""
+    H, V = cfg.hidden, cfg.vocab
+    KD, VD = cfg.heads * (cfg.qk_nope + cfg.qk_rope), cfg.heads * cfg.v_head
+    KVA, KVB = cfg.kv_rank + cfg.qk_rope, cfg.heads * (cfg.qk_nope + cfg.v_head)
+    attn = 2 * ((cfg.q_rank + KVA) * H + KD * cfg.q_rank + KVB * cfg.kv_rank + H * VD)
+    dense = 2 * 3 * cfg.dense_inter * H
+    per_matrix = cfg.moe_inter * H // 2 + cfg.moe_inter * H // 32 * 2
+    moe = distinct_per_layer * 3 * per_matrix + 2 * 3 * cfg.shared_inter * H + 2 * cfg.experts * H
+    n_moe = cfg.n_layers - cfg.first_dense
+    return cfg.n_layers * attn + cfg.first_dense * dense + n_moe * moe + 2 * V * H
+
+
+def run_stack(args):
+    """BASELINE config 5: the truncated Kimi-K2-shaped stack, greedy decode after a uniform-random prompt."""
+    import oracle as O
+    from blok_amd.lib import check, default_config, kx
+    lib = kx()
+    cfg = default_config()
+    B, P, K, W = args.batch, args.prompt, args.steps, args.warmup
+    cfg.n_layers, cfg.max_batch, cfg.max_context, cfg.seed = args.stack_layers, B, P + K + W + 1, args.seed
+    name = C.create_string_buffer(256)
+    cus, hbm = C.c_int32(), C.c_uint64()
+    check(lib.kx_device_info(name, 256, C.byref(cus), C.byref(hbm)))
+    wb, cb, sb = C.c_uint64(), C.c_uint64(), C.c_uint64()
+    check(lib.kx_model_bytes(C.byref(cfg), C.byref(wb), C.byref(cb), C.byref(sb)))
+    t0 = time.perf_counter()
+    model = C.c_void_p()
+    check(lib.kx_model_create(C.byref(cfg), C.byref(model)))
+    t_create = time.perf_counter() - t0
+    st = C.c_void_p()
+    check(lib.kx_model_stream(model, C.byref(st)))
+    prompt = O.tokens_u32(B * P, args.seed, 4, cfg.vocab).reshape(B, P)
+    e = [C.c_void_p() for _ in range(3)]
+    for ev in e:
+        check(lib.kx_event_create(C.byref(ev)))
+    check(lib.kx_event_record(e[0], st))
+    check(lib.kx_prefill(model, prompt.ctypes.data, B, P))
+    for _ in range(W):
+        check(lib.kx_decode_step(model, None))
+    check(lib.kx_event_record(e[1], st))
+    check(lib.kx_sync(st))
+    t0 = time.perf_counter()
+    ids = np.zeros((K, B), dtype=np.uint32)
+    for i in range(K):                      # K timed decode steps; ids stay on the device
+        check(lib.kx_decode_step(model, None))
+    check(lib.kx_event_record(e[2], st))
+    check(lib.kx_sync(st))
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    ms_pre, ms_dec = C.c_float(), C.c_float()
+    check(lib.kx_event_elapsed_ms(e[0], e[1], C.byref(ms_pre)))
+    check(lib.kx_event_elapsed_ms(e[1], e[2], C.byref(ms_dec)))
+    last = np.zeros(B, dtype=np.uint32)
+    check(lib.kx_greedy_sample(model, last.ctypes.data))
+    check(lib.kx_model_destroy(model))
+    ms_per_step = ms_dec.value / K
+    toks = B * 1e3 / ms_per_step
+    algo = stack_bytes_per_token(cfg, cfg.topk) if B == 1 else None
+    return {
+        "value": round(toks, 2), "ms_per_step": round(ms_per_step, 5), "wall_ms_per_step": round(wall_ms / K, 5),
+        "prefill_ms_per_token": round(ms_pre.value / (P + W), 5),
+        "workload": f"truncated Kimi-K2 stack (BASELINE config 5): {cfg.n_layers} layers (1 dense + {cfg.n_layers - 1} MoE), "
+                    f"vocab {cfg.vocab}, batch {B}, {P}-token uniform-random prompt prefilled token by token, then "
+                    f"{W} warm-up and {K} timed greedy decode steps; seeded random-init weights resident in HBM",
+        "resident_gb": {"weights": round(wb.value / 1e9, 2), "kv_cache": round(cb.value / 1e9, 3), "scratch": round(sb.value / 1e9, 3)},
+        "model_create_s": round(t_create, 2), "device": name.value.decode(), "compute_units": cus.value,
+        "last_ids": last.tolist(),
+        "stack_hbm": None if algo is None else {"algorithmic_bytes_per_token": int(algo),
+                                                "achieved_gbs": round(algo / (ms_per_step * 1e-3) / 1e9, 1),
+                                                "frac_of_peak": round(algo / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                                                "roof_tok_s": round(HBM_PEAK_GBS * 1e9 / algo, 1)},
+    }
+
+
+def run_cpu_stack(args):
+    """CPU baseline: the oracle's reference schedule on a bounded sample of config 5 (fewer layers, few tokens)."""
+    import oracle as O
+    from blok_amd.lib import default_config
+    cfg = default_config()
+    cfg.n_layers, cfg.max_batch, cfg.max_context, cfg.seed = args.cpu_layers, 1, 64, args.seed
+    P, K = 2, args.cpu_tokens
+    t0 = time.perf_counter()
+    m = O.OxModel(cfg, 0)
+    t_init = time.perf_counter() - t0
+    prompt = O.tokens_u32(P, args.seed, 4, cfg.vocab).reshape(1, P)
+    t0 = time.perf_counter()
+    rc, out, _ = m.generate(prompt, K + 1)      # P prefill steps (one sampled) + K sampled decode steps
+    dt = time.perf_counter() - t0
+    m.close()
+    steps = P + K
+    per_step = dt / steps
+    full = default_config()
+    scaled = per_step * ((full.n_layers - 1) / max(1, cfg.n_layers - 1))
+    return {"value": round(1.0 / per_step, 4), "unit": "tok/s", "cores": O.load().ox_num_threads(), "kind": "port",
+            "sample": f"oracle reference schedule (mode 0), {cfg.n_layers}-layer truncation of config 5 (1 dense + "
+                      f"{cfg.n_layers - 1} MoE, full vocabulary), {steps} token steps in {dt:.1f} s after {t_init:.1f} s of "
+                      f"weight generation; OpenMP over output rows; scaled by MoE-layer count to 24 layers this is about "
+                      f"{1.0 / scaled:.3f} tok/s"}
+
+
+def run_default(args):
+    """Config 5 for `value`, plus the routed INT4 gate/up kernel of config 2 (T = batch) for `roofline`."""
+    stack = run_stack(args)
+    margs = argparse.Namespace(**vars(args))
+    margs.tokens, margs.steps, margs.warmup, margs.no_cpu = args.batch, 40, 8, True
+    moe = run_moe_layer(margs, emit=False)
+    cpu = None if args.no_cpu else run_cpu_stack(args)
+    out = {
+        "metric": "decode tok/s + INT4 expert GEMV HBM GB/s (% of peak), Kimi-K2 shapes, 1 GPU",
+        "value": stack["value"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": stack["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int4 weights x bf16 activations, f32 accumulate", "data": "synthetic",
+        "config": {"workload": stack["workload"], "batch": args.batch, "prompt": args.prompt, "device": stack["device"],
+                   "compute_units": stack["compute_units"], "resident_gb": stack["resident_gb"]},
+        "roofline": moe["roofline"],
+        "int4_expert_gemv": dict(moe["int4_expert_gemv"], workload=moe["config"]["workload"], phase_ms=moe["phase_ms"]),
+        "stack": {k: stack[k] for k in ("wall_ms_per_step", "prefill_ms_per_token", "model_create_s", "stack_hbm", "last_ids")},
+        "cpu_baseline": cpu,
+    }
     print(json.dumps(out), flush=True)
+    return out
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=40)
+    ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--workload", default="moe_layer")
+    ap.add_argument("--workload", default="stack", choices=["stack", "moe_layer"])
+    ap.add_argument("--batch", type=int, default=1)
+    ap.add_argument("--prompt", type=int, default=1024)
+    ap.add_argument("--stack-layers", type=int, default=24)
+    ap.add_argument("--cpu-layers", type=int, default=2)
     ap.add_argument("--tokens", type=int, default=1)
     ap.add_argument("--layers", type=int, default=4, help="independent layers cycled to keep weights cold")
     ap.add_argument("--seed", type=int, default=0)
@@ -230,8 +362,7 @@ def main():
     if args.workload == "moe_layer":
         run_moe_layer(args)
     else:
-        print(f"unknown workload {args.workload}", file=sys.stderr)
-        sys.exit(2)
+        run_default(args)
 
 
 if __name__ == "__main__":

@@ -462,3 +462,8 @@ extern "C" int kx_model_latent(kx_model *m, int32_t layer, int32_t seq_index, in
   KX_HIP(hipStreamSynchronize(m->st));
   return KX_OK;
 }
+extern "C" int kx_model_stream(kx_model *m, void **stream) {
+  KX_REQUIRE(m && stream, "kx_model_stream: null argument");
+  *stream = (void *)m->st;
+  return KX_OK;
+}

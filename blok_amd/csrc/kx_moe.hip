@@ -30,6 +30,7 @@ struct kx_moe_workspace {
   uint16_t *mid;      // [T*topk, moe_inter]
   uint16_t *eout;     // [T*topk, hidden]
   uint16_t *smid;     // [T, shared_inter]
+  uint16_t *sy;       // [T, hidden] shared expert output (prefill path)
   hipEvent_t ev[6];
 };
 
@@ -58,7 +59,7 @@ extern "C" int kx_moe_workspace_create(const kx_config *cfg, int32_t max_tokens,
       {(void **)&ws->counts, E * 4}, {(void **)&ws->offsets, (E + 1) * 4}, {(void **)&ws->pairs, T * K * 4},
       {(void **)&ws->work, E * 16}, {(void **)&ws->n_active, 4},
       {(void **)&ws->mid, T * K * (size_t)cfg->moe_inter * 2}, {(void **)&ws->eout, T * K * (size_t)cfg->hidden * 2},
-      {(void **)&ws->smid, T * (size_t)cfg->shared_inter * 2}};
+      {(void **)&ws->smid, T * (size_t)cfg->shared_inter * 2}, {(void **)&ws->sy, T * (size_t)cfg->hidden * 2}};
   for (auto &al : allocs) {
     hipError_t e = hipMalloc(al.p, al.bytes);
     if (e != hipSuccess) {
@@ -75,7 +76,7 @@ extern "C" int kx_moe_workspace_create(const kx_config *cfg, int32_t max_tokens,
 extern "C" int kx_moe_workspace_destroy(kx_moe_workspace *ws) {
   if (!ws) return KX_OK;
   void *ptrs[] = {ws->logits, ws->ids, ws->weights, ws->counts, ws->offsets, ws->pairs,
-                  ws->work, ws->n_active, ws->mid, ws->eout, ws->smid};
+                  ws->work, ws->n_active, ws->mid, ws->eout, ws->smid, ws->sy};
   for (void *p : ptrs)
     if (p) (void)hipFree(p);
   for (auto &e : ws->ev)
@@ -173,4 +174,42 @@ extern "C" int kx_moe_decode_layer_timed(const kx_config *cfg, const kx_moe_weig
   KX_HIP(hipEventSynchronize(ws->ev[5]));
   for (int i = 0; i < 5; ++i) KX_HIP(hipEventElapsedTime(&ms5[i], ws->ev[i], ws->ev[i + 1]));
   return KX_OK;
+}
+
+// ---- prefill chunk through one MoE layer: grouped GEMMs on the matrix cores ------------------
+extern "C" int kx_moe_prefill_layer(const kx_config *c, const kx_moe_weights *w, kx_moe_workspace *ws, const void *d_n,
+                                    void *d_x, int32_t tokens, uint32_t flags, void *stream) {
+  int rc = check_cfg(c);
+  if (rc) return rc;
+  KX_REQUIRE(w && ws && d_n && d_x, "kx_moe_prefill_layer: null argument");
+  KX_REQUIRE(tokens > 0 && tokens <= ws->max_tokens, "kx_moe_prefill_layer: tokens=%d outside [1, %d]", tokens, ws->max_tokens);
+  KX_REQUIRE(c->hidden == ws->cfg.hidden && c->moe_inter == ws->cfg.moe_inter && c->experts == ws->cfg.experts &&
+                 c->topk == ws->cfg.topk && c->shared_inter == ws->cfg.shared_inter,
+             "kx_moe_prefill_layer: workspace was created for another shape");
+  hipStream_t st = kx_stream(stream);
+  const int H = c->hidden, I = c->moe_inter, SI = c->shared_inter, E = c->experts, K = c->topk;
+  const uint16_t *n = (const uint16_t *)d_n;
+  // router: fp32 logits through the decode GEMV (its summation order is reproducible), top-k, bucketing
+  KxGemvArgs g = {};
+  g.w0 = (const uint16_t *)w->d_router_gate; g.x = n; g.x_stride = H; g.out = ws->logits; g.out_stride = E;
+  g.rows = E; g.cols = H; g.tokens = tokens;
+  if ((rc = kx_gemv_launch(KX_EPI_F32, g, st))) return rc;
+  if ((rc = kx_router_topk_launch(ws->logits, (const float *)w->d_router_bias, ws->ids, ws->weights, tokens, E, K,
+                                  c->routed_scale, st))) return rc;
+  if ((rc = kx_bucket_launch(ws->ids, tokens, E, K, ws->counts, ws->offsets, ws->pairs, ws->work, ws->n_active, st)))
+    return rc;
+  const int n_slots = (long)tokens * K < E ? tokens * K : E;
+  // routed experts: gate/up + SwiGLU, then down
+  if ((rc = kx_grouped_gemm_launch(true, true, w->d_gate_packed, (const uint16_t *)w->d_gate_scale, w->d_up_packed,
+                                   (const uint16_t *)w->d_up_scale, n, ws->mid, ws->work, ws->pairs, 0, n_slots, I, H, K,
+                                   (size_t)I * (H / 8), (size_t)I * (H / 32), st))) return rc;
+  if ((rc = kx_grouped_gemm_launch(false, true, w->d_down_packed, (const uint16_t *)w->d_down_scale, nullptr, nullptr,
+                                   ws->mid, ws->eout, ws->work, ws->pairs, 0, n_slots, H, I, 1, (size_t)H * (I / 8),
+                                   (size_t)H * (I / 32), st))) return rc;
+  // shared expert: one group of all tokens, bf16 weights
+  if ((rc = kx_grouped_gemm_launch(true, false, w->d_shared_gate, nullptr, w->d_shared_up, nullptr, n, ws->smid, nullptr,
+                                   nullptr, tokens, 1, SI, H, 1, 0, 0, st))) return rc;
+  if ((rc = kx_grouped_gemm_launch(false, false, w->d_shared_down, nullptr, nullptr, nullptr, ws->smid, ws->sy, nullptr,
+                                   nullptr, tokens, 1, H, SI, 1, 0, 0, st))) return rc;
+  return kx_moe_combine_launch(ws->eout, ws->weights, ws->sy, (uint16_t *)d_x, tokens, H, K, flags, st);
 }

@@ -158,6 +158,13 @@ int kx_moe_workspace_views(kx_moe_workspace *ws, void **d_logits, void **d_ids, 
  * flags bit0: skip the residual add and write `down` to d_x instead.        */
 int kx_moe_decode_layer(const kx_config *cfg, const kx_moe_weights *w, kx_moe_workspace *ws,
                         const void *d_n, void *d_x, int32_t tokens, uint32_t flags, void *stream);
+/* The same layer for a prefill chunk of T tokens (BASELINE config 4): the tokens of each expert are
+ * gathered into a W4A16 grouped GEMM -- INT4 words dequantized into LDS tiles of bf16 feeding
+ * v_mfma_f32_32x32x16_bf16 with fp32 accumulators -- and the shared expert runs as a bf16 GEMM.
+ * The reference has no batched prefill (one run() per prompt token, :886); per token the result is
+ * that of kx_moe_decode_layer within max-rel 1e-2.                                               */
+int kx_moe_prefill_layer(const kx_config *cfg, const kx_moe_weights *w, kx_moe_workspace *ws,
+                         const void *d_n, void *d_x, int32_t tokens, uint32_t flags, void *stream);
 /* per-phase kernel time of the most recent kx_moe_decode_layer_timed call, ms:
  * [0] router+bucket [1] routed gate/up [2] routed down [3] shared gate/up
  * [4] shared down + combine.  Synchronises.                                 */
@@ -213,6 +220,8 @@ int kx_generate(kx_model *model, const uint32_t *h_prompt, int32_t batch, int32_
 int kx_model_hidden(kx_model *model, uint16_t *h_out);
 int kx_model_logits(kx_model *model, float *h_out);
 int kx_model_latent(kx_model *model, int32_t layer, int32_t seq_index, int32_t pos0, int32_t n, uint16_t *h_out);
+/* the model's private stream (hipStream_t), for event timing around its entry points          */
+int kx_model_stream(kx_model *model, void **stream);
 /* ms of GPU time of the last kx_generate: [0] prefill, [1] decode steps                         */
 int kx_model_timing(kx_model *model, float *ms2);
 /* bf(mean + sigma*z) fill used for the norm weights */

@@ -412,12 +412,21 @@ struct ox_moe_weights {
 // weights f32 [T,topk], mid bf16 [T*topk, moe_inter], eout bf16 [T*topk, hidden].
 void ox_moe_layer(const ox_moe_weights *w, const uint16_t *n, uint16_t *x, int tokens, int hidden, int moe_inter,
                   int shared_inter, int experts, int topk, float routed_scale, uint32_t flags, int mode,
-                  float *o_logits, uint16_t *o_ids, float *o_weights, uint16_t *o_mid, uint16_t *o_eout) {
+                  float *o_logits, uint16_t *o_ids, float *o_weights, uint16_t *o_mid, uint16_t *o_eout);
+static void moe_layer_impl(const ox_moe_weights *w, const uint16_t *n, uint16_t *x, int tokens, int hidden, int moe_inter,
+                           int shared_inter, int experts, int topk, float routed_scale, uint32_t flags, int mode,
+                           float *o_logits, uint16_t *o_ids, float *o_weights, uint16_t *o_mid, uint16_t *o_eout,
+                           const uint16_t *in_ids, const float *in_weights) {
   const int H = hidden, I = moe_inter, SI = shared_inter, E = experts, K = topk;
   std::vector<float> logits((size_t)tokens * E), weights((size_t)tokens * K);
   std::vector<uint16_t> ids((size_t)tokens * K);
-  ox_gemv_bf16(w->router_gate, n, logits.data(), E, H, tokens, 1, mode);  // :838
-  ox_router_topk(logits.data(), w->router_bias, ids.data(), weights.data(), tokens, E, K, routed_scale, mode);
+  if (in_ids) {  // routing decided elsewhere (checked separately): only the expert arithmetic is restated
+    memcpy(ids.data(), in_ids, ids.size() * 2);
+    memcpy(weights.data(), in_weights, weights.size() * 4);
+  } else {
+    ox_gemv_bf16(w->router_gate, n, logits.data(), E, H, tokens, 1, mode);  // :838
+    ox_router_topk(logits.data(), w->router_bias, ids.data(), weights.data(), tokens, E, K, routed_scale, mode);
+  }
   if (o_logits) memcpy(o_logits, logits.data(), logits.size() * 4);
   if (o_ids) memcpy(o_ids, ids.data(), ids.size() * 2);
   if (o_weights) memcpy(o_weights, weights.data(), weights.size() * 4);
@@ -910,6 +919,20 @@ int ox_generate(ox_model *m, const uint32_t *prompt, int B, int P, int n_tokens,
 const float *ox_model_logits(ox_model *m) { return m->last_logits.data(); }
 const uint16_t *ox_model_hidden(ox_model *m) { return m->x.data(); }
 const uint16_t *ox_model_latent(ox_model *m, int layer) { return m->layers[layer].latent.data(); }
+
+void ox_moe_layer(const ox_moe_weights *w, const uint16_t *n, uint16_t *x, int tokens, int hidden, int moe_inter,
+                  int shared_inter, int experts, int topk, float routed_scale, uint32_t flags, int mode,
+                  float *o_logits, uint16_t *o_ids, float *o_weights, uint16_t *o_mid, uint16_t *o_eout) {
+  moe_layer_impl(w, n, x, tokens, hidden, moe_inter, shared_inter, experts, topk, routed_scale, flags, mode, o_logits,
+                 o_ids, o_weights, o_mid, o_eout, nullptr, nullptr);
+}
+// the same layer with the expert ids u16 [T, topk] and routing weights f32 [T, topk] given
+void ox_moe_layer_routed(const ox_moe_weights *w, const uint16_t *n, uint16_t *x, int tokens, int hidden, int moe_inter,
+                         int shared_inter, int experts, int topk, uint32_t flags, int mode, const uint16_t *ids,
+                         const float *weights) {
+  moe_layer_impl(w, n, x, tokens, hidden, moe_inter, shared_inter, experts, topk, 0.0f, flags, mode, nullptr, nullptr,
+                 nullptr, nullptr, nullptr, ids, weights);
+}
 
 int ox_num_threads(void) {
 #ifdef _OPENMP

@@ -50,6 +50,7 @@ _SIGS = {
     "ox_model_logits": ([_P], C.POINTER(C.c_float)),
     "ox_model_hidden": ([_P], C.POINTER(C.c_uint16)),
     "ox_model_latent": ([_P, _I], C.POINTER(C.c_uint16)),
+    "ox_moe_layer_routed": ([C.POINTER(OxMoeWeights), _P, _P, _I, _I, _I, _I, _I, _I, C.c_uint32, _I, _P, _P], None),
     "ox_num_threads": ([], _I),
     "ox_set_threads": ([_I], None),
 }
