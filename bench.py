@@ -169,7 +169,7 @@ def run_moe_layer(args, emit=True):
         ox = O.load()
         host = layers.host_layer(0)
         wo = moe_oracle_weights(host)
-        tc = min(T, args.cpu_tokens)
+        tc = min(T, 4)
         xo = x_host[:tc].copy()
         t0 = time.perf_counter()
         reps = 0
@@ -338,12 +338,63 @@ def run_default(args):
     return out
 
 
+def run_prefill(args):
+    """BASELINE config 4: a 2048-token prefill chunk through one MoE layer on the matrix cores."""
+    import oracle as O
+    from blok_amd.lib import DevBuf, check, default_config, kx
+    lib = kx()
+    cfg = default_config()
+    T = args.tokens
+    layers = MoeLayerSet(lib, cfg, 2, args.seed)
+    # Zipf-like load: bias += c*ln(1/rank)
+    for li, w in enumerate(layers.layers):
+        bias = O.normal_f32(cfg.experts, args.seed + 1000 * li, 11, 0.01) + 0.1 * np.log(1.0 / np.arange(1, cfg.experts + 1))
+        check(lib.kx_h2d(w.d_router_bias, bias.astype(np.float32).ctypes.data, cfg.experts * 4))
+    ws = C.c_void_p()
+    check(lib.kx_moe_workspace_create(C.byref(cfg), T, C.byref(ws)))
+    n_host = O.normal_bf16(T * cfg.hidden, args.seed, 30, 1.0)
+    x_host = O.normal_bf16(T * cfg.hidden, args.seed, 31, 1.0)
+    dn, dx = DevBuf.from_numpy(n_host), DevBuf.from_numpy(x_host)
+    views = [C.c_void_p() for _ in range(8)]
+    check(lib.kx_moe_workspace_views(ws, *[C.byref(v) for v in views]))
+    e0, e1 = C.c_void_p(), C.c_void_p()
+    check(lib.kx_event_create(C.byref(e0)))
+    check(lib.kx_event_create(C.byref(e1)))
+    for i in range(args.warmup):
+        check(lib.kx_moe_prefill_layer(C.byref(cfg), C.byref(layers.layers[i % 2]), ws, dn.ptr, dx.ptr, T, 1, None))
+    check(lib.kx_sync(None))
+    check(lib.kx_event_record(e0, None))
+    for i in range(args.steps):
+        check(lib.kx_moe_prefill_layer(C.byref(cfg), C.byref(layers.layers[i % 2]), ws, dn.ptr, dx.ptr, T, 1, None))
+    check(lib.kx_event_record(e1, None))
+    ms = C.c_float()
+    check(lib.kx_event_elapsed_ms(e0, e1, C.byref(ms)))
+    counts = np.empty(cfg.experts, dtype=np.int32)
+    check(lib.kx_d2h(counts.ctypes.data, views[3].value, counts.nbytes))
+    check(lib.kx_moe_workspace_destroy(ws))
+    ms_step = ms.value / args.steps
+    U = int(np.count_nonzero(counts))
+    by = moe_layer_bytes(cfg, T, U)
+    flops = 2.0 * T * cfg.topk * 3 * cfg.moe_inter * cfg.hidden + 2.0 * T * 3 * cfg.shared_inter * cfg.hidden
+    out = {"metric": "prefill tok/s through one MoE layer (BASELINE config 4)", "value": round(T / (ms_step * 1e-3), 1),
+           "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4),
+           "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "dtype": "int4 weights dequantized to bf16, bf16 MFMA, f32 accumulate", "data": "synthetic",
+           "config": {"workload": f"moe_prefill_layer, T={T}, Zipf-skewed gate bias", "experts_used": U,
+                      "busiest_expert_tokens": int(counts.max())},
+           "roofline": {"bound": "mfma", "achieved": round(flops / (ms_step * 1e-3) / 1e12, 2), "peak": 2500.0,
+                        "unit": "TFLOP/s", "frac": round(flops / (ms_step * 1e-3) / 1e12 / 2500.0, 4), "traffic": None},
+           "hbm_gbs": round(by["layer"] / (ms_step * 1e-3) / 1e9, 1)}
+    print(json.dumps(out), flush=True)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--workload", default="stack", choices=["stack", "moe_layer"])
+    ap.add_argument("--workload", default="stack", choices=["stack", "moe_layer", "prefill"])
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--prompt", type=int, default=1024)
     ap.add_argument("--stack-layers", type=int, default=24)
@@ -352,14 +403,22 @@ def main():
     ap.add_argument("--layers", type=int, default=4, help="independent layers cycled to keep weights cold")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--cpu-tokens", type=int, default=4)
+    ap.add_argument("--cpu-tokens", type=int, default=40)
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
         sys.exit(2)
     build_if_missing()
-    if args.workload == "moe_layer":
+    if args.workload == "prefill":
+        if args.tokens == 1:
+            args.tokens = 2048
+        if args.steps == 256:
+            args.steps = 10
+        run_prefill(args)
+    elif args.workload == "moe_layer":
+        if args.steps == 256:
+            args.steps = 40
         run_moe_layer(args)
     else:
         run_default(args)

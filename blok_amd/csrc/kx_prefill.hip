@@ -74,7 +74,8 @@ __global__ void __launch_bounds__(256) grouped_gemm_k(PfArgs a) {
   const int xr = tid >> 2, xc = (tid & 3) * 16;   // activation tile: row, first of 16 columns
   const int wr = tid >> 1, wg = tid & 1;          // weight tile: row, group (32 columns) of the K step
 
-  for (int m0 = p_begin; m0 < p_end; m0 += BM) {
+  // token tiles of the expert are spread over blockIdx.z
+  for (int m0 = p_begin + blockIdx.z * BM; m0 < p_end; m0 += gridDim.z * BM) {
     kx_f32x16 acc[MATS][2];
 #pragma unroll
     for (int m = 0; m < MATS; ++m)
@@ -163,13 +164,16 @@ __global__ void __launch_bounds__(256) moe_combine_k(const uint16_t *__restrict_
 
 int kx_grouped_gemm_launch(bool dual, bool i4, const void *w0, const uint16_t *s0, const void *w1, const uint16_t *s1,
                            const uint16_t *x, uint16_t *out, const int4 *work, const int *pairs, int n_pairs, int n_slots,
-                           int N, int K, int x_div, size_t expert_w, size_t expert_s, hipStream_t st) {
+                           int N, int K, int x_div, size_t expert_w, size_t expert_s, int n_pairs_max, hipStream_t st) {
   KX_REQUIRE(K > 0 && K % 64 == 0, "kx_grouped_gemm: K=%d must be a positive multiple of 64", K);
   KX_REQUIRE(N > 0, "kx_grouped_gemm: N=%d must be positive", N);
   PfArgs a;
   a.w0 = w0; a.w1 = w1; a.s0 = s0; a.s1 = s1; a.x = x; a.out = out; a.work = work; a.pairs = pairs;
   a.n_pairs = n_pairs; a.N = N; a.K = K; a.x_div = x_div; a.expert_w = expert_w; a.expert_s = expert_s;
-  dim3 g(kx_cdiv(N, BN), work ? n_slots : 1), b(256);
+  const int max_rows = work ? n_pairs_max : n_pairs;
+  int mz = kx_cdiv(max_rows, BM);
+  mz = mz < 1 ? 1 : mz > 64 ? 64 : mz;
+  dim3 g(kx_cdiv(N, BN), work ? n_slots : 1, mz), b(256);
   if (dual && i4) hipLaunchKernelGGL((grouped_gemm_k<true, true>), g, b, 0, st, a);
   else if (dual) hipLaunchKernelGGL((grouped_gemm_k<true, false>), g, b, 0, st, a);
   else if (i4) hipLaunchKernelGGL((grouped_gemm_k<false, true>), g, b, 0, st, a);
