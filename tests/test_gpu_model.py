@@ -184,3 +184,18 @@ def test_mla_decode_operator(kxlib, ox, batch, seq):
     assert O.max_rel(O.bf16_to_f32(got), O.bf16_to_f32(exp0)) < 1e-2
     if seq == 1:
         assert (got == cache[:, 0:1, :R]).all()   # one position: the latent itself
+
+
+def test_executor_json_line(kxlib):
+    import json
+    import os
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    exe = os.path.join(root, "blok_amd", "kx-kimi-exec")
+    r = subprocess.run([exe, "--index", "ignored", "--prompt-tokens", "11,12,13", "--tokens", "3", "--layers", "2", "--seed", "7",
+                        "--ignore-eos"], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr
+    doc = json.loads(r.stdout)                       # blok/runtime.py:88-94
+    assert doc["status"] == "ok" and len(doc["token_ids"]) == 3
+    assert all(isinstance(t, int) and 0 <= t < 163840 for t in doc["token_ids"])
+    assert r.stdout.startswith('{"status":"ok","token_ids":[') and r.stdout.endswith("]}\n")
