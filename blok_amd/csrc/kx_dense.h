@@ -26,6 +26,14 @@ struct KxGemvArgs {
   // output rows [k*row_block, (k+1)*row_block) use weight rows k*w_block_stride + w_block_off + r
   // and the activation row at x + k*x_block_stride.  row_block == 0: plain matrix.
   int row_block, w_block_stride, w_block_off, x_block_stride;
+  // optional prologue: x is RMS-normed with these weights before use (at most 4 tokens);
+  // norm_out, if set, receives the normed rows [tokens][cols]
+  const uint16_t *norm_w;
+  float norm_eps;
+  uint16_t *norm_out;
+  // optional: x[t] of block (head) k is the merge of attention partials, bf(O/Z), instead of a.x
+  const float *mla_pm, *mla_pz, *mla_po;
+  int mla_spans, mla_heads;
   // KX_EPI_MOE_COMBINE
   const uint16_t *expert_out;  // bf16 [tokens*topk, rows]
   const float *route_w;        // f32 [tokens, topk]
@@ -36,7 +44,8 @@ struct KxGemvArgs {
 int kx_gemv_launch(int epi, KxGemvArgs a, hipStream_t st);
 int kx_rmsnorm_launch(const uint16_t *x, const uint16_t *w, uint16_t *y, int tokens, int n, int x_stride,
                       int y_stride, float eps, hipStream_t st);
-int kx_argmax_launch(const float *logits, int tokens, int n, int stride, uint32_t *out, hipStream_t st);
+int kx_argmax_launch(const float *logits, int tokens, int n, int stride, uint32_t *out, float *scratch, hipStream_t st);
+#define KX_ARGMAX_SCRATCH_FLOATS(tokens) ((size_t)(tokens) * 128)
 
 // kx_i4.hip
 int kx_i4_launch(bool dual, const uint32_t *packed0, const uint16_t *scale0, const uint32_t *packed1,
@@ -48,6 +57,9 @@ int kx_i4_launch(bool dual, const uint32_t *packed0, const uint16_t *scale0, con
 // kx_router.hip
 int kx_router_topk_launch(const float *logits, const float *bias, uint16_t *ids, float *weights, int tokens,
                           int experts, int topk, float routed_scale, hipStream_t st);
+int kx_route_launch(const float *logits, const float *bias, uint16_t *ids, float *weights, int tokens, int experts,
+                    int topk, float routed_scale, int *counts, int *offsets, int *pairs, int4 *work, int *n_active,
+                    hipStream_t st);
 int kx_bucket_launch(const uint16_t *ids, int tokens, int experts, int topk, int *counts, int *offsets,
                      int *pairs, int4 *work, int *n_active, hipStream_t st);
 
@@ -57,3 +69,9 @@ int kx_grouped_gemm_launch(bool dual, bool i4, const void *w0, const uint16_t *s
                            int N, int K, int x_div, size_t expert_w, size_t expert_s, int n_pairs_max, hipStream_t st);
 int kx_moe_combine_launch(const uint16_t *eout, const float *rw, const uint16_t *sy, uint16_t *x, int tokens, int hidden,
                           int topk, uint32_t flags, hipStream_t st);
+
+// kx_moe.hip: the decode layer with the post-attention RMSNorm fused into the router GEMV.
+// When norm_w is set, d_x is normed on the fly and the normed rows are written to d_n first.
+struct kx_moe_workspace;
+int kx_moe_layer_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_workspace *ws, void *d_n, void *d_x,
+                        int tokens, uint32_t flags, const uint16_t *norm_w, hipStream_t st, bool timed);

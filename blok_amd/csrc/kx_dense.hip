@@ -93,6 +93,49 @@ __global__ void __launch_bounds__(1024) gemv_bf16_k(KxGemvArgs a) {
   const bool x_once = T <= TT;  // activations stay in registers for the whole chunk
   const uint16_t *wm[2] = {a.w0, MATS == 2 ? a.w1 : a.w0};
 
+  // Optional prologue: RMSNorm of the activation rows (rmsnorm_k's schedule: 256 threads own the
+  // 8-element chunks t, t+256, ...; butterfly per wave; ((w0+w1)+w2)+w3).  Every workgroup
+  // computes the row scales; the normalised values are formed when the activations are loaded.
+  __shared__ float n_ws[4];
+  __shared__ float n_scale[4];
+  if (a.norm_w) {
+    const int chunks = a.cols >> 3;
+    for (int t = 0; t < T; ++t) {
+      const uint16_t *xr = a.x + (size_t)t * a.x_stride;
+      float v = 0.0f;
+      if (threadIdx.x < 256)
+        for (int c = threadIdx.x; c < chunks; c += 256) {
+          float f[8];
+          unpack8(f, ((const uint4 *)xr)[c]);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v = __builtin_fmaf(f[e], f[e], v);
+        }
+      float vv[1] = {v};
+      kxw::reduce<1, 64>(vv, lane);
+      if (lane == 0 && wave < 4) n_ws[wave] = vv[0];
+      __syncthreads();
+      if (threadIdx.x == 0) n_scale[t] = kx_rsqrtf((((n_ws[0] + n_ws[1]) + n_ws[2]) + n_ws[3]) / (float)a.cols + a.norm_eps);
+      __syncthreads();
+    }
+    if (a.norm_out && blockIdx.x == 0)  // one workgroup also stores the normalised rows for later kernels
+      for (int t = 0; t < T; ++t) {
+        const uint16_t *xr = a.x + (size_t)t * a.x_stride;
+        uint16_t *yr = a.norm_out + (size_t)t * a.cols;
+        const float sc = n_scale[t];
+        for (int c = threadIdx.x; c < chunks; c += blockDim.x) {
+          float f[8], g[8];
+          unpack8(f, ((const uint4 *)xr)[c]);
+          unpack8(g, ((const uint4 *)a.norm_w)[c]);
+          uint32_t o[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            o[e] = (uint32_t)kx_bf16_rne(kx_bfround(f[2 * e] * sc) * g[2 * e]) |
+                   ((uint32_t)kx_bf16_rne(kx_bfround(f[2 * e + 1] * sc) * g[2 * e + 1]) << 16);
+          ((uint4 *)yr)[c] = make_uint4(o[0], o[1], o[2], o[3]);
+        }
+      }
+  }
+
   for (int chunk = blockIdx.x; chunk < n_chunks; chunk += gridDim.x) {
     int c0 = chunk * CR;
     c0 = c0 + CR <= a.rows ? c0 : a.rows - CR;  // host guarantees rows >= CR
@@ -114,7 +157,35 @@ __global__ void __launch_bounds__(1024) gemv_bf16_k(KxGemvArgs a) {
 #pragma unroll
         for (int t = 0; t < TT; ++t) {
           const int tok = min(t0 + t, T - 1);
-          unpack8(xs[t], *(const uint4 *)(xb + (size_t)tok * a.x_stride + col));
+          if (a.mla_po) {
+            // activations = merged attention partials of head `blk` (mla_combine's arithmetic):
+            // M = max M_j; w_j = exp(M_j - M); Z = fma(Z_j, w_j, Z); O = fma(O_j, w_j, O); x = bf(O / Z)
+            float M = -__builtin_inff();
+            for (int j = 0; j < a.mla_spans; ++j) M = fmaxf(M, a.mla_pm[((size_t)tok * a.mla_spans + j) * a.mla_heads + blk]);
+            float Z = 0.0f, O[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+            for (int j = 0; j < a.mla_spans; ++j) {
+              const size_t idx = ((size_t)tok * a.mla_spans + j) * a.mla_heads + blk;
+              const float w = kx_expf(a.mla_pm[idx] - M);
+              Z = __builtin_fmaf(a.mla_pz[idx], w, Z);
+              const float4 *o = (const float4 *)(a.mla_po + idx * a.cols + col);
+              const float4 o0 = o[0], o1 = o[1];
+              O[0] = __builtin_fmaf(o0.x, w, O[0]); O[1] = __builtin_fmaf(o0.y, w, O[1]);
+              O[2] = __builtin_fmaf(o0.z, w, O[2]); O[3] = __builtin_fmaf(o0.w, w, O[3]);
+              O[4] = __builtin_fmaf(o1.x, w, O[4]); O[5] = __builtin_fmaf(o1.y, w, O[5]);
+              O[6] = __builtin_fmaf(o1.z, w, O[6]); O[7] = __builtin_fmaf(o1.w, w, O[7]);
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) xs[t][e] = kx_bfround(O[e] / Z);
+          } else {
+            unpack8(xs[t], *(const uint4 *)(xb + (size_t)tok * a.x_stride + col));
+            if (a.norm_w) {
+              float g[8];
+              unpack8(g, *(const uint4 *)(a.norm_w + col));
+              const float sc = n_scale[tok];
+#pragma unroll
+              for (int e = 0; e < 8; ++e) xs[t][e] = kx_bfround(kx_bfround(xs[t][e] * sc) * g[e]);
+            }
+          }
         }
       };
       auto compute_tile = [&](uint4 (&buf)[MATS][RI], int tile) {
@@ -207,30 +278,49 @@ __global__ void __launch_bounds__(1024) gemv_bf16_k(KxGemvArgs a) {
   }
 }
 
-// lowest-index argmax over bf16-rounded logits (sample_lm_head :718-734, argmax_k :477-493)
-__global__ void __launch_bounds__(1024) argmax_rows_k(const float *__restrict__ logits, int n, int stride,
-                                                      uint32_t *__restrict__ out) {
-  __shared__ float sv[16];
-  __shared__ uint32_t si[16];
-  const float *p = logits + (size_t)blockIdx.x * stride;
-  float best = -__builtin_inff();
-  uint32_t bi = 0;
-  for (int i = threadIdx.x; i < n; i += blockDim.x) {
-    float v = p[i];
-    if (v > best) { best = v; bi = (uint32_t)i; }
-  }
+// lowest-index argmax over bf16-rounded logits (sample_lm_head :718-734, argmax_k :477-493), in two
+// stages: ARGMAX_PARTS workgroups per row each reduce a slice, then one wave per row merges them
+constexpr int ARGMAX_PARTS = 64;
+
+__device__ __forceinline__ void argmax_merge(float &best, uint32_t &bi, float ov, uint32_t oi) {
+  if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
+}
+__device__ __forceinline__ void argmax_wave(float &best, uint32_t &bi) {
   for (int m = 32; m; m >>= 1) {
     float ov = __shfl_xor(best, m);
     uint32_t oi = (uint32_t)__shfl_xor((int)bi, m);
-    if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
+    argmax_merge(best, bi, ov, oi);
   }
+}
+
+__global__ void __launch_bounds__(256) argmax_part_k(const float *__restrict__ logits, int n, int stride,
+                                                     float *__restrict__ pv, uint32_t *__restrict__ pi) {
+  __shared__ float sv[4];
+  __shared__ uint32_t si[4];
+  const float *p = logits + (size_t)blockIdx.y * stride;
+  const int per = (n + ARGMAX_PARTS - 1) / ARGMAX_PARTS;
+  const int lo = blockIdx.x * per, hi = min(n, lo + per);
+  float best = -__builtin_inff();
+  uint32_t bi = 0xffffffffu;
+  for (int i = lo + threadIdx.x; i < hi; i += blockDim.x) {
+    float v = p[i];
+    if (v > best) { best = v; bi = (uint32_t)i; }
+  }
+  argmax_wave(best, bi);
   if ((threadIdx.x & 63) == 0) { sv[threadIdx.x >> 6] = best; si[threadIdx.x >> 6] = bi; }
   __syncthreads();
   if (threadIdx.x == 0) {
-    for (int w = 1; w < (int)(blockDim.x >> 6); ++w)
-      if (sv[w] > best || (sv[w] == best && si[w] < bi)) { best = sv[w]; bi = si[w]; }
-    out[blockIdx.x] = bi;
+    for (int w = 1; w < 4; ++w) argmax_merge(best, bi, sv[w], si[w]);
+    pv[blockIdx.y * ARGMAX_PARTS + blockIdx.x] = best;
+    pi[blockIdx.y * ARGMAX_PARTS + blockIdx.x] = bi;
   }
+}
+__global__ void __launch_bounds__(64) argmax_final_k(const float *__restrict__ pv, const uint32_t *__restrict__ pi,
+                                                     uint32_t *__restrict__ out) {
+  float best = pv[blockIdx.x * ARGMAX_PARTS + threadIdx.x];
+  uint32_t bi = pi[blockIdx.x * ARGMAX_PARTS + threadIdx.x];
+  argmax_wave(best, bi);
+  if (threadIdx.x == 0) out[blockIdx.x] = bi == 0xffffffffu ? 0u : bi;  // every logit -inf or NaN: id 0 as :481
 }
 
 template <int MATS, int RI>
@@ -283,6 +373,12 @@ int kx_gemv_launch(int epi, KxGemvArgs a, hipStream_t st) {
   }
   a.nt = nt;
   const int CR = rt * nt;
+  if (a.norm_w) {
+    KX_REQUIRE(a.tokens <= 4 && a.nw * a.rs * 64 >= 256 && !a.row_block, "kx_gemv: the fused RMSNorm needs at most 4 tokens and 256 threads");
+  }
+  if (a.mla_po) {
+    KX_REQUIRE(a.row_block && a.cols == 512 && !a.norm_w, "kx_gemv: attention partials feed a 512-column blocked matrix");
+  }
   const int all_tokens = a.tokens;
   const uint16_t *x0 = a.x;
   char *out0 = (char *)a.out;
@@ -317,8 +413,13 @@ int kx_rmsnorm_launch(const uint16_t *x, const uint16_t *w, uint16_t *y, int tok
   return KX_OK;
 }
 
-int kx_argmax_launch(const float *logits, int tokens, int n, int stride, uint32_t *out, hipStream_t st) {
-  hipLaunchKernelGGL(argmax_rows_k, dim3(tokens), dim3(1024), 0, st, logits, n, stride, out);
+// scratch: tokens * ARGMAX_PARTS floats and as many uint32
+int kx_argmax_launch(const float *logits, int tokens, int n, int stride, uint32_t *out, float *scratch, hipStream_t st) {
+  float *pv = scratch;
+  uint32_t *pi = (uint32_t *)(scratch + (size_t)tokens * ARGMAX_PARTS);
+  hipLaunchKernelGGL(argmax_part_k, dim3(ARGMAX_PARTS, tokens), dim3(256), 0, st, logits, n, stride, pv, pi);
+  KX_LAUNCH_CHECK();
+  hipLaunchKernelGGL(argmax_final_k, dim3(tokens), dim3(64), 0, st, pv, pi, out);
   KX_LAUNCH_CHECK();
   return KX_OK;
 }

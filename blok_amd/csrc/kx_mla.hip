@@ -85,37 +85,41 @@ __device__ __forceinline__ void unpack8(float (&f)[8], uint4 u) {
   f[4] = bf_lo(u.z); f[5] = bf_hi(u.z); f[6] = bf_lo(u.w); f[7] = bf_hi(u.w);
 }
 
-// RMSNorm of one row by a 256-thread workgroup; the schedule of rmsnorm_k (kx_dense.hip)
+// RMSNorm of one row by the first 256 threads of a workgroup; the schedule of rmsnorm_k (kx_dense.hip).
+// Every thread of the workgroup must call it (it contains barriers).
 __device__ __forceinline__ void rmsnorm_block(const uint16_t *xr, const uint16_t *w, uint16_t *yr, int n, float eps,
                                               float *ws /* 4 floats of LDS */) {
   const int chunks = n >> 3;
+  const bool active = threadIdx.x < 256;
   float v = 0.0f;
-  for (int c = threadIdx.x; c < chunks; c += 256) {
-    float f[8];
-    unpack8(f, ((const uint4 *)xr)[c]);
+  if (active)
+    for (int c = threadIdx.x; c < chunks; c += 256) {
+      float f[8];
+      unpack8(f, ((const uint4 *)xr)[c]);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) v = __builtin_fmaf(f[e], f[e], v);
-  }
+      for (int e = 0; e < 8; ++e) v = __builtin_fmaf(f[e], f[e], v);
+    }
   float vv[1] = {v};
   kxw::reduce<1, 64>(vv, threadIdx.x & 63);
   __syncthreads();  // ws may still be read from a previous call
-  if ((threadIdx.x & 63) == 0) ws[threadIdx.x >> 6] = vv[0];
+  if (active && (threadIdx.x & 63) == 0) ws[threadIdx.x >> 6] = vv[0];
   __syncthreads();
   const float total = ((ws[0] + ws[1]) + ws[2]) + ws[3];
   const float scale = kx_rsqrtf(total / (float)n + eps);
-  for (int c = threadIdx.x; c < chunks; c += 256) {
-    float f[8], g[8];
-    unpack8(f, ((const uint4 *)xr)[c]);
-    unpack8(g, ((const uint4 *)w)[c]);
-    uint32_t o[4];
+  if (active)
+    for (int c = threadIdx.x; c < chunks; c += 256) {
+      float f[8], g[8];
+      unpack8(f, ((const uint4 *)xr)[c]);
+      unpack8(g, ((const uint4 *)w)[c]);
+      uint32_t o[4];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      uint32_t a = kx_bf16_rne(kx_bfround(f[2 * e] * scale) * g[2 * e]);
-      uint32_t b = kx_bf16_rne(kx_bfround(f[2 * e + 1] * scale) * g[2 * e + 1]);
-      o[e] = a | (b << 16);
+      for (int e = 0; e < 4; ++e) {
+        uint32_t a = kx_bf16_rne(kx_bfround(f[2 * e] * scale) * g[2 * e]);
+        uint32_t b = kx_bf16_rne(kx_bfround(f[2 * e + 1] * scale) * g[2 * e + 1]);
+        o[e] = a | (b << 16);
+      }
+      ((uint4 *)yr)[c] = make_uint4(o[0], o[1], o[2], o[3]);
     }
-    ((uint4 *)yr)[c] = make_uint4(o[0], o[1], o[2], o[3]);
-  }
 }
 
 // interleaved-pair rotation of rope_k (:352-356): reads (2p, 2p+1), writes (p, half+p)
@@ -124,23 +128,15 @@ __device__ __forceinline__ void rope_pair(float x0, float x1, float c, float s, 
   y_hi = kx_bfround(kx_bfround(x1 * c) + kx_bfround(x0 * s));
 }
 
-// After the fused q_a / kv_a projection: q_a RMSNorm (:814), kv_a RMSNorm on the latent
-// part only (:817), RoPE of the shared rope key (:820-823), write of the cache row (:824).
-// qkv bf16 [T][q_rank + kv_rank + rope]; one workgroup per token (= sequence).
-__global__ void __launch_bounds__(256) kv_finish_k(const uint16_t *__restrict__ qkv, const uint16_t *__restrict__ w_qa_ln,
-                                                   const uint16_t *__restrict__ w_kv_ln, const uint16_t *__restrict__ rope_row,
-                                                   uint16_t *__restrict__ qa_out, uint16_t *__restrict__ cache, int q_rank,
-                                                   int kv_rank, int rope, size_t seq_stride, int pos, float eps) {
-  __shared__ float ws[4];
-  const int t = blockIdx.x, kva = kv_rank + rope;
-  const uint16_t *row = qkv + (size_t)t * (q_rank + kva);
-  uint16_t *crow = cache + (size_t)t * seq_stride + (size_t)pos * kva;
-  rmsnorm_block(row, w_qa_ln, qa_out + (size_t)t * q_rank, q_rank, eps, ws);
-  rmsnorm_block(row + q_rank, w_kv_ln, crow, kv_rank, eps, ws);
+// kv_a RMSNorm on the latent part only (:817), RoPE of the shared rope key (:820-823) and the write of
+// the cache row (:824) for token t; kva bf16 [kv_rank + rope] is the kv_a output of the token.
+__device__ __forceinline__ void kv_finish_block(const uint16_t *kva, const uint16_t *w_kv_ln, const uint16_t *rope_row,
+                                                uint16_t *crow, int kv_rank, int rope, float eps, float *ws) {
+  rmsnorm_block(kva, w_kv_ln, crow, kv_rank, eps, ws);
   const int half = rope >> 1;
   if ((int)threadIdx.x < half) {
     const int p = threadIdx.x;
-    const uint16_t *kr = row + q_rank + kv_rank;
+    const uint16_t *kr = kva + kv_rank;
     float lo, hi;
     rope_pair(kx_bf16_f32(kr[2 * p]), kx_bf16_f32(kr[2 * p + 1]), kx_bf16_f32(rope_row[p]), kx_bf16_f32(rope_row[half + p]),
               lo, hi);
@@ -149,19 +145,36 @@ __global__ void __launch_bounds__(256) kv_finish_k(const uint16_t *__restrict__ 
   }
 }
 
-// q_abs[t][h] = (bf(W_UK[h]^T q_nope[h]) | rope(q_rope[h])) as f32.  Grid (heads, T), 8 waves:
-// wave j runs the chain over d = j, j+8, ...; lane owns 8 latent columns.
-__global__ void __launch_bounds__(512) q_absorb_k(const uint16_t *__restrict__ q, const uint16_t *__restrict__ kvb,
-                                                  const uint16_t *__restrict__ rope_row, float *__restrict__ qabs,
-                                                  int heads, int nope, int rope, int v_head, int kv_rank) {
+// q_abs[t][h] = (bf(W_UK[h]^T q_nope[h]) | rope(q_rope[h])) as f32.  Grid (heads + 1, T), 8 waves:
+// wave j runs the chain over d = j, j+8, ...; lane owns 8 latent columns.  The extra block
+// (blockIdx.x == heads) finishes the token's kv_a output and writes its cache row.
+struct QAbsArgs {
+  const uint16_t *q, *kvb, *rope_row;
+  float *qabs;
+  const uint16_t *kva, *w_kv_ln;  // kva: first kv_a output row, kva_stride elements between tokens
+  uint16_t *cache;
+  size_t seq_stride;
+  int heads, nope, rope, v_head, kv_rank, kva_stride, pos;
+  float eps;
+};
+__global__ void __launch_bounds__(512) q_absorb_k(QAbsArgs a) {
   extern __shared__ float part[];  // [8][kv_rank]
+  __shared__ float ws[4];
   const int h = blockIdx.x, t = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int nope = a.nope, rope = a.rope, kv_rank = a.kv_rank;
   const int qk = nope + rope, kva = kv_rank + rope;
-  const uint16_t *qh = q + ((size_t)t * heads + h) * qk;
-  const uint16_t *wuk = kvb + (size_t)h * (nope + v_head) * kv_rank;
-  float *out = qabs + ((size_t)t * heads + h) * kva;
+  if (h == a.heads) {
+    if (a.cache)
+      kv_finish_block(a.kva + (size_t)t * a.kva_stride, a.w_kv_ln, a.rope_row, a.cache + (size_t)t * a.seq_stride + (size_t)a.pos * kva,
+                      kv_rank, rope, a.eps, ws);
+    return;
+  }
+  const uint16_t *qh = a.q + ((size_t)t * a.heads + h) * qk;
+  const uint16_t *wuk = a.kvb + (size_t)h * (nope + a.v_head) * kv_rank;
+  float *out = a.qabs + ((size_t)t * a.heads + h) * kva;
   for (int c0 = lane * 8; c0 < kv_rank; c0 += 512) {
     float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll 8
     for (int d = wave; d < nope; d += 8) {
       float wf[8];
       unpack8(wf, *(const uint4 *)(wuk + (size_t)d * kv_rank + c0));
@@ -183,8 +196,8 @@ __global__ void __launch_bounds__(512) q_absorb_k(const uint16_t *__restrict__ q
   if ((int)threadIdx.x < half) {
     const int p = threadIdx.x;
     float lo, hi;
-    rope_pair(kx_bf16_f32(qh[nope + 2 * p]), kx_bf16_f32(qh[nope + 2 * p + 1]), kx_bf16_f32(rope_row[p]),
-              kx_bf16_f32(rope_row[half + p]), lo, hi);
+    rope_pair(kx_bf16_f32(qh[nope + 2 * p]), kx_bf16_f32(qh[nope + 2 * p + 1]), kx_bf16_f32(a.rope_row[p]),
+              kx_bf16_f32(a.rope_row[half + p]), lo, hi);
     out[kv_rank + p] = lo;
     out[kv_rank + half + p] = hi;
   }
@@ -200,11 +213,16 @@ struct MlaArgs {
 };
 
 // kv_rank 512, rope 64 (the Kimi-K2 latent layout).  HG heads per wave, 4 waves per workgroup.
-// grid (spans, heads / (4*HG), B).
+// grid (spans, heads / (4*HG), B).  The 64 cache rows of a tile are staged in LDS once per
+// workgroup with coalesced 16-byte loads (row pitch 1168 B, so that both the row-per-lane reads
+// of the score pass and the column-per-lane reads of the PV pass are free of bank conflicts).
+constexpr int MLA_R = 512, MLA_KVA = 576, MLA_PITCH = 584;  // bf16 elements; 1168 B per staged row
+
 template <int HG>
 __global__ void __launch_bounds__(256) mla_partial_k(MlaArgs a) {
-  constexpr int R = 512, KVA = 576;
-  __shared__ float p_lds[4][HG][64];
+  constexpr int R = MLA_R, KVA = MLA_KVA, PITCH = MLA_PITCH;
+  extern __shared__ __attribute__((aligned(16))) uint16_t tile_lds[];  // [64][PITCH] then p [4][HG][64] floats
+  float(*p_lds)[HG][64] = (float(*)[HG][64])(tile_lds + 64 * PITCH);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int span = blockIdx.x, b = blockIdx.z;
   const int h0 = (blockIdx.y * 4 + wave) * HG;
@@ -222,14 +240,31 @@ __global__ void __launch_bounds__(256) mla_partial_k(MlaArgs a) {
   }
   for (int tile = span * a.span_tiles; tile < tile_end; ++tile) {
     const int t0 = tile << 6, n = min(64, a.seq - t0);
+    // stage rows t0 .. t0+n-1: 72 pieces of 16 bytes per row, 18 per thread
+    {
+      const uint4 *src = (const uint4 *)(cache + (size_t)t0 * KVA);
+      uint4 v[18];
+#pragma unroll
+      for (int i = 0; i < 18; ++i) {
+        const int idx = threadIdx.x + i * 256;  // piece (row, j) = (idx / 72, idx % 72)
+        v[i] = idx < n * 72 ? src[idx] : make_uint4(0, 0, 0, 0);
+      }
+#pragma unroll
+      for (int i = 0; i < 18; ++i) {
+        const int idx = threadIdx.x + i * 256, row = idx / 72, j = idx - row * 72;
+        *(uint4 *)(tile_lds + row * PITCH + j * 8) = v[i];
+      }
+    }
+    __syncthreads();
     // scores: lane = position, one fma chain over the 576 columns per head
-    const uint16_t *row = cache + (size_t)(t0 + min(lane, n - 1)) * KVA;
+    const uint16_t *row = tile_lds + lane * PITCH;
     float acc[HG];
 #pragma unroll
     for (int h = 0; h < HG; ++h) acc[h] = 0.0f;
+#pragma unroll 4
     for (int j = 0; j < KVA / 8; ++j) {
       float cf[8];
-      unpack8(cf, ((const uint4 *)row)[j]);
+      unpack8(cf, *(const uint4 *)(row + j * 8));
 #pragma unroll
       for (int h = 0; h < HG; ++h) {
         const float *qh = q + h * KVA + j * 8;
@@ -253,16 +288,15 @@ __global__ void __launch_bounds__(256) mla_partial_k(MlaArgs a) {
       M[h] = Mn;
       p_lds[wave][h][lane] = kx_bfround(p);
     }
-    __syncthreads();
-    // PV: lane = 8 latent columns, positions in order
+    // PV: lane = 8 latent columns, positions in order (p of this wave was written by this wave)
 #pragma unroll
     for (int h = 0; h < HG; ++h)
 #pragma unroll
       for (int e = 0; e < 8; ++e) O[h][e] = O[h][e] * alpha[h];
-    const uint16_t *col = cache + (size_t)t0 * KVA + lane * 8;
+    const uint16_t *col = tile_lds + lane * 8;
     for (int t = 0; t < n; ++t) {
       float cf[8];
-      unpack8(cf, *(const uint4 *)(col + (size_t)t * KVA));
+      unpack8(cf, *(const uint4 *)(col + t * PITCH));
 #pragma unroll
       for (int h = 0; h < HG; ++h) {
         const float p = p_lds[wave][h][t];
@@ -270,7 +304,7 @@ __global__ void __launch_bounds__(256) mla_partial_k(MlaArgs a) {
         for (int e = 0; e < 8; ++e) O[h][e] = __builtin_fmaf(p, cf[e], O[h][e]);
       }
     }
-    __syncthreads();
+    __syncthreads();  // the next tile overwrites the staged rows
   }
 #pragma unroll
   for (int h = 0; h < HG; ++h) {
@@ -311,21 +345,15 @@ __global__ void __launch_bounds__(64) mla_combine_k(const float *__restrict__ pm
 
 }  // namespace
 
-int kx_kv_finish_launch(const uint16_t *qkv, const uint16_t *w_qa_ln, const uint16_t *w_kv_ln, const uint16_t *rope_row,
-                        uint16_t *qa_out, uint16_t *cache, int tokens, int q_rank, int kv_rank, int rope,
-                        size_t seq_stride, int pos, float eps, hipStream_t st) {
-  KX_REQUIRE(q_rank % 8 == 0 && kv_rank % 8 == 0 && rope % 2 == 0 && rope / 2 <= 256, "kx_kv_finish: bad shape");
-  hipLaunchKernelGGL(kv_finish_k, dim3(tokens), dim3(256), 0, st, qkv, w_qa_ln, w_kv_ln, rope_row, qa_out, cache, q_rank,
-                     kv_rank, rope, seq_stride, pos, eps);
-  KX_LAUNCH_CHECK();
-  return KX_OK;
-}
-
 int kx_q_absorb_launch(const uint16_t *q, const uint16_t *kvb, const uint16_t *rope_row, float *qabs, int tokens,
-                       int heads, int nope, int rope, int v_head, int kv_rank, hipStream_t st) {
+                       int heads, int nope, int rope, int v_head, int kv_rank, const uint16_t *kva, int kva_stride,
+                       const uint16_t *w_kv_ln, uint16_t *cache, size_t seq_stride, int pos, float eps, hipStream_t st) {
   KX_REQUIRE(kv_rank % 8 == 0 && rope % 2 == 0 && rope / 2 <= 512, "kx_q_absorb: bad shape");
-  hipLaunchKernelGGL(q_absorb_k, dim3(heads, tokens), dim3(512), (size_t)8 * kv_rank * sizeof(float), st, q, kvb, rope_row,
-                     qabs, heads, nope, rope, v_head, kv_rank);
+  QAbsArgs a;
+  a.q = q; a.kvb = kvb; a.rope_row = rope_row; a.qabs = qabs; a.kva = kva; a.w_kv_ln = w_kv_ln; a.cache = cache;
+  a.seq_stride = seq_stride; a.heads = heads; a.nope = nope; a.rope = rope; a.v_head = v_head; a.kv_rank = kv_rank;
+  a.kva_stride = kva_stride; a.pos = pos; a.eps = eps;
+  hipLaunchKernelGGL(q_absorb_k, dim3(heads + (cache ? 1 : 0), tokens), dim3(512), (size_t)8 * kv_rank * sizeof(float), st, a);
   KX_LAUNCH_CHECK();
   return KX_OK;
 }
@@ -337,8 +365,8 @@ size_t kx_mla_partial_floats(int batch, int heads, int kv_rank, int max_seq) {
   return (size_t)batch * spans * heads * (kv_rank + 2);
 }
 
-int kx_mla_attend_launch(const kx_config *c, const uint16_t *cache, size_t seq_stride, const float *qabs, float *partial,
-                         uint16_t *o_lat, int batch, int seq, hipStream_t st) {
+int kx_mla_partials_launch(const kx_config *c, const uint16_t *cache, size_t seq_stride, const float *qabs, float *partial,
+                           int batch, int seq, KxMlaPartials *out, hipStream_t st) {
   KX_REQUIRE(c->kv_rank == 512 && c->qk_rope == 64, "kx_mla: the attention kernel is built for kv_rank 512, qk_rope 64 (got %d, %d)",
              c->kv_rank, c->qk_rope);
   KX_REQUIRE(c->heads % 4 == 0, "kx_mla: heads=%d must be a multiple of 4", c->heads);
@@ -358,12 +386,30 @@ int kx_mla_attend_launch(const kx_config *c, const uint16_t *cache, size_t seq_s
   int hg = 1;
   while (hg < 8 && c->heads % (4 * hg * 2) == 0 && waves1 / (hg * 2) >= 4096) hg *= 2;
   dim3 g(a.spans, c->heads / (4 * hg), batch), b(256);
-  if (hg == 1) hipLaunchKernelGGL(mla_partial_k<1>, g, b, 0, st, a);
-  else if (hg == 2) hipLaunchKernelGGL(mla_partial_k<2>, g, b, 0, st, a);
-  else if (hg == 4) hipLaunchKernelGGL(mla_partial_k<4>, g, b, 0, st, a);
-  else hipLaunchKernelGGL(mla_partial_k<8>, g, b, 0, st, a);
+  const size_t lds = (size_t)64 * MLA_PITCH * 2 + (size_t)4 * hg * 64 * sizeof(float);
+  static bool attr_set = false;
+  if (!attr_set) {  // more than 64 KB of dynamic LDS has to be allowed per kernel
+    KX_HIP(hipFuncSetAttribute((const void *)mla_partial_k<1>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
+    KX_HIP(hipFuncSetAttribute((const void *)mla_partial_k<2>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
+    KX_HIP(hipFuncSetAttribute((const void *)mla_partial_k<4>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
+    KX_HIP(hipFuncSetAttribute((const void *)mla_partial_k<8>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
+    attr_set = true;
+  }
+  if (hg == 1) hipLaunchKernelGGL(mla_partial_k<1>, g, b, lds, st, a);
+  else if (hg == 2) hipLaunchKernelGGL(mla_partial_k<2>, g, b, lds, st, a);
+  else if (hg == 4) hipLaunchKernelGGL(mla_partial_k<4>, g, b, lds, st, a);
+  else hipLaunchKernelGGL(mla_partial_k<8>, g, b, lds, st, a);
   KX_LAUNCH_CHECK();
-  hipLaunchKernelGGL(mla_combine_k, dim3(c->heads, batch), dim3(64), 0, st, a.pm, a.pz, a.po, o_lat, c->heads, a.spans);
+  out->pm = a.pm; out->pz = a.pz; out->po = a.po; out->spans = a.spans;
+  return KX_OK;
+}
+
+int kx_mla_attend_launch(const kx_config *c, const uint16_t *cache, size_t seq_stride, const float *qabs, float *partial,
+                         uint16_t *o_lat, int batch, int seq, hipStream_t st) {
+  KxMlaPartials p;
+  int rc = kx_mla_partials_launch(c, cache, seq_stride, qabs, partial, batch, seq, &p, st);
+  if (rc) return rc;
+  hipLaunchKernelGGL(mla_combine_k, dim3(c->heads, batch), dim3(64), 0, st, p.pm, p.pz, p.po, o_lat, c->heads, p.spans);
   KX_LAUNCH_CHECK();
   return KX_OK;
 }
@@ -388,5 +434,6 @@ extern "C" int kx_q_absorb(const kx_config *cfg, const void *d_q, const void *d_
                            int32_t tokens, void *stream) {
   KX_REQUIRE(cfg && d_q && d_kvb && d_rope_row && d_qabs, "kx_q_absorb: null argument");
   return kx_q_absorb_launch((const uint16_t *)d_q, (const uint16_t *)d_kvb, (const uint16_t *)d_rope_row, (float *)d_qabs,
-                            tokens, cfg->heads, cfg->qk_nope, cfg->qk_rope, cfg->v_head, cfg->kv_rank, kx_stream(stream));
+                            tokens, cfg->heads, cfg->qk_nope, cfg->qk_rope, cfg->v_head, cfg->kv_rank, nullptr, 0, nullptr,
+                            nullptr, 0, 0, 0.0f, kx_stream(stream));
 }

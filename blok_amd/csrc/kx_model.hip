@@ -58,7 +58,7 @@ struct kx_model {
   std::vector<Layer> layers;
   // scratch of one step
   uint16_t *x, *n, *qkv, *qa, *q, *o_lat, *att, *dmid;
-  float *qabs, *partial, *logits;
+  float *qabs, *partial, *logits, *argmax_scratch;
   uint32_t *ids, *next, *history;  // [max_context][B], [B], [max_context][B]
   kx_moe_workspace *moe_ws = nullptr;
   hipStream_t st = nullptr;
@@ -157,6 +157,7 @@ int layout(const kx_config *c, Plan &p, kx_model *m) {
   auto *qabs = KX_AT(float *, B * (size_t)c->heads * KVA * 4);
   auto *partial = KX_AT(float *, kx_mla_partial_floats(c->max_batch, c->heads, c->kv_rank, c->max_context) * 4);
   auto *logits = KX_AT(float *, B * V * 4);
+  auto *argmax_scratch = KX_AT(float *, KX_ARGMAX_SCRATCH_FLOATS(B) * 4);
   auto *ids = KX_AT(uint32_t *, (size_t)c->max_context * B * 4);
   auto *next = KX_AT(uint32_t *, B * 4);
   auto *history = KX_AT(uint32_t *, (size_t)c->max_context * B * 4);
@@ -164,7 +165,7 @@ int layout(const kx_config *c, Plan &p, kx_model *m) {
   p.scratch = p.total - p.weights - p.cache;
   if (m) {
     m->x = x; m->n = n; m->qkv = qkv; m->qa = qa; m->q = q; m->o_lat = o_lat; m->att = att; m->dmid = dmid;
-    m->qabs = qabs; m->partial = partial; m->logits = logits; m->ids = ids; m->next = next; m->history = history;
+    m->qabs = qabs; m->partial = partial; m->logits = logits; m->argmax_scratch = argmax_scratch; m->ids = ids; m->next = next; m->history = history;
   }
   return KX_OK;
 }
@@ -234,48 +235,57 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample) {
   KX_LAUNCH_CHECK();
   const uint16_t *rope_row = m->rope_tab + (size_t)pos * c.qk_rope;
   const size_t seq_stride = (size_t)c.max_context * KVA;
+  const bool fuse = B <= 4;  // RMSNorms ride in the prologue of the GEMV that consumes them
   for (int l = 0; l < c.n_layers; ++l) {
     Layer &L = m->layers[l];
-    KX_TRY(kx_rmsnorm_launch(m->x, L.input_ln, m->n, B, H, H, H, c.rms_eps, st));                      // :812
     KxGemvArgs g = {};
     g.w0 = L.qkv_a; g.x = m->n; g.x_stride = H; g.out = m->qkv; g.out_stride = QKV; g.rows = QKV; g.cols = H; g.tokens = B;
+    if (fuse) { g.x = m->x; g.norm_w = L.input_ln; g.norm_eps = c.rms_eps; }
+    else KX_TRY(kx_rmsnorm_launch(m->x, L.input_ln, m->n, B, H, H, H, c.rms_eps, st));                 // :812
     KX_TRY(kx_gemv_launch(KX_EPI_BF16, g, st));                                                         // :813, :816
-    KX_TRY(kx_kv_finish_launch(m->qkv, L.qa_ln, L.kv_ln, rope_row, m->qa, L.cache, B, c.q_rank, c.kv_rank, c.qk_rope,
-                               seq_stride, pos, c.rms_eps, st));                                        // :814, :817, :820-824
     g = {};
     g.w0 = L.qb; g.x = m->qa; g.x_stride = c.q_rank; g.out = m->q; g.out_stride = KD; g.rows = KD; g.cols = c.q_rank; g.tokens = B;
+    if (fuse) { g.x = m->qkv; g.x_stride = QKV; g.norm_w = L.qa_ln; g.norm_eps = c.rms_eps; }
+    else KX_TRY(kx_rmsnorm_launch(m->qkv, L.qa_ln, m->qa, B, c.q_rank, QKV, c.q_rank, c.rms_eps, st)); // :814
     KX_TRY(kx_gemv_launch(KX_EPI_BF16, g, st));                                                         // :815
-    KX_TRY(kx_q_absorb_launch(m->q, L.kvb, rope_row, m->qabs, B, c.heads, c.qk_nope, c.qk_rope, c.v_head, c.kv_rank, st));
-    KX_TRY(kx_mla_attend_launch(&c, L.cache, seq_stride, m->qabs, m->partial, m->o_lat, B, pos + 1, st));  // :825
-    g = {};
+    // W_UK absorb + rope(q); the extra block norms kv_a, rotates the rope key, writes the cache row (:817-824)
+    KX_TRY(kx_q_absorb_launch(m->q, L.kvb, rope_row, m->qabs, B, c.heads, c.qk_nope, c.qk_rope, c.v_head, c.kv_rank,
+                              m->qkv + c.q_rank, QKV, L.kv_ln, L.cache, seq_stride, pos, c.rms_eps, st));
+    KxMlaPartials mp;
+    KX_TRY(kx_mla_partials_launch(&c, L.cache, seq_stride, m->qabs, m->partial, B, pos + 1, &mp, st));  // :825
+    g = {};  // W_UV of :818 per head; its activations are the merged attention partials
     g.w0 = L.kvb; g.x = m->o_lat; g.x_stride = c.heads * c.kv_rank; g.out = m->att; g.out_stride = VD; g.rows = VD;
     g.cols = c.kv_rank; g.tokens = B; g.row_block = c.v_head; g.w_block_stride = c.qk_nope + c.v_head;
     g.w_block_off = c.qk_nope; g.x_block_stride = c.kv_rank;
-    KX_TRY(kx_gemv_launch(KX_EPI_BF16, g, st));                                                         // W_UV of :818
+    g.mla_pm = mp.pm; g.mla_pz = mp.pz; g.mla_po = mp.po; g.mla_spans = mp.spans; g.mla_heads = c.heads;
+    KX_TRY(kx_gemv_launch(KX_EPI_BF16, g, st));
     g = {};
     g.w0 = L.o; g.x = m->att; g.x_stride = VD; g.out = m->x; g.out_stride = H; g.rows = H; g.cols = VD; g.tokens = B;
     KX_TRY(kx_gemv_launch(KX_EPI_RESID, g, st));                                                        // :826-827
-    KX_TRY(kx_rmsnorm_launch(m->x, L.post_ln, m->n, B, H, H, H, c.rms_eps, st));                       // :829
     if (l < c.first_dense) {                                                                            // bf16_mlp (:674-686)
       g = {};
       g.w0 = L.dgate; g.w1 = L.dup; g.x = m->n; g.x_stride = H; g.out = m->dmid; g.out_stride = c.dense_inter;
       g.rows = c.dense_inter; g.cols = H; g.tokens = B;
+      if (fuse) { g.x = m->x; g.norm_w = L.post_ln; g.norm_eps = c.rms_eps; }
+      else KX_TRY(kx_rmsnorm_launch(m->x, L.post_ln, m->n, B, H, H, H, c.rms_eps, st));                // :829
       KX_TRY(kx_gemv_launch(KX_EPI_SWIGLU, g, st));
       g = {};
       g.w0 = L.ddown; g.x = m->dmid; g.x_stride = c.dense_inter; g.out = m->x; g.out_stride = H; g.rows = H;
       g.cols = c.dense_inter; g.tokens = B;
       KX_TRY(kx_gemv_launch(KX_EPI_RESID, g, st));                                                      // :684, :877
     } else {
-      KX_TRY(kx_moe_decode_layer(&c, &L.moe, m->moe_ws, m->n, m->x, B, 0, st));                         // :835-877
+      if (!fuse) KX_TRY(kx_rmsnorm_launch(m->x, L.post_ln, m->n, B, H, H, H, c.rms_eps, st));          // :829
+      KX_TRY(kx_moe_layer_launch(&c, &L.moe, m->moe_ws, m->n, m->x, B, 0, fuse ? L.post_ln : nullptr, st, false));  // :835-877
     }
   }
   if (sample) {                                                                                          // :880-881
-    KX_TRY(kx_rmsnorm_launch(m->x, m->final_norm, m->n, B, H, H, H, c.rms_eps, st));
     KxGemvArgs g = {};
     g.w0 = m->lm_head; g.x = m->n; g.x_stride = H; g.out = m->logits; g.out_stride = c.vocab; g.rows = c.vocab; g.cols = H;
     g.tokens = B;
+    if (fuse) { g.x = m->x; g.norm_w = m->final_norm; g.norm_eps = c.rms_eps; }
+    else KX_TRY(kx_rmsnorm_launch(m->x, m->final_norm, m->n, B, H, H, H, c.rms_eps, st));
     KX_TRY(kx_gemv_launch(KX_EPI_ARGMAX, g, st));
-    KX_TRY(kx_argmax_launch(m->logits, B, c.vocab, c.vocab, m->next, st));
+    KX_TRY(kx_argmax_launch(m->logits, B, c.vocab, c.vocab, m->next, m->argmax_scratch, st));
   }
 #undef KX_TRY
   m->sampled = sample;

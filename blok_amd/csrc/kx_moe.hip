@@ -109,8 +109,8 @@ static int routed_tt(int tokens, int topk, int experts) {
   return 4;
 }
 
-static int moe_layer(const kx_config *c, const kx_moe_weights *w, kx_moe_workspace *ws, const void *d_n, void *d_x,
-                     int tokens, uint32_t flags, hipStream_t st, bool timed) {
+int kx_moe_layer_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_workspace *ws, void *d_n, void *d_x,
+                        int tokens, uint32_t flags, const uint16_t *norm_w, hipStream_t st, bool timed) {
   int rc = check_cfg(c);
   if (rc) return rc;
   KX_REQUIRE(w && ws && d_n && d_x, "kx_moe_decode_layer: null argument");
@@ -125,11 +125,12 @@ static int moe_layer(const kx_config *c, const kx_moe_weights *w, kx_moe_workspa
   KxGemvArgs g = {};
   g.w0 = (const uint16_t *)w->d_router_gate; g.x = n; g.x_stride = H; g.out = ws->logits; g.out_stride = E;
   g.rows = E; g.cols = H; g.tokens = tokens;
+  if (norm_w) {  // the router GEMV norms the residual stream itself and leaves the normed rows in d_n
+    g.x = (const uint16_t *)d_x; g.norm_w = norm_w; g.norm_eps = c->rms_eps; g.norm_out = (uint16_t *)d_n;
+  }
   if ((rc = kx_gemv_launch(KX_EPI_F32, g, st))) return rc;
-  if ((rc = kx_router_topk_launch(ws->logits, (const float *)w->d_router_bias, ws->ids, ws->weights, tokens, E, K,
-                                  c->routed_scale, st))) return rc;
-  if ((rc = kx_bucket_launch(ws->ids, tokens, E, K, ws->counts, ws->offsets, ws->pairs, ws->work, ws->n_active, st)))
-    return rc;
+  if ((rc = kx_route_launch(ws->logits, (const float *)w->d_router_bias, ws->ids, ws->weights, tokens, E, K, c->routed_scale,
+                            ws->counts, ws->offsets, ws->pairs, ws->work, ws->n_active, st))) return rc;
   if (timed) KX_HIP(hipEventRecord(ws->ev[1], st));
   // 4 routed gate/up + SwiGLU
   const int tt = routed_tt(tokens, K, E);
@@ -162,14 +163,14 @@ static int moe_layer(const kx_config *c, const kx_moe_weights *w, kx_moe_workspa
 
 extern "C" int kx_moe_decode_layer(const kx_config *cfg, const kx_moe_weights *w, kx_moe_workspace *ws, const void *d_n,
                                    void *d_x, int32_t tokens, uint32_t flags, void *stream) {
-  return moe_layer(cfg, w, ws, d_n, d_x, tokens, flags, kx_stream(stream), false);
+  return kx_moe_layer_launch(cfg, w, ws, (void *)d_n, d_x, tokens, flags, nullptr, kx_stream(stream), false);
 }
 
 extern "C" int kx_moe_decode_layer_timed(const kx_config *cfg, const kx_moe_weights *w, kx_moe_workspace *ws,
                                          const void *d_n, void *d_x, int32_t tokens, uint32_t flags, void *stream,
                                          float *ms5) {
   KX_REQUIRE(ms5, "kx_moe_decode_layer_timed: null output");
-  int rc = moe_layer(cfg, w, ws, d_n, d_x, tokens, flags, kx_stream(stream), true);
+  int rc = kx_moe_layer_launch(cfg, w, ws, (void *)d_n, d_x, tokens, flags, nullptr, kx_stream(stream), true);
   if (rc) return rc;
   KX_HIP(hipEventSynchronize(ws->ev[5]));
   for (int i = 0; i < 5; ++i) KX_HIP(hipEventElapsedTime(&ms5[i], ws->ev[i], ws->ev[i + 1]));

@@ -21,13 +21,11 @@ namespace {
 using kxw::wave_max_f32;
 using kxw::wave_min_i32;
 
-// one wave per token; lane owns experts lane, lane+64, ... (EPL of them)
+// top-k of one token by one wave; lane owns experts lane, lane+64, ... (EPL of them)
 template <int EPL>
-__global__ void __launch_bounds__(64) router_topk_k(const float *__restrict__ logits, const float *__restrict__ bias,
-                                                    uint16_t *__restrict__ ids, float *__restrict__ weights, int E,
-                                                    int topk, float routed_scale) {
-  const int tok = blockIdx.x, lane = threadIdx.x;
-  const float *lg = logits + (size_t)tok * E;
+__device__ __forceinline__ void topk_token(const float *__restrict__ lg, const float *__restrict__ bias,
+                                           uint16_t *__restrict__ ids, float *__restrict__ weights, int E, int topk,
+                                           float routed_scale, int lane) {
   float sc[EPL], sel[EPL];
   const float NEG_INF = -__builtin_inff();
 #pragma unroll
@@ -55,20 +53,27 @@ __global__ void __launch_bounds__(64) router_topk_k(const float *__restrict__ lo
     s_win = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, s_win), win & 63));
     sum += s_win;
     if (lane == k) my_w = s_win;
-    if (lane == 0) ids[(size_t)tok * topk + k] = (uint16_t)win;
+    if (lane == 0) ids[k] = (uint16_t)win;
   }
-  if (lane < topk) weights[(size_t)tok * topk + lane] = my_w / (sum + 1.0e-20f) * routed_scale;
+  if (lane < topk) weights[lane] = my_w / (sum + 1.0e-20f) * routed_scale;
+}
+
+// one wave per token
+template <int EPL>
+__global__ void __launch_bounds__(64) router_topk_k(const float *__restrict__ logits, const float *__restrict__ bias,
+                                                    uint16_t *__restrict__ ids, float *__restrict__ weights, int E,
+                                                    int topk, float routed_scale) {
+  const int tok = blockIdx.x;
+  topk_token<EPL>(logits + (size_t)tok * E, bias, ids + (size_t)tok * topk, weights + (size_t)tok * topk, E, topk,
+                  routed_scale, threadIdx.x);
 }
 
 // one workgroup, thread e owns expert e: count, exclusive scan, stable placement.
 // The ids are staged in LDS (padded with 0xffff to a multiple of 8) and scanned 8 at a time.
-__global__ void __launch_bounds__(1024) bucket_k(const uint16_t *__restrict__ ids, int n_pairs, int E,
-                                                 int *__restrict__ counts, int *__restrict__ offsets,
-                                                 int *__restrict__ pairs, int4 *__restrict__ work,
-                                                 int *__restrict__ n_active) {
-  extern __shared__ uint4 s_ids4[];  // ceil(n_pairs / 8) pieces
-  __shared__ int s_cnt[1024];
-  __shared__ int s_act[1024];
+__device__ __forceinline__ void bucket_block(const uint16_t *__restrict__ ids, int n_pairs, int E,
+                                             int *__restrict__ counts, int *__restrict__ offsets,
+                                             int *__restrict__ pairs, int4 *__restrict__ work,
+                                             int *__restrict__ n_active, uint4 *s_ids4, int *s_cnt, int *s_act) {
   const int e = threadIdx.x, n = blockDim.x;
   const int n8 = (n_pairs + 7) >> 3;
   uint16_t *s_ids = (uint16_t *)s_ids4;
@@ -120,6 +125,35 @@ __global__ void __launch_bounds__(1024) bucket_k(const uint16_t *__restrict__ id
   }
 }
 
+__global__ void __launch_bounds__(1024) bucket_k(const uint16_t *__restrict__ ids, int n_pairs, int E,
+                                                 int *__restrict__ counts, int *__restrict__ offsets,
+                                                 int *__restrict__ pairs, int4 *__restrict__ work,
+                                                 int *__restrict__ n_active) {
+  extern __shared__ uint4 s_ids4[];  // ceil(n_pairs / 8) pieces
+  __shared__ int s_cnt[1024];
+  __shared__ int s_act[1024];
+  bucket_block(ids, n_pairs, E, counts, offsets, pairs, work, n_active, s_ids4, s_cnt, s_act);
+}
+
+// top-k of up to blockDim/64 tokens (one wave each), then the bucketing, in one workgroup
+template <int EPL>
+__global__ void __launch_bounds__(1024) topk_bucket_k(const float *__restrict__ logits, const float *__restrict__ bias,
+                                                      uint16_t *__restrict__ ids, float *__restrict__ weights, int tokens,
+                                                      int E, int topk, float routed_scale, int *__restrict__ counts,
+                                                      int *__restrict__ offsets, int *__restrict__ pairs,
+                                                      int4 *__restrict__ work, int *__restrict__ n_active) {
+  extern __shared__ uint4 s_ids4[];
+  __shared__ int s_cnt[1024];
+  __shared__ int s_act[1024];
+  const int wave = threadIdx.x >> 6;
+  if (wave < tokens)
+    topk_token<EPL>(logits + (size_t)wave * E, bias, ids + (size_t)wave * topk, weights + (size_t)wave * topk, E, topk,
+                    routed_scale, threadIdx.x & 63);
+  __threadfence_block();
+  __syncthreads();  // the ids written above are read back by bucket_block
+  bucket_block(ids, tokens * topk, E, counts, offsets, pairs, work, n_active, s_ids4, s_cnt, s_act);
+}
+
 }  // namespace
 
 int kx_router_topk_launch(const float *logits, const float *bias, uint16_t *ids, float *weights, int tokens,
@@ -146,7 +180,7 @@ int kx_bucket_launch(const uint16_t *ids, int tokens, int experts, int topk, int
   KX_REQUIRE(experts > 0 && experts <= 1024, "kx_bucket: experts=%d outside [1, 1024]", experts);
   int threads = kx_cdiv(experts, 64) * 64;
   const size_t lds = (size_t)kx_cdiv(tokens * topk, 8) * 16;
-  KX_REQUIRE(lds <= 128 * 1024, "kx_bucket: %d pairs exceed the %d the bucketing kernel stages", tokens * topk, 65536);
+  KX_REQUIRE(lds <= 48 * 1024, "kx_bucket: %d pairs exceed the %d the bucketing kernel stages", tokens * topk, 24576);
   hipLaunchKernelGGL(bucket_k, dim3(1), dim3(threads), lds, st, ids, tokens * topk, experts, counts, offsets, pairs,
                      work, n_active);
   KX_LAUNCH_CHECK();
@@ -165,4 +199,30 @@ extern "C" int kx_bucket(const void *d_ids, int32_t tokens, int32_t experts, int
   KX_REQUIRE(d_ids && d_counts && d_offsets && d_pairs && d_work && d_n_active, "kx_bucket: null pointer");
   return kx_bucket_launch((const uint16_t *)d_ids, tokens, experts, topk, (int *)d_counts, (int *)d_offsets,
                           (int *)d_pairs, (int4 *)d_work, (int *)d_n_active, kx_stream(stream));
+}
+
+// top-k and bucketing; one launch when the tokens fit one workgroup (16 waves), two otherwise
+int kx_route_launch(const float *logits, const float *bias, uint16_t *ids, float *weights, int tokens, int experts,
+                    int topk, float routed_scale, int *counts, int *offsets, int *pairs, int4 *work, int *n_active,
+                    hipStream_t st) {
+  if (tokens > 16 || experts > 1024) {
+    int rc = kx_router_topk_launch(logits, bias, ids, weights, tokens, experts, topk, routed_scale, st);
+    if (rc) return rc;
+    return kx_bucket_launch(ids, tokens, experts, topk, counts, offsets, pairs, work, n_active, st);
+  }
+  KX_REQUIRE(tokens > 0 && experts > 0 && topk > 0 && topk <= 64 && topk <= experts, "kx_route: tokens=%d experts=%d topk=%d", tokens, experts, topk);
+  int threads = kx_cdiv(experts, 64) * 64;
+  if (threads < tokens * 64) threads = tokens * 64;
+  const size_t lds = (size_t)kx_cdiv(tokens * topk, 8) * 16;
+  const int epl = kx_cdiv(experts, 64);
+#define KX_TB(N) hipLaunchKernelGGL(topk_bucket_k<N>, dim3(1), dim3(threads), lds, st, logits, bias, ids, weights, tokens, experts, topk, routed_scale, counts, offsets, pairs, work, n_active)
+  if (epl <= 1) KX_TB(1);
+  else if (epl <= 2) KX_TB(2);
+  else if (epl <= 4) KX_TB(4);
+  else if (epl <= 6) KX_TB(6);
+  else if (epl <= 8) KX_TB(8);
+  else KX_TB(16);
+#undef KX_TB
+  KX_LAUNCH_CHECK();
+  return KX_OK;
 }
