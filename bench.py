@@ -389,12 +389,43 @@ def run_prefill(args):
     return out
 
 
+def run_copy(args):
+    """Plain copy of a known size: the kernel whose FETCH_SIZE / WRITE_SIZE readings calibrate the traffic figures."""
+    from blok_amd.lib import check, kx
+    lib = kx()
+    nbytes = args.copy_mib << 20
+    src, dst = C.c_void_p(), C.c_void_p()
+    check(lib.kx_dev_malloc(C.byref(src), nbytes))
+    check(lib.kx_dev_malloc(C.byref(dst), nbytes))
+    check(lib.kx_fill_words_u32(src, nbytes // 4, 1, 1, None))
+    e0, e1 = C.c_void_p(), C.c_void_p()
+    check(lib.kx_event_create(C.byref(e0)))
+    check(lib.kx_event_create(C.byref(e1)))
+    for _ in range(args.warmup):
+        check(lib.kx_dev_copy(dst, src, nbytes, None))
+    check(lib.kx_sync(None))
+    check(lib.kx_event_record(e0, None))
+    for _ in range(args.steps):
+        check(lib.kx_dev_copy(dst, src, nbytes, None))
+    check(lib.kx_event_record(e1, None))
+    check(lib.kx_sync(None))
+    ms = C.c_float()
+    check(lib.kx_event_elapsed_ms(e0, e1, C.byref(ms)))
+    per = ms.value / args.steps
+    print(json.dumps({"metric": "copy16_k read+write GB/s", "value": round(2 * nbytes / (per * 1e-3) / 1e9, 1),
+                      "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+                      "ms_per_step": round(per, 5), "higher_is_better": True,
+                      "config": {"workload": f"kx_dev_copy of {args.copy_mib} MiB (reads {nbytes} B, writes {nbytes} B per launch)"}}),
+          flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--workload", default="stack", choices=["stack", "moe_layer", "prefill"])
+    ap.add_argument("--workload", default="stack", choices=["stack", "moe_layer", "prefill", "copy"])
+    ap.add_argument("--copy-mib", type=int, default=1024)
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--prompt", type=int, default=1024)
     ap.add_argument("--stack-layers", type=int, default=24)
@@ -410,6 +441,9 @@ def main():
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
         sys.exit(2)
     build_if_missing()
+    if args.workload == "copy":
+        run_copy(args)
+        return
     if args.workload == "prefill":
         if args.tokens == 1:
             args.tokens = 2048

@@ -93,6 +93,34 @@ __global__ void __launch_bounds__(1024) gemv_bf16_k(KxGemvArgs a) {
   const bool x_once = T <= TT;  // activations stay in registers for the whole chunk
   const uint16_t *wm[2] = {a.w0, MATS == 2 ? a.w1 : a.w0};
 
+  // (chunk, slice) -> first row of the chunk, its row block, this lane's column, this wave's weight rows
+  struct Item { int c0, blk; uint32_t col; const uint16_t *wb[2]; };
+  auto item = [&](int chunk, int s) {
+    Item it;
+    it.c0 = chunk * CR;
+    it.c0 = it.c0 + CR <= a.rows ? it.c0 : a.rows - CR;  // host guarantees rows >= CR
+    it.col = (uint32_t)s * 512u + (uint32_t)lane * 8u;
+    it.blk = a.row_block ? it.c0 / a.row_block : 0;
+    const int wrow0 = a.row_block ? it.blk * a.w_block_stride + a.w_block_off + (it.c0 - it.blk * a.row_block) : it.c0;
+    it.wb[0] = wm[0] + (size_t)(wrow0 + rset * RI) * a.cols;
+    it.wb[1] = wm[1] + (size_t)(wrow0 + rset * RI) * a.cols;
+    return it;
+  };
+  auto load_tile = [&](uint4 (&buf)[MATS][RI], const Item &it, int tile) {
+#pragma unroll
+    for (int i = 0; i < RI; ++i)
+#pragma unroll
+      for (int m = 0; m < MATS; ++m)
+        buf[m][i] = ld_stream16(it.wb[m] + (size_t)((tile * RT + i) * a.cols) + it.col);
+  };
+  uint4 bufA[MATS][RI], bufB[MATS][RI];
+  // the first weight tile is requested before the prologue so that its latency overlaps it
+  bool preloaded = false;
+  if (a.norm_w && (int)blockIdx.x < n_chunks && wslot < S) {
+    load_tile(bufA, item(blockIdx.x, wslot), 0);
+    preloaded = true;
+  }
+
   // Optional prologue: RMSNorm of the activation rows (rmsnorm_k's schedule: 256 threads own the
   // 8-element chunks t, t+256, ...; butterfly per wave; ((w0+w1)+w2)+w3).  Every workgroup
   // computes the row scales; the normalised values are formed when the activations are loaded.
@@ -138,20 +166,12 @@ __global__ void __launch_bounds__(1024) gemv_bf16_k(KxGemvArgs a) {
 
   for (int chunk = blockIdx.x; chunk < n_chunks; chunk += gridDim.x) {
     int c0 = chunk * CR;
-    c0 = c0 + CR <= a.rows ? c0 : a.rows - CR;  // host guarantees rows >= CR
+    c0 = c0 + CR <= a.rows ? c0 : a.rows - CR;
     for (int s = wslot; s < S; s += a.nw) {
-      const uint32_t col = (uint32_t)s * 512u + (uint32_t)lane * 8u;
-      const int blk = a.row_block ? c0 / a.row_block : 0;
-      const int wrow0 = a.row_block ? blk * a.w_block_stride + a.w_block_off + (c0 - blk * a.row_block) : c0;
+      const Item it = item(chunk, s);
+      const uint32_t col = it.col;
+      const int blk = it.blk;
       const uint16_t *xb = a.x + (size_t)blk * a.x_block_stride;
-      const uint16_t *wb[2] = {wm[0] + (size_t)(wrow0 + rset * RI) * a.cols, wm[1] + (size_t)(wrow0 + rset * RI) * a.cols};
-      auto load_tile = [&](uint4 (&buf)[MATS][RI], int tile) {
-#pragma unroll
-        for (int i = 0; i < RI; ++i)
-#pragma unroll
-          for (int m = 0; m < MATS; ++m)
-            buf[m][i] = ld_stream16(wb[m] + (size_t)((tile * RT + i) * a.cols) + col);
-      };
       float xs[TT][8];
       auto load_x = [&](int t0) {
 #pragma unroll
@@ -159,20 +179,36 @@ __global__ void __launch_bounds__(1024) gemv_bf16_k(KxGemvArgs a) {
           const int tok = min(t0 + t, T - 1);
           if (a.mla_po) {
             // activations = merged attention partials of head `blk` (mla_combine's arithmetic):
-            // M = max M_j; w_j = exp(M_j - M); Z = fma(Z_j, w_j, Z); O = fma(O_j, w_j, O); x = bf(O / Z)
-            float M = -__builtin_inff();
-            for (int j = 0; j < a.mla_spans; ++j) M = fmaxf(M, a.mla_pm[((size_t)tok * a.mla_spans + j) * a.mla_heads + blk]);
+            // M = max M_j; w_j = exp(M_j - M); Z = fma(Z_j, w_j, Z); O = fma(O_j, w_j, O); x = bf(O / Z).
+            // Lane j holds span j's (M_j, Z_j, w_j); the O_j rows are fetched four spans at a time.
+            const int spans = a.mla_spans;
+            const size_t idx0 = (size_t)tok * spans * a.mla_heads + blk;
+            const size_t my = idx0 + (size_t)min(lane, spans - 1) * a.mla_heads;
+            const float mj = a.mla_pm[my], zj = a.mla_pz[my];
+            const float M = kxw::wave_max_f32(lane < spans ? mj : -__builtin_inff());
+            const float wj = kx_expf(mj - M);
             float Z = 0.0f, O[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-            for (int j = 0; j < a.mla_spans; ++j) {
-              const size_t idx = ((size_t)tok * a.mla_spans + j) * a.mla_heads + blk;
-              const float w = kx_expf(a.mla_pm[idx] - M);
-              Z = __builtin_fmaf(a.mla_pz[idx], w, Z);
-              const float4 *o = (const float4 *)(a.mla_po + idx * a.cols + col);
-              const float4 o0 = o[0], o1 = o[1];
-              O[0] = __builtin_fmaf(o0.x, w, O[0]); O[1] = __builtin_fmaf(o0.y, w, O[1]);
-              O[2] = __builtin_fmaf(o0.z, w, O[2]); O[3] = __builtin_fmaf(o0.w, w, O[3]);
-              O[4] = __builtin_fmaf(o1.x, w, O[4]); O[5] = __builtin_fmaf(o1.y, w, O[5]);
-              O[6] = __builtin_fmaf(o1.z, w, O[6]); O[7] = __builtin_fmaf(o1.w, w, O[7]);
+            for (int j = 0; j < spans; ++j)
+              Z = __builtin_fmaf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, zj), j)),
+                                 __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wj), j)), Z);
+            for (int j0 = 0; j0 < spans; j0 += 4) {
+              float4 o0[4], o1[4];
+#pragma unroll
+              for (int u = 0; u < 4; ++u) {
+                const float4 *o = (const float4 *)(a.mla_po + (idx0 + (size_t)min(j0 + u, spans - 1) * a.mla_heads) * a.cols + col);
+                o0[u] = o[0];
+                o1[u] = o[1];
+              }
+#pragma unroll
+              for (int u = 0; u < 4; ++u) {
+                if (j0 + u < spans) {
+                  const float w = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wj), j0 + u));
+                  O[0] = __builtin_fmaf(o0[u].x, w, O[0]); O[1] = __builtin_fmaf(o0[u].y, w, O[1]);
+                  O[2] = __builtin_fmaf(o0[u].z, w, O[2]); O[3] = __builtin_fmaf(o0[u].w, w, O[3]);
+                  O[4] = __builtin_fmaf(o1[u].x, w, O[4]); O[5] = __builtin_fmaf(o1[u].y, w, O[5]);
+                  O[6] = __builtin_fmaf(o1[u].z, w, O[6]); O[7] = __builtin_fmaf(o1[u].w, w, O[7]);
+                }
+              }
             }
 #pragma unroll
             for (int e = 0; e < 8; ++e) xs[t][e] = kx_bfround(O[e] / Z);
@@ -218,13 +254,13 @@ __global__ void __launch_bounds__(1024) gemv_bf16_k(KxGemvArgs a) {
           }
         }
       };
-      uint4 bufA[MATS][RI], bufB[MATS][RI];
-      load_tile(bufA, 0);
+      if (!preloaded) load_tile(bufA, it, 0);
+      preloaded = false;
       if (x_once) load_x(0);
       for (int tile = 0; tile < a.nt; tile += 2) {
-        if (tile + 1 < a.nt) load_tile(bufB, tile + 1);
+        if (tile + 1 < a.nt) load_tile(bufB, it, tile + 1);
         compute_tile(bufA, tile);
-        if (tile + 2 < a.nt) load_tile(bufA, tile + 2);
+        if (tile + 2 < a.nt) load_tile(bufA, it, tile + 2);
         if (tile + 1 < a.nt) compute_tile(bufB, tile + 1);
       }
     }
@@ -378,6 +414,7 @@ int kx_gemv_launch(int epi, KxGemvArgs a, hipStream_t st) {
   }
   if (a.mla_po) {
     KX_REQUIRE(a.row_block && a.cols == 512 && !a.norm_w, "kx_gemv: attention partials feed a 512-column blocked matrix");
+    KX_REQUIRE(a.tokens <= 4 && a.mla_spans >= 1 && a.mla_spans <= 64, "kx_gemv: the fused attention merge takes at most 4 tokens and 64 spans (got %d, %d)", a.tokens, a.mla_spans);
   }
   const int all_tokens = a.tokens;
   const uint16_t *x0 = a.x;

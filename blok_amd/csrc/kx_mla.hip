@@ -86,7 +86,8 @@ __device__ __forceinline__ void unpack8(float (&f)[8], uint4 u) {
 }
 
 // RMSNorm of one row by the first 256 threads of a workgroup; the schedule of rmsnorm_k (kx_dense.hip).
-// Every thread of the workgroup must call it (it contains barriers).
+// Every thread of the workgroup must call it (it contains barriers).  A workgroup of fewer than 256
+// threads must cover the row's n/8 chunks with one chunk per thread (the missing waves add +0).
 __device__ __forceinline__ void rmsnorm_block(const uint16_t *xr, const uint16_t *w, uint16_t *yr, int n, float eps,
                                               float *ws /* 4 floats of LDS */) {
   const int chunks = n >> 3;
@@ -102,6 +103,8 @@ __device__ __forceinline__ void rmsnorm_block(const uint16_t *xr, const uint16_t
   float vv[1] = {v};
   kxw::reduce<1, 64>(vv, threadIdx.x & 63);
   __syncthreads();  // ws may still be read from a previous call
+  if (threadIdx.x < 4) ws[threadIdx.x] = 0.0f;
+  __syncthreads();
   if (active && (threadIdx.x & 63) == 0) ws[threadIdx.x >> 6] = vv[0];
   __syncthreads();
   const float total = ((ws[0] + ws[1]) + ws[2]) + ws[3];
@@ -145,9 +148,11 @@ __device__ __forceinline__ void kv_finish_block(const uint16_t *kva, const uint1
   }
 }
 
-// q_abs[t][h] = (bf(W_UK[h]^T q_nope[h]) | rope(q_rope[h])) as f32.  Grid (heads + 1, T), 8 waves:
-// wave j runs the chain over d = j, j+8, ...; lane owns 8 latent columns.  The extra block
-// (blockIdx.x == heads) finishes the token's kv_a output and writes its cache row.
+// q_abs[t][h] = (bf(W_UK[h]^T q_nope[h]) | rope(q_rope[h])) as f32.  A workgroup of 128 threads takes
+// 128 latent columns of one head: thread (chain, cl) = (tid / 16, tid % 16) runs the fma chain over
+// d = chain, chain+8, ... for columns 8 cl .. 8 cl + 7; the 8 chains are then summed pairwise.
+// Grid (heads * ceil(kv_rank / 128) + 1, T): the extra workgroup finishes the token's kv_a output and
+// writes its cache row.
 struct QAbsArgs {
   const uint16_t *q, *kvb, *rope_row;
   float *qabs;
@@ -157,25 +162,29 @@ struct QAbsArgs {
   int heads, nope, rope, v_head, kv_rank, kva_stride, pos;
   float eps;
 };
-__global__ void __launch_bounds__(512) q_absorb_k(QAbsArgs a) {
-  extern __shared__ float part[];  // [8][kv_rank]
+__global__ void __launch_bounds__(128) q_absorb_k(QAbsArgs a) {
+  __shared__ float part[8][128];
   __shared__ float ws[4];
-  const int h = blockIdx.x, t = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int t = blockIdx.y;
   const int nope = a.nope, rope = a.rope, kv_rank = a.kv_rank;
   const int qk = nope + rope, kva = kv_rank + rope;
-  if (h == a.heads) {
+  const int cq_n = (kv_rank + 127) >> 7;
+  if ((int)blockIdx.x == a.heads * cq_n) {
     if (a.cache)
       kv_finish_block(a.kva + (size_t)t * a.kva_stride, a.w_kv_ln, a.rope_row, a.cache + (size_t)t * a.seq_stride + (size_t)a.pos * kva,
                       kv_rank, rope, a.eps, ws);
     return;
   }
+  const int h = blockIdx.x / cq_n, cq = blockIdx.x - h * cq_n;
+  const int cl = threadIdx.x & 15, chain = threadIdx.x >> 4;
   const uint16_t *qh = a.q + ((size_t)t * a.heads + h) * qk;
   const uint16_t *wuk = a.kvb + (size_t)h * (nope + a.v_head) * kv_rank;
   float *out = a.qabs + ((size_t)t * a.heads + h) * kva;
-  for (int c0 = lane * 8; c0 < kv_rank; c0 += 512) {
+  const int c0 = cq * 128 + cl * 8;
+  if (c0 < kv_rank) {
     float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll 8
-    for (int d = wave; d < nope; d += 8) {
+#pragma unroll 16
+    for (int d = chain; d < nope; d += 8) {
       float wf[8];
       unpack8(wf, *(const uint4 *)(wuk + (size_t)d * kv_rank + c0));
       const float qd = kx_bf16_f32(qh[d]);
@@ -183,17 +192,18 @@ __global__ void __launch_bounds__(512) q_absorb_k(QAbsArgs a) {
       for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(wf[e], qd, acc[e]);
     }
 #pragma unroll
-    for (int e = 0; e < 8; ++e) part[wave * kv_rank + c0 + e] = acc[e];
+    for (int e = 0; e < 8; ++e) part[chain][cl * 8 + e] = acc[e];
   }
   __syncthreads();
-  for (int c = threadIdx.x; c < kv_rank; c += blockDim.x) {
-    const float *p = part + c;
-    const float s = ((p[0] + p[kv_rank]) + (p[2 * kv_rank] + p[3 * kv_rank])) +
-                    ((p[4 * kv_rank] + p[5 * kv_rank]) + (p[6 * kv_rank] + p[7 * kv_rank]));
-    out[c] = kx_bfround(s);
+  {
+    const int c = threadIdx.x;
+    if (cq * 128 + c < kv_rank) {
+      const float s = ((part[0][c] + part[1][c]) + (part[2][c] + part[3][c])) + ((part[4][c] + part[5][c]) + (part[6][c] + part[7][c]));
+      out[cq * 128 + c] = kx_bfround(s);
+    }
   }
   const int half = rope >> 1;
-  if ((int)threadIdx.x < half) {
+  if (cq == 0 && (int)threadIdx.x < half) {
     const int p = threadIdx.x;
     float lo, hi;
     rope_pair(kx_bf16_f32(qh[nope + 2 * p]), kx_bf16_f32(qh[nope + 2 * p + 1]), kx_bf16_f32(a.rope_row[p]),
@@ -348,12 +358,12 @@ __global__ void __launch_bounds__(64) mla_combine_k(const float *__restrict__ pm
 int kx_q_absorb_launch(const uint16_t *q, const uint16_t *kvb, const uint16_t *rope_row, float *qabs, int tokens,
                        int heads, int nope, int rope, int v_head, int kv_rank, const uint16_t *kva, int kva_stride,
                        const uint16_t *w_kv_ln, uint16_t *cache, size_t seq_stride, int pos, float eps, hipStream_t st) {
-  KX_REQUIRE(kv_rank % 8 == 0 && rope % 2 == 0 && rope / 2 <= 512, "kx_q_absorb: bad shape");
+  KX_REQUIRE(kv_rank % 8 == 0 && kv_rank <= 1024 && rope % 2 == 0 && rope / 2 <= 128, "kx_q_absorb: kv_rank=%d (multiple of 8, at most 1024), rope=%d (even, at most 256)", kv_rank, rope);
   QAbsArgs a;
   a.q = q; a.kvb = kvb; a.rope_row = rope_row; a.qabs = qabs; a.kva = kva; a.w_kv_ln = w_kv_ln; a.cache = cache;
   a.seq_stride = seq_stride; a.heads = heads; a.nope = nope; a.rope = rope; a.v_head = v_head; a.kv_rank = kv_rank;
   a.kva_stride = kva_stride; a.pos = pos; a.eps = eps;
-  hipLaunchKernelGGL(q_absorb_k, dim3(heads + (cache ? 1 : 0), tokens), dim3(512), (size_t)8 * kv_rank * sizeof(float), st, a);
+  hipLaunchKernelGGL(q_absorb_k, dim3(heads * ((kv_rank + 127) / 128) + (cache ? 1 : 0), tokens), dim3(128), 0, st, a);
   KX_LAUNCH_CHECK();
   return KX_OK;
 }

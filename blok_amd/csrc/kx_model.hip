@@ -251,13 +251,17 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample) {
     // W_UK absorb + rope(q); the extra block norms kv_a, rotates the rope key, writes the cache row (:817-824)
     KX_TRY(kx_q_absorb_launch(m->q, L.kvb, rope_row, m->qabs, B, c.heads, c.qk_nope, c.qk_rope, c.v_head, c.kv_rank,
                               m->qkv + c.q_rank, QKV, L.kv_ln, L.cache, seq_stride, pos, c.rms_eps, st));
-    KxMlaPartials mp;
-    KX_TRY(kx_mla_partials_launch(&c, L.cache, seq_stride, m->qabs, m->partial, B, pos + 1, &mp, st));  // :825
-    g = {};  // W_UV of :818 per head; its activations are the merged attention partials
+    g = {};  // W_UV of :818 per head
     g.w0 = L.kvb; g.x = m->o_lat; g.x_stride = c.heads * c.kv_rank; g.out = m->att; g.out_stride = VD; g.rows = VD;
     g.cols = c.kv_rank; g.tokens = B; g.row_block = c.v_head; g.w_block_stride = c.qk_nope + c.v_head;
     g.w_block_off = c.qk_nope; g.x_block_stride = c.kv_rank;
-    g.mla_pm = mp.pm; g.mla_pz = mp.pz; g.mla_po = mp.po; g.mla_spans = mp.spans; g.mla_heads = c.heads;
+    if (fuse) {  // its activations are the attention partials, merged as they are loaded      // :825
+      KxMlaPartials mp;
+      KX_TRY(kx_mla_partials_launch(&c, L.cache, seq_stride, m->qabs, m->partial, B, pos + 1, &mp, st));
+      g.mla_pm = mp.pm; g.mla_pz = mp.pz; g.mla_po = mp.po; g.mla_spans = mp.spans; g.mla_heads = c.heads;
+    } else {
+      KX_TRY(kx_mla_attend_launch(&c, L.cache, seq_stride, m->qabs, m->partial, m->o_lat, B, pos + 1, st));
+    }
     KX_TRY(kx_gemv_launch(KX_EPI_BF16, g, st));
     g = {};
     g.w0 = L.o; g.x = m->att; g.x_stride = VD; g.out = m->x; g.out_stride = H; g.rows = H; g.cols = VD; g.tokens = B;

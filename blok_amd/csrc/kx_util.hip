@@ -144,6 +144,19 @@ extern "C" int kx_fill_normal_f32(void *d_out, uint64_t n, uint64_t seed, uint64
   KX_LAUNCH_CHECK();
   return KX_OK;
 }
+// plain 16-byte-per-lane copy: the known-traffic kernel that HBM counters are calibrated against
+__global__ void __launch_bounds__(256) copy16_k(uint4 *__restrict__ dst, const uint4 *__restrict__ src, uint64_t n16) {
+  for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (uint64_t)gridDim.x * 256) dst[i] = src[i];
+}
+extern "C" int kx_dev_copy(void *d_dst, const void *d_src, uint64_t bytes, void *stream) {
+  KX_REQUIRE((d_dst && d_src) || !bytes, "kx_dev_copy: null pointer");
+  KX_REQUIRE(bytes % 16 == 0 && ((uintptr_t)d_dst | (uintptr_t)d_src) % 16 == 0, "kx_dev_copy: 16-byte granularity");
+  if (!bytes) return KX_OK;
+  hipLaunchKernelGGL(copy16_k, dim3(fill_grid(bytes / 16)), dim3(256), 0, kx_stream(stream), (uint4 *)d_dst,
+                     (const uint4 *)d_src, bytes / 16);
+  KX_LAUNCH_CHECK();
+  return KX_OK;
+}
 extern "C" int kx_fill_words_u32(void *d_out, uint64_t n, uint64_t seed, uint64_t tensor_id, void *stream) {
   KX_REQUIRE(d_out || !n, "kx_fill_words_u32: null pointer");
   if (!n) return KX_OK;

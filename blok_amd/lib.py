@@ -56,6 +56,7 @@ _SIGS = {
     "kx_fill_normal_bf16": [_P, _U64, _U64, _U64, _F, C.c_int, _P],
     "kx_fill_normal_f32": [_P, _U64, _U64, _U64, _F, _P],
     "kx_fill_words_u32": [_P, _U64, _U64, _U64, _P],
+    "kx_dev_copy": [_P, _P, _U64, _P],
     "kx_i4_unpack": [_P, _P, _I, _I, _P],
     "kx_i4_dequant": [_P, _P, _P, _I, _I, _P],
     "kx_i4_gemv": [_P, _P, _P, _P, _I, _I, _I, _P],

@@ -79,6 +79,10 @@ int kx_event_destroy(void *event);
 int kx_event_record(void *event, void *stream);
 int kx_event_elapsed_ms(void *start, void *stop, float *ms); /* waits for stop */
 
+/* Device-to-device copy by a plain kernel (16 bytes per lane); bytes and both pointers multiples of 16.
+ * No counterpart in the reference: it is the known-size kernel that HBM traffic counters are scaled by. */
+int kx_dev_copy(void *d_dst, const void *d_src, uint64_t bytes, void *stream);
+
 /* ---- synthetic tensors: value = f(seed, tensor_id, index) --------------- */
 int kx_fill_normal_bf16(void *d_out, uint64_t n, uint64_t seed, uint64_t tensor_id, float sigma,
                         int absval, void *stream);
