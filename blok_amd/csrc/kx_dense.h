@@ -38,8 +38,10 @@ struct KxGemvArgs {
   const uint16_t *expert_out;  // bf16 [tokens*topk, rows]
   const float *route_w;        // f32 [tokens, topk]
   int topk;
-  uint32_t flags;
+  uint32_t flags;              // bit 0: MOE_COMBINE overwrites x; KX_GEMV_COHERENT_OUT: see below
 };
+// F32 epilogue: store the outputs with device-scope stores (another workgroup of the launch reads them)
+#define KX_GEMV_COHERENT_OUT 2u
 
 int kx_gemv_launch(int epi, KxGemvArgs a, hipStream_t st);
 int kx_rmsnorm_launch(const uint16_t *x, const uint16_t *w, uint16_t *y, int tokens, int n, int x_stride,
@@ -57,6 +59,9 @@ int kx_i4_launch(bool dual, const uint32_t *packed0, const uint16_t *scale0, con
 // kx_router.hip
 int kx_router_topk_launch(const float *logits, const float *bias, uint16_t *ids, float *weights, int tokens,
                           int experts, int topk, float routed_scale, hipStream_t st);
+int kx_gemv_pair_route_launch(KxGemvArgs shared_gate_up, KxGemvArgs router, const float *bias, uint16_t *ids, float *weights,
+                              int experts, int topk, float routed_scale, int *counts, int *offsets, int *pairs, int4 *work,
+                              int *n_active, int *counter, bool *fused, hipStream_t st);
 int kx_route_launch(const float *logits, const float *bias, uint16_t *ids, float *weights, int tokens, int experts,
                     int topk, float routed_scale, int *counts, int *offsets, int *pairs, int4 *work, int *n_active,
                     hipStream_t st);

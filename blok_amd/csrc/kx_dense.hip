@@ -16,6 +16,7 @@
 #include "kx_common.h"
 #include "kx_dense.h"
 #include "kx_math.h"
+#include "kx_route.h"
 #include "kx_wave.h"
 
 namespace {
@@ -81,8 +82,8 @@ __global__ void __launch_bounds__(256) rmsnorm_k(const uint16_t *__restrict__ x,
 // moved back to end at the last row; the rows it shares with the previous chunk are
 // computed twice but written once, by the previous chunk.
 template <int MATS, int RI, int TT>
-__global__ void __launch_bounds__(1024) gemv_bf16_k(KxGemvArgs a) {
-  extern __shared__ float part[];  // [mats][CR][tokens][S]
+__device__ __forceinline__ void gemv_body(const KxGemvArgs &a, const int bid, const int nblocks,
+                                          float *part /* LDS [mats][CR][tokens][S] */) {
   constexpr int NV = RI * MATS * TT;
   constexpr int NOUT = kxw::reduce_out<NV, 64>();
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -116,8 +117,8 @@ __global__ void __launch_bounds__(1024) gemv_bf16_k(KxGemvArgs a) {
   uint4 bufA[MATS][RI], bufB[MATS][RI];
   // the first weight tile is requested before the prologue so that its latency overlaps it
   bool preloaded = false;
-  if (a.norm_w && (int)blockIdx.x < n_chunks && wslot < S) {
-    load_tile(bufA, item(blockIdx.x, wslot), 0);
+  if (a.norm_w && bid < n_chunks && wslot < S) {
+    load_tile(bufA, item(bid, wslot), 0);
     preloaded = true;
   }
 
@@ -145,7 +146,7 @@ __global__ void __launch_bounds__(1024) gemv_bf16_k(KxGemvArgs a) {
       if (threadIdx.x == 0) n_scale[t] = kx_rsqrtf((((n_ws[0] + n_ws[1]) + n_ws[2]) + n_ws[3]) / (float)a.cols + a.norm_eps);
       __syncthreads();
     }
-    if (a.norm_out && blockIdx.x == 0)  // one workgroup also stores the normalised rows for later kernels
+    if (a.norm_out && bid == 0)  // one workgroup also stores the normalised rows for later kernels
       for (int t = 0; t < T; ++t) {
         const uint16_t *xr = a.x + (size_t)t * a.x_stride;
         uint16_t *yr = a.norm_out + (size_t)t * a.cols;
@@ -164,7 +165,7 @@ __global__ void __launch_bounds__(1024) gemv_bf16_k(KxGemvArgs a) {
       }
   }
 
-  for (int chunk = blockIdx.x; chunk < n_chunks; chunk += gridDim.x) {
+  for (int chunk = bid; chunk < n_chunks; chunk += nblocks) {
     int c0 = chunk * CR;
     c0 = c0 + CR <= a.rows ? c0 : a.rows - CR;
     for (int s = wslot; s < S; s += a.nw) {
@@ -283,7 +284,10 @@ __global__ void __launch_bounds__(1024) gemv_bf16_k(KxGemvArgs a) {
           ((uint16_t *)a.out)[(size_t)tok * a.out_stride + row] = kx_bf16_rne(y0);
           break;
         case KX_EPI_F32:
-          ((float *)a.out)[(size_t)tok * a.out_stride + row] = y0;
+          if (a.flags & KX_GEMV_COHERENT_OUT)  // read back by another workgroup of this launch: store through to memory
+            __hip_atomic_store((float *)a.out + (size_t)tok * a.out_stride + row, y0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          else
+            ((float *)a.out)[(size_t)tok * a.out_stride + row] = y0;
           break;
         case KX_EPI_SWIGLU:
           ((uint16_t *)a.out)[(size_t)tok * a.out_stride + row] = kx_bf16_rne(kx_swiglu(kx_bfround(y0), kx_bfround(y1)));
@@ -312,6 +316,55 @@ __global__ void __launch_bounds__(1024) gemv_bf16_k(KxGemvArgs a) {
     }
     __syncthreads();
   }
+}
+
+template <int MATS, int RI, int TT>
+__global__ void __launch_bounds__(TT > 1 ? 512 : 1024) gemv_bf16_k(KxGemvArgs a) {
+  extern __shared__ float part[];
+  gemv_body<MATS, RI, TT>(a, blockIdx.x, gridDim.x, part);
+}
+
+// Two GEMVs over the same activations in one launch: the first gridDim.x - n0 workgroups run the
+// second problem (the router gate, f32 logits), the other n0 the first (two matrices, SwiGLU:
+// the shared expert's gate and up).  The router workgroup that finishes last routes the tokens: top-k and
+// bucketing, from the logits that all of them have written by then.
+struct KxRouteArgs {
+  int *counter;  // zero before the launch; the routing workgroup leaves it at zero
+  const float *bias;
+  uint16_t *ids;
+  float *weights;
+  int experts, topk;
+  float routed_scale;
+  int *counts, *offsets, *pairs;
+  int4 *work;
+  int *n_active;
+};
+template <int RI0, int TT>
+__global__ void __launch_bounds__(TT > 1 ? 512 : 1024) gemv_pair_k(KxGemvArgs a0, KxGemvArgs a1, int n0, KxRouteArgs r) {
+  extern __shared__ float part[];
+  const int n1 = gridDim.x - n0;  // the router's workgroups come first: its routing tail overlaps the rest
+  if ((int)blockIdx.x >= n1) {
+    gemv_body<2, RI0, TT>(a0, blockIdx.x - n1, n0, part);
+    return;
+  }
+  gemv_body<1, 1, TT>(a1, blockIdx.x, n1, part);
+  if (!r.counter) return;
+  __shared__ int s_last;
+  __shared__ int s_cnt[1024];
+  __shared__ int s_act[1024];
+  __shared__ uint4 s_ids4[4];
+  // The logits were stored through to memory (device-scope stores).  Every wave waits for its stores
+  // to be acknowledged; after the barrier one thread counts the workgroup in.  The workgroup that
+  // counts in last reads all logits with device-scope loads, so no cache has to be flushed.
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+  if (threadIdx.x == 0)
+    s_last = __hip_atomic_fetch_add(r.counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == n1 - 1;
+  __syncthreads();
+  if (!s_last) return;
+  kxr::route_block_any<true>((const float *)a1.out, r.bias, r.ids, r.weights, a1.tokens, r.experts, r.topk, r.routed_scale,
+                       r.counts, r.offsets, r.pairs, r.work, r.n_active, s_ids4, s_cnt, s_act);
+  if (threadIdx.x == 0) *r.counter = 0;
 }
 
 // lowest-index argmax over bf16-rounded logits (sample_lm_head :718-734, argmax_k :477-493), in two
@@ -381,11 +434,13 @@ void launch_ri(const KxGemvArgs &a, int ri, int tt, dim3 g, dim3 b, size_t lds, 
 
 }  // namespace
 
-// Tokens are taken in blocks of at most 32 (LDS holds a partial per token and slice).
-int kx_gemv_launch(int epi, KxGemvArgs a, hipStream_t st) {
-  KX_REQUIRE(a.cols > 0 && a.cols % 512 == 0, "kx_gemv: cols=%d must be a positive multiple of 512", a.cols);
-  KX_REQUIRE(a.rows > 0 && a.tokens > 0, "kx_gemv: rows=%d tokens=%d must be positive", a.rows, a.tokens);
-  KX_REQUIRE(epi >= KX_EPI_BF16 && epi <= KX_EPI_ARGMAX, "kx_gemv: unknown epilogue %d", epi);
+namespace {
+// Fills in the launch shape of a GEMV (a.epi, a.nw, a.rs, a.nt) and returns rows per wave and tile in
+// ri; ri_max caps it.  Returns the rows per chunk, or -1 after setting the error.
+int gemv_plan(int epi, KxGemvArgs &a, int &ri, int ri_max, int target_chunks = 256) {
+  if (!(a.cols > 0 && a.cols % 512 == 0)) { kx_set_error("kx_gemv: cols=%d must be a positive multiple of 512", a.cols); return -1; }
+  if (!(a.rows > 0 && a.tokens > 0)) { kx_set_error("kx_gemv: rows=%d tokens=%d must be positive", a.rows, a.tokens); return -1; }
+  if (!(epi >= KX_EPI_BF16 && epi <= KX_EPI_ARGMAX)) { kx_set_error("kx_gemv: unknown epilogue %d", epi); return -1; }
   const int S = a.cols / 512;
   const int mats = epi == KX_EPI_SWIGLU ? 2 : 1;
   a.epi = epi;
@@ -397,25 +452,40 @@ int kx_gemv_launch(int epi, KxGemvArgs a, hipStream_t st) {
   a.rs = 8 / a.nw;
   while (a.rs > 1 && a.rs > a.rows) a.rs >>= 1;
   // rows per wave and tile, tiles per chunk: a few hundred chunks when the matrix allows
-  int ri = a.rows >= 2048 * a.rs ? 4 : a.rows >= 768 * a.rs ? 2 : 1;
+  ri = a.rows >= 2048 * a.rs ? 4 : a.rows >= 768 * a.rs ? 2 : 1;
   while (ri > 1 && ri * a.rs > a.rows) ri >>= 1;
   if (ri * mats > 4) ri = 4 / mats;
+  if (ri > ri_max) ri = ri_max;
   const int rt = a.rs * ri;
-  int nt = a.rows / (rt * 256);
+  int nt = a.rows / (rt * target_chunks);
   nt = nt < 1 ? 1 : nt > 8 ? 8 : nt;
   if (a.row_block) {  // a chunk must not straddle blocks
-    KX_REQUIRE(a.rows % a.row_block == 0 && a.row_block % rt == 0, "kx_gemv: row_block=%d does not fit tiles of %d rows", a.row_block, rt);
+    if (!(a.rows % a.row_block == 0 && a.row_block % rt == 0)) { kx_set_error("kx_gemv: row_block=%d does not fit tiles of %d rows", a.row_block, rt); return -1; }
     while (a.row_block % (rt * nt)) --nt;
   }
   a.nt = nt;
-  const int CR = rt * nt;
-  if (a.norm_w) {
-    KX_REQUIRE(a.tokens <= 4 && a.nw * a.rs * 64 >= 256 && !a.row_block, "kx_gemv: the fused RMSNorm needs at most 4 tokens and 256 threads");
+  if (a.norm_w && !(a.tokens <= 4 && a.nw * a.rs * 64 >= 256 && !a.row_block)) {
+    kx_set_error("kx_gemv: the fused RMSNorm needs at most 4 tokens and 256 threads");
+    return -1;
   }
   if (a.mla_po) {
-    KX_REQUIRE(a.row_block && a.cols == 512 && !a.norm_w, "kx_gemv: attention partials feed a 512-column blocked matrix");
-    KX_REQUIRE(a.tokens <= 4 && a.mla_spans >= 1 && a.mla_spans <= 64, "kx_gemv: the fused attention merge takes at most 4 tokens and 64 spans (got %d, %d)", a.tokens, a.mla_spans);
+    if (!(a.row_block && a.cols == 512 && !a.norm_w)) { kx_set_error("kx_gemv: attention partials feed a 512-column blocked matrix"); return -1; }
+    if (!(a.tokens <= 4 && a.mla_spans >= 1 && a.mla_spans <= 64)) {
+      kx_set_error("kx_gemv: the fused attention merge takes at most 4 tokens and 64 spans (got %d, %d)", a.tokens, a.mla_spans);
+      return -1;
+    }
   }
+  return rt * nt;
+}
+}  // namespace
+
+// Tokens are taken in blocks of at most 32 (LDS holds a partial per token and slice).
+int kx_gemv_launch(int epi, KxGemvArgs a, hipStream_t st) {
+  int ri;
+  const int CR = gemv_plan(epi, a, ri, 4);
+  if (CR < 0) return KX_ERR_ARG;
+  const int S = a.cols / 512;
+  const int mats = epi == KX_EPI_SWIGLU ? 2 : 1;
   const int all_tokens = a.tokens;
   const uint16_t *x0 = a.x;
   char *out0 = (char *)a.out;
@@ -438,6 +508,40 @@ int kx_gemv_launch(int epi, KxGemvArgs a, hipStream_t st) {
     else launch_ri<1>(b, ri, tt, g, blk, lds, st);
     KX_LAUNCH_CHECK();
   }
+  return KX_OK;
+}
+
+// The shared expert's gate/up GEMV (SwiGLU epilogue) and the router's logits GEMV in one launch,
+// with the routing (top-k, bucketing) done by the last router workgroup.  Returns KX_OK with
+// *fused = false, having launched nothing, when the shapes do not allow the combination.
+int kx_gemv_pair_route_launch(KxGemvArgs a0, KxGemvArgs a1, const float *bias, uint16_t *ids, float *weights, int experts,
+                              int topk, float routed_scale, int *counts, int *offsets, int *pairs, int4 *work,
+                              int *n_active, int *counter, bool *fused, hipStream_t st) {
+  *fused = false;
+  if (a0.tokens != a1.tokens || a0.tokens > 4 || a0.tokens * topk > 32 || a0.cols != a1.cols || topk > 64 || topk > experts) return KX_OK;
+  int ri0, ri1;
+  const int CR0 = gemv_plan(KX_EPI_SWIGLU, a0, ri0, 2), CR1 = gemv_plan(KX_EPI_F32, a1, ri1, 1, 128);
+  if (CR0 < 0 || CR1 < 0) return KX_ERR_ARG;
+  const int threads = a0.nw * a0.rs * 64;
+  if (threads != a1.nw * a1.rs * 64 || experts > threads || experts > 1024) return KX_OK;
+  const int S = a0.cols / 512, T = a0.tokens;
+  const size_t lds0 = (size_t)2 * CR0 * T * S * sizeof(float), lds1 = (size_t)CR1 * T * S * sizeof(float);
+  const size_t lds = lds0 > lds1 ? lds0 : lds1;
+  if (lds > 120 * 1024) return KX_OK;
+  const int n0 = kx_cdiv(a0.rows, CR0), n1 = kx_cdiv(a1.rows, CR1);
+  if (n0 + n1 > 4096) return KX_OK;
+  KxRouteArgs r;
+  r.counter = counter; r.bias = bias; r.ids = ids; r.weights = weights; r.experts = experts; r.topk = topk;
+  a1.flags |= KX_GEMV_COHERENT_OUT;
+  r.routed_scale = routed_scale; r.counts = counts; r.offsets = offsets; r.pairs = pairs; r.work = work; r.n_active = n_active;
+  const int tt = T >= 4 ? 4 : T >= 2 ? 2 : 1;
+  dim3 g(n0 + n1), blk(threads);
+#define KX_PAIR(R, TT_) hipLaunchKernelGGL((gemv_pair_k<R, TT_>), g, blk, lds, st, a0, a1, n0, r)
+  if (ri0 == 2) { if (tt == 4) KX_PAIR(2, 4); else if (tt == 2) KX_PAIR(2, 2); else KX_PAIR(2, 1); }
+  else          { if (tt == 4) KX_PAIR(1, 4); else if (tt == 2) KX_PAIR(1, 2); else KX_PAIR(1, 1); }
+#undef KX_PAIR
+  KX_LAUNCH_CHECK();
+  *fused = true;
   return KX_OK;
 }
 

@@ -27,6 +27,7 @@ struct kx_moe_workspace {
   int *pairs;         // [T*topk]
   int4 *work;         // [E] {expert, first, last, first pair}
   int *n_active;      // [1]
+  int *route_counter; // [1] zero between launches: workgroups of the router GEMV count themselves in
   uint16_t *mid;      // [T*topk, moe_inter]
   uint16_t *eout;     // [T*topk, hidden]
   uint16_t *smid;     // [T, shared_inter]
@@ -57,7 +58,7 @@ extern "C" int kx_moe_workspace_create(const kx_config *cfg, int32_t max_tokens,
   struct { void **p; size_t bytes; } allocs[] = {
       {(void **)&ws->logits, T * E * 4}, {(void **)&ws->ids, T * K * 2}, {(void **)&ws->weights, T * K * 4},
       {(void **)&ws->counts, E * 4}, {(void **)&ws->offsets, (E + 1) * 4}, {(void **)&ws->pairs, T * K * 4},
-      {(void **)&ws->work, E * 16}, {(void **)&ws->n_active, 4},
+      {(void **)&ws->work, E * 16}, {(void **)&ws->n_active, 8},
       {(void **)&ws->mid, T * K * (size_t)cfg->moe_inter * 2}, {(void **)&ws->eout, T * K * (size_t)cfg->hidden * 2},
       {(void **)&ws->smid, T * (size_t)cfg->shared_inter * 2}, {(void **)&ws->sy, T * (size_t)cfg->hidden * 2}};
   for (auto &al : allocs) {
@@ -68,6 +69,8 @@ extern "C" int kx_moe_workspace_create(const kx_config *cfg, int32_t max_tokens,
       return KX_ERR_HIP;
     }
   }
+  ws->route_counter = ws->n_active + 1;
+  KX_HIP(hipMemset(ws->n_active, 0, 8));
   for (auto &e : ws->ev) KX_HIP(hipEventCreate(&e));
   *out = ws;
   return KX_OK;
@@ -121,18 +124,28 @@ int kx_moe_layer_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_work
   const int H = c->hidden, I = c->moe_inter, E = c->experts, K = c->topk;
   const uint16_t *n = (const uint16_t *)d_n;
   if (timed) KX_HIP(hipEventRecord(ws->ev[0], st));
-  // 1-3 router
+  // router logits, top-k, bucketing; shared gate/up + SwiGLU.  Up to 4 tokens: one launch for all of it.
   KxGemvArgs g = {};
   g.w0 = (const uint16_t *)w->d_router_gate; g.x = n; g.x_stride = H; g.out = ws->logits; g.out_stride = E;
   g.rows = E; g.cols = H; g.tokens = tokens;
-  if (norm_w) {  // the router GEMV norms the residual stream itself and leaves the normed rows in d_n
+  KxGemvArgs s = {};
+  s.w0 = (const uint16_t *)w->d_shared_gate; s.w1 = (const uint16_t *)w->d_shared_up; s.x = n; s.x_stride = H;
+  s.out = ws->smid; s.out_stride = c->shared_inter; s.rows = c->shared_inter; s.cols = H; s.tokens = tokens;
+  if (norm_w) {  // both GEMVs norm the residual stream themselves; the router leaves the normed rows in d_n
     g.x = (const uint16_t *)d_x; g.norm_w = norm_w; g.norm_eps = c->rms_eps; g.norm_out = (uint16_t *)d_n;
+    s.x = (const uint16_t *)d_x; s.norm_w = norm_w; s.norm_eps = c->rms_eps;
   }
-  if ((rc = kx_gemv_launch(KX_EPI_F32, g, st))) return rc;
-  if ((rc = kx_route_launch(ws->logits, (const float *)w->d_router_bias, ws->ids, ws->weights, tokens, E, K, c->routed_scale,
-                            ws->counts, ws->offsets, ws->pairs, ws->work, ws->n_active, st))) return rc;
+  bool paired = false;
+  if ((rc = kx_gemv_pair_route_launch(s, g, (const float *)w->d_router_bias, ws->ids, ws->weights, E, K, c->routed_scale,
+                                      ws->counts, ws->offsets, ws->pairs, ws->work, ws->n_active, ws->route_counter, &paired,
+                                      st))) return rc;
+  if (!paired) {
+    if ((rc = kx_gemv_launch(KX_EPI_F32, g, st))) return rc;
+    if ((rc = kx_route_launch(ws->logits, (const float *)w->d_router_bias, ws->ids, ws->weights, tokens, E, K, c->routed_scale,
+                              ws->counts, ws->offsets, ws->pairs, ws->work, ws->n_active, st))) return rc;
+  }
   if (timed) KX_HIP(hipEventRecord(ws->ev[1], st));
-  // 4 routed gate/up + SwiGLU
+  // routed gate/up + SwiGLU
   const int tt = routed_tt(tokens, K, E);
   const int max_active = (long)tokens * K < E ? tokens * K : E;
   if ((rc = kx_i4_launch(true, (const uint32_t *)w->d_gate_packed, (const uint16_t *)w->d_gate_scale,
@@ -140,18 +153,18 @@ int kx_moe_layer_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_work
                          ws->pairs, 0, I, H, K, (size_t)I * (H / 8), (size_t)I * (H / 32),
                          tt, max_active, st))) return rc;
   if (timed) KX_HIP(hipEventRecord(ws->ev[2], st));
-  // 5 routed down
+  // routed down
   if ((rc = kx_i4_launch(false, (const uint32_t *)w->d_down_packed, (const uint16_t *)w->d_down_scale, nullptr, nullptr,
                          ws->mid, ws->eout, ws->work, ws->pairs, 0, H, I, 1,
                          (size_t)H * (I / 8), (size_t)H * (I / 32), tt, max_active, st))) return rc;
   if (timed) KX_HIP(hipEventRecord(ws->ev[3], st));
-  // 6 shared gate/up + SwiGLU
-  KxGemvArgs s = {};
-  s.w0 = (const uint16_t *)w->d_shared_gate; s.w1 = (const uint16_t *)w->d_shared_up; s.x = n; s.x_stride = H;
-  s.out = ws->smid; s.out_stride = c->shared_inter; s.rows = c->shared_inter; s.cols = H; s.tokens = tokens;
-  if ((rc = kx_gemv_launch(KX_EPI_SWIGLU, s, st))) return rc;
+  // shared gate/up + SwiGLU when it did not ride with the router
+  if (!paired) {
+    if (norm_w) { s.x = n; s.norm_w = nullptr; }  // d_n holds the normed rows by now
+    if ((rc = kx_gemv_launch(KX_EPI_SWIGLU, s, st))) return rc;
+  }
   if (timed) KX_HIP(hipEventRecord(ws->ev[4], st));
-  // 7 shared down + combine + residual
+  // shared down + combine + residual
   KxGemvArgs d = {};
   d.w0 = (const uint16_t *)w->d_shared_down; d.x = ws->smid; d.x_stride = c->shared_inter; d.out = d_x;
   d.out_stride = H; d.rows = H; d.cols = c->shared_inter; d.tokens = tokens; d.expert_out = ws->eout;

@@ -1,0 +1,152 @@
+// kx_route.h -- device-side pieces of the router: top-k of one token by one wave, and
+// the token -> expert bucketing by one workgroup.  Shared by the stand-alone router
+// kernels and by the GEMV whose last workgroup routes the logits it has just produced.
+#pragma once
+#include "kx_common.h"
+#include "kx_math.h"
+#include "kx_wave.h"
+
+namespace kxr {
+
+using kxw::wave_max_f32;
+using kxw::wave_min_i32;
+
+// top-k of one token by one wave; lane owns experts lane, lane+64, ... (EPL of them)
+template <int EPL, bool COHERENT = false>
+__device__ __forceinline__ void topk_token(const float *lg, const float *__restrict__ bias,
+                                           uint16_t *__restrict__ ids, float *__restrict__ weights, int E, int topk,
+                                           float routed_scale, int lane, uint16_t *s_ids = nullptr) {
+  float sc[EPL], sel[EPL];
+  const float NEG_INF = -__builtin_inff();
+#pragma unroll
+  for (int j = 0; j < EPL; ++j) {
+    int e = lane + 64 * j;
+    float x = 0.0f, b = e < E ? bias[e] : 0.0f;
+    if (e < E) x = COHERENT ? __hip_atomic_load(lg + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : lg[e];
+    sc[j] = kx_sigmoidf(x);
+    sel[j] = e < E ? sc[j] + b : NEG_INF;
+  }
+  float sum = 0.0f;
+  float my_w = 0.0f;  // lane k keeps the k-th winner's score
+  for (int k = 0; k < topk; ++k) {
+    float best = NEG_INF;
+    int bi = 0x7fffffff;
+#pragma unroll
+    for (int j = 0; j < EPL; ++j)
+      if (sel[j] > best) { best = sel[j]; bi = lane + 64 * j; }
+    const float m = wave_max_f32(best);
+    int win = wave_min_i32(best == m ? bi : 0x7fffffff);
+    if (win == 0x7fffffff) win = 0;  // every candidate was -inf: the reference keeps id 0 (:391-393)
+    float s_win = 0.0f;
+#pragma unroll
+    for (int j = 0; j < EPL; ++j)
+      if (win == lane + 64 * j) { s_win = sc[j]; sel[j] = NEG_INF; }
+    s_win = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, s_win), win & 63));
+    sum += s_win;
+    if (lane == k) my_w = s_win;
+    if (lane == 0) {
+      ids[k] = (uint16_t)win;
+      if (s_ids) s_ids[k] = (uint16_t)win;
+    }
+  }
+  if (lane < topk) weights[lane] = my_w / (sum + 1.0e-20f) * routed_scale;
+}
+
+// one workgroup, thread e owns expert e: count, exclusive scan, stable placement.
+// The ids are staged in LDS (padded with 0xffff to a multiple of 8) and scanned 8 at a time;
+// `staged` says the caller has already put them there.
+__device__ __forceinline__ void bucket_block(const uint16_t *__restrict__ ids, int n_pairs, int E,
+                                             int *__restrict__ counts, int *__restrict__ offsets,
+                                             int *__restrict__ pairs, int4 *__restrict__ work,
+                                             int *__restrict__ n_active, uint4 *s_ids4, int *s_cnt, int *s_act,
+                                             bool staged = false) {
+  const int e = threadIdx.x, n = blockDim.x;
+  const int n8 = (n_pairs + 7) >> 3;
+  uint16_t *s_ids = (uint16_t *)s_ids4;
+  if (!staged) {
+    for (int p = threadIdx.x; p < n8 * 8; p += n) s_ids[p] = p < n_pairs ? ids[p] : (uint16_t)0xffff;
+    __syncthreads();
+  }
+  const uint32_t me = (uint32_t)e, me2 = me | (me << 16);
+  int cnt = 0;
+  if (e < E)
+    for (int q = 0; q < n8; ++q) {
+      const uint4 u = s_ids4[q];
+      const uint32_t w[4] = {u.x ^ me2, u.y ^ me2, u.z ^ me2, u.w ^ me2};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) cnt += ((w[j] & 0xffffu) == 0) + ((w[j] >> 16) == 0);
+    }
+  s_cnt[e] = cnt;
+  s_act[e] = cnt > 0 ? 1 : 0;
+  __syncthreads();
+  for (int d = 1; d < n; d <<= 1) {  // inclusive Hillis-Steele scans of both arrays
+    int a = e >= d ? s_cnt[e - d] : 0, b = e >= d ? s_act[e - d] : 0;
+    __syncthreads();
+    s_cnt[e] += a;
+    s_act[e] += b;
+    __syncthreads();
+  }
+  const int off = s_cnt[e] - cnt, slot = s_act[e] - (cnt > 0 ? 1 : 0), total_active = s_act[n - 1];
+  if (e < E) {
+    counts[e] = cnt;
+    offsets[e] = off;
+    int pos = off, first = 0;
+    if (cnt > 0)
+      for (int q = 0; q < n8 && pos < off + cnt; ++q) {
+        const uint4 u = s_ids4[q];
+        const uint32_t w[4] = {u.x ^ me2, u.y ^ me2, u.z ^ me2, u.w ^ me2};
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const uint32_t h = (j & 1) ? (w[j >> 1] >> 16) : (w[j >> 1] & 0xffffu);
+          if (h == 0) {
+            if (pos == off) first = q * 8 + j;
+            pairs[pos++] = q * 8 + j;
+          }
+        }
+      }
+    if (cnt > 0) work[slot] = make_int4(e, off, off + cnt, first);
+    if (e >= total_active) work[e] = make_int4(-1, 0, 0, 0);
+  }
+  if (e == 0) {
+    offsets[E] = s_cnt[n - 1];
+    *n_active = total_active;
+  }
+}
+
+// top-k of `tokens` tokens (wave w takes tokens w, w + waves, ...), then the bucketing, by one workgroup
+// of at least E threads.  s_ids4 holds ceil(tokens * topk / 8) pieces; s_cnt and s_act blockDim ints each.
+template <int EPL, bool COHERENT = false>
+__device__ __forceinline__ void route_block(const float *__restrict__ logits, const float *__restrict__ bias,
+                                            uint16_t *__restrict__ ids, float *__restrict__ weights, int tokens, int E,
+                                            int topk, float routed_scale, int *__restrict__ counts,
+                                            int *__restrict__ offsets, int *__restrict__ pairs, int4 *__restrict__ work,
+                                            int *__restrict__ n_active, uint4 *s_ids4, int *s_cnt, int *s_act) {
+  uint16_t *s_ids = (uint16_t *)s_ids4;
+  const int n_pairs = tokens * topk, n8 = (n_pairs + 7) >> 3;
+  for (int p = n_pairs + threadIdx.x; p < n8 * 8; p += blockDim.x) s_ids[p] = (uint16_t)0xffff;
+  const int wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+  for (int t = wave; t < tokens; t += waves)
+    topk_token<EPL, COHERENT>(logits + (size_t)t * E, bias, ids + (size_t)t * topk, weights + (size_t)t * topk, E, topk,
+                              routed_scale, threadIdx.x & 63, s_ids + t * topk);
+  __syncthreads();
+  bucket_block(ids, n_pairs, E, counts, offsets, pairs, work, n_active, s_ids4, s_cnt, s_act, true);
+}
+
+// route_block with the per-lane expert count chosen at run time; COHERENT: the logits were written by other
+// workgroups of the same launch and are read with device-scope loads
+template <bool COHERENT = false>
+__device__ __forceinline__ void route_block_any(const float *logits, const float *bias, uint16_t *ids, float *weights,
+                                                int tokens, int E, int topk, float routed_scale, int *counts, int *offsets,
+                                                int *pairs, int4 *work, int *n_active, uint4 *s_ids4, int *s_cnt, int *s_act) {
+  const int epl = (E + 63) >> 6;
+#define KX_RB(N) route_block<N, COHERENT>(logits, bias, ids, weights, tokens, E, topk, routed_scale, counts, offsets, pairs, work, n_active, s_ids4, s_cnt, s_act)
+  if (epl <= 1) KX_RB(1);
+  else if (epl <= 2) KX_RB(2);
+  else if (epl <= 4) KX_RB(4);
+  else if (epl <= 6) KX_RB(6);
+  else if (epl <= 8) KX_RB(8);
+  else KX_RB(16);
+#undef KX_RB
+}
+
+}  // namespace kxr

@@ -14,49 +14,13 @@
 #include "kx_common.h"
 #include "kx_dense.h"
 #include "kx_math.h"
+#include "kx_route.h"
 #include "kx_wave.h"
 
 namespace {
 
-using kxw::wave_max_f32;
-using kxw::wave_min_i32;
-
-// top-k of one token by one wave; lane owns experts lane, lane+64, ... (EPL of them)
-template <int EPL>
-__device__ __forceinline__ void topk_token(const float *__restrict__ lg, const float *__restrict__ bias,
-                                           uint16_t *__restrict__ ids, float *__restrict__ weights, int E, int topk,
-                                           float routed_scale, int lane) {
-  float sc[EPL], sel[EPL];
-  const float NEG_INF = -__builtin_inff();
-#pragma unroll
-  for (int j = 0; j < EPL; ++j) {
-    int e = lane + 64 * j;
-    float x = e < E ? lg[e] : 0.0f, b = e < E ? bias[e] : 0.0f;
-    sc[j] = kx_sigmoidf(x);
-    sel[j] = e < E ? sc[j] + b : NEG_INF;
-  }
-  float sum = 0.0f;
-  float my_w = 0.0f;  // lane k keeps the k-th winner's score
-  for (int k = 0; k < topk; ++k) {
-    float best = NEG_INF;
-    int bi = 0x7fffffff;
-#pragma unroll
-    for (int j = 0; j < EPL; ++j)
-      if (sel[j] > best) { best = sel[j]; bi = lane + 64 * j; }
-    const float m = wave_max_f32(best);
-    int win = wave_min_i32(best == m ? bi : 0x7fffffff);
-    if (win == 0x7fffffff) win = 0;  // every candidate was -inf: the reference keeps id 0 (:391-393)
-    float s_win = 0.0f;
-#pragma unroll
-    for (int j = 0; j < EPL; ++j)
-      if (win == lane + 64 * j) { s_win = sc[j]; sel[j] = NEG_INF; }
-    s_win = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, s_win), win & 63));
-    sum += s_win;
-    if (lane == k) my_w = s_win;
-    if (lane == 0) ids[k] = (uint16_t)win;
-  }
-  if (lane < topk) weights[lane] = my_w / (sum + 1.0e-20f) * routed_scale;
-}
+using kxr::bucket_block;
+using kxr::topk_token;
 
 // one wave per token
 template <int EPL>
@@ -66,63 +30,6 @@ __global__ void __launch_bounds__(64) router_topk_k(const float *__restrict__ lo
   const int tok = blockIdx.x;
   topk_token<EPL>(logits + (size_t)tok * E, bias, ids + (size_t)tok * topk, weights + (size_t)tok * topk, E, topk,
                   routed_scale, threadIdx.x);
-}
-
-// one workgroup, thread e owns expert e: count, exclusive scan, stable placement.
-// The ids are staged in LDS (padded with 0xffff to a multiple of 8) and scanned 8 at a time.
-__device__ __forceinline__ void bucket_block(const uint16_t *__restrict__ ids, int n_pairs, int E,
-                                             int *__restrict__ counts, int *__restrict__ offsets,
-                                             int *__restrict__ pairs, int4 *__restrict__ work,
-                                             int *__restrict__ n_active, uint4 *s_ids4, int *s_cnt, int *s_act) {
-  const int e = threadIdx.x, n = blockDim.x;
-  const int n8 = (n_pairs + 7) >> 3;
-  uint16_t *s_ids = (uint16_t *)s_ids4;
-  for (int p = threadIdx.x; p < n8 * 8; p += n) s_ids[p] = p < n_pairs ? ids[p] : (uint16_t)0xffff;
-  __syncthreads();
-  const uint32_t me = (uint32_t)e, me2 = me | (me << 16);
-  int cnt = 0;
-  if (e < E)
-    for (int q = 0; q < n8; ++q) {
-      const uint4 u = s_ids4[q];
-      const uint32_t w[4] = {u.x ^ me2, u.y ^ me2, u.z ^ me2, u.w ^ me2};
-#pragma unroll
-      for (int j = 0; j < 4; ++j) cnt += ((w[j] & 0xffffu) == 0) + ((w[j] >> 16) == 0);
-    }
-  s_cnt[e] = cnt;
-  s_act[e] = cnt > 0 ? 1 : 0;
-  __syncthreads();
-  for (int d = 1; d < n; d <<= 1) {  // inclusive Hillis-Steele scans of both arrays
-    int a = e >= d ? s_cnt[e - d] : 0, b = e >= d ? s_act[e - d] : 0;
-    __syncthreads();
-    s_cnt[e] += a;
-    s_act[e] += b;
-    __syncthreads();
-  }
-  const int off = s_cnt[e] - cnt, slot = s_act[e] - (cnt > 0 ? 1 : 0), total_active = s_act[n - 1];
-  if (e < E) {
-    counts[e] = cnt;
-    offsets[e] = off;
-    int pos = off, first = 0;
-    if (cnt > 0)
-      for (int q = 0; q < n8 && pos < off + cnt; ++q) {
-        const uint4 u = s_ids4[q];
-        const uint32_t w[4] = {u.x ^ me2, u.y ^ me2, u.z ^ me2, u.w ^ me2};
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const uint32_t h = (j & 1) ? (w[j >> 1] >> 16) : (w[j >> 1] & 0xffffu);
-          if (h == 0) {
-            if (pos == off) first = q * 8 + j;
-            pairs[pos++] = q * 8 + j;
-          }
-        }
-      }
-    if (cnt > 0) work[slot] = make_int4(e, off, off + cnt, first);
-    if (e >= total_active) work[e] = make_int4(-1, 0, 0, 0);
-  }
-  if (e == 0) {
-    offsets[E] = s_cnt[n - 1];
-    *n_active = total_active;
-  }
 }
 
 __global__ void __launch_bounds__(1024) bucket_k(const uint16_t *__restrict__ ids, int n_pairs, int E,
@@ -135,7 +42,7 @@ __global__ void __launch_bounds__(1024) bucket_k(const uint16_t *__restrict__ id
   bucket_block(ids, n_pairs, E, counts, offsets, pairs, work, n_active, s_ids4, s_cnt, s_act);
 }
 
-// top-k of up to blockDim/64 tokens (one wave each), then the bucketing, in one workgroup
+// top-k of the tokens (one wave each, in turns), then the bucketing, in one workgroup
 template <int EPL>
 __global__ void __launch_bounds__(1024) topk_bucket_k(const float *__restrict__ logits, const float *__restrict__ bias,
                                                       uint16_t *__restrict__ ids, float *__restrict__ weights, int tokens,
@@ -145,13 +52,8 @@ __global__ void __launch_bounds__(1024) topk_bucket_k(const float *__restrict__ 
   extern __shared__ uint4 s_ids4[];
   __shared__ int s_cnt[1024];
   __shared__ int s_act[1024];
-  const int wave = threadIdx.x >> 6;
-  if (wave < tokens)
-    topk_token<EPL>(logits + (size_t)wave * E, bias, ids + (size_t)wave * topk, weights + (size_t)wave * topk, E, topk,
-                    routed_scale, threadIdx.x & 63);
-  __threadfence_block();
-  __syncthreads();  // the ids written above are read back by bucket_block
-  bucket_block(ids, tokens * topk, E, counts, offsets, pairs, work, n_active, s_ids4, s_cnt, s_act);
+  kxr::route_block<EPL>(logits, bias, ids, weights, tokens, E, topk, routed_scale, counts, offsets, pairs, work, n_active,
+                        s_ids4, s_cnt, s_act);
 }
 
 }  // namespace
