@@ -114,13 +114,33 @@ __device__ __forceinline__ void gemv_body(const KxGemvArgs &a, const int bid, co
       for (int m = 0; m < MATS; ++m)
         buf[m][i] = ld_stream16(it.wb[m] + (size_t)((tile * RT + i) * a.cols) + it.col);
   };
+  // The work of a wave is one sequence of steps (chunk, slice, tile), tiles innermost, in which the
+  // loads of step i+1 (weights, and the raw activations when it starts a slice) are in flight while
+  // step i is computed; the first step's loads are requested before the prologue.
+  struct Pos { int chunk, s, tile; };
+  auto advance = [&](Pos p) {
+    if (++p.tile == a.nt) {
+      p.tile = 0;
+      p.s += a.nw;
+      if (p.s >= S) { p.s = wslot; p.chunk += nblocks; }
+    }
+    return p;
+  };
+  struct XRaw { uint4 x[TT]; uint4 g; };
+  const bool x_pref = x_once && !a.mla_po;  // activations of a slice are fetched one step ahead
+  auto load_xraw = [&](XRaw &r, const Item &it) {
+    const uint16_t *xb = a.x + (size_t)it.blk * a.x_block_stride;
+#pragma unroll
+    for (int t = 0; t < TT; ++t) r.x[t] = *(const uint4 *)(xb + (size_t)min(t, T - 1) * a.x_stride + it.col);
+    if (a.norm_w) r.g = *(const uint4 *)(a.norm_w + it.col);
+  };
   uint4 bufA[MATS][RI], bufB[MATS][RI];
-  // the first weight tile is requested before the prologue so that its latency overlaps it
-  bool preloaded = false;
-  if (a.norm_w && bid < n_chunks && wslot < S) {
-    load_tile(bufA, item(bid, wslot), 0);
-    preloaded = true;
-  }
+  XRaw xrA, xrB;
+  Pos cur = {bid, wslot, 0};
+  if (cur.chunk >= n_chunks) return;  // whole workgroups only: the host launches at most n_chunks of them
+  Item itc = item(cur.chunk, cur.s);
+  load_tile(bufA, itc, 0);
+  if (x_pref) load_xraw(xrA, itc);
 
   // Optional prologue: RMSNorm of the activation rows (rmsnorm_k's schedule: 256 threads own the
   // 8-element chunks t, t+256, ...; butterfly per wave; ((w0+w1)+w2)+w3).  Every workgroup
@@ -165,20 +185,16 @@ __device__ __forceinline__ void gemv_body(const KxGemvArgs &a, const int bid, co
       }
   }
 
-  for (int chunk = bid; chunk < n_chunks; chunk += nblocks) {
-    int c0 = chunk * CR;
-    c0 = c0 + CR <= a.rows ? c0 : a.rows - CR;
-    for (int s = wslot; s < S; s += a.nw) {
-      const Item it = item(chunk, s);
-      const uint32_t col = it.col;
-      const int blk = it.blk;
-      const uint16_t *xb = a.x + (size_t)blk * a.x_block_stride;
-      float xs[TT][8];
-      auto load_x = [&](int t0) {
+  float xs[TT][8];
+  // activations of tokens t0 .. t0+TT-1 for the slice of `it`, straight from memory
+  auto load_x = [&](const Item &it, int t0) {
+    const uint32_t col = it.col;
+    const int blk = it.blk;
+    const uint16_t *xb = a.x + (size_t)blk * a.x_block_stride;
 #pragma unroll
-        for (int t = 0; t < TT; ++t) {
-          const int tok = min(t0 + t, T - 1);
-          if (a.mla_po) {
+    for (int t = 0; t < TT; ++t) {
+      const int tok = min(t0 + t, T - 1);
+      if (a.mla_po) {
             // activations = merged attention partials of head `blk` (mla_combine's arithmetic):
             // M = max M_j; w_j = exp(M_j - M); Z = fma(Z_j, w_j, Z); O = fma(O_j, w_j, O); x = bf(O / Z).
             // Lane j holds span j's (M_j, Z_j, w_j); the O_j rows are fetched four spans at a time.
@@ -213,58 +229,64 @@ __device__ __forceinline__ void gemv_body(const KxGemvArgs &a, const int bid, co
             }
 #pragma unroll
             for (int e = 0; e < 8; ++e) xs[t][e] = kx_bfround(O[e] / Z);
-          } else {
-            unpack8(xs[t], *(const uint4 *)(xb + (size_t)tok * a.x_stride + col));
-            if (a.norm_w) {
-              float g[8];
-              unpack8(g, *(const uint4 *)(a.norm_w + col));
-              const float sc = n_scale[tok];
+      } else {
+        unpack8(xs[t], *(const uint4 *)(xb + (size_t)tok * a.x_stride + col));
+        if (a.norm_w) {
+          float g[8];
+          unpack8(g, *(const uint4 *)(a.norm_w + col));
+          const float sc = n_scale[tok];
 #pragma unroll
-              for (int e = 0; e < 8; ++e) xs[t][e] = kx_bfround(kx_bfround(xs[t][e] * sc) * g[e]);
-            }
-          }
+          for (int e = 0; e < 8; ++e) xs[t][e] = kx_bfround(kx_bfround(xs[t][e] * sc) * g[e]);
         }
-      };
-      auto compute_tile = [&](uint4 (&buf)[MATS][RI], int tile) {
-        for (int t0 = 0; t0 < T; t0 += TT) {
-          if (!x_once) load_x(t0);
-          float v[NV];
-#pragma unroll
-          for (int i = 0; i < RI; ++i)
-#pragma unroll
-            for (int m = 0; m < MATS; ++m) {
-              float wf[8];
-              unpack8(wf, buf[m][i]);
-#pragma unroll
-              for (int t = 0; t < TT; ++t) {
-                float acc = 0.0f;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) acc = __builtin_fmaf(wf[e], xs[t][e], acc);
-                v[(i * MATS + m) * TT + t] = acc;
-              }
-            }
-          kxw::reduce<NV, 64>(v, lane);
-          if (kxw::reduce_writer<NV, 64>(lane)) {
-#pragma unroll
-            for (int j = 0; j < NOUT; ++j) {
-              const int idx = kxw::reduce_index<NV, 64>(lane, j);  // (i*MATS + m)*TT + t
-              const int t = idx % TT, m = (idx / TT) % MATS, i = idx / (TT * MATS);
-              const int rc = tile * RT + rset * RI + i, tok = t0 + t;
-              if (tok < T) part[((m * CR + rc) * T + tok) * S + s] = v[j];
-            }
-          }
-        }
-      };
-      if (!preloaded) load_tile(bufA, it, 0);
-      preloaded = false;
-      if (x_once) load_x(0);
-      for (int tile = 0; tile < a.nt; tile += 2) {
-        if (tile + 1 < a.nt) load_tile(bufB, it, tile + 1);
-        compute_tile(bufA, tile);
-        if (tile + 2 < a.nt) load_tile(bufA, it, tile + 2);
-        if (tile + 1 < a.nt) compute_tile(bufB, tile + 1);
       }
     }
+  };
+  // the same from the prefetched raw values
+  auto form_x = [&](const XRaw &r) {
+    float g[8];
+    if (a.norm_w) unpack8(g, r.g);
+#pragma unroll
+    for (int t = 0; t < TT; ++t) {
+      unpack8(xs[t], r.x[t]);
+      if (a.norm_w) {
+        const float sc = n_scale[min(t, T - 1)];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) xs[t][e] = kx_bfround(kx_bfround(xs[t][e] * sc) * g[e]);
+      }
+    }
+  };
+  auto compute_tile = [&](uint4 (&buf)[MATS][RI], const Item &it, int s, int tile) {
+    for (int t0 = 0; t0 < T; t0 += TT) {
+      if (!x_once) load_x(it, t0);
+      float v[NV];
+#pragma unroll
+      for (int i = 0; i < RI; ++i)
+#pragma unroll
+        for (int m = 0; m < MATS; ++m) {
+          float wf[8];
+          unpack8(wf, buf[m][i]);
+#pragma unroll
+          for (int t = 0; t < TT; ++t) {
+            float acc = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc = __builtin_fmaf(wf[e], xs[t][e], acc);
+            v[(i * MATS + m) * TT + t] = acc;
+          }
+        }
+      kxw::reduce<NV, 64>(v, lane);
+      if (kxw::reduce_writer<NV, 64>(lane)) {
+#pragma unroll
+        for (int j = 0; j < NOUT; ++j) {
+          const int idx = kxw::reduce_index<NV, 64>(lane, j);  // (i*MATS + m)*TT + t
+          const int t = idx % TT, m = (idx / TT) % MATS, i = idx / (TT * MATS);
+          const int rc = tile * RT + rset * RI + i, tok = t0 + t;
+          if (tok < T) part[((m * CR + rc) * T + tok) * S + s] = v[j];
+        }
+      }
+    }
+  };
+  // end of a chunk: the slices of every (row, token) are summed left to right and the epilogue runs
+  auto chunk_end = [&](int chunk, int c0) {
     __syncthreads();
     for (int idx = threadIdx.x; idx < CR * T; idx += blockDim.x) {
       const int rc = idx % CR, tok = idx / CR;
@@ -315,6 +337,39 @@ __device__ __forceinline__ void gemv_body(const KxGemvArgs &a, const int bid, co
       }
     }
     __syncthreads();
+  };
+  auto step = [&](uint4 (&buf)[MATS][RI], const XRaw &xr, const Pos &p, const Item &it, bool last_of_chunk) {
+    if (x_once && p.tile == 0) {
+      if (x_pref) form_x(xr);
+      else load_x(it, 0);
+    }
+    compute_tile(buf, it, p.s, p.tile);
+    if (last_of_chunk) chunk_end(p.chunk, it.c0);
+  };
+  while (true) {
+    Pos nxt = advance(cur);
+    bool more = nxt.chunk < n_chunks;
+    Item itn = itc;
+    if (more) {
+      if (nxt.tile == 0) itn = item(nxt.chunk, nxt.s);
+      load_tile(bufB, itn, nxt.tile);
+      if (x_pref && nxt.tile == 0) load_xraw(xrB, itn);
+    }
+    step(bufA, xrA, cur, itc, nxt.chunk != cur.chunk);
+    if (!more) break;
+    cur = nxt;
+    itc = itn;
+    nxt = advance(cur);
+    more = nxt.chunk < n_chunks;
+    if (more) {
+      if (nxt.tile == 0) itn = item(nxt.chunk, nxt.s);
+      load_tile(bufA, itn, nxt.tile);
+      if (x_pref && nxt.tile == 0) load_xraw(xrA, itn);
+    }
+    step(bufB, xrB, cur, itc, nxt.chunk != cur.chunk);
+    if (!more) break;
+    cur = nxt;
+    itc = itn;
   }
 }
 
