@@ -36,6 +36,11 @@ def build_if_missing():
         __graft_entry__.build()
 
 
+# HBM bytes of one i4_gemv_k<dual> launch at T=1 (8 experts) from rocprofv3 counters: FETCH_SIZE 64,630 KiB x 2.0
+# (a 1 GiB kx_dev_copy reads 524,288 on that counter) + WRITE_SIZE 32 KiB x 1.0; see profiles/
+GATE_UP_TRAFFIC_T1 = 132395008
+
+
 def moe_layer_bytes(cfg, tokens, distinct):
     """Algorithmic HBM bytes of one MoE decode layer (unique bytes that must cross once)."""
     H, I, SI, E = cfg.hidden, cfg.moe_inter, cfg.shared_inter, cfg.experts
@@ -157,9 +162,26 @@ def run_moe_layer(args, emit=True):
     phases /= args.steps
     U = float(np.mean(distinct))
     by = moe_layer_bytes(cfg, T, U)
-    gate_up_gbs = U * by["gate_up"] / (phases[1] * 1e-3) / 1e9
-    down_gbs = U * by["down"] / (phases[2] * 1e-3) / 1e9
-    routed_gbs = by["routed"] / ((phases[1] + phases[2]) * 1e-3) / 1e9
+    # the two routed-expert kernels alone, launched back to back over the cycled layers (cold weights), on the
+    # routing of the last step: average launch duration = elapsed / launches, events on the launch stream
+    alone = []
+    for which in (0, 1):
+        for i in range(n_layers):
+            check(lib.kx_moe_routed_only(C.byref(cfg), C.byref(layers.layers[i]), ws, dn.ptr, T, which, None))
+        check(lib.kx_sync(None))
+        reps = max(args.steps, 20)
+        check(lib.kx_event_record(e0, None))
+        for i in range(reps):
+            check(lib.kx_moe_routed_only(C.byref(cfg), C.byref(layers.layers[i % n_layers]), ws, dn.ptr, T, which, None))
+        check(lib.kx_event_record(e1, None))
+        check(lib.kx_sync(None))
+        check(lib.kx_event_elapsed_ms(e0, e1, C.byref(ms)))
+        alone.append(ms.value / reps)
+    check(lib.kx_d2h(counts.ctypes.data, views[3].value, counts.nbytes))
+    U_last = int(np.count_nonzero(counts))
+    gate_up_gbs = U_last * by["gate_up"] / (alone[0] * 1e-3) / 1e9
+    down_gbs = U_last * by["down"] / (alone[1] * 1e-3) / 1e9
+    routed_gbs = U_last * (by["gate_up"] + by["down"]) / ((alone[0] + alone[1]) * 1e-3) / 1e9
     layer_gbs = by["layer"] / (ms_per_step * 1e-3) / 1e9
 
     # CPU baseline: the oracle's reference schedule on the same layer-0 weights, bounded sample
@@ -197,16 +219,19 @@ def run_moe_layer(args, emit=True):
                    "tokens": T, "distinct_experts_per_step": round(U, 2), "device": name.value.decode(),
                    "compute_units": cus.value},
         "roofline": {"bound": "hbm", "achieved": round(gate_up_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gate_up_gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(gate_up_gbs / HBM_PEAK_GBS, 4),
+                     "traffic": GATE_UP_TRAFFIC_T1 if (T == 1 and U_last == cfg.topk) else None,
                      "kernel": "i4_gemv_k<dual> (routed gate+up + SwiGLU)",
-                     "algorithmic_bytes_per_launch": int(U * by["gate_up"]),
-                     "avg_launch_ms": round(float(phases[1]), 5)},
+                     "algorithmic_bytes_per_launch": int(U_last * by["gate_up"]),
+                     "avg_launch_ms": round(alone[0], 5),
+                     "how": "launched back to back over the cycled layers, HIP events on the launch stream"},
         "int4_expert_gemv": {"routed_gbs": round(routed_gbs, 1), "routed_frac_of_peak": round(routed_gbs / HBM_PEAK_GBS, 4),
                              "gate_up_gbs": round(gate_up_gbs, 1), "down_gbs": round(down_gbs, 1),
-                             "layer_gbs": round(layer_gbs, 1)},
-        "phase_ms": {"router_bucket": round(float(phases[0]), 5), "routed_gate_up": round(float(phases[1]), 5),
-                     "routed_down": round(float(phases[2]), 5), "shared_gate_up": round(float(phases[3]), 5),
-                     "shared_down_combine": round(float(phases[4]), 5)},
+                             "gate_up_ms": round(alone[0], 5), "down_ms": round(alone[1], 5),
+                             "distinct_experts": U_last, "layer_gbs": round(layer_gbs, 1)},
+        "phase_ms": {"shared_gate_up_router_route": round(float(phases[0]), 5), "routed_gate_up": round(float(phases[1]), 5),
+                     "routed_down": round(float(phases[2]), 5), "shared_down_combine": round(float(phases[3] + phases[4]), 5),
+                     "note": "events around each launch inside the layer; they include the event commands themselves"},
         "wall_ms_per_step": round(wall_ms / args.steps, 5),
         "cpu_baseline": cpu,
     }
@@ -389,6 +414,52 @@ def run_prefill(args):
     return out
 
 
+def run_mla(args):
+    """BASELINE config 3: MLA decode attention on the latent cache, one query position per sequence."""
+    from blok_amd.lib import check, default_config, kx
+    lib = kx()
+    cfg = default_config()
+    B, L = args.batch, args.context
+    kva = cfg.kv_rank + cfg.qk_rope
+    cache_bytes = B * L * kva * 2
+    cache, qabs, wsp, o_lat = C.c_void_p(), C.c_void_p(), C.c_void_p(), C.c_void_p()
+    check(lib.kx_dev_malloc(C.byref(cache), cache_bytes))
+    check(lib.kx_fill_normal_bf16(cache, B * L * kva, args.seed, 40, 1.0, 0, None))
+    check(lib.kx_dev_malloc(C.byref(qabs), B * cfg.heads * kva * 4))
+    check(lib.kx_fill_normal_f32(qabs, B * cfg.heads * kva, args.seed, 41, 1.0, None))
+    ws_bytes = C.c_size_t()
+    check(lib.kx_mla_workspace_bytes(C.byref(cfg), B, L, C.byref(ws_bytes)))
+    check(lib.kx_dev_malloc(C.byref(wsp), ws_bytes.value))
+    check(lib.kx_dev_malloc(C.byref(o_lat), B * cfg.heads * cfg.kv_rank * 2))
+    e0, e1 = C.c_void_p(), C.c_void_p()
+    check(lib.kx_event_create(C.byref(e0)))
+    check(lib.kx_event_create(C.byref(e1)))
+    steps = args.steps if args.steps != 256 else 20
+    for _ in range(min(args.warmup, 3)):
+        check(lib.kx_mla_decode(C.byref(cfg), cache, L * kva, qabs, wsp, o_lat, B, L, None))
+    check(lib.kx_sync(None))
+    check(lib.kx_event_record(e0, None))
+    for _ in range(steps):
+        check(lib.kx_mla_decode(C.byref(cfg), cache, L * kva, qabs, wsp, o_lat, B, L, None))
+    check(lib.kx_event_record(e1, None))
+    check(lib.kx_sync(None))
+    ms = C.c_float()
+    check(lib.kx_event_elapsed_ms(e0, e1, C.byref(ms)))
+    per = ms.value / steps
+    flops = 2.0 * B * L * cfg.heads * (kva + cfg.kv_rank)
+    gbs = cache_bytes / (per * 1e-3) / 1e9
+    print(json.dumps({"metric": "MLA decode attention, latent-cache GB/s (BASELINE config 3)", "value": round(gbs, 1),
+                      "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": min(args.warmup, 3), "ms_per_step": round(per, 4),
+                      "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16 cache, f32 accumulate",
+                      "data": "synthetic",
+                      "config": {"workload": f"kx_mla_decode, B={B}, L={L}, 64 heads, latent 512+64", "batch": B, "context": L},
+                      "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                   "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                                   "algorithmic_bytes_per_launch": cache_bytes},
+                      "valu": {"tflops": round(flops / (per * 1e-3) / 1e12, 2), "peak_fp32_tflops": 157.3,
+                               "frac": round(flops / (per * 1e-3) / 1e12 / 157.3, 4)}}), flush=True)
+
+
 def run_copy(args):
     """Plain copy of a known size: the kernel whose FETCH_SIZE / WRITE_SIZE readings calibrate the traffic figures."""
     from blok_amd.lib import check, kx
@@ -424,7 +495,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--workload", default="stack", choices=["stack", "moe_layer", "prefill", "copy"])
+    ap.add_argument("--workload", default="stack", choices=["stack", "moe_layer", "prefill", "mla", "copy"])
+    ap.add_argument("--context", type=int, default=32768)
     ap.add_argument("--copy-mib", type=int, default=1024)
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--prompt", type=int, default=1024)
@@ -443,6 +515,9 @@ def main():
     build_if_missing()
     if args.workload == "copy":
         run_copy(args)
+        return
+    if args.workload == "mla":
+        run_mla(args)
         return
     if args.workload == "prefill":
         if args.tokens == 1:

@@ -127,7 +127,8 @@ __device__ __forceinline__ void gemv_body(const KxGemvArgs &a, const int bid, co
     return p;
   };
   struct XRaw { uint4 x[TT]; uint4 g; };
-  const bool x_pref = x_once && !a.mla_po;  // activations of a slice are fetched one step ahead
+  // activations of a slice are fetched one step ahead (not in the variant whose registers are full)
+  const bool x_pref = x_once && !a.mla_po && !(MATS == 2 && RI == 2);
   auto load_xraw = [&](XRaw &r, const Item &it) {
     const uint16_t *xb = a.x + (size_t)it.blk * a.x_block_stride;
 #pragma unroll

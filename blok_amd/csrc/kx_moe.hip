@@ -190,6 +190,28 @@ extern "C" int kx_moe_decode_layer_timed(const kx_config *cfg, const kx_moe_weig
   return KX_OK;
 }
 
+// One routed-expert kernel alone, on the routing the most recent decode-layer call left in the workspace
+// (for timing the kernel back to back): which = 0 gate/up + SwiGLU (d_n -> mid), 1 down (mid -> expert outputs).
+extern "C" int kx_moe_routed_only(const kx_config *c, const kx_moe_weights *w, kx_moe_workspace *ws, const void *d_n,
+                                  int32_t tokens, int32_t which, void *stream) {
+  int rc = check_cfg(c);
+  if (rc) return rc;
+  KX_REQUIRE(w && ws && d_n, "kx_moe_routed_only: null argument");
+  KX_REQUIRE(tokens > 0 && tokens <= ws->max_tokens, "kx_moe_routed_only: tokens=%d outside [1, %d]", tokens, ws->max_tokens);
+  KX_REQUIRE(which == 0 || which == 1, "kx_moe_routed_only: which=%d", which);
+  const int H = c->hidden, I = c->moe_inter, E = c->experts, K = c->topk;
+  const int tt = routed_tt(tokens, K, E);
+  const int max_active = (long)tokens * K < E ? tokens * K : E;
+  if (which == 0)
+    return kx_i4_launch(true, (const uint32_t *)w->d_gate_packed, (const uint16_t *)w->d_gate_scale,
+                        (const uint32_t *)w->d_up_packed, (const uint16_t *)w->d_up_scale, (const uint16_t *)d_n, ws->mid,
+                        ws->work, ws->pairs, 0, I, H, K, (size_t)I * (H / 8), (size_t)I * (H / 32), tt, max_active,
+                        kx_stream(stream));
+  return kx_i4_launch(false, (const uint32_t *)w->d_down_packed, (const uint16_t *)w->d_down_scale, nullptr, nullptr,
+                      ws->mid, ws->eout, ws->work, ws->pairs, 0, H, I, 1, (size_t)H * (I / 8), (size_t)H * (I / 32), tt,
+                      max_active, kx_stream(stream));
+}
+
 // ---- prefill chunk through one MoE layer: grouped GEMMs on the matrix cores ------------------
 extern "C" int kx_moe_prefill_layer(const kx_config *c, const kx_moe_weights *w, kx_moe_workspace *ws, const void *d_n,
                                     void *d_x, int32_t tokens, uint32_t flags, void *stream) {

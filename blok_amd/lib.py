@@ -89,6 +89,7 @@ _SIGS = {
     "kx_moe_prefill_layer": [C.POINTER(KxConfig), C.POINTER(KxMoeWeights), _P, _P, _P, _I, C.c_uint32, _P],
     "kx_moe_decode_layer_timed": [C.POINTER(KxConfig), C.POINTER(KxMoeWeights), _P, _P, _P, _I,
                                   C.c_uint32, _P, C.POINTER(C.c_float)],
+    "kx_moe_routed_only": [C.POINTER(KxConfig), C.POINTER(KxMoeWeights), _P, _P, _I, _I, _P],
 }
 
 _lib = None

@@ -175,6 +175,11 @@ int kx_moe_prefill_layer(const kx_config *cfg, const kx_moe_weights *w, kx_moe_w
 int kx_moe_decode_layer_timed(const kx_config *cfg, const kx_moe_weights *w, kx_moe_workspace *ws,
                               const void *d_n, void *d_x, int32_t tokens, uint32_t flags,
                               void *stream, float *ms5);
+/* One routed-expert kernel alone, on the routing that the most recent kx_moe_decode_layer call left in
+ * the workspace: which = 0 gate/up + SwiGLU (:845-861), 1 down (:863-866).  For timing a kernel back
+ * to back; it has no counterpart of its own in the reference.                                    */
+int kx_moe_routed_only(const kx_config *cfg, const kx_moe_weights *w, kx_moe_workspace *ws,
+                       const void *d_n, int32_t tokens, int32_t which, void *stream);
 
 /* ---- MLA decode attention (tiled_attention, :692-716, on the absorbed latent cache) ----
  * kx_rope_table   : rope_k's cos/sin (:351) with the YaRN frequencies (:325-344) for positions
