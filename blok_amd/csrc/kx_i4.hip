@@ -152,11 +152,14 @@ constexpr int I4_RI = 2;  // rows per half-wave per tile
 
 // A workgroup of ks*rs waves takes chunks of nt tiles of RT = rs*4 rows of one expert.
 // Wave (s, rset): slice s of rows rset*4 .. rset*4+3 of each tile; its half-waves take
-// alternate rows.  Per chunk: the group scales of all its rows are staged in LDS once,
-// the packed words stream through two register buffers (tile i+1 is in flight while
-// tile i is computed), partial sums go to LDS and are summed over the slices at the end
-// of the chunk.  A last chunk that would run past the matrix is moved back to end at
-// the last row (the overlap is computed twice, with identical results).
+// alternate rows.  Per chunk: the group scales of all its rows are copied into LDS (global ->
+// LDS loads, no registers), the packed words stream through two register buffers (tile i+1
+// is in flight while tile i is computed), partial sums go to LDS and are summed over the
+// slices at the end of the chunk.  While a chunk is computed the next one is prepared: its
+// work record is read and its scales are copied into the second scale buffer at the start;
+// the first tile and activations of whatever comes next (a further pass, the next chunk) are requested before the epilogue.  A last chunk that would
+// run past the matrix is moved back to end at the last row (the overlap is computed twice,
+// with identical results, and written once).
 // KS_T > 0 fixes ks (and rs, nt) at compile time; 0 reads them from the arguments.
 template <bool DUAL, int TT, int KS_T, int MAXT, int WPE>
 __global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) i4_gemv_k(I4Args a) {
@@ -165,7 +168,6 @@ __global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(WPE, 
   constexpr int RI = I4_RI;
   constexpr int NV = RI * MATS * TT;
   constexpr int NOUT = kxw::reduce_out<NV, 32>();
-  constexpr int SC_ITERS = 4;  // scale staging: 16-byte pieces per thread and matrix
   const int ks = KS_T ? KS_T : a.ks;
   const int rs = KS_T ? (KS_T >= 5 ? 1 : 8 / KS_T) : a.rs;
   const int RT = rs * 2 * RI;
@@ -175,73 +177,96 @@ __global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(WPE, 
   const int l = lane & 31, h = lane >> 5;
   const int s = wave % ks, rset = wave / ks;
   const int groups = ks * 32, row_words = ks * 128;
+  const int n16 = CR * groups / 8;                                // 16-byte pieces of one matrix's chunk scales
+  const int sc_pieces = (MATS * n16 + 63) & ~63;                  // per buffer, whole 1 KB runs
   float *part = lds;                                              // [mats][CR][TT][ks]
-  uint16_t *sc_lds = (uint16_t *)(lds + MATS * CR * TT * ks);     // [mats][CR][groups]
+  uint4 *sc_base = (uint4 *)(lds + ((MATS * CR * TT * ks + 3) & ~3));  // 2 x [mats][CR][groups] bf16
   const int cpe = (a.rows + CR - 1) / CR;                         // chunks per expert
   const int n_chunks = (a.work ? a.n_slots : 1) * cpe;
   const int row_lane = rset * RI * 2 + h;                         // row of this lane in tile 0, i = 0
   const uint32_t w_off = (uint32_t)row_lane * (uint32_t)row_words + (uint32_t)(s * 32 + l) * 4;
-  const uint16_t *sc_lane = sc_lds + row_lane * groups + s * 32 + l;
+  const int sc_off = row_lane * groups + s * 32 + l;
   uint32_t magic;
   asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(magic));
 
-  for (int chunk = blockIdx.x; chunk < n_chunks; chunk += gridDim.x) {
+  struct Work { int e, p_begin, p_end, first_pair, c0, c_first; };
+  auto load_work = [&](int chunk) {
+    Work w;
     const int ai = chunk / cpe;
-    int c0 = (chunk - ai * cpe) * CR;
-    c0 = c0 + CR <= a.rows ? c0 : a.rows - CR;  // host guarantees rows >= CR
-    int4 wk = a.work ? a.work[ai] : make_int4(0, 0, a.n_pairs, 0);
-    const int e = __builtin_amdgcn_readfirstlane(wk.x);
-    if (e < 0) break;  // records with work come first
-    const int p_begin = __builtin_amdgcn_readfirstlane(wk.y), p_end = __builtin_amdgcn_readfirstlane(wk.z);
-    const int first_pair = __builtin_amdgcn_readfirstlane(wk.w);
-    const uint32_t *pk[2] = {a.packed0 + (size_t)e * a.expert_words + (size_t)c0 * row_words,
-                             DUAL ? a.packed1 + (size_t)e * a.expert_words + (size_t)c0 * row_words : nullptr};
-
-    auto load_tile = [&](uint4 (&buf)[MATS][RI], int tile) {
+    const int4 wk = a.work ? a.work[ai] : make_int4(0, 0, a.n_pairs, 0);
+    w.e = __builtin_amdgcn_readfirstlane(wk.x);
+    w.p_begin = __builtin_amdgcn_readfirstlane(wk.y);
+    w.p_end = __builtin_amdgcn_readfirstlane(wk.z);
+    w.first_pair = __builtin_amdgcn_readfirstlane(wk.w);
+    w.c_first = (chunk - ai * cpe) * CR;
+    w.c0 = w.c_first + CR <= a.rows ? w.c_first : a.rows - CR;  // host guarantees rows >= CR
+    return w;
+  };
+  // group scales of a chunk: CR*groups contiguous bf16 per matrix, copied piece i -> piece i of the buffer
+  auto copy_scales = [&](const Work &w, uint4 *dst) {
+    const int nwaves = blockDim.x >> 6;
+    for (int m = 0; m < MATS; ++m) {
+      const uint4 *sg = (const uint4 *)((m ? a.scale1 : a.scale0) + (size_t)w.e * a.expert_scales + (size_t)w.c0 * groups);
+      for (int i0 = wave * 64; i0 < n16; i0 += nwaves * 64)
+        if (i0 + lane < n16)
+          __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)(sg + i0 + lane),
+                                           (void __attribute__((address_space(3))) *)(dst + m * n16 + i0), 16, 0, 0);
+    }
+  };
+  auto tile_ptr = [&](const Work &w, int m) {
+    return (m ? a.packed1 : a.packed0) + (size_t)w.e * a.expert_words + (size_t)w.c0 * row_words;
+  };
+  auto load_tile = [&](uint4 (&buf)[MATS][RI], const Work &w, int tile) {
 #pragma unroll
-      for (int i = 0; i < RI; ++i)
+    for (int i = 0; i < RI; ++i)
 #pragma unroll
-        for (int m = 0; m < MATS; ++m)
-          buf[m][i] = ld_stream(pk[m] + (size_t)((tile * RT + i * 2) * row_words) + w_off);
-    };
+      for (int m = 0; m < MATS; ++m)
+        buf[m][i] = ld_stream(tile_ptr(w, m) + (size_t)((tile * RT + i * 2) * row_words) + w_off);
+  };
+  auto load_xraw = [&](uint4 (&xraw)[TT][4], const Work &w, int pc) {
+#pragma unroll
+    for (int t = 0; t < TT; ++t) {
+      const int pi = min(pc + t, w.p_end - 1);
+      const int pair = !a.work ? pi : (pi == w.p_begin ? w.first_pair : a.pairs[pi]);
+      const uint4 *xp = (const uint4 *)(a.x + (size_t)(pair / a.x_div) * a.cols) + (s * 32 + l) * 4;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) xraw[t][q] = xp[q];
+    }
+  };
 
-    for (int pc = p_begin; pc < p_end; pc += TT) {
-      uint4 bufA[MATS][RI], bufB[MATS][RI];
-      load_tile(bufA, 0);
+  int chunk = blockIdx.x;
+  if (chunk >= n_chunks) return;
+  Work cur = load_work(chunk);
+  if (cur.e < 0) return;  // records with work come first
+  uint4 bufA[MATS][RI], bufB[MATS][RI];
+  uint4 xraw[TT][4];
+  int sb = 0;
+  copy_scales(cur, sc_base);
+  load_tile(bufA, cur, 0);
+  load_xraw(xraw, cur, cur.p_begin);
+  bool fresh = true;  // the scales of `cur` have not been made visible to the workgroup yet
+
+  while (true) {
+    const int nchunk = chunk + gridDim.x;
+    bool more = nchunk < n_chunks;
+    Work nxt = cur;
+    if (more) {
+      nxt = load_work(nchunk);
+      more = nxt.e >= 0;
+    }
+    // the other scale buffer was last read in the chunk before this one; every wave is past that chunk's barriers
+    if (more) copy_scales(nxt, sc_base + (sb ^ 1) * sc_pieces);
+    const uint16_t *sc_lane = (const uint16_t *)(sc_base + sb * sc_pieces) + sc_off;
+
+    for (int pc = cur.p_begin; pc < cur.p_end; pc += TT) {
       XGroup xg[TT];
-      uint4 xraw[TT][4];
-#pragma unroll
-      for (int t = 0; t < TT; ++t) {
-        const int pi = min(pc + t, p_end - 1);
-        const int pair = !a.work ? pi : (pi == p_begin ? first_pair : a.pairs[pi]);
-        const uint4 *xp = (const uint4 *)(a.x + (size_t)(pair / a.x_div) * a.cols) + (s * 32 + l) * 4;
-#pragma unroll
-        for (int w = 0; w < 4; ++w) xraw[t][w] = xp[w];
-      }
-      if (pc == p_begin) {
-        // group scales of the chunk: CR*groups contiguous bf16 per matrix; every load is
-        // issued before the first LDS write
-        const int n16 = CR * groups / 8;
-        uint4 stg[MATS][SC_ITERS];
-#pragma unroll
-        for (int m = 0; m < MATS; ++m) {
-          const uint4 *sg = (const uint4 *)((m ? a.scale1 : a.scale0) + (size_t)e * a.expert_scales + (size_t)c0 * groups);
-#pragma unroll
-          for (int it = 0; it < SC_ITERS; ++it) stg[m][it] = sg[min((int)(threadIdx.x + it * blockDim.x), n16 - 1)];
-        }
-#pragma unroll
-        for (int m = 0; m < MATS; ++m) {
-          uint4 *dst = (uint4 *)(sc_lds + (size_t)m * CR * groups);
-#pragma unroll
-          for (int it = 0; it < SC_ITERS; ++it) {
-            const int i = threadIdx.x + it * blockDim.x;
-            if (i < n16) dst[i] = stg[m][it];
-          }
-        }
-      }
 #pragma unroll
       for (int t = 0; t < TT; ++t) prep_xgroup(xg[t], xraw[t]);
-      __syncthreads();  // scales visible; previous pass has consumed `part`
+      if (fresh) {  // first chunk of the workgroup: wait for the scale copies of every wave
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        fresh = false;
+      }
 
       auto compute_tile = [&](uint4 (&buf)[MATS][RI], int tile) {
         float v[NV];
@@ -268,16 +293,30 @@ __global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(WPE, 
       };
 
       for (int tile = 0; tile < nt; tile += 2) {
-        if (tile + 1 < nt) load_tile(bufB, tile + 1);
+        if (tile + 1 < nt) load_tile(bufB, cur, tile + 1);
         compute_tile(bufA, tile);
-        if (tile + 2 < nt) load_tile(bufA, tile + 2);
+        if (tile + 2 < nt) load_tile(bufA, cur, tile + 2);
         if (tile + 1 < nt) compute_tile(bufB, tile + 1);
+      }
+      // every load of this wave has landed, the scale copies for the next chunk included; its first tile
+      // and activations are requested now and arrive during the epilogue
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      const bool last_pass = pc + TT >= cur.p_end;
+      if (!last_pass || more) {  // a further pass over this chunk (an expert with more than TT pairs), or the next chunk
+        const Work &t = last_pass ? nxt : cur;
+        load_tile(bufA, t, 0);
+        load_xraw(xraw, t, last_pass ? nxt.p_begin : pc + TT);
+      } else {  // nothing follows: end the registers' live ranges here
+#pragma unroll
+        for (int t = 0; t < TT; ++t)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) xraw[t][q] = make_uint4(0, 0, 0, 0);
       }
       __syncthreads();
       // sequential sum over the slices, rounding and epilogue
       for (int idx = threadIdx.x; idx < CR * TT; idx += blockDim.x) {
         const int rc = idx % CR, t = idx / CR;
-        if (pc + t < p_end && c0 + rc >= (chunk - ai * cpe) * CR) {  // a moved-back chunk skips the rows it shares
+        if (pc + t < cur.p_end && cur.c0 + rc >= cur.c_first) {  // a moved-back chunk skips the rows it shares
           const int pair = !a.work ? pc + t : a.pairs[pc + t];
           const float *p0 = part + ((0 * CR + rc) * TT + t) * ks;
           float y0 = p0[0];
@@ -289,11 +328,15 @@ __global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(WPE, 
             for (int q = 1; q < ks; ++q) y1 += p1[q];
             res = kx_swiglu(kx_bfround(y0), kx_bfround(y1));
           }
-          a.out[(size_t)pair * a.rows + c0 + rc] = kx_bf16_rne(res);
+          a.out[(size_t)pair * a.rows + cur.c0 + rc] = kx_bf16_rne(res);
         }
       }
+      __syncthreads();  // `part` is free again; the next chunk's scale copies are visible to every wave
     }
-    __syncthreads();  // the next chunk overwrites the staged scales
+    if (!more) break;
+    cur = nxt;
+    chunk = nchunk;
+    sb ^= 1;
   }
 }
 
@@ -317,10 +360,9 @@ int plan(int cols, int rows, int mats, int tt, I4Launch &pl) {
   while (nt > 1 && rt * nt > rows) --nt;
   pl.nt = nt;
   pl.cr = rt * nt;
-  pl.lds = (size_t)mats * pl.cr * tt * pl.ks * sizeof(float) + (size_t)mats * pl.cr * (cols / 32) * 2;
+  const size_t sc_pieces = ((size_t)mats * pl.cr * (cols / 32) / 8 + 63) & ~(size_t)63;  // 16-byte pieces per scale buffer
+  pl.lds = (((size_t)mats * pl.cr * tt * pl.ks + 3) & ~(size_t)3) * sizeof(float) + 2 * sc_pieces * 16;
   KX_REQUIRE(pl.lds <= 160 * 1024, "kx_i4: cols=%d needs %zu bytes of LDS", cols, pl.lds);
-  // scale staging moves cr*groups/8 16-byte pieces per matrix with at most 4 per thread
-  KX_REQUIRE(pl.cr * (cols / 32) / 8 <= 4 * pl.threads, "kx_i4: chunk of %d rows x %d columns exceeds the scale staging", pl.cr, cols);
   return KX_OK;
 }
 
