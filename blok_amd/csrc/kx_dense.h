@@ -70,8 +70,9 @@ int kx_bucket_launch(const uint16_t *ids, int tokens, int experts, int topk, int
 
 // kx_prefill.hip
 int kx_grouped_gemm_launch(bool dual, bool i4, const void *w0, const uint16_t *s0, const void *w1, const uint16_t *s1,
-                           const uint16_t *x, uint16_t *out, const int4 *work, const int *pairs, int n_pairs, int n_slots,
-                           int N, int K, int x_div, size_t expert_w, size_t expert_s, int n_pairs_max, hipStream_t st);
+                           const uint16_t *x, void *out, bool out_f32, const int4 *work, const int *pairs, int n_pairs,
+                           int n_slots, int N, int K, int x_div, size_t expert_w, size_t expert_s, int n_pairs_max,
+                           hipStream_t st);
 int kx_moe_combine_launch(const uint16_t *eout, const float *rw, const uint16_t *sy, uint16_t *x, int tokens, int hidden,
                           int topk, uint32_t flags, hipStream_t st);
 

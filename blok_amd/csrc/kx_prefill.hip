@@ -7,13 +7,25 @@
 // combine (:868,:871), the shared expert (:872-875) and the residual add (:877) --
 // with the tokens of each expert gathered into one GEMM.
 //
-// The only place MFMA is used.  Per workgroup: one expert, 128 weight rows, the
-// expert's tokens in tiles of 64.  Per K step of 64 columns the packed INT4 words
-// are unpacked and dequantized exactly as the reference does, w = bf((n-8)*scale)
-// (:311-312), into an LDS tile of bf16; the gathered activation rows go into a
-// second LDS tile; four waves each run v_mfma_f32_32x32x16_bf16 on a 64x32 slab of
-// the output with fp32 accumulators.  The bf16 shared expert uses the same kernel
-// with a plain copy in place of the dequant.
+// The only place MFMA is used.  Per workgroup (4 waves): one expert, 128 weight rows, the
+// expert's tokens in tiles of 128.  Wave w owns weight rows 32 w .. +31 for all 128 tokens
+// (fp32 accumulators of v_mfma_f32_32x32x16_bf16).  Per K step of 64 columns:
+//  * weights never touch LDS: lane (r, h) = (lane % 32, lane / 32) loads the 16 bytes of row r
+//    that hold columns 32 h .. +31 of the step -- one quantization group, four packed words --
+//    and dequantizes word j to the reference's values, w = bf((n-8)*scale) (:311-312), which
+//    is exactly the B operand of the step's j-th MFMA when that MFMA contracts over columns
+//    {8 j .. +7} and {32 + 8 j .. +7} (the contraction order within a step is free, the
+//    activation operand uses the same columns);
+//  * the gathered activation rows go through a double-buffered LDS tile, one barrier per step;
+//  * the global loads of step k+1 are in flight while step k is computed.
+// The bf16 shared expert and the router gate use the same kernel with plain loads in place
+// of the dequant.
+//
+// Dequant without integer conversion: (w & 0x000F000F) | 0x64006400 is the f16 pair
+// (1024+n0, 1024+n4), (w & 0x00F000F0) | 0x64006400 is (1024+16 n1, 1024+16 n5), w >> 8 gives
+// n2,n6,n3,n7 the same way; fma(f16, s, -1032 s) = (n-8) s and fma(f16, s/16, -72 s) = (n-8) s
+// are exact in fp32 (4-bit times 8-bit significands), and one v_cvt_pk_bf16_f32 rounds two of
+// them to nearest-even.
 //
 // MFMA's internal summation order is not documented, so this path is held to the
 // max-rel 1e-2 bar and is never used for the token-identity runs.
@@ -24,125 +36,192 @@
 namespace {
 
 typedef __bf16 kx_bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 kx_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float kx_f32x2 __attribute__((ext_vector_type(2)));
 typedef float kx_f32x16 __attribute__((ext_vector_type(16)));
+typedef _Float16 kx_h2 __attribute__((ext_vector_type(2)));
 
-constexpr int BM = 64, BN = 128, BK = 64;
+constexpr int BM = 128, BN = 128, BK = 64;
 constexpr int LDS_STRIDE = BK + 8;  // bf16 elements per LDS row: 144 B keeps 16-byte reads of a column of rows spread over banks
+constexpr int PF_THREADS = 256;
 
 struct PfArgs {
   const void *w0, *w1;          // INT4: packed i32 [E][N][K/8]; BF16: bf16 [E][N][K]
   const uint16_t *s0, *s1;      // INT4: bf16 scales [E][N][K/32]
   const uint16_t *x;            // bf16 activation rows of K
-  uint16_t *out;                // bf16 [pairs][N]
+  void *out;                    // bf16 [pairs][N], or f32 when out_f32
   const int4 *work;             // {expert, first, last, _} per expert with work; nullptr: one group of n_pairs rows
   const int *pairs;             // pair ids sorted by expert; nullptr: identity
   int n_pairs, N, K, x_div;     // activation row = pair / x_div
   size_t expert_w, expert_s;    // elements between experts (words or bf16; scales)
+  int out_f32;                  // single matrix only: store the fp32 accumulators unrounded
 };
 
-__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-  return (uint32_t)kx_bf16_rne(lo) | ((uint32_t)kx_bf16_rne(hi) << 16);
+__device__ __forceinline__ uint32_t pf_and_or(uint32_t a, uint32_t mask, uint32_t magic) {
+  uint32_t r;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "s"(mask), "v"(magic));
+  return r;
+}
+__device__ __forceinline__ uint32_t pf_pack(float lo, float hi) {
+  kx_f32x2 v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, kx_bf16x2));
 }
 
-// dequantize one group (4 packed words, 32 weights) to 32 bf16 = 4 uint4, columns ascending
-__device__ __forceinline__ void dequant_group(const uint4 v, float sc, uint4 (&o)[4]) {
-  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-  const float m8 = -8.0f * sc;  // exact
-#pragma unroll
-  for (int p = 0; p < 4; ++p) {
-    float f[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) f[j] = __builtin_fmaf((float)((w[p] >> (4 * j)) & 0xfu), sc, m8);  // == (n-8)*sc exactly
-    o[p] = make_uint4(pack_bf16(f[0], f[1]), pack_bf16(f[2], f[3]), pack_bf16(f[4], f[5]), pack_bf16(f[6], f[7]));
-  }
+// dequantize one packed word (8 weights) to 8 bf16, columns ascending
+__device__ __forceinline__ kx_bf16x8 dequant_word(uint32_t w, float sc, float sc16, float c0, float c1, uint32_t magic) {
+  const uint32_t w8 = w >> 8;
+  const kx_h2 a = __builtin_bit_cast(kx_h2, pf_and_or(w, 0x000F000Fu, magic));   // n0, n4
+  const kx_h2 b = __builtin_bit_cast(kx_h2, pf_and_or(w, 0x00F000F0u, magic));   // 16 n1, 16 n5
+  const kx_h2 c = __builtin_bit_cast(kx_h2, pf_and_or(w8, 0x000F000Fu, magic));  // n2, n6
+  const kx_h2 d = __builtin_bit_cast(kx_h2, pf_and_or(w8, 0x00F000F0u, magic));  // 16 n3, 16 n7
+  const float f0 = __builtin_fmaf((float)a.x, sc, c0), f4 = __builtin_fmaf((float)a.y, sc, c0);
+  const float f1 = __builtin_fmaf((float)b.x, sc16, c1), f5 = __builtin_fmaf((float)b.y, sc16, c1);
+  const float f2 = __builtin_fmaf((float)c.x, sc, c0), f6 = __builtin_fmaf((float)c.y, sc, c0);
+  const float f3 = __builtin_fmaf((float)d.x, sc16, c1), f7 = __builtin_fmaf((float)d.y, sc16, c1);
+  return __builtin_bit_cast(kx_bf16x8, make_uint4(pf_pack(f0, f1), pf_pack(f2, f3), pf_pack(f4, f5), pf_pack(f6, f7)));
 }
 
 template <bool DUAL, bool I4>
-__global__ void __launch_bounds__(256) grouped_gemm_k(PfArgs a) {
+__global__ void __launch_bounds__(PF_THREADS, 2) grouped_gemm_k(PfArgs a) {
   constexpr int MATS = DUAL ? 2 : 1;
-  __shared__ __attribute__((aligned(16))) uint16_t xs[BM * LDS_STRIDE];
-  __shared__ __attribute__((aligned(16))) uint16_t ws[MATS][BN * LDS_STRIDE];
+  constexpr int XT = BM * LDS_STRIDE;  // elements of one activation tile
+  __shared__ __attribute__((aligned(16))) uint16_t xs_lds[2 * XT];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lr = lane & 31, lh = lane >> 5;
   const int n0 = blockIdx.x * BN;
   int4 wk = a.work ? a.work[blockIdx.y] : make_int4(0, 0, a.n_pairs, 0);
   const int e = __builtin_amdgcn_readfirstlane(wk.x);
   if (e < 0) return;
   const int p_begin = __builtin_amdgcn_readfirstlane(wk.y), p_end = __builtin_amdgcn_readfirstlane(wk.z);
-  const void *wbase[2] = {a.w0, a.w1};
-  const uint16_t *sbase[2] = {a.s0, a.s1};
-  // staging roles
-  const int xr = tid >> 2, xc = (tid & 3) * 16;   // activation tile: row, first of 16 columns
-  const int wr = tid >> 1, wg = tid & 1;          // weight tile: row, group (32 columns) of the K step
+  uint32_t magic;
+  asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(magic));
+  const int nk = a.K / BK;
+  // this lane's weight row and its 32-column half of every K step
+  const int wrow = min(n0 + wave * 32 + lr, a.N - 1);
+  const uint32_t *wq_ptr[MATS];
+  const uint16_t *wb_ptr[MATS], *sc_ptr[MATS];
+#pragma unroll
+  for (int m = 0; m < MATS; ++m) {
+    const void *wbase = m ? a.w1 : a.w0;
+    wq_ptr[m] = (const uint32_t *)wbase + (size_t)e * a.expert_w + (size_t)wrow * (a.K >> 3) + lh * 4;
+    wb_ptr[m] = (const uint16_t *)wbase + (size_t)e * a.expert_w + (size_t)wrow * a.K + lh * 32;
+    sc_ptr[m] = (m ? a.s1 : a.s0) + (I4 ? (size_t)e * a.expert_s + (size_t)wrow * (a.K >> 5) + lh : 0);
+  }
+  // activation staging: thread -> rows tid/4 and 64 + tid/4, 16 columns from (tid%4)*16
+  const int xr = tid >> 2, xc = (tid & 3) * 16;
 
-  // token tiles of the expert are spread over blockIdx.z
   for (int m0 = p_begin + blockIdx.z * BM; m0 < p_end; m0 += gridDim.z * BM) {
-    kx_f32x16 acc[MATS][2];
+    const int nb = min(4, (p_end - m0 + 31) >> 5);  // 32-token blocks that hold tokens
+    kx_f32x16 acc[MATS][4];
 #pragma unroll
     for (int m = 0; m < MATS; ++m)
 #pragma unroll
-      for (int t = 0; t < 2; ++t)
+      for (int t = 0; t < 4; ++t)
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[m][t][i] = 0.0f;
-    const int pi = m0 + xr;
-    const bool x_valid = pi < p_end;
-    const int pair = x_valid ? (a.pairs ? a.pairs[pi] : pi) : 0;
-    const uint16_t *xrow = a.x + (size_t)(pair / a.x_div) * a.K + xc;
-    const int wrow = min(n0 + wr, a.N - 1);
-    for (int k0 = 0; k0 < a.K; k0 += BK) {
-      // global loads of this K step
-      uint4 xv0 = make_uint4(0, 0, 0, 0), xv1 = xv0;
-      if (x_valid) { xv0 = *(const uint4 *)(xrow + k0); xv1 = *(const uint4 *)(xrow + k0 + 8); }
-      uint4 wq[MATS][4];
+    const uint16_t *xrow[2];
+    bool x_valid[2];
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      const int pi = m0 + q * 64 + xr;
+      x_valid[q] = pi < p_end;
+      const int pair = x_valid[q] ? (a.pairs ? a.pairs[pi] : pi) : 0;
+      xrow[q] = a.x + (size_t)(pair / a.x_div) * a.K + xc;
+    }
+
+    uint4 xv[2][2];
+    uint4 wq[MATS];      // INT4: the group's four packed words
+    float wsc[MATS];
+    uint4 wb[MATS][4];   // BF16: 32 columns
+    auto load_global = [&](int ks) {
+      const int k0 = ks * BK;
+#pragma unroll
+      for (int q = 0; q < 2; ++q) {
+        xv[q][0] = xv[q][1] = make_uint4(0, 0, 0, 0);
+        if (x_valid[q]) { xv[q][0] = *(const uint4 *)(xrow[q] + k0); xv[q][1] = *(const uint4 *)(xrow[q] + k0 + 8); }
+      }
 #pragma unroll
       for (int m = 0; m < MATS; ++m) {
         if (I4) {
-          const uint32_t *pw = (const uint32_t *)wbase[m] + (size_t)e * a.expert_w + (size_t)wrow * (a.K >> 3) + ((k0 >> 3) + wg * 4);
-          const float sc = kx_bf16_f32(sbase[m][(size_t)e * a.expert_s + (size_t)wrow * (a.K >> 5) + (k0 >> 5) + wg]);
-          dequant_group(*(const uint4 *)pw, sc, wq[m]);
+          wq[m] = *(const uint4 *)(wq_ptr[m] + ks * 8);
+          wsc[m] = kx_bf16_f32(sc_ptr[m][ks * 2]);
         } else {
-          const uint16_t *pw = (const uint16_t *)wbase[m] + (size_t)e * a.expert_w + (size_t)wrow * a.K + k0 + wg * 32;
 #pragma unroll
-          for (int p = 0; p < 4; ++p) wq[m][p] = ((const uint4 *)pw)[p];
+          for (int j = 0; j < 4; ++j) wb[m][j] = *(const uint4 *)(wb_ptr[m] + k0 + j * 8);
         }
       }
-      __syncthreads();  // the previous K step's fragments have been read
-      *(uint4 *)(xs + xr * LDS_STRIDE + xc) = xv0;
-      *(uint4 *)(xs + xr * LDS_STRIDE + xc + 8) = xv1;
+    };
+    auto store_x = [&](uint16_t *st) {
 #pragma unroll
-      for (int m = 0; m < MATS; ++m)
+      for (int q = 0; q < 2; ++q) {
+        *(uint4 *)(st + (q * 64 + xr) * LDS_STRIDE + xc) = xv[q][0];
+        *(uint4 *)(st + (q * 64 + xr) * LDS_STRIDE + xc + 8) = xv[q][1];
+      }
+    };
+
+    load_global(0);
+    store_x(xs_lds);
+    __syncthreads();
+    for (int ks = 0; ks < nk; ++ks) {
+      const uint16_t *xs = xs_lds + (ks & 1) * XT;
+      // this step's weights leave the load registers before the next step's loads are issued
+      uint32_t cw[MATS][4];
+      float csc[MATS];
+      kx_bf16x8 cb[MATS][4];
 #pragma unroll
-        for (int p = 0; p < 4; ++p) *(uint4 *)(ws[m] + wr * LDS_STRIDE + wg * 32 + p * 8) = wq[m][p];
-      __syncthreads();
+      for (int m = 0; m < MATS; ++m) {
+        if (I4) {
+          cw[m][0] = wq[m].x; cw[m][1] = wq[m].y; cw[m][2] = wq[m].z; cw[m][3] = wq[m].w;
+          csc[m] = wsc[m];
+        } else {
 #pragma unroll
-      for (int kk = 0; kk < BK; kk += 16) {
-        // operand layout of v_mfma_f32_32x32x16_bf16: lane l holds row (l % 32), k = 8*(l / 32) .. +7
-        const int kcol = kk + (lane >> 5) * 8;
-        const kx_bf16x8 a0 = *(const kx_bf16x8 *)(xs + (lane & 31) * LDS_STRIDE + kcol);
-        const kx_bf16x8 a1 = *(const kx_bf16x8 *)(xs + (32 + (lane & 31)) * LDS_STRIDE + kcol);
+          for (int j = 0; j < 4; ++j) cb[m][j] = __builtin_bit_cast(kx_bf16x8, wb[m][j]);
+        }
+      }
+      if (ks + 1 < nk) load_global(ks + 1);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        // MFMA j of the step contracts over columns 8 j .. +7 (lanes 0-31) and 32 + 8 j .. +7 (lanes 32-63)
+        kx_bf16x8 b[MATS];
 #pragma unroll
         for (int m = 0; m < MATS; ++m) {
-          const kx_bf16x8 b = *(const kx_bf16x8 *)(ws[m] + (wave * 32 + (lane & 31)) * LDS_STRIDE + kcol);
-          acc[m][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b, acc[m][0], 0, 0, 0);
-          acc[m][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b, acc[m][1], 0, 0, 0);
+          if (I4) {
+            const float sc = csc[m];
+            b[m] = dequant_word(cw[m][j], sc, sc * 0.0625f, -1032.0f * sc, -72.0f * sc, magic);
+          } else {
+            b[m] = cb[m][j];
+          }
+        }
+        const int kcol = lh * 32 + j * 8;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          if (t < nb) {
+            const kx_bf16x8 av = *(const kx_bf16x8 *)(xs + (t * 32 + lr) * LDS_STRIDE + kcol);
+#pragma unroll
+            for (int m = 0; m < MATS; ++m) acc[m][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, b[m], acc[m][t], 0, 0, 0);
+          }
         }
       }
+      if (ks + 1 < nk) store_x(xs_lds + ((ks + 1) & 1) * XT);
+      __syncthreads();  // the other tile is complete; this one may be overwritten in the next step
     }
-    // epilogue: D[i][j], j = lane % 32 (weight row), i = 8*(v/4) + 4*(lane/32) + v%4 (token of the tile)
-    const int n = n0 + wave * 32 + (lane & 31);
+    // epilogue: D[i][j], j = lane % 32 (weight row), i = 8*(v/4) + 4*(lane/32) + v%4 (token of the 32-token block)
+    const int n = n0 + wave * 32 + lr;
+    if (n < a.N) {
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+      for (int t = 0; t < 4; ++t)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int i = t * 32 + 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-        const int po = m0 + i;
-        if (po < p_end && n < a.N) {
-          const int pr = a.pairs ? a.pairs[po] : po;
-          float r = acc[0][t][v];
-          if (DUAL) r = kx_swiglu(kx_bfround(r), kx_bfround(acc[1][t][v]));
-          a.out[(size_t)pr * a.N + n] = kx_bf16_rne(r);
+        for (int v = 0; v < 16; ++v) {
+          const int po = m0 + t * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+          if (po < p_end) {
+            const int pr = a.pairs ? a.pairs[po] : po;
+            float r = acc[0][t][v];
+            if (DUAL) r = kx_swiglu(kx_bfround(r), kx_bfround(acc[1][t][v]));
+            if (!DUAL && a.out_f32) ((float *)a.out)[(size_t)pr * a.N + n] = r;
+            else ((uint16_t *)a.out)[(size_t)pr * a.N + n] = kx_bf16_rne(r);
+          }
         }
-      }
-    __syncthreads();
+    }
   }
 }
 
@@ -163,21 +242,25 @@ __global__ void __launch_bounds__(256) moe_combine_k(const uint16_t *__restrict_
 }  // namespace
 
 int kx_grouped_gemm_launch(bool dual, bool i4, const void *w0, const uint16_t *s0, const void *w1, const uint16_t *s1,
-                           const uint16_t *x, uint16_t *out, const int4 *work, const int *pairs, int n_pairs, int n_slots,
-                           int N, int K, int x_div, size_t expert_w, size_t expert_s, int n_pairs_max, hipStream_t st) {
+                           const uint16_t *x, void *out, bool out_f32, const int4 *work, const int *pairs, int n_pairs,
+                           int n_slots, int N, int K, int x_div, size_t expert_w, size_t expert_s, int n_pairs_max,
+                           hipStream_t st) {
   KX_REQUIRE(K > 0 && K % 64 == 0, "kx_grouped_gemm: K=%d must be a positive multiple of 64", K);
   KX_REQUIRE(N > 0, "kx_grouped_gemm: N=%d must be positive", N);
+  KX_REQUIRE(!(dual && out_f32), "kx_grouped_gemm: fp32 output is for a single matrix");
   PfArgs a;
   a.w0 = w0; a.w1 = w1; a.s0 = s0; a.s1 = s1; a.x = x; a.out = out; a.work = work; a.pairs = pairs;
   a.n_pairs = n_pairs; a.N = N; a.K = K; a.x_div = x_div; a.expert_w = expert_w; a.expert_s = expert_s;
+  a.out_f32 = out_f32 ? 1 : 0;
   const int max_rows = work ? n_pairs_max : n_pairs;
   int mz = kx_cdiv(max_rows, BM);
   mz = mz < 1 ? 1 : mz > 64 ? 64 : mz;
-  dim3 g(kx_cdiv(N, BN), work ? n_slots : 1, mz), b(256);
-  if (dual && i4) hipLaunchKernelGGL((grouped_gemm_k<true, true>), g, b, 0, st, a);
-  else if (dual) hipLaunchKernelGGL((grouped_gemm_k<true, false>), g, b, 0, st, a);
-  else if (i4) hipLaunchKernelGGL((grouped_gemm_k<false, true>), g, b, 0, st, a);
-  else hipLaunchKernelGGL((grouped_gemm_k<false, false>), g, b, 0, st, a);
+  dim3 g(kx_cdiv(N, BN), work ? n_slots : 1, mz), b(PF_THREADS);
+  const size_t lds = 0;
+  if (dual && i4) hipLaunchKernelGGL((grouped_gemm_k<true, true>), g, b, lds, st, a);
+  else if (dual) hipLaunchKernelGGL((grouped_gemm_k<true, false>), g, b, lds, st, a);
+  else if (i4) hipLaunchKernelGGL((grouped_gemm_k<false, true>), g, b, lds, st, a);
+  else hipLaunchKernelGGL((grouped_gemm_k<false, false>), g, b, lds, st, a);
   KX_LAUNCH_CHECK();
   return KX_OK;
 }
