@@ -33,6 +33,8 @@
 #include "kx_dense.h"
 #include "kx_math.h"
 
+#include <type_traits>
+
 namespace {
 
 typedef __bf16 kx_bf16x8 __attribute__((ext_vector_type(8)));
@@ -112,13 +114,6 @@ __global__ void __launch_bounds__(PF_THREADS, 2) grouped_gemm_k(PfArgs a) {
 
   for (int m0 = p_begin + blockIdx.z * BM; m0 < p_end; m0 += gridDim.z * BM) {
     const int nb = min(4, (p_end - m0 + 31) >> 5);  // 32-token blocks that hold tokens
-    kx_f32x16 acc[MATS][4];
-#pragma unroll
-    for (int m = 0; m < MATS; ++m)
-#pragma unroll
-      for (int t = 0; t < 4; ++t)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc[m][t][i] = 0.0f;
     const uint16_t *xrow[2];
     bool x_valid[2];
 #pragma unroll
@@ -129,99 +124,141 @@ __global__ void __launch_bounds__(PF_THREADS, 2) grouped_gemm_k(PfArgs a) {
       xrow[q] = a.x + (size_t)(pair / a.x_div) * a.K + xc;
     }
 
-    uint4 xv[2][2];
-    uint4 wq[MATS];      // INT4: the group's four packed words
-    float wsc[MATS];
-    uint4 wb[MATS][4];   // BF16: 32 columns
-    auto load_global = [&](int ks) {
-      const int k0 = ks * BK;
+    // the tile with NB token blocks, NB a compile-time constant so that the K loop has no branches
+    auto run = [&](auto nb_c) {
+      constexpr int NB = decltype(nb_c)::value;
+      constexpr int XQ = NB > 2 ? 2 : 1;  // halves of the activation tile that are staged
+      kx_f32x16 acc[MATS][NB];
 #pragma unroll
-      for (int q = 0; q < 2; ++q) {
-        xv[q][0] = xv[q][1] = make_uint4(0, 0, 0, 0);
-        if (x_valid[q]) { xv[q][0] = *(const uint4 *)(xrow[q] + k0); xv[q][1] = *(const uint4 *)(xrow[q] + k0 + 8); }
-      }
+      for (int m = 0; m < MATS; ++m)
 #pragma unroll
-      for (int m = 0; m < MATS; ++m) {
-        if (I4) {
-          wq[m] = *(const uint4 *)(wq_ptr[m] + ks * 8);
-          wsc[m] = kx_bf16_f32(sc_ptr[m][ks * 2]);
-        } else {
+        for (int t = 0; t < NB; ++t)
 #pragma unroll
-          for (int j = 0; j < 4; ++j) wb[m][j] = *(const uint4 *)(wb_ptr[m] + k0 + j * 8);
-        }
-      }
-    };
-    auto store_x = [&](uint16_t *st) {
-#pragma unroll
-      for (int q = 0; q < 2; ++q) {
-        *(uint4 *)(st + (q * 64 + xr) * LDS_STRIDE + xc) = xv[q][0];
-        *(uint4 *)(st + (q * 64 + xr) * LDS_STRIDE + xc + 8) = xv[q][1];
-      }
-    };
-
-    load_global(0);
-    store_x(xs_lds);
-    __syncthreads();
-    for (int ks = 0; ks < nk; ++ks) {
-      const uint16_t *xs = xs_lds + (ks & 1) * XT;
-      // this step's weights leave the load registers before the next step's loads are issued
-      uint32_t cw[MATS][4];
-      float csc[MATS];
-      kx_bf16x8 cb[MATS][4];
-#pragma unroll
-      for (int m = 0; m < MATS; ++m) {
-        if (I4) {
-          cw[m][0] = wq[m].x; cw[m][1] = wq[m].y; cw[m][2] = wq[m].z; cw[m][3] = wq[m].w;
-          csc[m] = wsc[m];
-        } else {
-#pragma unroll
-          for (int j = 0; j < 4; ++j) cb[m][j] = __builtin_bit_cast(kx_bf16x8, wb[m][j]);
-        }
-      }
-      if (ks + 1 < nk) load_global(ks + 1);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        // MFMA j of the step contracts over columns 8 j .. +7 (lanes 0-31) and 32 + 8 j .. +7 (lanes 32-63)
-        kx_bf16x8 b[MATS];
+          for (int i = 0; i < 16; ++i) acc[m][t][i] = 0.0f;
+      struct WRaw {
+        uint4 q[MATS];      // INT4: the group's four packed words
+        float sc[MATS];
+        uint4 b[MATS][I4 ? 1 : 4];  // BF16: 32 columns
+      };
+      uint4 xv[XQ][2];
+      auto load_w = [&](WRaw &r, int ks) {
 #pragma unroll
         for (int m = 0; m < MATS; ++m) {
           if (I4) {
-            const float sc = csc[m];
-            b[m] = dequant_word(cw[m][j], sc, sc * 0.0625f, -1032.0f * sc, -72.0f * sc, magic);
+            r.q[m] = *(const uint4 *)(wq_ptr[m] + ks * 8);
+            r.sc[m] = kx_bf16_f32(sc_ptr[m][ks * 2]);
           } else {
-            b[m] = cb[m][j];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) r.b[m][j] = *(const uint4 *)(wb_ptr[m] + ks * BK + j * 8);
           }
         }
+      };
+      auto load_x = [&](int ks) {
+#pragma unroll
+        for (int q = 0; q < XQ; ++q) {
+          xv[q][0] = xv[q][1] = make_uint4(0, 0, 0, 0);
+          if (x_valid[q]) { xv[q][0] = *(const uint4 *)(xrow[q] + ks * BK); xv[q][1] = *(const uint4 *)(xrow[q] + ks * BK + 8); }
+        }
+      };
+      auto store_x = [&](uint16_t *st) {
+#pragma unroll
+        for (int q = 0; q < XQ; ++q) {
+          *(uint4 *)(st + (q * 64 + xr) * LDS_STRIDE + xc) = xv[q][0];
+          *(uint4 *)(st + (q * 64 + xr) * LDS_STRIDE + xc + 8) = xv[q][1];
+        }
+      };
+      // one K step on the weights in r; the activations of step ks are in LDS tile ks % 2.
+      // MFMA j of the step contracts over columns 8 j .. +7 (lanes 0-31) and 32 + 8 j .. +7 (lanes 32-63).
+      // Software pipeline: the operands of MFMA group j+1 (LDS reads of the activations, dequant of the
+      // weights) are produced while the matrix cores run group j.
+      auto dequant_j = [&](const WRaw &r, int j, kx_bf16x8 (&b)[MATS]) {
+#pragma unroll
+        for (int m = 0; m < MATS; ++m) {
+          if (I4) {
+            const float sc = r.sc[m];
+            const uint32_t w = j == 0 ? r.q[m].x : j == 1 ? r.q[m].y : j == 2 ? r.q[m].z : r.q[m].w;
+            b[m] = dequant_word(w, sc, sc * 0.0625f, -1032.0f * sc, -72.0f * sc, magic);
+          } else {
+            b[m] = __builtin_bit_cast(kx_bf16x8, r.b[m][j]);
+          }
+        }
+      };
+      auto read_a = [&](const uint16_t *xs, int j, kx_bf16x8 (&av)[NB]) {
         const int kcol = lh * 32 + j * 8;
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          if (t < nb) {
-            const kx_bf16x8 av = *(const kx_bf16x8 *)(xs + (t * 32 + lr) * LDS_STRIDE + kcol);
+        for (int t = 0; t < NB; ++t) av[t] = *(const kx_bf16x8 *)(xs + (t * 32 + lr) * LDS_STRIDE + kcol);
+      };
+      constexpr int VPER = I4 ? (34 * MATS + NB * MATS - 1) / (NB * MATS) : 0;  // VALU instructions per MFMA
+      auto mfma_group = [&](const kx_bf16x8 (&av)[NB], const kx_bf16x8 (&b)[MATS], auto with_valu) {
 #pragma unroll
-            for (int m = 0; m < MATS; ++m) acc[m][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, b[m], acc[m][t], 0, 0, 0);
-          }
+        for (int t = 0; t < NB; ++t)
+#pragma unroll
+          for (int m = 0; m < MATS; ++m) acc[m][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[t], b[m], acc[m][t], 0, 0, 0);
+        // scheduling: one MFMA, then a share of the VALU work that prepares the next group
+#pragma unroll
+        for (int i = 0; i < NB * MATS; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          if constexpr (decltype(with_valu)::value) __builtin_amdgcn_sched_group_barrier(0x002, VPER, 0);
+        }
+      };
+      auto step = [&](const WRaw &r, int ks) {
+        const uint16_t *xs = xs_lds + (ks & 1) * XT;
+        kx_bf16x8 b0[MATS], b1[MATS], a0[NB], a1[NB];
+        dequant_j(r, 0, b0);
+        read_a(xs, 0, a0);
+        read_a(xs, 1, a1);
+        dequant_j(r, 1, b1);
+        mfma_group(a0, b0, std::true_type{});
+        read_a(xs, 2, a0);
+        dequant_j(r, 2, b0);
+        mfma_group(a1, b1, std::true_type{});
+        read_a(xs, 3, a1);
+        dequant_j(r, 3, b1);
+        mfma_group(a0, b0, std::true_type{});
+        mfma_group(a1, b1, std::false_type{});
+      };
+
+      // weights and activations are fetched one K step ahead (registers; two LDS tiles)
+      WRaw w0, w1;
+      load_w(w0, 0);
+      load_x(0);
+      store_x(xs_lds);
+      __syncthreads();
+      for (int ks = 0; ks < nk; ks += 2) {
+        if (ks + 1 < nk) { load_w(w1, ks + 1); load_x(ks + 1); }
+        step(w0, ks);
+        if (ks + 1 < nk) store_x(xs_lds + XT);
+        __syncthreads();
+        if (ks + 1 < nk) {
+          if (ks + 2 < nk) { load_w(w0, ks + 2); load_x(ks + 2); }
+          step(w1, ks + 1);
+          if (ks + 2 < nk) store_x(xs_lds);
+          __syncthreads();
         }
       }
-      if (ks + 1 < nk) store_x(xs_lds + ((ks + 1) & 1) * XT);
-      __syncthreads();  // the other tile is complete; this one may be overwritten in the next step
-    }
-    // epilogue: D[i][j], j = lane % 32 (weight row), i = 8*(v/4) + 4*(lane/32) + v%4 (token of the 32-token block)
-    const int n = n0 + wave * 32 + lr;
-    if (n < a.N) {
+      // epilogue: D[i][j], j = lane % 32 (weight row), i = 8*(v/4) + 4*(lane/32) + v%4 (token of the 32-token block)
+      const int n = n0 + wave * 32 + lr;
+      if (n < a.N) {
 #pragma unroll
-      for (int t = 0; t < 4; ++t)
+        for (int t = 0; t < NB; ++t)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const int po = m0 + t * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
-          if (po < p_end) {
-            const int pr = a.pairs ? a.pairs[po] : po;
-            float r = acc[0][t][v];
-            if (DUAL) r = kx_swiglu(kx_bfround(r), kx_bfround(acc[1][t][v]));
-            if (!DUAL && a.out_f32) ((float *)a.out)[(size_t)pr * a.N + n] = r;
-            else ((uint16_t *)a.out)[(size_t)pr * a.N + n] = kx_bf16_rne(r);
+          for (int v = 0; v < 16; ++v) {
+            const int po = m0 + t * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+            if (po < p_end) {
+              const int pr = a.pairs ? a.pairs[po] : po;
+              float r = acc[0][t][v];
+              if (DUAL) r = kx_swiglu(kx_bfround(r), kx_bfround(acc[1][t][v]));
+              if (!DUAL && a.out_f32) ((float *)a.out)[(size_t)pr * a.N + n] = r;
+              else ((uint16_t *)a.out)[(size_t)pr * a.N + n] = kx_bf16_rne(r);
+            }
           }
-        }
-    }
+      }
+      __syncthreads();  // the next token tile starts by overwriting LDS tile 0
+    };
+    if (nb == 1) run(std::integral_constant<int, 1>{});
+    else if (nb == 2) run(std::integral_constant<int, 2>{});
+    else if (nb == 3) run(std::integral_constant<int, 3>{});
+    else run(std::integral_constant<int, 4>{});
   }
 }
 

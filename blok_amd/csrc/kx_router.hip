@@ -56,6 +56,113 @@ __global__ void __launch_bounds__(1024) topk_bucket_k(const float *__restrict__ 
                         s_ids4, s_cnt, s_act);
 }
 
+// ---- bucketing of a prefill chunk: one workgroup per expert instead of one per launch ------------
+// ids of segment `seg` (seg_len a multiple of 8) compared with expert e; calls f(pair index) for every match, in order
+template <typename F>
+__device__ __forceinline__ void for_matches(const uint16_t *__restrict__ ids, int n_pairs, int begin, int end, uint32_t e, F f) {
+  for (int p0 = begin; p0 < end; p0 += 8) {
+    uint16_t v[8];
+    if (p0 + 8 <= n_pairs) {
+      const uint4 u = *(const uint4 *)(ids + p0);
+      const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = (uint16_t)((j & 1) ? (w[j >> 1] >> 16) : (w[j >> 1] & 0xffffu));
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = p0 + j < n_pairs ? ids[p0 + j] : (uint16_t)0xffff;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (v[j] == e) f(p0 + j);
+  }
+}
+
+__device__ __forceinline__ int block_sum_256(int v, int *s_red) {  // sum over the 256 threads, returned to all
+  for (int m = 32; m; m >>= 1) v += __shfl_xor(v, m);
+  if ((threadIdx.x & 63) == 0) s_red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  const int t = s_red[0] + s_red[1] + s_red[2] + s_red[3];
+  __syncthreads();
+  return t;
+}
+
+// grid (E), 256 threads: counts[e]
+__global__ void __launch_bounds__(256) bucket_count_k(const uint16_t *__restrict__ ids, int n_pairs, int *__restrict__ counts) {
+  __shared__ int s_red[4];
+  const int seg = (((n_pairs + 255) >> 8) + 7) & ~7;
+  int cnt = 0;
+  for_matches(ids, n_pairs, threadIdx.x * seg, min(n_pairs, (threadIdx.x + 1) * seg), blockIdx.x, [&](int) { ++cnt; });
+  cnt = block_sum_256(cnt, s_red);
+  if (threadIdx.x == 0) counts[blockIdx.x] = cnt;
+}
+
+// one workgroup of at least E threads: offsets, the list of experts with work, n_active
+__global__ void __launch_bounds__(1024) bucket_scan_k(const int *__restrict__ counts, int E, int *__restrict__ offsets,
+                                                      int4 *__restrict__ work, int *__restrict__ n_active) {
+  __shared__ int s_cnt[1024];
+  __shared__ int s_act[1024];
+  const int e = threadIdx.x, n = blockDim.x;
+  const int cnt = e < E ? counts[e] : 0;
+  s_cnt[e] = cnt;
+  s_act[e] = cnt > 0 ? 1 : 0;
+  __syncthreads();
+  for (int d = 1; d < n; d <<= 1) {
+    int a = e >= d ? s_cnt[e - d] : 0, b = e >= d ? s_act[e - d] : 0;
+    __syncthreads();
+    s_cnt[e] += a;
+    s_act[e] += b;
+    __syncthreads();
+  }
+  const int off = s_cnt[e] - cnt, slot = s_act[e] - (cnt > 0 ? 1 : 0), total_active = s_act[n - 1];
+  if (e < E) {
+    offsets[e] = off;
+    if (cnt > 0) work[slot] = make_int4(e, off, off + cnt, 0);  // the first pair is filled in by bucket_place_k
+    if (e >= total_active) work[e] = make_int4(-1, 0, 0, 0);
+  }
+  if (e == 0) {
+    offsets[E] = s_cnt[n - 1];
+    *n_active = total_active;
+  }
+}
+
+// grid (E), 256 threads: the pairs of expert e in ascending order at pairs[offsets[e] ..]
+__global__ void __launch_bounds__(256) bucket_place_k(const uint16_t *__restrict__ ids, int n_pairs, const int *__restrict__ counts,
+                                                      const int *__restrict__ offsets, const int *__restrict__ n_active,
+                                                      int *__restrict__ pairs, int4 *__restrict__ work) {
+  __shared__ int s_scan[256];
+  const int e = blockIdx.x, t = threadIdx.x;
+  if (counts[e] == 0) return;
+  const int off = offsets[e];
+  const int seg = (((n_pairs + 255) >> 8) + 7) & ~7;
+  const int begin = t * seg, end = min(n_pairs, (t + 1) * seg);
+  int cnt = 0;
+  for_matches(ids, n_pairs, begin, end, e, [&](int) { ++cnt; });
+  s_scan[t] = cnt;
+  __syncthreads();
+  for (int d = 1; d < 256; d <<= 1) {
+    const int a = t >= d ? s_scan[t - d] : 0;
+    __syncthreads();
+    s_scan[t] += a;
+    __syncthreads();
+  }
+  int pos = off + s_scan[t] - cnt;
+  const bool has_first = cnt > 0 && pos == off;
+  int first = 0;
+  for_matches(ids, n_pairs, begin, end, e, [&](int p) {
+    if (pos == off) first = p;
+    pairs[pos++] = p;
+  });
+  if (has_first) {  // the record of expert e: the list is sorted by expert id
+    int lo = 0, hi = *n_active - 1;
+    while (lo < hi) {
+      const int mid = (lo + hi) >> 1;
+      if (work[mid].x < e) lo = mid + 1;
+      else hi = mid;
+    }
+    work[lo].w = first;
+  }
+}
+
 }  // namespace
 
 int kx_router_topk_launch(const float *logits, const float *bias, uint16_t *ids, float *weights, int tokens,
@@ -81,9 +188,19 @@ int kx_bucket_launch(const uint16_t *ids, int tokens, int experts, int topk, int
   KX_REQUIRE(tokens > 0 && topk > 0, "kx_bucket: tokens=%d topk=%d must be positive", tokens, topk);
   KX_REQUIRE(experts > 0 && experts <= 1024, "kx_bucket: experts=%d outside [1, 1024]", experts);
   int threads = kx_cdiv(experts, 64) * 64;
-  const size_t lds = (size_t)kx_cdiv(tokens * topk, 8) * 16;
-  KX_REQUIRE(lds <= 48 * 1024, "kx_bucket: %d pairs exceed the %d the bucketing kernel stages", tokens * topk, 24576);
-  hipLaunchKernelGGL(bucket_k, dim3(1), dim3(threads), lds, st, ids, tokens * topk, experts, counts, offsets, pairs,
+  const long n_pairs = (long)tokens * topk;
+  KX_REQUIRE(n_pairs < (1L << 30), "kx_bucket: %ld pairs", n_pairs);
+  if (n_pairs > 1024) {  // a chunk: one workgroup per expert counts, one scans, one per expert places
+    hipLaunchKernelGGL(bucket_count_k, dim3(experts), dim3(256), 0, st, ids, (int)n_pairs, counts);
+    KX_LAUNCH_CHECK();
+    hipLaunchKernelGGL(bucket_scan_k, dim3(1), dim3(threads), 0, st, counts, experts, offsets, work, n_active);
+    KX_LAUNCH_CHECK();
+    hipLaunchKernelGGL(bucket_place_k, dim3(experts), dim3(256), 0, st, ids, (int)n_pairs, counts, offsets, n_active, pairs, work);
+    KX_LAUNCH_CHECK();
+    return KX_OK;
+  }
+  const size_t lds = (size_t)kx_cdiv((int)n_pairs, 8) * 16;
+  hipLaunchKernelGGL(bucket_k, dim3(1), dim3(threads), lds, st, ids, (int)n_pairs, experts, counts, offsets, pairs,
                      work, n_active);
   KX_LAUNCH_CHECK();
   return KX_OK;

@@ -56,7 +56,7 @@ def test_router_ties_take_lowest_index(kxlib, ox):
     assert (ids == ids1).all() and (w.view(np.uint32) == w1.view(np.uint32)).all()
 
 
-@pytest.mark.parametrize("T,E,topk", [(1, 384, 8), (8, 384, 8), (64, 384, 8), (2048, 384, 8), (7, 16, 4)])
+@pytest.mark.parametrize("T,E,topk", [(1, 384, 8), (8, 384, 8), (64, 384, 8), (2048, 384, 8), (7, 16, 4), (301, 384, 8), (259, 16, 4)])
 def test_bucket_bit_exact(kxlib, ox, T, E, topk):
     say(f"bucket T={T} E={E} topk={topk}")
     logits = O.normal_f32(T * E, 6, 1, 1.0).reshape(T, E)
