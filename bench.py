@@ -36,9 +36,9 @@ def build_if_missing():
         __graft_entry__.build()
 
 
-# HBM bytes of one i4_gemv_k<dual> launch at T=1 (8 experts) from rocprofv3 counters: FETCH_SIZE 64,630 KiB x 2.0
-# (a 1 GiB kx_dev_copy reads 524,288 on that counter) + WRITE_SIZE 32 KiB x 1.0; see profiles/
-GATE_UP_TRAFFIC_T1 = 132395008
+# HBM bytes of one i4_gemv_k<dual> launch at T=1 (8 experts) from rocprofv3 counters: FETCH_SIZE 64,645 KiB x 2.0
+# (a 1 GiB kx_dev_copy reads 524,300 on that counter) + WRITE_SIZE 32 KiB x 1.0; see profiles/
+GATE_UP_TRAFFIC_T1 = 132423000
 
 
 def moe_layer_bytes(cfg, tokens, distinct):
