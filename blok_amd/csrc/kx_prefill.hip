@@ -7,19 +7,23 @@
 // combine (:868,:871), the shared expert (:872-875) and the residual add (:877) --
 // with the tokens of each expert gathered into one GEMM.
 //
-// The only place MFMA is used.  Per workgroup (4 waves): one expert, 128 weight rows, the
+// The only place MFMA is used.  Per workgroup (8 waves): one expert, 256 weight rows, the
 // expert's tokens in tiles of 128.  Wave w owns weight rows 32 w .. +31 for all 128 tokens
 // (fp32 accumulators of v_mfma_f32_32x32x16_bf16).  Per K step of 64 columns:
-//  * weights never touch LDS: lane (r, h) = (lane % 32, lane / 32) loads the 16 bytes of row r
-//    that hold columns 32 h .. +31 of the step -- one quantization group, four packed words --
-//    and dequantizes word j to the reference's values, w = bf((n-8)*scale) (:311-312), which
-//    is exactly the B operand of the step's j-th MFMA when that MFMA contracts over columns
-//    {8 j .. +7} and {32 + 8 j .. +7} (the contraction order within a step is free, the
-//    activation operand uses the same columns);
-//  * the gathered activation rows go through a double-buffered LDS tile, one barrier per step;
-//  * the global loads of step k+1 are in flight while step k is computed.
-// The bf16 shared expert and the router gate use the same kernel with plain loads in place
-// of the dequant.
+//  * INT4 weights reach the lanes through LDS as packed words: for every two K steps the
+//    64-byte runs of the 256 rows (both matrices) are copied by global -> LDS loads, which
+//    take no registers and use every byte they fetch, into a ring of two stages; lane
+//    (r, h) = (lane % 32, lane / 32) reads the 16 bytes of row r that hold columns 32 h .. +31
+//    of the step -- one quantization group, four packed words -- and dequantizes word j to
+//    the reference's values, w = bf((n-8)*scale) (:311-312), which is exactly the B operand
+//    of the step's j-th MFMA when that MFMA contracts over columns {8 j .. +7} and
+//    {32 + 8 j .. +7} (the contraction order within a step is free, the activation operand
+//    uses the same columns).  The 16-byte pieces of a row are stored xor-swizzled by the row
+//    so that the lanes' reads are free of bank conflicts.  Group scales are staged in LDS
+//    for eight K steps at a time (32 bytes per row and matrix, one load per thread);
+//  * bf16 weights (shared expert, router gate) are loaded by the lanes themselves, 64
+//    contiguous bytes per lane and step, one step ahead;
+//  * the gathered activation rows go through a double-buffered LDS tile, one barrier per step.
 //
 // Dequant without integer conversion: (w & 0x000F000F) | 0x64006400 is the f16 pair
 // (1024+n0, 1024+n4), (w & 0x00F000F0) | 0x64006400 is (1024+16 n1, 1024+16 n5), w >> 8 gives
@@ -43,9 +47,11 @@ typedef float kx_f32x2 __attribute__((ext_vector_type(2)));
 typedef float kx_f32x16 __attribute__((ext_vector_type(16)));
 typedef _Float16 kx_h2 __attribute__((ext_vector_type(2)));
 
-constexpr int BM = 128, BN = 128, BK = 64;
+constexpr int BN = 256, BK = 64;  // a token tile has up to 4 blocks of 32 tokens (PfArgs::nb_max)
 constexpr int LDS_STRIDE = BK + 8;  // bf16 elements per LDS row: 144 B keeps 16-byte reads of a column of rows spread over banks
-constexpr int PF_THREADS = 256;
+constexpr int PF_THREADS = 512;
+constexpr int W_STAGE = BN * 64;               // bytes of one matrix's packed words for two K steps
+constexpr int SC_STRIDE = 40;                  // bytes per (row, matrix) of staged scales: 16 bf16 + pad against bank conflicts
 
 struct PfArgs {
   const void *w0, *w1;          // INT4: packed i32 [E][N][K/8]; BF16: bf16 [E][N][K]
@@ -57,6 +63,7 @@ struct PfArgs {
   int n_pairs, N, K, x_div;     // activation row = pair / x_div
   size_t expert_w, expert_s;    // elements between experts (words or bf16; scales)
   int out_f32;                  // single matrix only: store the fp32 accumulators unrounded
+  int nb_max;                   // 32-token blocks per token tile (1..4): sizes the activation tiles in LDS
 };
 
 __device__ __forceinline__ uint32_t pf_and_or(uint32_t a, uint32_t mask, uint32_t magic) {
@@ -84,10 +91,13 @@ __device__ __forceinline__ kx_bf16x8 dequant_word(uint32_t w, float sc, float sc
 }
 
 template <bool DUAL, bool I4>
-__global__ void __launch_bounds__(PF_THREADS, 2) grouped_gemm_k(PfArgs a) {
+__global__ void __launch_bounds__(PF_THREADS, I4 ? 1 : 2) grouped_gemm_k(PfArgs a) {
   constexpr int MATS = DUAL ? 2 : 1;
-  constexpr int XT = BM * LDS_STRIDE;  // elements of one activation tile
-  __shared__ __attribute__((aligned(16))) uint16_t xs_lds[2 * XT];
+  extern __shared__ __attribute__((aligned(16))) uint8_t pf_lds[];
+  const int BM = a.nb_max * 32, XT = BM * LDS_STRIDE;   // tokens and elements of one activation tile
+  uint16_t *xs_lds = (uint16_t *)pf_lds;                 // two activation tiles
+  uint8_t *w_ring = pf_lds + 2 * XT * 2;                 // INT4: [2 stages][MATS][256 rows][4 pieces of 16 B]
+  uint8_t *sc_lds = w_ring + 2 * MATS * W_STAGE;         // INT4: [2][256 rows * MATS][SC_STRIDE]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int lr = lane & 31, lh = lane >> 5;
   const int n0 = blockIdx.x * BN;
@@ -98,36 +108,65 @@ __global__ void __launch_bounds__(PF_THREADS, 2) grouped_gemm_k(PfArgs a) {
   uint32_t magic;
   asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(magic));
   const int nk = a.K / BK;
-  // this lane's weight row and its 32-column half of every K step
-  const int wrow = min(n0 + wave * 32 + lr, a.N - 1);
-  const uint32_t *wq_ptr[MATS];
-  const uint16_t *wb_ptr[MATS], *sc_ptr[MATS];
+  const int trow = wave * 32 + lr;                       // this lane's weight row within the tile
+  const int wrow = min(n0 + trow, a.N - 1);
+  // bf16 weights: this lane's row and its 32-column half of every K step
+  const uint16_t *wb_ptr[MATS];
 #pragma unroll
-  for (int m = 0; m < MATS; ++m) {
-    const void *wbase = m ? a.w1 : a.w0;
-    wq_ptr[m] = (const uint32_t *)wbase + (size_t)e * a.expert_w + (size_t)wrow * (a.K >> 3) + lh * 4;
-    wb_ptr[m] = (const uint16_t *)wbase + (size_t)e * a.expert_w + (size_t)wrow * a.K + lh * 32;
-    sc_ptr[m] = (m ? a.s1 : a.s0) + (I4 ? (size_t)e * a.expert_s + (size_t)wrow * (a.K >> 5) + lh : 0);
+  for (int m = 0; m < MATS; ++m)
+    wb_ptr[m] = (const uint16_t *)(m ? a.w1 : a.w0) + (size_t)e * a.expert_w + (size_t)wrow * a.K + lh * 32;
+  // INT4: global -> LDS copies of this wave for one stage: MATS*2 instructions of 64 pieces
+  const uint32_t *dma_src[MATS * 2];
+  int dma_dst[MATS * 2];
+#pragma unroll
+  for (int u = 0; u < MATS * 2; ++u) {
+    const int g = (wave * MATS * 2 + u) * 64 + lane;     // piece index over [MATS][256 rows][4]
+    const int m = g >> 10, sl = g & 1023, row = sl >> 2, ps = sl & 3;
+    const int p = ps ^ ((row >> 2) & 3);                 // the piece of the row that lives in slot ps
+    dma_src[u] = (const uint32_t *)(m ? a.w1 : a.w0) + (size_t)e * a.expert_w + (size_t)min(n0 + row, a.N - 1) * (a.K >> 3) + p * 4;
+    dma_dst[u] = (wave * MATS * 2 + u) * 1024;           // byte offset within a stage, the same for the whole wave
   }
-  // activation staging: thread -> rows tid/4 and 64 + tid/4, 16 columns from (tid%4)*16
+  auto dma_stage = [&](int ss) {  // packed words of K steps 2 ss, 2 ss + 1 into stage ss % 2
+    if (I4) {
+#pragma unroll
+      for (int u = 0; u < MATS * 2; ++u)
+        __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)(dma_src[u] + ss * 16),
+                                         (void __attribute__((address_space(3))) *)(w_ring + (ss & 1) * MATS * W_STAGE + dma_dst[u]),
+                                         16, 0, 0);
+    }
+  };
+  // scale staging: thread -> (row, matrix), 16 scales = 8 K steps per load
+  const int sc_row = MATS == 2 ? tid >> 1 : tid, sc_m = MATS == 2 ? (tid & 1) : 0;
+  const bool sc_active = I4 && sc_row < BN;
+  const uint16_t *sc_src = (sc_m ? a.s1 : a.s0) + (I4 ? (size_t)e * a.expert_s + (size_t)min(n0 + sc_row, a.N - 1) * (a.K >> 5) : 0);
+  uint2 sc_regs[4];
+  auto load_scales = [&](int blk) {
+    if (sc_active) {
+      const uint2 *p = (const uint2 *)(sc_src + blk * 16);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sc_regs[i] = p[i];
+    }
+  };
+  auto store_scales = [&](int blk) {
+    if (sc_active) {
+      uint2 *d = (uint2 *)(sc_lds + (blk & 1) * (BN * MATS * SC_STRIDE) + (sc_row * MATS + sc_m) * SC_STRIDE);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) d[i] = sc_regs[i];
+    }
+  };
+  // activation staging: thread -> row tid/4, 16 columns from (tid%4)*16
   const int xr = tid >> 2, xc = (tid & 3) * 16;
 
   for (int m0 = p_begin + blockIdx.z * BM; m0 < p_end; m0 += gridDim.z * BM) {
-    const int nb = min(4, (p_end - m0 + 31) >> 5);  // 32-token blocks that hold tokens
-    const uint16_t *xrow[2];
-    bool x_valid[2];
-#pragma unroll
-    for (int q = 0; q < 2; ++q) {
-      const int pi = m0 + q * 64 + xr;
-      x_valid[q] = pi < p_end;
-      const int pair = x_valid[q] ? (a.pairs ? a.pairs[pi] : pi) : 0;
-      xrow[q] = a.x + (size_t)(pair / a.x_div) * a.K + xc;
-    }
+    const int nb = min(a.nb_max, (p_end - m0 + 31) >> 5);  // 32-token blocks that hold tokens
+    const int pi = m0 + xr;
+    const bool x_valid = pi < p_end;
+    const int pair = x_valid ? (a.pairs ? a.pairs[pi] : pi) : 0;
+    const uint16_t *xrow = a.x + (size_t)(pair / a.x_div) * a.K + xc;
 
     // the tile with NB token blocks, NB a compile-time constant so that the K loop has no branches
     auto run = [&](auto nb_c) {
       constexpr int NB = decltype(nb_c)::value;
-      constexpr int XQ = NB > 2 ? 2 : 1;  // halves of the activation tile that are staged
       kx_f32x16 acc[MATS][NB];
 #pragma unroll
       for (int m = 0; m < MATS; ++m)
@@ -136,41 +175,37 @@ __global__ void __launch_bounds__(PF_THREADS, 2) grouped_gemm_k(PfArgs a) {
 #pragma unroll
           for (int i = 0; i < 16; ++i) acc[m][t][i] = 0.0f;
       struct WRaw {
-        uint4 q[MATS];      // INT4: the group's four packed words
+        uint4 q[MATS];              // INT4: the group's four packed words
         float sc[MATS];
         uint4 b[MATS][I4 ? 1 : 4];  // BF16: 32 columns
       };
-      uint4 xv[XQ][2];
-      auto load_w = [&](WRaw &r, int ks) {
+      uint4 xv[2];
+      auto load_x = [&](int ks) {
+        xv[0] = xv[1] = make_uint4(0, 0, 0, 0);
+        if (x_valid && xr < NB * 32) { xv[0] = *(const uint4 *)(xrow + ks * BK); xv[1] = *(const uint4 *)(xrow + ks * BK + 8); }
+      };
+      auto store_x = [&](uint16_t *st) {
+        if (xr < NB * 32) {
+          *(uint4 *)(st + xr * LDS_STRIDE + xc) = xv[0];
+          *(uint4 *)(st + xr * LDS_STRIDE + xc + 8) = xv[1];
+        }
+      };
+      // this lane's weights of K step ks: INT4 from the LDS ring and the staged scales, bf16 from memory
+      auto fetch_w = [&](WRaw &r, int ks) {
 #pragma unroll
         for (int m = 0; m < MATS; ++m) {
           if (I4) {
-            r.q[m] = *(const uint4 *)(wq_ptr[m] + ks * 8);
-            r.sc[m] = kx_bf16_f32(sc_ptr[m][ks * 2]);
+            const int q = (ks & 1) * 2 + lh;
+            const uint8_t *st = w_ring + ((ks >> 1) & 1) * MATS * W_STAGE + m * W_STAGE;
+            r.q[m] = *(const uint4 *)(st + (trow * 4 + (q ^ ((trow >> 2) & 3))) * 16);
+            const uint8_t *sb = sc_lds + ((ks >> 3) & 1) * (BN * MATS * SC_STRIDE) + (trow * MATS + m) * SC_STRIDE;
+            r.sc[m] = kx_bf16_f32(*(const uint16_t *)(sb + ((ks & 7) * 2 + lh) * 2));
           } else {
 #pragma unroll
             for (int j = 0; j < 4; ++j) r.b[m][j] = *(const uint4 *)(wb_ptr[m] + ks * BK + j * 8);
           }
         }
       };
-      auto load_x = [&](int ks) {
-#pragma unroll
-        for (int q = 0; q < XQ; ++q) {
-          xv[q][0] = xv[q][1] = make_uint4(0, 0, 0, 0);
-          if (x_valid[q]) { xv[q][0] = *(const uint4 *)(xrow[q] + ks * BK); xv[q][1] = *(const uint4 *)(xrow[q] + ks * BK + 8); }
-        }
-      };
-      auto store_x = [&](uint16_t *st) {
-#pragma unroll
-        for (int q = 0; q < XQ; ++q) {
-          *(uint4 *)(st + (q * 64 + xr) * LDS_STRIDE + xc) = xv[q][0];
-          *(uint4 *)(st + (q * 64 + xr) * LDS_STRIDE + xc + 8) = xv[q][1];
-        }
-      };
-      // one K step on the weights in r; the activations of step ks are in LDS tile ks % 2.
-      // MFMA j of the step contracts over columns 8 j .. +7 (lanes 0-31) and 32 + 8 j .. +7 (lanes 32-63).
-      // Software pipeline: the operands of MFMA group j+1 (LDS reads of the activations, dequant of the
-      // weights) are produced while the matrix cores run group j.
       auto dequant_j = [&](const WRaw &r, int j, kx_bf16x8 (&b)[MATS]) {
 #pragma unroll
         for (int m = 0; m < MATS; ++m) {
@@ -201,6 +236,8 @@ __global__ void __launch_bounds__(PF_THREADS, 2) grouped_gemm_k(PfArgs a) {
           if constexpr (decltype(with_valu)::value) __builtin_amdgcn_sched_group_barrier(0x002, VPER, 0);
         }
       };
+      // one K step.  MFMA j contracts over columns 8 j .. +7 (lanes 0-31) and 32 + 8 j .. +7 (lanes 32-63); the
+      // operands of group j+1 (LDS reads, dequant) are produced while the matrix cores run group j.
       auto step = [&](const WRaw &r, int ks) {
         const uint16_t *xs = xs_lds + (ks & 1) * XT;
         kx_bf16x8 b0[MATS], b1[MATS], a0[NB], a1[NB];
@@ -218,26 +255,39 @@ __global__ void __launch_bounds__(PF_THREADS, 2) grouped_gemm_k(PfArgs a) {
         mfma_group(a1, b1, std::false_type{});
       };
 
-      // weights and activations are fetched one K step ahead (registers; two LDS tiles)
+      // prologue: stage 0 of the ring, the first scale block, the first activation tile
       WRaw w0, w1;
-      load_w(w0, 0);
+      dma_stage(0);
+      load_scales(0);
       load_x(0);
+      if (!I4) fetch_w(w0, 0);
+      store_scales(0);
       store_x(xs_lds);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
       for (int ks = 0; ks < nk; ks += 2) {
-        if (ks + 1 < nk) { load_w(w1, ks + 1); load_x(ks + 1); }
+        // even step: the other ring stage was last read two steps ago, behind a barrier
+        if (ks + 2 < nk) dma_stage((ks >> 1) + 1);
+        if ((ks & 7) == 0 && ks + 8 < nk) load_scales((ks >> 3) + 1);
+        if (ks + 1 < nk) load_x(ks + 1);
+        if (I4) fetch_w(w0, ks);
+        if (!I4 && ks + 1 < nk) fetch_w(w1, ks + 1);
         step(w0, ks);
         if (ks + 1 < nk) store_x(xs_lds + XT);
         __syncthreads();
         if (ks + 1 < nk) {
-          if (ks + 2 < nk) { load_w(w0, ks + 2); load_x(ks + 2); }
+          if (ks + 2 < nk) load_x(ks + 2);
+          if (I4) fetch_w(w1, ks + 1);
+          if (!I4 && ks + 2 < nk) fetch_w(w0, ks + 2);
           step(w1, ks + 1);
           if (ks + 2 < nk) store_x(xs_lds);
+          if ((ks & 7) == 6 && ks + 2 < nk) store_scales((ks >> 3) + 1);
+          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's copies into the ring have landed
           __syncthreads();
         }
       }
       // epilogue: D[i][j], j = lane % 32 (weight row), i = 8*(v/4) + 4*(lane/32) + v%4 (token of the 32-token block)
-      const int n = n0 + wave * 32 + lr;
+      const int n = n0 + trow;
       if (n < a.N) {
 #pragma unroll
         for (int t = 0; t < NB; ++t)
@@ -253,10 +303,10 @@ __global__ void __launch_bounds__(PF_THREADS, 2) grouped_gemm_k(PfArgs a) {
             }
           }
       }
-      __syncthreads();  // the next token tile starts by overwriting LDS tile 0
+      __syncthreads();  // the next token tile starts by overwriting the LDS tiles
     };
     if (nb == 1) run(std::integral_constant<int, 1>{});
-    else if (nb == 2) run(std::integral_constant<int, 2>{});
+    else if (nb == 2 || !I4) run(std::integral_constant<int, 2>{});  // bf16 weights are launched with nb_max 2
     else if (nb == 3) run(std::integral_constant<int, 3>{});
     else run(std::integral_constant<int, 4>{});
   }
@@ -282,18 +332,29 @@ int kx_grouped_gemm_launch(bool dual, bool i4, const void *w0, const uint16_t *s
                            const uint16_t *x, void *out, bool out_f32, const int4 *work, const int *pairs, int n_pairs,
                            int n_slots, int N, int K, int x_div, size_t expert_w, size_t expert_s, int n_pairs_max,
                            hipStream_t st) {
-  KX_REQUIRE(K > 0 && K % 64 == 0, "kx_grouped_gemm: K=%d must be a positive multiple of 64", K);
+  KX_REQUIRE(K > 0 && K % 128 == 0 && (!i4 || K % 512 == 0), "kx_grouped_gemm: K=%d must be a positive multiple of %d", K, i4 ? 512 : 128);
   KX_REQUIRE(N > 0, "kx_grouped_gemm: N=%d must be positive", N);
   KX_REQUIRE(!(dual && out_f32), "kx_grouped_gemm: fp32 output is for a single matrix");
   PfArgs a;
   a.w0 = w0; a.w1 = w1; a.s0 = s0; a.s1 = s1; a.x = x; a.out = out; a.work = work; a.pairs = pairs;
   a.n_pairs = n_pairs; a.N = N; a.K = K; a.x_div = x_div; a.expert_w = expert_w; a.expert_s = expert_s;
   a.out_f32 = out_f32 ? 1 : 0;
+  // token tile: 128 tokens for the INT4 kernels, whose dequant work per weight tile is amortised over the tokens;
+  // 64 for the bf16 ones (more workgroups for the one-group GEMMs of the shared expert and the router)
+  a.nb_max = i4 ? 4 : 2;
+  const int BM = a.nb_max * 32;
   const int max_rows = work ? n_pairs_max : n_pairs;
   int mz = kx_cdiv(max_rows, BM);
   mz = mz < 1 ? 1 : mz > 64 ? 64 : mz;
   dim3 g(kx_cdiv(N, BN), work ? n_slots : 1, mz), b(PF_THREADS);
-  const size_t lds = 0;
+  const int mats = dual ? 2 : 1;
+  const size_t lds = (size_t)2 * BM * LDS_STRIDE * 2 + (i4 ? (size_t)2 * mats * W_STAGE + (size_t)2 * BN * mats * SC_STRIDE : 0);
+  static bool attr_set = false;
+  if (!attr_set) {  // more than 64 KB of dynamic LDS has to be allowed per kernel
+    KX_HIP(hipFuncSetAttribute((const void *)grouped_gemm_k<true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+    KX_HIP(hipFuncSetAttribute((const void *)grouped_gemm_k<false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+    attr_set = true;
+  }
   if (dual && i4) hipLaunchKernelGGL((grouped_gemm_k<true, true>), g, b, lds, st, a);
   else if (dual) hipLaunchKernelGGL((grouped_gemm_k<true, false>), g, b, lds, st, a);
   else if (i4) hipLaunchKernelGGL((grouped_gemm_k<false, true>), g, b, lds, st, a);
