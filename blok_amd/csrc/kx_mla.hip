@@ -233,7 +233,8 @@ __global__ void __launch_bounds__(256) mla_partial_k(MlaArgs a) {
   constexpr int R = MLA_R, KVA = MLA_KVA, PITCH = MLA_PITCH;
   extern __shared__ __attribute__((aligned(16))) uint16_t tile_lds[];  // [64][PITCH] then p [4][HG][64] floats
   float(*p_lds)[HG][64] = (float(*)[HG][64])(tile_lds + 64 * PITCH);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: q is then read through the scalar path
   const int span = blockIdx.x, b = blockIdx.z;
   const int h0 = (blockIdx.y * 4 + wave) * HG;
   const uint16_t *cache = a.cache + (size_t)b * a.seq_stride;
@@ -303,8 +304,10 @@ __global__ void __launch_bounds__(256) mla_partial_k(MlaArgs a) {
     for (int h = 0; h < HG; ++h)
 #pragma unroll
       for (int e = 0; e < 8; ++e) O[h][e] = O[h][e] * alpha[h];
+    // all 64 rows: rows past the sequence are staged as zeros and carry p = 0, which leaves O unchanged
     const uint16_t *col = tile_lds + lane * 8;
-    for (int t = 0; t < n; ++t) {
+#pragma unroll 8
+    for (int t = 0; t < 64; ++t) {
       float cf[8];
       unpack8(cf, *(const uint4 *)(col + t * PITCH));
 #pragma unroll
