@@ -456,8 +456,10 @@ def run_mla(args):
                       "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                    "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
                                    "algorithmic_bytes_per_launch": cache_bytes},
-                      "valu": {"tflops": round(flops / (per * 1e-3) / 1e12, 2), "peak_fp32_tflops": 157.3,
-                               "frac": round(flops / (per * 1e-3) / 1e12 / 157.3, 4)}}), flush=True)
+                      "compute": {"tflops": round(flops / (per * 1e-3) / 1e12, 2),
+                                  "kernel": "mla_partial_mfma_k (bf16 MFMA)" if L >= 2048 else "mla_partial_k (fp32 VALU)",
+                                  "frac_of_mfma_bf16_peak": round(flops / (per * 1e-3) / 1e12 / 2500.0, 4),
+                                  "frac_of_valu_fp32_peak": round(flops / (per * 1e-3) / 1e12 / 157.3, 4)}}), flush=True)
 
 
 def run_copy(args):

@@ -70,6 +70,14 @@ extern "C" int kx_softmax_scale(const kx_config *cfg, float *rs, float *mscale) 
   return KX_OK;
 }
 
+// 0: matrix-core kernel from 2048 positions on, 1: VALU kernel always, 2: matrix-core kernel always
+static int g_mla_kernel = 0;
+extern "C" int kx_mla_set_kernel(int32_t mode) {
+  KX_REQUIRE(mode >= 0 && mode <= 2, "kx_mla_set_kernel: mode=%d outside [0, 2]", mode);
+  g_mla_kernel = mode;
+  return KX_OK;
+}
+
 int kx_mla_span_tiles(int seq) {
   int tiles = (seq + 63) / 64, st = 1;
   while (tiles > 64 * st) st *= 2;
@@ -329,25 +337,223 @@ __global__ void __launch_bounds__(256) mla_partial_k(MlaArgs a) {
   }
 }
 
+// ---- the same partials on the matrix cores, for long contexts -----------------------------------
+// q_abs and p = bf(exp(s - m)) are bf16-representable and the cache is bf16, so q.c and p.c are exact
+// products summed in fp32: v_mfma_f32_16x16x32_bf16 computes what mla_partial_k computes with another
+// summation order (held to the 1e-2 bar, not bit-exact; the token-identity runs use mla_partial_k).
+// Workgroup = (sequence, span), 8 waves; wave (hw, cw) owns heads 16 hw .. +15 and, in the second product,
+// latent columns 256 cw .. +255 (both column halves compute the scores of their heads); 32-position tiles.
+//  * the 32 cache rows of tile t+1 are copied global -> LDS (no registers) while tile t is computed;
+//    rows sit at their natural pitch of 1152 B with the 16-byte pieces xor-swizzled by the row, so the
+//    row-per-lane operand reads are free of bank conflicts;
+//  * scores: S^T[pos, head] = C[pos, 576] Q^T[576, head], A operand = cache rows from LDS, B operand =
+//    this lane's head of q in registers (18 K steps of 32);
+//  * the lane that owns head h in the result holds, per K step of the second product, exactly the 8
+//    probabilities a B operand lane needs if MFMA K index 8 g + 4 a + v stands for position
+//    16 a + 4 g + v of the tile -- so p never leaves the registers;
+//  * O^T[col, head] += C^T[col, pos] P^T[pos, head]: the A operand needs 8 positions of one column, so
+//    the 512 latent columns of the tile are transposed once per tile into a second LDS buffer, in that
+//    K index order (LDS -> LDS, lanes = positions, conflict-free both ways).
+constexpr int MM_T = 32;                      // positions per tile
+constexpr int MM_NAT = MM_T * MLA_KVA * 2;    // bytes of one staged tile
+constexpr int MM_CT_PITCH = 80;               // bytes per transposed column: 32 positions + pad
+constexpr int MM_CT = MLA_R * MM_CT_PITCH;
+typedef __bf16 kx_bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 kx_bf16x2v __attribute__((ext_vector_type(2)));
+typedef float kx_f32x2v __attribute__((ext_vector_type(2)));
+typedef float kx_f32x4 __attribute__((ext_vector_type(4)));
+// two f32 -> packed bf16 pair, round to nearest even (v_cvt_pk_bf16_f32; the same values as kx_bf16_rne for finite inputs)
+__device__ __forceinline__ uint32_t mm_pack_bf16(float lo, float hi) {
+  kx_f32x2v v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, kx_bf16x2v));
+}
+
+__global__ void __launch_bounds__(512, 1) mla_partial_mfma_k(MlaArgs a) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t mm_lds[];
+  uint8_t *nat = mm_lds;               // [2][32 rows][72 pieces of 16 B]
+  uint8_t *ct = mm_lds + 2 * MM_NAT;   // [512 columns][MM_CT_PITCH]
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int hw = wave & 3, cw = wave >> 2;  // heads 16 hw .. +15, latent columns 256 cw .. +255 of the second product
+  const int c16 = lane & 15, g = lane >> 4;
+  const int span = blockIdx.x, b = blockIdx.z;
+  const int head = hw * 16 + c16;
+  const uint16_t *cache = a.cache + (size_t)b * a.seq_stride;
+  const int pos0 = span * a.span_tiles * 64, pos_end = min(a.seq, (span + 1) * a.span_tiles * 64);
+  const int n_tiles = (pos_end - pos0 + MM_T - 1) / MM_T;
+  const float scale = a.rs * a.mscale * a.mscale;
+  constexpr float LOG2E = 1.44269504088896341f;
+
+  // q of this lane's head as B operands: K step ks covers columns 32 ks .. +31, lane group g its 8 g .. +7
+  kx_bf16x8 qf[18];
+  {
+    const float *q = a.qabs + ((size_t)b * a.heads + head) * MLA_KVA;
+#pragma unroll
+    for (int ks = 0; ks < 18; ++ks) {
+      const float4 lo = *(const float4 *)(q + ks * 32 + g * 8), hi = *(const float4 *)(q + ks * 32 + g * 8 + 4);
+      const uint4 u = make_uint4((kx_f32_bits(lo.x) >> 16) | (kx_f32_bits(lo.y) & 0xffff0000u),
+                                 (kx_f32_bits(lo.z) >> 16) | (kx_f32_bits(lo.w) & 0xffff0000u),
+                                 (kx_f32_bits(hi.x) >> 16) | (kx_f32_bits(hi.y) & 0xffff0000u),
+                                 (kx_f32_bits(hi.z) >> 16) | (kx_f32_bits(hi.w) & 0xffff0000u));
+      qf[ks] = __builtin_bit_cast(kx_bf16x8, u);
+    }
+  }
+  // global -> LDS copy of a tile: 2304 pieces = 36 instructions over the 8 waves; slot (row p, j') holds
+  // piece j' ^ ((p >> 1) & 7) (low three bits) of the row; rows past the sequence repeat its last row
+  auto copy_tile = [&](int t) {
+#pragma unroll
+    for (int u = 0; u < 5; ++u) {
+      const int ii = wave + 8 * u;
+      if (ii < 36) {
+        const int slot = ii * 64 + lane;
+        const int p = slot / 72, js = slot - p * 72;
+        const int j = (js & ~7) | ((js ^ (p >> 1)) & 7);
+        const int row = min(pos0 + t * MM_T + p, a.seq - 1);
+        __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)(cache + (size_t)row * MLA_KVA + j * 8),
+                                         (void __attribute__((address_space(3))) *)(nat + (t & 1) * MM_NAT + ii * 1024), 16, 0, 0);
+      }
+    }
+  };
+  auto nat_piece = [&](const uint8_t *st, int p, int j) {  // address of piece j of staged row p
+    return st + p * (MLA_KVA * 2) + (((j & ~7) | ((j ^ (p >> 1)) & 7)) << 4);
+  };
+
+  // byte offsets of this lane's A operands of the first product: row 16 pb + c16, piece 4 ks + g = 8 (ks / 2) + (4 (ks % 2) + g)
+  int s_off[2][2];
+#pragma unroll
+  for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+    for (int o = 0; o < 2; ++o) {
+      const int pr = pb * 16 + c16;
+      s_off[pb][o] = pr * (MLA_KVA * 2) + (((4 * o + g) ^ (pr >> 1)) & 7) * 16;
+    }
+  float M = -__builtin_inff(), Z = 0.0f;
+  kx_f32x4 O[16];
+#pragma unroll
+  for (int cb = 0; cb < 16; ++cb) O[cb] = kx_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+  copy_tile(0);
+  for (int t = 0; t < n_tiles; ++t) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of tile t has landed
+    __syncthreads();                                   // ... and everybody's; the previous tile is done with both buffers
+    if (t + 1 < n_tiles) copy_tile(t + 1);
+    const uint8_t *st = nat + (t & 1) * MM_NAT;
+    // transpose the latent columns 64 wave .. +63: lanes 0-31 take piece j, lanes 32-63 piece j+1, position = lane % 32
+    {
+      const int p = lane & 31;
+      const int kidx = ((p >> 2) & 3) * 8 + (p >> 4) * 4 + (p & 3);  // position 16 a + 4 g + v -> K index 8 g + 4 a + v
+      uint4 u[4];
+#pragma unroll
+      for (int it = 0; it < 4; ++it) u[it] = *(const uint4 *)nat_piece(st, p, wave * 8 + it * 2 + (lane >> 5));
+#pragma unroll
+      for (int it = 0; it < 4; ++it) {
+        const int j = wave * 8 + it * 2 + (lane >> 5);
+        uint8_t *d = ct + (j * 8) * MM_CT_PITCH + kidx * 2;
+        const uint32_t w[4] = {u[it].x, u[it].y, u[it].z, u[it].w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          *(uint16_t *)(d + (2 * e) * MM_CT_PITCH) = (uint16_t)(w[e] & 0xffffu);
+          *(uint16_t *)(d + (2 * e + 1) * MM_CT_PITCH) = (uint16_t)(w[e] >> 16);
+        }
+      }
+    }
+    // scores of positions 16 pb + 4 g + v for this lane's head (both column halves compute them)
+    kx_f32x4 sacc[2] = {kx_f32x4{0.0f, 0.0f, 0.0f, 0.0f}, kx_f32x4{0.0f, 0.0f, 0.0f, 0.0f}};
+#pragma unroll
+    for (int ks = 0; ks < 18; ++ks)
+#pragma unroll
+      for (int pb = 0; pb < 2; ++pb) {
+        const kx_bf16x8 av = *(const kx_bf16x8 *)(st + s_off[pb][ks & 1] + (ks >> 1) * 128);
+        sacc[pb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, qf[ks], sacc[pb], 0, 0, 0);
+      }
+    float sv[8];
+    float mt = -__builtin_inff();
+#pragma unroll
+    for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+      for (int v = 0; v < 4; v += 2) {
+        const int pos = pos0 + t * MM_T + pb * 16 + g * 4 + v;
+        const uint32_t r0 = mm_pack_bf16(sacc[pb][v], sacc[pb][v + 1]);                                       // bf(q.k)
+        const uint32_t r1 = mm_pack_bf16(kx_bits_f32(r0 << 16) * scale, kx_bits_f32(r0 & 0xffff0000u) * scale);  // bf(. * scale), :429
+        float s0 = kx_bits_f32(r1 << 16), s1 = kx_bits_f32(r1 & 0xffff0000u);
+        if (pos >= pos_end) s0 = -__builtin_inff();
+        if (pos + 1 >= pos_end) s1 = -__builtin_inff();
+        sv[pb * 4 + v] = s0;
+        sv[pb * 4 + v + 1] = s1;
+        mt = fmaxf(mt, fmaxf(s0, s1));
+      }
+    mt = fmaxf(mt, __shfl_xor(mt, 16));
+    mt = fmaxf(mt, __shfl_xor(mt, 32));
+    const float Mn = fmaxf(M, mt);
+    // exponentials through v_exp_f32: this path is held to a tolerance, not to the bits of kx_expf
+    const float alpha = __builtin_amdgcn_exp2f((M - Mn) * LOG2E);
+    float ps = 0.0f;
+    uint32_t pk[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float e0 = __builtin_amdgcn_exp2f((sv[2 * i] - Mn) * LOG2E), e1 = __builtin_amdgcn_exp2f((sv[2 * i + 1] - Mn) * LOG2E);
+      ps += e0 + e1;
+      pk[i] = mm_pack_bf16(e0, e1);
+    }
+    ps += __shfl_xor(ps, 16);
+    ps += __shfl_xor(ps, 32);
+    Z = __builtin_fmaf(Z, alpha, ps);
+    M = Mn;
+    const kx_bf16x8 pf = __builtin_bit_cast(kx_bf16x8, make_uint4(pk[0], pk[1], pk[2], pk[3]));
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {  // the running maximum of some head of the wave moved
+#pragma unroll
+      for (int cb = 0; cb < 16; ++cb) O[cb] *= alpha;
+    }
+    __syncthreads();  // the transposed tile is complete
+#pragma unroll
+    for (int cb = 0; cb < 16; ++cb) {
+      const kx_bf16x8 av = *(const kx_bf16x8 *)(ct + ((cw * 16 + cb) * 16 + c16) * MM_CT_PITCH + g * 16);
+      O[cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, pf, O[cb], 0, 0, 0);
+    }
+  }
+  // partials: lane = (head, columns 256 cw + 16 cb + 4 g .. +3)
+  const size_t idx = ((size_t)b * a.spans + span) * a.heads + head;
+  if (g == 0 && cw == 0) { a.pm[idx] = M; a.pz[idx] = Z; }
+#pragma unroll
+  for (int cb = 0; cb < 16; ++cb)
+    *(float4 *)(a.po + idx * MLA_R + (cw * 16 + cb) * 16 + g * 4) = make_float4(O[cb][0], O[cb][1], O[cb][2], O[cb][3]);
+}
+
 // merge of the spans; grid (heads, B), one wave, lane = 8 latent columns
 __global__ void __launch_bounds__(64) mla_combine_k(const float *__restrict__ pm, const float *__restrict__ pz,
                                                     const float *__restrict__ po, uint16_t *__restrict__ o_lat, int heads,
                                                     int spans) {
+  // M = max M_j; w_j = exp(M_j - M); Z = fma(Z_j, w_j, Z); O = fma(O_j, w_j, O) in span order; lane j holds span
+  // j's (M_j, Z_j, w_j) (at most 64 spans), the O_j rows are fetched four spans at a time
   constexpr int R = 512;
   const int h = blockIdx.x, b = blockIdx.y, lane = threadIdx.x;
-  float M = -__builtin_inff();
-  for (int j = 0; j < spans; ++j) M = fmaxf(M, pm[((size_t)b * spans + j) * heads + h]);
+  const size_t idx0 = (size_t)b * spans * heads + h;
+  const size_t my = idx0 + (size_t)min(lane, spans - 1) * heads;
+  const float mj = pm[my], zj = pz[my];
+  const float M = kxw::wave_max_f32(lane < spans ? mj : -__builtin_inff());
+  const float wj = kx_expf(mj - M);
   float Z = 0.0f, O[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-  for (int j = 0; j < spans; ++j) {
-    const size_t idx = ((size_t)b * spans + j) * heads + h;
-    const float w = kx_expf(pm[idx] - M);
-    Z = __builtin_fmaf(pz[idx], w, Z);
-    const float4 *o = (const float4 *)(po + idx * R + lane * 8);
-    const float4 o0 = o[0], o1 = o[1];
-    O[0] = __builtin_fmaf(o0.x, w, O[0]); O[1] = __builtin_fmaf(o0.y, w, O[1]);
-    O[2] = __builtin_fmaf(o0.z, w, O[2]); O[3] = __builtin_fmaf(o0.w, w, O[3]);
-    O[4] = __builtin_fmaf(o1.x, w, O[4]); O[5] = __builtin_fmaf(o1.y, w, O[5]);
-    O[6] = __builtin_fmaf(o1.z, w, O[6]); O[7] = __builtin_fmaf(o1.w, w, O[7]);
+  for (int j = 0; j < spans; ++j)
+    Z = __builtin_fmaf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, zj), j)),
+                       __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wj), j)), Z);
+  for (int j0 = 0; j0 < spans; j0 += 4) {
+    float4 o0[4], o1[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const float4 *o = (const float4 *)(po + (idx0 + (size_t)min(j0 + u, spans - 1) * heads) * R + lane * 8);
+      o0[u] = o[0];
+      o1[u] = o[1];
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (j0 + u < spans) {
+        const float w = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wj), j0 + u));
+        O[0] = __builtin_fmaf(o0[u].x, w, O[0]); O[1] = __builtin_fmaf(o0[u].y, w, O[1]);
+        O[2] = __builtin_fmaf(o0[u].z, w, O[2]); O[3] = __builtin_fmaf(o0[u].w, w, O[3]);
+        O[4] = __builtin_fmaf(o1[u].x, w, O[4]); O[5] = __builtin_fmaf(o1[u].y, w, O[5]);
+        O[6] = __builtin_fmaf(o1[u].z, w, O[6]); O[7] = __builtin_fmaf(o1[u].w, w, O[7]);
+      }
+    }
   }
   uint32_t r[4];
 #pragma unroll
@@ -407,6 +613,19 @@ int kx_mla_partials_launch(const kx_config *c, const uint16_t *cache, size_t seq
     KX_HIP(hipFuncSetAttribute((const void *)mla_partial_k<4>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
     KX_HIP(hipFuncSetAttribute((const void *)mla_partial_k<8>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
     attr_set = true;
+  }
+  const bool use_mfma = g_mla_kernel == 2 || (g_mla_kernel == 0 && seq >= 2048);
+  if (use_mfma) {
+    KX_REQUIRE(c->heads == 64, "kx_mla: the matrix-core kernel is built for 64 heads (got %d)", c->heads);
+    static bool mfma_attr = false;
+    if (!mfma_attr) {
+      KX_HIP(hipFuncSetAttribute((const void *)mla_partial_mfma_k, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * MM_NAT + MM_CT));
+      mfma_attr = true;
+    }
+    hipLaunchKernelGGL(mla_partial_mfma_k, dim3(a.spans, 1, batch), dim3(512), 2 * MM_NAT + MM_CT, st, a);
+    KX_LAUNCH_CHECK();
+    out->pm = a.pm; out->pz = a.pz; out->po = a.po; out->spans = a.spans;
+    return KX_OK;
   }
   if (hg == 1) hipLaunchKernelGGL(mla_partial_k<1>, g, b, lds, st, a);
   else if (hg == 2) hipLaunchKernelGGL(mla_partial_k<2>, g, b, lds, st, a);

@@ -72,6 +72,7 @@ _SIGS = {
     "kx_rope_table": [C.POINTER(KxConfig), _I, _I, _P],
     "kx_softmax_scale": [C.POINTER(KxConfig), C.POINTER(C.c_float), C.POINTER(C.c_float)],
     "kx_q_absorb": [C.POINTER(KxConfig), _P, _P, _P, _P, _I, _P],
+    "kx_mla_set_kernel": [_I],
     "kx_mla_workspace_bytes": [C.POINTER(KxConfig), _I, _I, C.POINTER(_SZ)],
     "kx_mla_decode": [C.POINTER(KxConfig), _P, _SZ, _P, _P, _P, _I, _I, _P],
     "kx_model_bytes": [C.POINTER(KxConfig), C.POINTER(C.c_uint64), C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)],

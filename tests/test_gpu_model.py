@@ -174,8 +174,12 @@ def test_mla_decode_operator(kxlib, ox, batch, seq):
     nbytes = C.c_size_t()
     check(kxlib.kx_mla_workspace_bytes(C.byref(cfg), batch, seq, C.byref(nbytes)))
     dc, dq, dw, do = dev(cache), dev(qabs), DevBuf(nbytes.value), DevBuf(batch * H * R * 2)
-    check(kxlib.kx_mla_decode(C.byref(cfg), dc.ptr, seq * KVA, dq.ptr, dw.ptr, do.ptr, batch, seq, None))
-    check(kxlib.kx_sync(None))
+    check(kxlib.kx_mla_set_kernel(1))   # the VALU kernel, whose summation order the oracle's mode 1 restates
+    try:
+        check(kxlib.kx_mla_decode(C.byref(cfg), dc.ptr, seq * KVA, dq.ptr, dw.ptr, do.ptr, batch, seq, None))
+        check(kxlib.kx_sync(None))
+    finally:
+        check(kxlib.kx_mla_set_kernel(0))
     got = do.to_numpy(np.uint16, (batch, H, R))
     exp1, exp0 = np.empty_like(got), np.empty_like(got)
     ox.ox_mla_decode(C.byref(cfg), ptr(cache), seq * KVA, ptr(qabs), ptr(exp1), batch, seq, 1)
@@ -184,6 +188,35 @@ def test_mla_decode_operator(kxlib, ox, batch, seq):
     assert O.max_rel(O.bf16_to_f32(got), O.bf16_to_f32(exp0)) < 1e-2
     if seq == 1:
         assert (got == cache[:, 0:1, :R]).all()   # one position: the latent itself
+
+
+@pytest.mark.parametrize("batch,seq", [(1, 1), (1, 31), (1, 100), (2, 700), (1, 4133), (1, 5000)])
+def test_mla_decode_matrix_core_kernel(kxlib, ox, batch, seq):
+    # the MFMA variant sums in another order: max-rel 1e-2 against both oracle schedules, and against the VALU kernel
+    say(f"mla decode (matrix cores) batch={batch} seq={seq}")
+    cfg = default_config()
+    H, KVA, R = cfg.heads, 576, 512
+    cache = O.normal_bf16(batch * seq * KVA, 5, 1, 1.0).reshape(batch, seq, KVA)
+    qabs = O.bf16_to_f32(O.normal_bf16(batch * H * KVA, 5, 2, 0.5)).reshape(batch, H, KVA)
+    nbytes = C.c_size_t()
+    check(kxlib.kx_mla_workspace_bytes(C.byref(cfg), batch, seq, C.byref(nbytes)))
+    dc, dq, dw, do = dev(cache), dev(qabs), DevBuf(nbytes.value), DevBuf(batch * H * R * 2)
+    outs = {}
+    try:
+        for mode in (2, 1):
+            check(kxlib.kx_mla_set_kernel(mode))
+            check(kxlib.kx_mla_decode(C.byref(cfg), dc.ptr, seq * KVA, dq.ptr, dw.ptr, do.ptr, batch, seq, None))
+            check(kxlib.kx_sync(None))
+            outs[mode] = O.bf16_to_f32(do.to_numpy(np.uint16, (batch, H, R)))
+    finally:
+        check(kxlib.kx_mla_set_kernel(0))
+    exp1, exp0 = np.empty((batch, H, R), dtype=np.uint16), np.empty((batch, H, R), dtype=np.uint16)
+    ox.ox_mla_decode(C.byref(cfg), ptr(cache), seq * KVA, ptr(qabs), ptr(exp1), batch, seq, 1)
+    ox.ox_mla_decode(C.byref(cfg), ptr(cache), seq * KVA, ptr(qabs), ptr(exp0), batch, seq, 0)
+    e_valu = O.max_rel(outs[2], outs[1])
+    e1, e0 = O.max_rel(outs[2], O.bf16_to_f32(exp1)), O.max_rel(outs[2], O.bf16_to_f32(exp0))
+    print(f"matrix-core MLA seq={seq}: max-rel {e_valu:.2e} vs VALU kernel, {e1:.2e} vs mode 1, {e0:.2e} vs mode 0", flush=True)
+    assert e_valu < 1e-2 and e1 < 1e-2 and e0 < 1e-2
 
 
 def test_executor_json_line(kxlib):
