@@ -371,7 +371,7 @@ void launch_tt(const I4Args &a, int tt, dim3 g, dim3 b, size_t lds, hipStream_t 
   // waves per SIMD the register budget is held to: two 7- or 8-wave workgroups per CU
   // for one token per pass, fewer when more activations live in registers
   if (tt == 1) hipLaunchKernelGGL((i4_gemv_k<DUAL, 1, KS_T, MAXT, 4>), g, b, lds, st, a);
-  else if (tt == 2) hipLaunchKernelGGL((i4_gemv_k<DUAL, 2, KS_T, MAXT, (MAXT > 512 ? 4 : 3)>), g, b, lds, st, a);
+  else if (tt == 2) hipLaunchKernelGGL((i4_gemv_k<DUAL, 2, KS_T, MAXT, 4>), g, b, lds, st, a);
   else hipLaunchKernelGGL((i4_gemv_k<DUAL, 4, KS_T, MAXT, (MAXT > 512 ? 4 : 2)>), g, b, lds, st, a);
 }
 
