@@ -69,8 +69,10 @@ int kx_bucket_launch(const uint16_t *ids, int tokens, int experts, int topk, int
                      int *pairs, int4 *work, int *n_active, hipStream_t st);
 
 // kx_prefill.hip
+// outputs of the grouped GEMM: bf16; fp32 unrounded; fp32 holding the bf16-rounded value; bf16 residual add into out
+enum { KX_GG_BF16 = 0, KX_GG_F32 = 1, KX_GG_F32_OF_BF16 = 2, KX_GG_RESID = 3 };
 int kx_grouped_gemm_launch(bool dual, bool i4, const void *w0, const uint16_t *s0, const void *w1, const uint16_t *s1,
-                           const uint16_t *x, void *out, bool out_f32, const int4 *work, const int *pairs, int n_pairs,
+                           const uint16_t *x, void *out, int out_mode, const int4 *work, const int *pairs, int n_pairs,
                            int n_slots, int N, int K, int x_div, size_t expert_w, size_t expert_s, int n_pairs_max,
                            hipStream_t st);
 int kx_moe_combine_launch(const uint16_t *eout, const float *rw, const uint16_t *sy, uint16_t *x, int tokens, int hidden,

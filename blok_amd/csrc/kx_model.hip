@@ -236,18 +236,28 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample) {
   const uint16_t *rope_row = m->rope_tab + (size_t)pos * c.qk_rope;
   const size_t seq_stride = (size_t)c.max_context * KVA;
   const bool fuse = B <= 4;  // RMSNorms ride in the prologue of the GEMV that consumes them
+  // From 16 sequences on, the dense projections run as GEMMs on the matrix cores (one group of B rows): the
+  // GEMV is bound by its fma count there.  Same values, another summation order (the bf16 rounding points stay).
+  const bool mm = B >= 16;
+  auto dense = [&](int epi, const KxGemvArgs &g) -> int {
+    if (!mm) return kx_gemv_launch(epi, g, st);
+    const bool dual = epi == KX_EPI_SWIGLU;
+    const int mode = epi == KX_EPI_RESID ? KX_GG_RESID : epi == KX_EPI_ARGMAX ? KX_GG_F32_OF_BF16 : epi == KX_EPI_F32 ? KX_GG_F32 : KX_GG_BF16;
+    return kx_grouped_gemm_launch(dual, false, g.w0, nullptr, dual ? g.w1 : nullptr, nullptr, g.x, g.out, mode, nullptr, nullptr,
+                                  g.tokens, 1, g.rows, g.cols, 1, 0, 0, g.tokens, st);
+  };
   for (int l = 0; l < c.n_layers; ++l) {
     Layer &L = m->layers[l];
     KxGemvArgs g = {};
     g.w0 = L.qkv_a; g.x = m->n; g.x_stride = H; g.out = m->qkv; g.out_stride = QKV; g.rows = QKV; g.cols = H; g.tokens = B;
     if (fuse) { g.x = m->x; g.norm_w = L.input_ln; g.norm_eps = c.rms_eps; }
     else KX_TRY(kx_rmsnorm_launch(m->x, L.input_ln, m->n, B, H, H, H, c.rms_eps, st));                 // :812
-    KX_TRY(kx_gemv_launch(KX_EPI_BF16, g, st));                                                         // :813, :816
+    KX_TRY(dense(KX_EPI_BF16, g));                                                                      // :813, :816
     g = {};
     g.w0 = L.qb; g.x = m->qa; g.x_stride = c.q_rank; g.out = m->q; g.out_stride = KD; g.rows = KD; g.cols = c.q_rank; g.tokens = B;
     if (fuse) { g.x = m->qkv; g.x_stride = QKV; g.norm_w = L.qa_ln; g.norm_eps = c.rms_eps; }
     else KX_TRY(kx_rmsnorm_launch(m->qkv, L.qa_ln, m->qa, B, c.q_rank, QKV, c.q_rank, c.rms_eps, st)); // :814
-    KX_TRY(kx_gemv_launch(KX_EPI_BF16, g, st));                                                         // :815
+    KX_TRY(dense(KX_EPI_BF16, g));                                                                      // :815
     // W_UK absorb + rope(q); the extra block norms kv_a, rotates the rope key, writes the cache row (:817-824)
     KX_TRY(kx_q_absorb_launch(m->q, L.kvb, rope_row, m->qabs, B, c.heads, c.qk_nope, c.qk_rope, c.v_head, c.kv_rank,
                               m->qkv + c.q_rank, QKV, L.kv_ln, L.cache, seq_stride, pos, c.rms_eps, st));
@@ -265,18 +275,18 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample) {
     KX_TRY(kx_gemv_launch(KX_EPI_BF16, g, st));
     g = {};
     g.w0 = L.o; g.x = m->att; g.x_stride = VD; g.out = m->x; g.out_stride = H; g.rows = H; g.cols = VD; g.tokens = B;
-    KX_TRY(kx_gemv_launch(KX_EPI_RESID, g, st));                                                        // :826-827
+    KX_TRY(dense(KX_EPI_RESID, g));                                                                     // :826-827
     if (l < c.first_dense) {                                                                            // bf16_mlp (:674-686)
       g = {};
       g.w0 = L.dgate; g.w1 = L.dup; g.x = m->n; g.x_stride = H; g.out = m->dmid; g.out_stride = c.dense_inter;
       g.rows = c.dense_inter; g.cols = H; g.tokens = B;
       if (fuse) { g.x = m->x; g.norm_w = L.post_ln; g.norm_eps = c.rms_eps; }
       else KX_TRY(kx_rmsnorm_launch(m->x, L.post_ln, m->n, B, H, H, H, c.rms_eps, st));                // :829
-      KX_TRY(kx_gemv_launch(KX_EPI_SWIGLU, g, st));
+      KX_TRY(dense(KX_EPI_SWIGLU, g));
       g = {};
       g.w0 = L.ddown; g.x = m->dmid; g.x_stride = c.dense_inter; g.out = m->x; g.out_stride = H; g.rows = H;
       g.cols = c.dense_inter; g.tokens = B;
-      KX_TRY(kx_gemv_launch(KX_EPI_RESID, g, st));                                                      // :684, :877
+      KX_TRY(dense(KX_EPI_RESID, g));                                                                   // :684, :877
     } else {
       if (!fuse) KX_TRY(kx_rmsnorm_launch(m->x, L.post_ln, m->n, B, H, H, H, c.rms_eps, st));          // :829
       KX_TRY(kx_moe_layer_launch(&c, &L.moe, m->moe_ws, m->n, m->x, B, 0, fuse ? L.post_ln : nullptr, st, false));  // :835-877
@@ -288,7 +298,7 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample) {
     g.tokens = B;
     if (fuse) { g.x = m->x; g.norm_w = m->final_norm; g.norm_eps = c.rms_eps; }
     else KX_TRY(kx_rmsnorm_launch(m->x, m->final_norm, m->n, B, H, H, H, c.rms_eps, st));
-    KX_TRY(kx_gemv_launch(KX_EPI_ARGMAX, g, st));
+    KX_TRY(dense(KX_EPI_ARGMAX, g));
     KX_TRY(kx_argmax_launch(m->logits, B, c.vocab, c.vocab, m->next, m->argmax_scratch, st));
   }
 #undef KX_TRY

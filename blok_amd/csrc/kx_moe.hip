@@ -233,7 +233,7 @@ extern "C" int kx_moe_prefill_layer(const kx_config *c, const kx_moe_weights *w,
     g.rows = E; g.cols = H; g.tokens = tokens;
     if ((rc = kx_gemv_launch(KX_EPI_F32, g, st))) return rc;
   } else {
-    if ((rc = kx_grouped_gemm_launch(false, false, w->d_router_gate, nullptr, nullptr, nullptr, n, ws->logits, true, nullptr,
+    if ((rc = kx_grouped_gemm_launch(false, false, w->d_router_gate, nullptr, nullptr, nullptr, n, ws->logits, KX_GG_F32, nullptr,
                                      nullptr, tokens, 1, E, H, 1, 0, 0, tokens, st))) return rc;
   }
   if ((rc = kx_router_topk_launch(ws->logits, (const float *)w->d_router_bias, ws->ids, ws->weights, tokens, E, K,
@@ -243,15 +243,15 @@ extern "C" int kx_moe_prefill_layer(const kx_config *c, const kx_moe_weights *w,
   const int n_slots = (long)tokens * K < E ? tokens * K : E;
   // routed experts: gate/up + SwiGLU, then down
   if ((rc = kx_grouped_gemm_launch(true, true, w->d_gate_packed, (const uint16_t *)w->d_gate_scale, w->d_up_packed,
-                                   (const uint16_t *)w->d_up_scale, n, ws->mid, false, ws->work, ws->pairs, 0, n_slots, I, H,
+                                   (const uint16_t *)w->d_up_scale, n, ws->mid, KX_GG_BF16, ws->work, ws->pairs, 0, n_slots, I, H,
                                    K, (size_t)I * (H / 8), (size_t)I * (H / 32), tokens, st))) return rc;
   if ((rc = kx_grouped_gemm_launch(false, true, w->d_down_packed, (const uint16_t *)w->d_down_scale, nullptr, nullptr,
-                                   ws->mid, ws->eout, false, ws->work, ws->pairs, 0, n_slots, H, I, 1, (size_t)H * (I / 8),
+                                   ws->mid, ws->eout, KX_GG_BF16, ws->work, ws->pairs, 0, n_slots, H, I, 1, (size_t)H * (I / 8),
                                    (size_t)H * (I / 32), tokens, st))) return rc;
   // shared expert: one group of all tokens, bf16 weights
-  if ((rc = kx_grouped_gemm_launch(true, false, w->d_shared_gate, nullptr, w->d_shared_up, nullptr, n, ws->smid, false,
+  if ((rc = kx_grouped_gemm_launch(true, false, w->d_shared_gate, nullptr, w->d_shared_up, nullptr, n, ws->smid, KX_GG_BF16,
                                    nullptr, nullptr, tokens, 1, SI, H, 1, 0, 0, tokens, st))) return rc;
-  if ((rc = kx_grouped_gemm_launch(false, false, w->d_shared_down, nullptr, nullptr, nullptr, ws->smid, ws->sy, false,
+  if ((rc = kx_grouped_gemm_launch(false, false, w->d_shared_down, nullptr, nullptr, nullptr, ws->smid, ws->sy, KX_GG_BF16,
                                    nullptr, nullptr, tokens, 1, H, SI, 1, 0, 0, tokens, st))) return rc;
   return kx_moe_combine_launch(ws->eout, ws->weights, ws->sy, (uint16_t *)d_x, tokens, H, K, flags, st);
 }

@@ -49,7 +49,6 @@ typedef _Float16 kx_h2 __attribute__((ext_vector_type(2)));
 
 constexpr int BN = 256, BK = 64;  // a token tile has up to 4 blocks of 32 tokens (PfArgs::nb_max)
 constexpr int LDS_STRIDE = BK + 8;  // bf16 elements per LDS row: 144 B keeps 16-byte reads of a column of rows spread over banks
-constexpr int PF_THREADS = 512;
 constexpr int W_STAGE = BN * 64;               // bytes of one matrix's packed words for two K steps
 constexpr int SC_STRIDE = 40;                  // bytes per (row, matrix) of staged scales: 16 bf16 + pad against bank conflicts
 
@@ -57,12 +56,12 @@ struct PfArgs {
   const void *w0, *w1;          // INT4: packed i32 [E][N][K/8]; BF16: bf16 [E][N][K]
   const uint16_t *s0, *s1;      // INT4: bf16 scales [E][N][K/32]
   const uint16_t *x;            // bf16 activation rows of K
-  void *out;                    // bf16 [pairs][N], or f32 when out_f32
+  void *out;                    // bf16 [pairs][N], or f32 (see out_mode)
   const int4 *work;             // {expert, first, last, _} per expert with work; nullptr: one group of n_pairs rows
   const int *pairs;             // pair ids sorted by expert; nullptr: identity
   int n_pairs, N, K, x_div;     // activation row = pair / x_div
   size_t expert_w, expert_s;    // elements between experts (words or bf16; scales)
-  int out_f32;                  // single matrix only: store the fp32 accumulators unrounded
+  int out_mode;                 // single matrix only: KX_GG_BF16, KX_GG_F32, KX_GG_F32_OF_BF16 or KX_GG_RESID
   int nb_max;                   // 32-token blocks per token tile (1..4): sizes the activation tiles in LDS
 };
 
@@ -90,8 +89,10 @@ __device__ __forceinline__ kx_bf16x8 dequant_word(uint32_t w, float sc, float sc
   return __builtin_bit_cast(kx_bf16x8, make_uint4(pf_pack(f0, f1), pf_pack(f2, f3), pf_pack(f4, f5), pf_pack(f6, f7)));
 }
 
-template <bool DUAL, bool I4>
-__global__ void __launch_bounds__(PF_THREADS, I4 ? 1 : 2) grouped_gemm_k(PfArgs a) {
+// WAVES waves per workgroup, 32 weight rows each (INT4: 8, the ring and the scale staging are laid out for 256 rows)
+template <bool DUAL, bool I4, int WAVES>
+__global__ void __launch_bounds__(WAVES * 64, (I4 || WAVES < 8) ? 1 : 2) grouped_gemm_k(PfArgs a) {
+  static_assert(!I4 || WAVES == 8, "the INT4 path is laid out for 8 waves");
   constexpr int MATS = DUAL ? 2 : 1;
   extern __shared__ __attribute__((aligned(16))) uint8_t pf_lds[];
   const int BM = a.nb_max * 32, XT = BM * LDS_STRIDE;   // tokens and elements of one activation tile
@@ -100,7 +101,7 @@ __global__ void __launch_bounds__(PF_THREADS, I4 ? 1 : 2) grouped_gemm_k(PfArgs 
   uint8_t *sc_lds = w_ring + 2 * MATS * W_STAGE;         // INT4: [2][256 rows * MATS][SC_STRIDE]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int lr = lane & 31, lh = lane >> 5;
-  const int n0 = blockIdx.x * BN;
+  const int n0 = blockIdx.x * (WAVES * 32);
   int4 wk = a.work ? a.work[blockIdx.y] : make_int4(0, 0, a.n_pairs, 0);
   const int e = __builtin_amdgcn_readfirstlane(wk.x);
   if (e < 0) return;
@@ -154,15 +155,22 @@ __global__ void __launch_bounds__(PF_THREADS, I4 ? 1 : 2) grouped_gemm_k(PfArgs 
       for (int i = 0; i < 4; ++i) d[i] = sc_regs[i];
     }
   };
-  // activation staging: thread -> row tid/4, 16 columns from (tid%4)*16
+  // activation staging: thread -> rows tid/4 + q * (16 WAVES), 16 columns from (tid%4)*16
+  constexpr int XROWS = WAVES * 16;  // rows staged per pass of the workgroup
   const int xr = tid >> 2, xc = (tid & 3) * 16;
 
   for (int m0 = p_begin + blockIdx.z * BM; m0 < p_end; m0 += gridDim.z * BM) {
     const int nb = min(a.nb_max, (p_end - m0 + 31) >> 5);  // 32-token blocks that hold tokens
-    const int pi = m0 + xr;
-    const bool x_valid = pi < p_end;
-    const int pair = x_valid ? (a.pairs ? a.pairs[pi] : pi) : 0;
-    const uint16_t *xrow = a.x + (size_t)(pair / a.x_div) * a.K + xc;
+    constexpr int XQMAX = (128 + XROWS - 1) / XROWS;
+    const uint16_t *xrow[XQMAX];
+    bool x_valid[XQMAX];
+#pragma unroll
+    for (int q = 0; q < XQMAX; ++q) {
+      const int pi = m0 + q * XROWS + xr;
+      x_valid[q] = pi < p_end && q * XROWS + xr < a.nb_max * 32;
+      const int pair = x_valid[q] ? (a.pairs ? a.pairs[pi] : pi) : 0;
+      xrow[q] = a.x + (size_t)(pair / a.x_div) * a.K + xc;
+    }
 
     // the tile with NB token blocks, NB a compile-time constant so that the K loop has no branches
     auto run = [&](auto nb_c) {
@@ -179,16 +187,25 @@ __global__ void __launch_bounds__(PF_THREADS, I4 ? 1 : 2) grouped_gemm_k(PfArgs 
         float sc[MATS];
         uint4 b[MATS][I4 ? 1 : 4];  // BF16: 32 columns
       };
-      uint4 xv[2];
+      constexpr int XQ = (NB * 32 + XROWS - 1) / XROWS;  // staging passes that hold rows of this tile
+      uint4 xv[XQ][2];
       auto load_x = [&](int ks) {
-        xv[0] = xv[1] = make_uint4(0, 0, 0, 0);
-        if (x_valid && xr < NB * 32) { xv[0] = *(const uint4 *)(xrow + ks * BK); xv[1] = *(const uint4 *)(xrow + ks * BK + 8); }
+#pragma unroll
+        for (int q = 0; q < XQ; ++q) {
+          xv[q][0] = xv[q][1] = make_uint4(0, 0, 0, 0);
+          if (x_valid[q] && q * XROWS + xr < NB * 32) {
+            xv[q][0] = *(const uint4 *)(xrow[q] + ks * BK);
+            xv[q][1] = *(const uint4 *)(xrow[q] + ks * BK + 8);
+          }
+        }
       };
       auto store_x = [&](uint16_t *st) {
-        if (xr < NB * 32) {
-          *(uint4 *)(st + xr * LDS_STRIDE + xc) = xv[0];
-          *(uint4 *)(st + xr * LDS_STRIDE + xc + 8) = xv[1];
-        }
+#pragma unroll
+        for (int q = 0; q < XQ; ++q)
+          if (q * XROWS + xr < NB * 32) {
+            *(uint4 *)(st + (q * XROWS + xr) * LDS_STRIDE + xc) = xv[q][0];
+            *(uint4 *)(st + (q * XROWS + xr) * LDS_STRIDE + xc + 8) = xv[q][1];
+          }
       };
       // this lane's weights of K step ks: INT4 from the LDS ring and the staged scales, bf16 from memory
       auto fetch_w = [&](WRaw &r, int ks) {
@@ -298,8 +315,16 @@ __global__ void __launch_bounds__(PF_THREADS, I4 ? 1 : 2) grouped_gemm_k(PfArgs 
               const int pr = a.pairs ? a.pairs[po] : po;
               float r = acc[0][t][v];
               if (DUAL) r = kx_swiglu(kx_bfround(r), kx_bfround(acc[1][t][v]));
-              if (!DUAL && a.out_f32) ((float *)a.out)[(size_t)pr * a.N + n] = r;
-              else ((uint16_t *)a.out)[(size_t)pr * a.N + n] = kx_bf16_rne(r);
+              if (DUAL || a.out_mode == KX_GG_BF16) {
+                ((uint16_t *)a.out)[(size_t)pr * a.N + n] = kx_bf16_rne(r);
+              } else if (a.out_mode == KX_GG_F32) {
+                ((float *)a.out)[(size_t)pr * a.N + n] = r;
+              } else if (a.out_mode == KX_GG_F32_OF_BF16) {
+                ((float *)a.out)[(size_t)pr * a.N + n] = kx_bfround(r);
+              } else {  // x = bf(x + bf(y))  (add_k, :248-251)
+                uint16_t *xo = (uint16_t *)a.out + (size_t)pr * a.N + n;
+                *xo = kx_bf16_rne(kx_bf16_f32(*xo) + kx_bfround(r));
+              }
             }
           }
       }
@@ -329,16 +354,16 @@ __global__ void __launch_bounds__(256) moe_combine_k(const uint16_t *__restrict_
 }  // namespace
 
 int kx_grouped_gemm_launch(bool dual, bool i4, const void *w0, const uint16_t *s0, const void *w1, const uint16_t *s1,
-                           const uint16_t *x, void *out, bool out_f32, const int4 *work, const int *pairs, int n_pairs,
+                           const uint16_t *x, void *out, int out_mode, const int4 *work, const int *pairs, int n_pairs,
                            int n_slots, int N, int K, int x_div, size_t expert_w, size_t expert_s, int n_pairs_max,
                            hipStream_t st) {
   KX_REQUIRE(K > 0 && K % 128 == 0 && (!i4 || K % 512 == 0), "kx_grouped_gemm: K=%d must be a positive multiple of %d", K, i4 ? 512 : 128);
   KX_REQUIRE(N > 0, "kx_grouped_gemm: N=%d must be positive", N);
-  KX_REQUIRE(!(dual && out_f32), "kx_grouped_gemm: fp32 output is for a single matrix");
+  KX_REQUIRE(out_mode >= KX_GG_BF16 && out_mode <= KX_GG_RESID && !(dual && out_mode != KX_GG_BF16), "kx_grouped_gemm: out_mode=%d", out_mode);
   PfArgs a;
   a.w0 = w0; a.w1 = w1; a.s0 = s0; a.s1 = s1; a.x = x; a.out = out; a.work = work; a.pairs = pairs;
   a.n_pairs = n_pairs; a.N = N; a.K = K; a.x_div = x_div; a.expert_w = expert_w; a.expert_s = expert_s;
-  a.out_f32 = out_f32 ? 1 : 0;
+  a.out_mode = out_mode;
   // token tile: 128 tokens for the INT4 kernels, whose dequant work per weight tile is amortised over the tokens;
   // 64 for the bf16 ones (more workgroups for the one-group GEMMs of the shared expert and the router)
   a.nb_max = i4 ? 4 : 2;
@@ -346,19 +371,25 @@ int kx_grouped_gemm_launch(bool dual, bool i4, const void *w0, const uint16_t *s
   const int max_rows = work ? n_pairs_max : n_pairs;
   int mz = kx_cdiv(max_rows, BM);
   mz = mz < 1 ? 1 : mz > 64 ? 64 : mz;
-  dim3 g(kx_cdiv(N, BN), work ? n_slots : 1, mz), b(PF_THREADS);
+  // waves per workgroup (32 weight rows each): 8 for INT4; for bf16 as few as it takes to get a couple of hundred
+  // workgroups (a decode batch is one token tile, so the N rows are the only source of parallelism there)
+  const long tiles = (long)mz * (work ? n_slots : 1);
+  const int waves = i4 ? 8 : (N / 256 * tiles >= 192 ? 8 : N / 64 * tiles >= 192 ? 2 : 1);
+  dim3 g(kx_cdiv(N, waves * 32), work ? n_slots : 1, mz), b(waves * 64);
   const int mats = dual ? 2 : 1;
   const size_t lds = (size_t)2 * BM * LDS_STRIDE * 2 + (i4 ? (size_t)2 * mats * W_STAGE + (size_t)2 * BN * mats * SC_STRIDE : 0);
   static bool attr_set = false;
   if (!attr_set) {  // more than 64 KB of dynamic LDS has to be allowed per kernel
-    KX_HIP(hipFuncSetAttribute((const void *)grouped_gemm_k<true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-    KX_HIP(hipFuncSetAttribute((const void *)grouped_gemm_k<false, true>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+    KX_HIP(hipFuncSetAttribute((const void *)grouped_gemm_k<true, true, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+    KX_HIP(hipFuncSetAttribute((const void *)grouped_gemm_k<false, true, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     attr_set = true;
   }
-  if (dual && i4) hipLaunchKernelGGL((grouped_gemm_k<true, true>), g, b, lds, st, a);
-  else if (dual) hipLaunchKernelGGL((grouped_gemm_k<true, false>), g, b, lds, st, a);
-  else if (i4) hipLaunchKernelGGL((grouped_gemm_k<false, true>), g, b, lds, st, a);
-  else hipLaunchKernelGGL((grouped_gemm_k<false, false>), g, b, lds, st, a);
+#define KX_GG(D, W) hipLaunchKernelGGL((grouped_gemm_k<D, false, W>), g, b, lds, st, a)
+  if (dual && i4) hipLaunchKernelGGL((grouped_gemm_k<true, true, 8>), g, b, lds, st, a);
+  else if (i4) hipLaunchKernelGGL((grouped_gemm_k<false, true, 8>), g, b, lds, st, a);
+  else if (dual) { if (waves == 8) KX_GG(true, 8); else if (waves == 2) KX_GG(true, 2); else KX_GG(true, 1); }
+  else { if (waves == 8) KX_GG(false, 8); else if (waves == 2) KX_GG(false, 2); else KX_GG(false, 1); }
+#undef KX_GG
   KX_LAUNCH_CHECK();
   return KX_OK;
 }
