@@ -50,11 +50,12 @@ int kx_argmax_launch(const float *logits, int tokens, int n, int stride, uint32_
 #define KX_ARGMAX_SCRATCH_FLOATS(tokens) ((size_t)(tokens) * 128)
 
 // kx_i4.hip
+// cnt_lo..cnt_hi: only the experts of the work list with that many pairs are processed (0, INT_MAX: all)
 int kx_i4_launch(bool dual, const uint32_t *packed0, const uint16_t *scale0, const uint32_t *packed1,
                  const uint16_t *scale1, const uint16_t *x, uint16_t *out, const int4 *work,
                  const int *pairs, int n_pairs, int rows,
-                 int cols, int x_div, size_t expert_words, size_t expert_scales, int tt, int grid,
-                 hipStream_t st);
+                 int cols, int x_div, size_t expert_words, size_t expert_scales, int tt, int n_slots,
+                 int cnt_lo, int cnt_hi, hipStream_t st);
 
 // kx_router.hip
 int kx_router_topk_launch(const float *logits, const float *bias, uint16_t *ids, float *weights, int tokens,

@@ -146,6 +146,7 @@ struct I4Args {
   int ks, rs;  // 1024-column slices, row sets; ks*rs waves per workgroup
   int nt;      // tiles per chunk
   size_t expert_words, expert_scales;
+  int cnt_lo, cnt_hi;  // only experts with cnt_lo <= pairs <= cnt_hi are processed by this launch
 };
 
 constexpr int I4_RI = 2;  // rows per half-wave per tile
@@ -161,7 +162,8 @@ constexpr int I4_RI = 2;  // rows per half-wave per tile
 // run past the matrix is moved back to end at the last row (the overlap is computed twice,
 // with identical results, and written once).
 // KS_T > 0 fixes ks (and rs, nt) at compile time; 0 reads them from the arguments.
-template <bool DUAL, int TT, int KS_T, int MAXT, int WPE>
+// FILTER: the launch processes only the experts whose pair count lies in [cnt_lo, cnt_hi]
+template <bool DUAL, int TT, int KS_T, int MAXT, int WPE, bool FILTER>
 __global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) i4_gemv_k(I4Args a) {
   extern __shared__ float lds[];
   constexpr int MATS = DUAL ? 2 : 1;
@@ -234,10 +236,23 @@ __global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(WPE, 
     }
   };
 
+  // the work of the first chunk at or after c (stride gridDim.x) whose expert this launch processes; e < 0: none
+  auto next_work = [&](int &c) {
+    Work w = load_work(c < n_chunks ? c : 0);
+    if (c >= n_chunks) w.e = -1;
+    if (FILTER) {
+      while (w.e >= 0 && (w.p_end - w.p_begin < a.cnt_lo || w.p_end - w.p_begin > a.cnt_hi)) {
+        c += gridDim.x;
+        if (c >= n_chunks) { w.e = -1; break; }
+        w = load_work(c);
+      }
+    }
+    return w;  // records with work come first: e < 0 ends the list
+  };
   int chunk = blockIdx.x;
   if (chunk >= n_chunks) return;
-  Work cur = load_work(chunk);
-  if (cur.e < 0) return;  // records with work come first
+  Work cur = next_work(chunk);
+  if (cur.e < 0) return;
   uint4 bufA[MATS][RI], bufB[MATS][RI];
   uint4 xraw[TT][4];
   int sb = 0;
@@ -247,11 +262,11 @@ __global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(WPE, 
   bool fresh = true;  // the scales of `cur` have not been made visible to the workgroup yet
 
   while (true) {
-    const int nchunk = chunk + gridDim.x;
+    int nchunk = chunk + gridDim.x;
     bool more = nchunk < n_chunks;
     Work nxt = cur;
     if (more) {
-      nxt = load_work(nchunk);
+      nxt = next_work(nchunk);
       more = nxt.e >= 0;
     }
     // the other scale buffer was last read in the chunk before this one; every wave is past that chunk's barriers
@@ -369,10 +384,16 @@ int plan(int cols, int rows, int mats, int tt, I4Launch &pl) {
 template <bool DUAL, int KS_T, int MAXT>
 void launch_tt(const I4Args &a, int tt, dim3 g, dim3 b, size_t lds, hipStream_t st) {
   // waves per SIMD the register budget is held to: two 7- or 8-wave workgroups per CU
-  // for one token per pass, fewer when more activations live in registers
-  if (tt == 1) hipLaunchKernelGGL((i4_gemv_k<DUAL, 1, KS_T, MAXT, 4>), g, b, lds, st, a);
-  else if (tt == 2) hipLaunchKernelGGL((i4_gemv_k<DUAL, 2, KS_T, MAXT, 4>), g, b, lds, st, a);
-  else hipLaunchKernelGGL((i4_gemv_k<DUAL, 4, KS_T, MAXT, (MAXT > 512 ? 4 : 2)>), g, b, lds, st, a);
+  // for one or two tokens per pass, fewer when four tokens' activations live in registers
+  const bool filter = a.cnt_lo > 0 || a.cnt_hi != 0x7fffffff;
+  if (tt == 1) {
+    if (filter) hipLaunchKernelGGL((i4_gemv_k<DUAL, 1, KS_T, MAXT, 4, true>), g, b, lds, st, a);
+    else hipLaunchKernelGGL((i4_gemv_k<DUAL, 1, KS_T, MAXT, 4, false>), g, b, lds, st, a);
+  } else if (tt == 2) {
+    hipLaunchKernelGGL((i4_gemv_k<DUAL, 2, KS_T, MAXT, 4, true>), g, b, lds, st, a);
+  } else {
+    hipLaunchKernelGGL((i4_gemv_k<DUAL, 4, KS_T, MAXT, (MAXT > 512 ? 4 : 2), true>), g, b, lds, st, a);
+  }
 }
 
 }  // namespace
@@ -382,7 +403,7 @@ void launch_tt(const I4Args &a, int tt, dim3 g, dim3 b, size_t lds, hipStream_t 
 int kx_i4_launch(bool dual, const uint32_t *packed0, const uint16_t *scale0, const uint32_t *packed1,
                  const uint16_t *scale1, const uint16_t *x, uint16_t *out, const int4 *work,
                  const int *pairs, int n_pairs, int rows, int cols, int x_div, size_t expert_words,
-                 size_t expert_scales, int tt, int n_slots, hipStream_t st) {
+                 size_t expert_scales, int tt, int n_slots, int cnt_lo, int cnt_hi, hipStream_t st) {
   I4Launch pl;
   int rc = plan(cols, rows, dual ? 2 : 1, tt, pl);
   if (rc) return rc;
@@ -391,8 +412,9 @@ int kx_i4_launch(bool dual, const uint32_t *packed0, const uint16_t *scale0, con
   a.x = x; a.out = out; a.work = work; a.pairs = pairs; a.n_pairs = n_pairs; a.n_slots = n_slots;
   a.rows = rows; a.cols = cols; a.x_div = x_div; a.ks = pl.ks; a.rs = pl.rs; a.nt = pl.nt;
   a.expert_words = expert_words; a.expert_scales = expert_scales;
+  a.cnt_lo = cnt_lo; a.cnt_hi = cnt_hi;
   long chunks = (long)n_slots * kx_cdiv(rows, pl.cr);
-  dim3 g((unsigned)(chunks < 4096 ? chunks : 4096)), b(pl.threads);
+  dim3 g((unsigned)(chunks < 32768 ? chunks : 32768)), b(pl.threads);
   const bool full = pl.rs == (pl.ks >= 5 ? 1 : 8 / pl.ks) && pl.nt == (dual ? 32 : 64) / (pl.rs * 4);
   if (full && pl.ks == 7) {        // Kimi-K2 gate/up: K = 7168
     if (dual) launch_tt<true, 7, 448>(a, tt, g, b, pl.lds, st);
@@ -438,6 +460,6 @@ extern "C" int kx_i4_gemv(const void *d_packed, const void *d_scale, const void 
   KX_REQUIRE(tokens > 0, "kx_i4_gemv: tokens=%d must be positive", tokens);
   int tt = tokens >= 4 ? 4 : tokens >= 2 ? 2 : 1;
   return kx_i4_launch(false, (const uint32_t *)d_packed, (const uint16_t *)d_scale, nullptr, nullptr,
-                      (const uint16_t *)d_x, (uint16_t *)d_y, nullptr, nullptr, tokens, rows, cols, 1, 0, 0, tt, 1,
+                      (const uint16_t *)d_x, (uint16_t *)d_y, nullptr, nullptr, tokens, rows, cols, 1, 0, 0, tt, 1, 0, 0x7fffffff,
                       kx_stream(stream));
 }

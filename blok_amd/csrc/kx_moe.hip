@@ -103,13 +103,45 @@ extern "C" int kx_moe_workspace_views(kx_moe_workspace *ws, void **d_logits, voi
   return KX_OK;
 }
 
-// tokens per pass of the routed kernels: with T tokens and topk of E experts the
-// expected tokens per active expert stays near 1 until T*topk approaches E.
-static int routed_tt(int tokens, int topk, int experts) {
-  long pairs = (long)tokens * topk;
-  if (pairs <= experts) return 1;
-  if (pairs <= 4L * experts) return 2;
-  return 4;
+// How the routed kernels go over the experts.  Every pass over an expert streams its weights again, so an expert
+// with n pairs wants n tokens per pass; more tokens per pass cost registers and speed.  Up to T*topk = E pairs one
+// launch with one token per pass is fastest (measured: splitting pays from about 48 tokens on); beyond that the
+// experts with one pair take the one-token kernel and the others a second launch with 2 (or 4) tokens per pass.
+struct RoutedPlan {
+  int n, tt[2], lo[2], hi[2];
+};
+static RoutedPlan routed_plan(int tokens, int topk, int experts) {
+  const long pairs = (long)tokens * topk;
+  RoutedPlan p;
+  if (pairs <= experts) {
+    p.n = 1; p.tt[0] = 1; p.lo[0] = 0; p.hi[0] = 0x7fffffff;
+  } else {
+    p.n = 2;
+    p.tt[0] = 1; p.lo[0] = 1; p.hi[0] = 1;
+    p.tt[1] = pairs <= 4L * experts ? 2 : 4; p.lo[1] = 2; p.hi[1] = 0x7fffffff;
+  }
+  return p;
+}
+
+// the routed gate/up (which = 0) or down (which = 1) kernel(s) over the work list in the workspace
+static int routed_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_workspace *ws, const uint16_t *n, int tokens,
+                         int which, hipStream_t st) {
+  const int H = c->hidden, I = c->moe_inter, E = c->experts, K = c->topk;
+  const int max_active = (long)tokens * K < E ? tokens * K : E;
+  const RoutedPlan p = routed_plan(tokens, K, E);
+  for (int i = 0; i < p.n; ++i) {
+    int rc;
+    if (which == 0)
+      rc = kx_i4_launch(true, (const uint32_t *)w->d_gate_packed, (const uint16_t *)w->d_gate_scale,
+                        (const uint32_t *)w->d_up_packed, (const uint16_t *)w->d_up_scale, n, ws->mid, ws->work, ws->pairs, 0, I,
+                        H, K, (size_t)I * (H / 8), (size_t)I * (H / 32), p.tt[i], max_active, p.lo[i], p.hi[i], st);
+    else
+      rc = kx_i4_launch(false, (const uint32_t *)w->d_down_packed, (const uint16_t *)w->d_down_scale, nullptr, nullptr,
+                        ws->mid, ws->eout, ws->work, ws->pairs, 0, H, I, 1, (size_t)H * (I / 8), (size_t)H * (I / 32),
+                        p.tt[i], max_active, p.lo[i], p.hi[i], st);
+    if (rc) return rc;
+  }
+  return KX_OK;
 }
 
 int kx_moe_layer_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_workspace *ws, void *d_n, void *d_x,
@@ -121,7 +153,7 @@ int kx_moe_layer_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_work
   KX_REQUIRE(c->hidden == ws->cfg.hidden && c->moe_inter == ws->cfg.moe_inter && c->experts == ws->cfg.experts &&
                  c->topk == ws->cfg.topk && c->shared_inter == ws->cfg.shared_inter,
              "kx_moe_decode_layer: workspace was created for another shape");
-  const int H = c->hidden, I = c->moe_inter, E = c->experts, K = c->topk;
+  const int H = c->hidden, E = c->experts, K = c->topk;
   const uint16_t *n = (const uint16_t *)d_n;
   if (timed) KX_HIP(hipEventRecord(ws->ev[0], st));
   // router logits, top-k, bucketing; shared gate/up + SwiGLU.  Up to 4 tokens: one launch for all of it.
@@ -146,17 +178,10 @@ int kx_moe_layer_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_work
   }
   if (timed) KX_HIP(hipEventRecord(ws->ev[1], st));
   // routed gate/up + SwiGLU
-  const int tt = routed_tt(tokens, K, E);
-  const int max_active = (long)tokens * K < E ? tokens * K : E;
-  if ((rc = kx_i4_launch(true, (const uint32_t *)w->d_gate_packed, (const uint16_t *)w->d_gate_scale,
-                         (const uint32_t *)w->d_up_packed, (const uint16_t *)w->d_up_scale, n, ws->mid, ws->work,
-                         ws->pairs, 0, I, H, K, (size_t)I * (H / 8), (size_t)I * (H / 32),
-                         tt, max_active, st))) return rc;
+  if ((rc = routed_launch(c, w, ws, n, tokens, 0, st))) return rc;
   if (timed) KX_HIP(hipEventRecord(ws->ev[2], st));
   // routed down
-  if ((rc = kx_i4_launch(false, (const uint32_t *)w->d_down_packed, (const uint16_t *)w->d_down_scale, nullptr, nullptr,
-                         ws->mid, ws->eout, ws->work, ws->pairs, 0, H, I, 1,
-                         (size_t)H * (I / 8), (size_t)H * (I / 32), tt, max_active, st))) return rc;
+  if ((rc = routed_launch(c, w, ws, n, tokens, 1, st))) return rc;
   if (timed) KX_HIP(hipEventRecord(ws->ev[3], st));
   // shared gate/up + SwiGLU when it did not ride with the router
   if (!paired) {
@@ -199,17 +224,7 @@ extern "C" int kx_moe_routed_only(const kx_config *c, const kx_moe_weights *w, k
   KX_REQUIRE(w && ws && d_n, "kx_moe_routed_only: null argument");
   KX_REQUIRE(tokens > 0 && tokens <= ws->max_tokens, "kx_moe_routed_only: tokens=%d outside [1, %d]", tokens, ws->max_tokens);
   KX_REQUIRE(which == 0 || which == 1, "kx_moe_routed_only: which=%d", which);
-  const int H = c->hidden, I = c->moe_inter, E = c->experts, K = c->topk;
-  const int tt = routed_tt(tokens, K, E);
-  const int max_active = (long)tokens * K < E ? tokens * K : E;
-  if (which == 0)
-    return kx_i4_launch(true, (const uint32_t *)w->d_gate_packed, (const uint16_t *)w->d_gate_scale,
-                        (const uint32_t *)w->d_up_packed, (const uint16_t *)w->d_up_scale, (const uint16_t *)d_n, ws->mid,
-                        ws->work, ws->pairs, 0, I, H, K, (size_t)I * (H / 8), (size_t)I * (H / 32), tt, max_active,
-                        kx_stream(stream));
-  return kx_i4_launch(false, (const uint32_t *)w->d_down_packed, (const uint16_t *)w->d_down_scale, nullptr, nullptr,
-                      ws->mid, ws->eout, ws->work, ws->pairs, 0, H, I, 1, (size_t)H * (I / 8), (size_t)H * (I / 32), tt,
-                      max_active, kx_stream(stream));
+  return routed_launch(c, w, ws, (const uint16_t *)d_n, tokens, which, kx_stream(stream));
 }
 
 // ---- prefill chunk through one MoE layer: grouped GEMMs on the matrix cores ------------------
