@@ -459,13 +459,26 @@ __global__ void __launch_bounds__(512, 1) mla_partial_mfma_k(MlaArgs a) {
     }
     // scores of positions 16 pb + 4 g + v for this lane's head (both column halves compute them)
     kx_f32x4 sacc[2] = {kx_f32x4{0.0f, 0.0f, 0.0f, 0.0f}, kx_f32x4{0.0f, 0.0f, 0.0f, 0.0f}};
+    {
+      // the A operands are read three K steps ahead of the MFMAs that consume them
+      constexpr int AH = 3;
+      kx_bf16x8 av[AH + 1][2];
 #pragma unroll
-    for (int ks = 0; ks < 18; ++ks)
+      for (int ks = 0; ks < AH; ++ks)
 #pragma unroll
-      for (int pb = 0; pb < 2; ++pb) {
-        const kx_bf16x8 av = *(const kx_bf16x8 *)(st + s_off[pb][ks & 1] + (ks >> 1) * 128);
-        sacc[pb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, qf[ks], sacc[pb], 0, 0, 0);
+        for (int pb = 0; pb < 2; ++pb) av[ks][pb] = *(const kx_bf16x8 *)(st + s_off[pb][ks & 1] + (ks >> 1) * 128);
+#pragma unroll
+      for (int ks = 0; ks < 18; ++ks) {
+        if (ks + AH < 18) {
+#pragma unroll
+          for (int pb = 0; pb < 2; ++pb)
+            av[(ks + AH) % (AH + 1)][pb] = *(const kx_bf16x8 *)(st + s_off[pb][(ks + AH) & 1] + ((ks + AH) >> 1) * 128);
+        }
+#pragma unroll
+        for (int pb = 0; pb < 2; ++pb)
+          sacc[pb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[ks % (AH + 1)][pb], qf[ks], sacc[pb], 0, 0, 0);
       }
+    }
     float sv[8];
     float mt = -__builtin_inff();
 #pragma unroll
@@ -501,14 +514,22 @@ __global__ void __launch_bounds__(512, 1) mla_partial_mfma_k(MlaArgs a) {
     M = Mn;
     const kx_bf16x8 pf = __builtin_bit_cast(kx_bf16x8, make_uint4(pk[0], pk[1], pk[2], pk[3]));
     if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {  // the running maximum of some head of the wave moved
+      asm volatile("" ::: "memory");                         // keep this a branch: it is rarely taken after the first tiles
 #pragma unroll
       for (int cb = 0; cb < 16; ++cb) O[cb] *= alpha;
     }
     __syncthreads();  // the transposed tile is complete
+    {
+      constexpr int AH = 4;  // operands read four column blocks ahead
+      kx_bf16x8 av[AH + 1];
+      const uint8_t *cbase = ct + (cw * 256 + c16) * MM_CT_PITCH + g * 16;
 #pragma unroll
-    for (int cb = 0; cb < 16; ++cb) {
-      const kx_bf16x8 av = *(const kx_bf16x8 *)(ct + ((cw * 16 + cb) * 16 + c16) * MM_CT_PITCH + g * 16);
-      O[cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, pf, O[cb], 0, 0, 0);
+      for (int cb = 0; cb < AH; ++cb) av[cb] = *(const kx_bf16x8 *)(cbase + cb * 16 * MM_CT_PITCH);
+#pragma unroll
+      for (int cb = 0; cb < 16; ++cb) {
+        if (cb + AH < 16) av[(cb + AH) % (AH + 1)] = *(const kx_bf16x8 *)(cbase + (cb + AH) * 16 * MM_CT_PITCH);
+        O[cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[cb % (AH + 1)], pf, O[cb], 0, 0, 0);
+      }
     }
   }
   // partials: lane = (head, columns 256 cw + 16 cb + 4 g .. +3)
