@@ -13,8 +13,10 @@
 //   o_lat[h] = softmax(s)[t] . c_t ;  o[h] = bf(W_UV[h] o_lat[h])   (rows h*256+128 ..)
 // One pass over the cache with an online softmax; the sequence is cut into spans
 // of span_tiles 64-position tiles that run in parallel and are merged afterwards.
+// Two kernels compute the span partials: mla_partial_k (fp32 VALU, the fixed summation
+// order below) and, for long contexts, mla_partial_mfma_k on the matrix cores.
 //
-// Summation order (fixed; span_tiles depends on the sequence length only):
+// Summation order of the VALU path (fixed; span_tiles depends on the sequence length only):
 //   score      one fma chain over the 576 cache columns, ascending
 //   tile       m = max s; p = exp(s - M'); z = xor-butterfly(64) of p;
 //              running: M' = max(M, m), a = exp(M - M'), Z = fma(Z, a, z),

@@ -8,11 +8,15 @@
 // cache and the scratch of a step for `max_batch` sequences; a step enqueues
 // kernels on one stream and never waits for the host.
 //
-// Per layer (T = batch tokens, all at the same position):
-//   rmsnorm -> [q_a ; kv_a] GEMV -> q_a norm, kv_a norm, rope(k), cache write
-//   -> q_b GEMV -> W_UK absorb + rope(q) -> attention over the latent cache
-//   -> W_UV GEMV per head -> o_proj GEMV with the residual add
-//   rmsnorm -> dense SwiGLU MLP (layers < first_dense) or the routed MoE layer.
+// Per layer (T = batch tokens, all at the same position; up to 4 tokens the RMSNorms run in the
+// prologue of the GEMV that consumes them):
+//   [q_a ; kv_a] GEMV (input norm) -> q_b GEMV (q_a norm) -> W_UK absorb + rope(q), with one
+//   workgroup that norms kv_a, rotates the rope key and writes the cache row -> attention
+//   partials over the latent cache -> W_UV GEMV per head (merges the partials as it loads
+//   them) -> o_proj GEMV with the residual add
+//   -> dense SwiGLU MLP (layers < first_dense) or the routed MoE layer (post-attention norm
+//   in their first GEMV).
+// From 16 sequences on the dense projections run as GEMMs on the matrix cores.
 #include <math.h>
 #include <string.h>
 #include <vector>

@@ -4,15 +4,17 @@
 // matvec (fp32 logits), sigmoid + bias + top-8, a blocking copy of the 8 ids to
 // the host, then per slot 32+112 tile launches each preceded by NVMe reads,
 // expert_accum_k per tile, round_bf16_k, the shared expert through bf16_mlp and
-// the residual add.  Here: six launches, no host round trip.
-//   1 router logits  (bf16 GEMV, fp32 out)
-//   2 sigmoid/bias/top-k
-//   3 bucketing (pairs sorted by expert, list of active experts)
-//   4 routed gate+up INT4 GEMV with the SwiGLU epilogue   -> mid  [T*topk, moe_inter]
-//   5 routed down INT4 GEMV                               -> eout [T*topk, hidden]
-//   6 shared gate+up bf16 GEMV with SwiGLU                -> smid [T, shared_inter]
-//   7 shared down bf16 GEMV; epilogue combines the topk routed outputs in slot
+// the residual add.  Here, no host round trip, and for up to 4 tokens four launches:
+//   1 shared gate+up bf16 GEMV with SwiGLU (-> smid [T, shared_inter]) and the router's logits
+//     GEMV in one launch; the router workgroup that finishes last does sigmoid/bias/top-k and
+//     the bucketing (pairs sorted by expert, list of active experts)
+//   2 routed gate+up INT4 GEMV with the SwiGLU epilogue   -> mid  [T*topk, moe_inter]
+//   3 routed down INT4 GEMV                               -> eout [T*topk, hidden]
+//   4 shared down bf16 GEMV; epilogue combines the topk routed outputs in slot
 //     order, adds the shared output and the residual.
+// More tokens: router GEMV, top-k + bucketing, and the shared gate+up GEMV are launches of
+// their own; beyond T*topk = E pairs the routed kernels run as two launches each (experts
+// with one pair, experts with more).
 #include "kx_common.h"
 #include "kx_dense.h"
 
