@@ -343,23 +343,27 @@ __global__ void __launch_bounds__(256) mla_partial_k(MlaArgs a) {
 // q_abs and p = bf(exp(s - m)) are bf16-representable and the cache is bf16, so q.c and p.c are exact
 // products summed in fp32: v_mfma_f32_16x16x32_bf16 computes what mla_partial_k computes with another
 // summation order (held to the 1e-2 bar, not bit-exact; the token-identity runs use mla_partial_k).
-// Workgroup = (sequence, span), 8 waves; wave (hw, cw) owns heads 16 hw .. +15 and, in the second product,
-// latent columns 256 cw .. +255 (both column halves compute the scores of their heads); 32-position tiles.
-//  * the 32 cache rows of tile t+1 are copied global -> LDS (no registers) while tile t is computed;
-//    rows sit at their natural pitch of 1152 B with the 16-byte pieces xor-swizzled by the row, so the
-//    row-per-lane operand reads are free of bank conflicts;
-//  * scores: S^T[pos, head] = C[pos, 576] Q^T[576, head], A operand = cache rows from LDS, B operand =
-//    this lane's head of q in registers (18 K steps of 32);
-//  * the lane that owns head h in the result holds, per K step of the second product, exactly the 8
-//    probabilities a B operand lane needs if MFMA K index 8 g + 4 a + v stands for position
-//    16 a + 4 g + v of the tile -- so p never leaves the registers;
-//  * O^T[col, head] += C^T[col, pos] P^T[pos, head]: the A operand needs 8 positions of one column, so
-//    the 512 latent columns of the tile are transposed once per tile into a second LDS buffer, in that
-//    K index order (LDS -> LDS, lanes = positions, conflict-free both ways).
+// Workgroup = (sequence, span), 8 waves, 32-position tiles; the two products split the work differently and
+// hand p, the running-maximum factor and the row sums over through LDS:
+//  * scores: wave (hw, pb) computes heads 16 hw .. +15 against positions 16 pb .. +15 of the tile,
+//    S^T[pos, head] = C[pos, 576] Q^T[576, head] with v_mfma_f32_16x16x32_bf16 (A = cache rows from LDS, B = the
+//    lane's head of q in registers, 18 K steps); the two waves of a head group exchange their maxima, then each
+//    writes p = bf(exp(s - m)) of its 16 positions in the K order of the second product;
+//  * O^T[col, head] += C^T[col, pos] P^T[pos, head]: wave (hb, cq) owns heads 32 hb .. +31 and latent columns
+//    128 cq .. +127 (v_mfma_f32_32x32x16_bf16, two K steps per tile).  The A operand needs 8 positions of one
+//    column, so the 512 latent columns of the tile are transposed once per tile into a second LDS buffer
+//    (LDS -> LDS, lanes = positions, conflict-free both ways), position 16 a + 4 g + v at K index 8 g + 4 a + v --
+//    the order in which the score accumulators hold the positions, so p is stored without any shuffle;
+//  * the 32 cache rows of tile t+2 are copied global -> LDS (no registers) while tile t is computed; rows sit at
+//    their natural pitch of 1152 B with the 16-byte pieces xor-swizzled by the row, so the row-per-lane operand
+//    reads are free of bank conflicts.
 constexpr int MM_T = 32;                      // positions per tile
 constexpr int MM_NAT = MM_T * MLA_KVA * 2;    // bytes of one staged tile
 constexpr int MM_CT_PITCH = 80;               // bytes per transposed column: 32 positions + pad
 constexpr int MM_CT = MLA_R * MM_CT_PITCH;
+constexpr int MM_P_PITCH = 80;                // bytes per head of the staged probabilities: 32 K indices + pad
+constexpr int MM_XCH = 64 * MM_P_PITCH + 5 * 64 * 4;  // p, two maxima, two row sums and the rescale factor per head
+typedef float kx_f32x16v __attribute__((ext_vector_type(16)));
 typedef __bf16 kx_bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 kx_bf16x2v __attribute__((ext_vector_type(2)));
 typedef float kx_f32x2v __attribute__((ext_vector_type(2)));
@@ -372,14 +376,23 @@ __device__ __forceinline__ uint32_t mm_pack_bf16(float lo, float hi) {
 
 __global__ void __launch_bounds__(512, 1) mla_partial_mfma_k(MlaArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t mm_lds[];
-  uint8_t *nat = mm_lds;               // [2][32 rows][72 pieces of 16 B]
-  uint8_t *ct = mm_lds + 2 * MM_NAT;   // [512 columns][MM_CT_PITCH]
+  uint8_t *nat = mm_lds;                       // [3][32 rows][72 pieces of 16 B]
+  uint8_t *ct = mm_lds + 3 * MM_NAT;           // [512 columns][MM_CT_PITCH]
+  uint8_t *p_lds = ct + MM_CT;                 // [64 heads][MM_P_PITCH]: bf16 p at K index order
+  float *mx_lds = (float *)(p_lds + 64 * MM_P_PITCH);  // [2][64] tile maxima of the two position halves
+  float *ps_lds = mx_lds + 128;                // [2][64] row sums of the two position halves
+  float *al_lds = ps_lds + 128;                // [64] exp(M_old - M_new)
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int hw = wave & 3, cw = wave >> 2;  // heads 16 hw .. +15, latent columns 256 cw .. +255 of the second product
-  const int c16 = lane & 15, g = lane >> 4;
   const int span = blockIdx.x, b = blockIdx.z;
+  // role in the score product
+  const int hw = wave & 3, pb = wave >> 2;
+  const int c16 = lane & 15, g = lane >> 4;
   const int head = hw * 16 + c16;
+  // role in the PV product
+  const int hb = wave & 1, cq = wave >> 1;
+  const int l32 = lane & 31, half = lane >> 5;
+  const int head2 = hb * 32 + l32;
   const uint16_t *cache = a.cache + (size_t)b * a.seq_stride;
   const int pos0 = span * a.span_tiles * 64, pos_end = min(a.seq, (span + 1) * a.span_tiles * 64);
   const int n_tiles = (pos_end - pos0 + MM_T - 1) / MM_T;
@@ -412,34 +425,54 @@ __global__ void __launch_bounds__(512, 1) mla_partial_mfma_k(MlaArgs a) {
         const int j = (js & ~7) | ((js ^ (p >> 1)) & 7);
         const int row = min(pos0 + t * MM_T + p, a.seq - 1);
         __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)(cache + (size_t)row * MLA_KVA + j * 8),
-                                         (void __attribute__((address_space(3))) *)(nat + (t & 1) * MM_NAT + ii * 1024), 16, 0, 0);
+                                         (void __attribute__((address_space(3))) *)(nat + (t % 3) * MM_NAT + ii * 1024), 16, 0, 0);
       }
     }
   };
   auto nat_piece = [&](const uint8_t *st, int p, int j) {  // address of piece j of staged row p
     return st + p * (MLA_KVA * 2) + (((j & ~7) | ((j ^ (p >> 1)) & 7)) << 4);
   };
+  // byte offsets of this lane's A operands of the score product: row 16 pb + c16, piece 4 ks + g = 8 (ks / 2) + (4 (ks % 2) + g)
+  int s_off[2];
+#pragma unroll
+  for (int o = 0; o < 2; ++o) {
+    const int pr = pb * 16 + c16;
+    s_off[o] = pr * (MLA_KVA * 2) + (((4 * o + g) ^ (pr >> 1)) & 7) * 16;
+  }
+  float M = -__builtin_inff(), Z = 0.0f;  // of `head`; the two waves of a head group keep identical copies
+  kx_f32x16v O[4];                        // heads 32 hb .. +31 x columns 128 cq + 32 cbk .. +31
+#pragma unroll
+  for (int cbk = 0; cbk < 4; ++cbk)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) O[cbk][i] = 0.0f;
 
-  // byte offsets of this lane's A operands of the first product: row 16 pb + c16, piece 4 ks + g = 8 (ks / 2) + (4 (ks % 2) + g)
-  int s_off[2][2];
-#pragma unroll
-  for (int pb = 0; pb < 2; ++pb)
-#pragma unroll
-    for (int o = 0; o < 2; ++o) {
-      const int pr = pb * 16 + c16;
-      s_off[pb][o] = pr * (MLA_KVA * 2) + (((4 * o + g) ^ (pr >> 1)) & 7) * 16;
-    }
-  float M = -__builtin_inff(), Z = 0.0f;
-  kx_f32x4 O[16];
-#pragma unroll
-  for (int cb = 0; cb < 16; ++cb) O[cb] = kx_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-
+  // tiles are copied two ahead into a ring of three buffers; loads complete in order, so waiting until only the
+  // copies of the newest tile (5 instructions for waves 0-3, 4 for the others) are outstanding means tile t has landed
   copy_tile(0);
+  if (n_tiles > 1) copy_tile(1);
   for (int t = 0; t < n_tiles; ++t) {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of tile t has landed
-    __syncthreads();                                   // ... and everybody's; the previous tile is done with both buffers
-    if (t + 1 < n_tiles) copy_tile(t + 1);
-    const uint8_t *st = nat + (t & 1) * MM_NAT;
+    if (t + 1 < n_tiles) {
+      if (wave < 4) asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    __syncthreads();  // everybody's share of tile t has landed; the previous tile is done with every buffer
+    if (t + 2 < n_tiles) copy_tile(t + 2);
+    const uint8_t *st = nat + (t % 3) * MM_NAT;
+    // scores of positions 16 pb + 4 g + v for this lane's head
+    kx_f32x4 sacc = kx_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    {
+      constexpr int AH = 4;  // operands are read four K steps ahead of the MFMAs that consume them
+      kx_bf16x8 av[AH + 1];
+#pragma unroll
+      for (int ks = 0; ks < AH; ++ks) av[ks] = *(const kx_bf16x8 *)(st + s_off[ks & 1] + (ks >> 1) * 128);
+#pragma unroll
+      for (int ks = 0; ks < 18; ++ks) {
+        if (ks + AH < 18) av[(ks + AH) % (AH + 1)] = *(const kx_bf16x8 *)(st + s_off[(ks + AH) & 1] + ((ks + AH) >> 1) * 128);
+        sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[ks % (AH + 1)], qf[ks], sacc, 0, 0, 0);
+      }
+    }
     // transpose the latent columns 64 wave .. +63: lanes 0-31 take piece j, lanes 32-63 piece j+1, position = lane % 32
     {
       const int p = lane & 31;
@@ -459,87 +492,79 @@ __global__ void __launch_bounds__(512, 1) mla_partial_mfma_k(MlaArgs a) {
         }
       }
     }
-    // scores of positions 16 pb + 4 g + v for this lane's head (both column halves compute them)
-    kx_f32x4 sacc[2] = {kx_f32x4{0.0f, 0.0f, 0.0f, 0.0f}, kx_f32x4{0.0f, 0.0f, 0.0f, 0.0f}};
-    {
-      // the A operands are read three K steps ahead of the MFMAs that consume them
-      constexpr int AH = 3;
-      kx_bf16x8 av[AH + 1][2];
+    float sv[4];
+    float mloc = -__builtin_inff();
 #pragma unroll
-      for (int ks = 0; ks < AH; ++ks)
-#pragma unroll
-        for (int pb = 0; pb < 2; ++pb) av[ks][pb] = *(const kx_bf16x8 *)(st + s_off[pb][ks & 1] + (ks >> 1) * 128);
-#pragma unroll
-      for (int ks = 0; ks < 18; ++ks) {
-        if (ks + AH < 18) {
-#pragma unroll
-          for (int pb = 0; pb < 2; ++pb)
-            av[(ks + AH) % (AH + 1)][pb] = *(const kx_bf16x8 *)(st + s_off[pb][(ks + AH) & 1] + ((ks + AH) >> 1) * 128);
-        }
-#pragma unroll
-        for (int pb = 0; pb < 2; ++pb)
-          sacc[pb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[ks % (AH + 1)][pb], qf[ks], sacc[pb], 0, 0, 0);
-      }
+    for (int v = 0; v < 4; v += 2) {
+      const int pos = pos0 + t * MM_T + pb * 16 + g * 4 + v;
+      const uint32_t r0 = mm_pack_bf16(sacc[v], sacc[v + 1]);                                                  // bf(q.k)
+      const uint32_t r1 = mm_pack_bf16(kx_bits_f32(r0 << 16) * scale, kx_bits_f32(r0 & 0xffff0000u) * scale);  // bf(. * scale), :429
+      float s0 = kx_bits_f32(r1 << 16), s1 = kx_bits_f32(r1 & 0xffff0000u);
+      if (pos >= pos_end) s0 = -__builtin_inff();
+      if (pos + 1 >= pos_end) s1 = -__builtin_inff();
+      sv[v] = s0;
+      sv[v + 1] = s1;
+      mloc = fmaxf(mloc, fmaxf(s0, s1));
     }
-    float sv[8];
-    float mt = -__builtin_inff();
-#pragma unroll
-    for (int pb = 0; pb < 2; ++pb)
-#pragma unroll
-      for (int v = 0; v < 4; v += 2) {
-        const int pos = pos0 + t * MM_T + pb * 16 + g * 4 + v;
-        const uint32_t r0 = mm_pack_bf16(sacc[pb][v], sacc[pb][v + 1]);                                       // bf(q.k)
-        const uint32_t r1 = mm_pack_bf16(kx_bits_f32(r0 << 16) * scale, kx_bits_f32(r0 & 0xffff0000u) * scale);  // bf(. * scale), :429
-        float s0 = kx_bits_f32(r1 << 16), s1 = kx_bits_f32(r1 & 0xffff0000u);
-        if (pos >= pos_end) s0 = -__builtin_inff();
-        if (pos + 1 >= pos_end) s1 = -__builtin_inff();
-        sv[pb * 4 + v] = s0;
-        sv[pb * 4 + v + 1] = s1;
-        mt = fmaxf(mt, fmaxf(s0, s1));
-      }
-    mt = fmaxf(mt, __shfl_xor(mt, 16));
-    mt = fmaxf(mt, __shfl_xor(mt, 32));
-    const float Mn = fmaxf(M, mt);
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 16));
+    mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
+    if (g == 0) mx_lds[pb * 64 + head] = mloc;
+    __syncthreads();  // the maxima of both position halves and the transposed tile are complete
+    const float Mn = fmaxf(M, fmaxf(mloc, mx_lds[(pb ^ 1) * 64 + head]));
     // exponentials through v_exp_f32: this path is held to a tolerance, not to the bits of kx_expf
     const float alpha = __builtin_amdgcn_exp2f((M - Mn) * LOG2E);
-    float ps = 0.0f;
-    uint32_t pk[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const float e0 = __builtin_amdgcn_exp2f((sv[2 * i] - Mn) * LOG2E), e1 = __builtin_amdgcn_exp2f((sv[2 * i + 1] - Mn) * LOG2E);
-      ps += e0 + e1;
-      pk[i] = mm_pack_bf16(e0, e1);
-    }
+    const float e0 = __builtin_amdgcn_exp2f((sv[0] - Mn) * LOG2E), e1 = __builtin_amdgcn_exp2f((sv[1] - Mn) * LOG2E);
+    const float e2 = __builtin_amdgcn_exp2f((sv[2] - Mn) * LOG2E), e3 = __builtin_amdgcn_exp2f((sv[3] - Mn) * LOG2E);
+    float ps = (e0 + e1) + (e2 + e3);
     ps += __shfl_xor(ps, 16);
     ps += __shfl_xor(ps, 32);
-    Z = __builtin_fmaf(Z, alpha, ps);
-    M = Mn;
-    const kx_bf16x8 pf = __builtin_bit_cast(kx_bf16x8, make_uint4(pk[0], pk[1], pk[2], pk[3]));
-    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {  // the running maximum of some head of the wave moved
-      asm volatile("" ::: "memory");                         // keep this a branch: it is rarely taken after the first tiles
-#pragma unroll
-      for (int cb = 0; cb < 16; ++cb) O[cb] *= alpha;
+    // positions 16 pb + 4 g + v sit at K indices 8 g + 4 pb + v
+    *(uint2 *)(p_lds + head * MM_P_PITCH + (8 * g + 4 * pb) * 2) = make_uint2(mm_pack_bf16(e0, e1), mm_pack_bf16(e2, e3));
+    if (g == 0) {
+      ps_lds[pb * 64 + head] = ps;
+      if (pb == 0) al_lds[head] = alpha;
     }
-    __syncthreads();  // the transposed tile is complete
+    M = Mn;
+    __syncthreads();  // p, row sums and rescale factors are complete
+    Z = __builtin_fmaf(Z, alpha, ps_lds[head] + ps_lds[64 + head]);
+    // second product, for heads 32 hb .. +31 and columns 128 cq .. +127
+    const float alpha2 = al_lds[head2];
+    if (__builtin_amdgcn_ballot_w64(alpha2 != 1.0f) != 0) {  // the running maximum of some head of the wave moved
+      asm volatile("" ::: "memory");                          // keep this a branch: it is rarely taken after the first tiles
+#pragma unroll
+      for (int cbk = 0; cbk < 4; ++cbk) O[cbk] *= alpha2;
+    }
     {
-      constexpr int AH = 4;  // operands read four column blocks ahead
-      kx_bf16x8 av[AH + 1];
-      const uint8_t *cbase = ct + (cw * 256 + c16) * MM_CT_PITCH + g * 16;
+      const kx_bf16x8 pf0 = *(const kx_bf16x8 *)(p_lds + head2 * MM_P_PITCH + half * 16);
+      const kx_bf16x8 pf1 = *(const kx_bf16x8 *)(p_lds + head2 * MM_P_PITCH + 32 + half * 16);
+      const uint8_t *cbase = ct + (cq * 128 + l32) * MM_CT_PITCH + half * 16;
+      kx_bf16x8 av[4][2];
 #pragma unroll
-      for (int cb = 0; cb < AH; ++cb) av[cb] = *(const kx_bf16x8 *)(cbase + cb * 16 * MM_CT_PITCH);
+      for (int cbk = 0; cbk < 4; ++cbk) {
+        av[cbk][0] = *(const kx_bf16x8 *)(cbase + cbk * 32 * MM_CT_PITCH);
+        av[cbk][1] = *(const kx_bf16x8 *)(cbase + cbk * 32 * MM_CT_PITCH + 32);
+      }
 #pragma unroll
-      for (int cb = 0; cb < 16; ++cb) {
-        if (cb + AH < 16) av[(cb + AH) % (AH + 1)] = *(const kx_bf16x8 *)(cbase + (cb + AH) * 16 * MM_CT_PITCH);
-        O[cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[cb % (AH + 1)], pf, O[cb], 0, 0, 0);
+      for (int cbk = 0; cbk < 4; ++cbk) {
+        O[cbk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[cbk][0], pf0, O[cbk], 0, 0, 0);
+        O[cbk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[cbk][1], pf1, O[cbk], 0, 0, 0);
       }
     }
   }
-  // partials: lane = (head, columns 256 cw + 16 cb + 4 g .. +3)
-  const size_t idx = ((size_t)b * a.spans + span) * a.heads + head;
-  if (g == 0 && cw == 0) { a.pm[idx] = M; a.pz[idx] = Z; }
+  // partials.  Maxima and sums: the score lanes of the first position half; O: lane = (head, column
+  // 128 cq + 32 cbk + 8 q + 4 half + c) for accumulator register 4 q + c
+  if (pb == 0 && g == 0) {
+    const size_t idx = ((size_t)b * a.spans + span) * a.heads + head;
+    a.pm[idx] = M;
+    a.pz[idx] = Z;
+  }
+  const size_t idx2 = ((size_t)b * a.spans + span) * a.heads + head2;
 #pragma unroll
-  for (int cb = 0; cb < 16; ++cb)
-    *(float4 *)(a.po + idx * MLA_R + (cw * 16 + cb) * 16 + g * 4) = make_float4(O[cb][0], O[cb][1], O[cb][2], O[cb][3]);
+  for (int cbk = 0; cbk < 4; ++cbk)
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      *(float4 *)(a.po + idx2 * MLA_R + cq * 128 + cbk * 32 + q * 8 + half * 4) =
+          make_float4(O[cbk][4 * q], O[cbk][4 * q + 1], O[cbk][4 * q + 2], O[cbk][4 * q + 3]);
 }
 
 // merge of the spans; grid (heads, B), one wave, lane = 8 latent columns
@@ -642,10 +667,10 @@ int kx_mla_partials_launch(const kx_config *c, const uint16_t *cache, size_t seq
     KX_REQUIRE(c->heads == 64, "kx_mla: the matrix-core kernel is built for 64 heads (got %d)", c->heads);
     static bool mfma_attr = false;
     if (!mfma_attr) {
-      KX_HIP(hipFuncSetAttribute((const void *)mla_partial_mfma_k, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * MM_NAT + MM_CT));
+      KX_HIP(hipFuncSetAttribute((const void *)mla_partial_mfma_k, hipFuncAttributeMaxDynamicSharedMemorySize, 3 * MM_NAT + MM_CT + MM_XCH));
       mfma_attr = true;
     }
-    hipLaunchKernelGGL(mla_partial_mfma_k, dim3(a.spans, 1, batch), dim3(512), 2 * MM_NAT + MM_CT, st, a);
+    hipLaunchKernelGGL(mla_partial_mfma_k, dim3(a.spans, 1, batch), dim3(512), 3 * MM_NAT + MM_CT + MM_XCH, st, a);
     KX_LAUNCH_CHECK();
     out->pm = a.pm; out->pz = a.pz; out->po = a.po; out->spans = a.spans;
     return KX_OK;
