@@ -151,6 +151,10 @@ struct I4Args {
 
 constexpr int I4_RI = 2;  // rows per half-wave per tile
 
+// Rows of a chunk for tiles of rt rows: 32 for the fused gate/up kernel; for one matrix 112 when rt divides it
+// (7168 rows / 112 = 64 chunks per expert: 8 experts fill the 512 resident workgroups exactly once), else 64.
+__host__ __device__ constexpr int i4_chunk_rows(bool dual, int rt) { return dual ? 32 : (112 % rt == 0 ? 112 : 64); }
+
 // A workgroup of ks*rs waves takes chunks of nt tiles of RT = rs*4 rows of one expert.
 // Wave (s, rset): slice s of rows rset*4 .. rset*4+3 of each tile; its half-waves take
 // alternate rows.  Per chunk: the group scales of all its rows are copied into LDS (global ->
@@ -173,7 +177,7 @@ __global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(WPE, 
   const int ks = KS_T ? KS_T : a.ks;
   const int rs = KS_T ? (KS_T >= 5 ? 1 : 8 / KS_T) : a.rs;
   const int RT = rs * 2 * RI;
-  const int nt = KS_T ? (DUAL ? 32 : 64) / (KS_T >= 5 ? 4 : 32 / KS_T) : a.nt;
+  const int nt = KS_T ? i4_chunk_rows(DUAL, KS_T >= 5 ? 4 : 32 / KS_T) / (KS_T >= 5 ? 4 : 32 / KS_T) : a.nt;
   const int CR = RT * nt;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int l = lane & 31, h = lane >> 5;
@@ -370,7 +374,7 @@ int plan(int cols, int rows, int mats, int tt, I4Launch &pl) {
   pl.threads = pl.ks * pl.rs * 64;
   const int rt = pl.rs * 2 * I4_RI;
   // chunk: 32 rows of both matrices (gate/up) or 64 rows of one
-  int nt = (mats == 2 ? 32 : 64) / rt;
+  int nt = i4_chunk_rows(mats == 2, rt) / rt;
   nt = nt < 1 ? 1 : nt;
   while (nt > 1 && rt * nt > rows) --nt;
   pl.nt = nt;
@@ -415,7 +419,7 @@ int kx_i4_launch(bool dual, const uint32_t *packed0, const uint16_t *scale0, con
   a.cnt_lo = cnt_lo; a.cnt_hi = cnt_hi;
   long chunks = (long)n_slots * kx_cdiv(rows, pl.cr);
   dim3 g((unsigned)(chunks < 32768 ? chunks : 32768)), b(pl.threads);
-  const bool full = pl.rs == (pl.ks >= 5 ? 1 : 8 / pl.ks) && pl.nt == (dual ? 32 : 64) / (pl.rs * 4);
+  const bool full = pl.rs == (pl.ks >= 5 ? 1 : 8 / pl.ks) && pl.nt == i4_chunk_rows(dual, pl.rs * 4) / (pl.rs * 4);
   if (full && pl.ks == 7) {        // Kimi-K2 gate/up: K = 7168
     if (dual) launch_tt<true, 7, 448>(a, tt, g, b, pl.lds, st);
     else launch_tt<false, 7, 448>(a, tt, g, b, pl.lds, st);
