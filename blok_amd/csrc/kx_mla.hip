@@ -662,7 +662,8 @@ int kx_mla_partials_launch(const kx_config *c, const uint16_t *cache, size_t seq
     KX_HIP(hipFuncSetAttribute((const void *)mla_partial_k<8>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
     attr_set = true;
   }
-  const bool use_mfma = g_mla_kernel == 2 || (g_mla_kernel == 0 && seq >= 2048);
+  // automatic choice: the matrix-core kernel from 2048 positions on, where it is built for the shape (64 heads)
+  const bool use_mfma = g_mla_kernel == 2 || (g_mla_kernel == 0 && seq >= 2048 && c->heads == 64);
   if (use_mfma) {
     KX_REQUIRE(c->heads == 64, "kx_mla: the matrix-core kernel is built for 64 heads (got %d)", c->heads);
     static bool mfma_attr = false;
