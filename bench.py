@@ -492,12 +492,85 @@ def run_copy(args):
           flush=True)
 
 
+def run_load(args):
+    """kx_model_load on a Kimi-K2-shaped checkpoint of --stack-layers layers whose shards are sparse files
+    (headers written, data holes): what the reader threads, staging buffers and host-to-device copies sustain
+    when the disk is not the limit.  Not a disk benchmark."""
+    import struct
+    import tempfile
+    from blok_amd import model_index
+    from blok_amd.lib import check, default_config, kx
+    lib = kx()
+    cfg = default_config()
+    cfg.n_layers = args.stack_layers if args.stack_layers != 24 else 2
+    cfg.max_batch, cfg.max_context = 1, 64
+    H, V, E, I, SI, D = cfg.hidden, cfg.vocab, cfg.experts, cfg.moe_inter, cfg.shared_inter, cfg.dense_inter
+    KD, VD = cfg.heads * (cfg.qk_nope + cfg.qk_rope), cfg.heads * cfg.v_head
+    KVA, KVB = cfg.kv_rank + cfg.qk_rope, cfg.heads * (cfg.qk_nope + cfg.v_head)
+    lm = "language_model."
+    shards = [[(lm + "model.embed_tokens.weight", "BF16", (V, H)), (lm + "model.norm.weight", "BF16", (H,)),
+               (lm + "lm_head.weight", "BF16", (V, H))]]
+    for l in range(cfg.n_layers):
+        p, t = f"{lm}model.layers.{l}.", []
+        for n, shp in (("input_layernorm", (H,)), ("post_attention_layernorm", (H,)), ("self_attn.q_a_proj", (cfg.q_rank, H)),
+                       ("self_attn.q_a_layernorm", (cfg.q_rank,)), ("self_attn.q_b_proj", (KD, cfg.q_rank)),
+                       ("self_attn.kv_a_proj_with_mqa", (KVA, H)), ("self_attn.kv_a_layernorm", (cfg.kv_rank,)),
+                       ("self_attn.kv_b_proj", (KVB, cfg.kv_rank)), ("self_attn.o_proj", (H, VD))):
+            t.append((p + n + ".weight", "BF16", shp))
+        if l < cfg.first_dense:
+            t += [(p + "mlp.gate_proj.weight", "BF16", (D, H)), (p + "mlp.up_proj.weight", "BF16", (D, H)),
+                  (p + "mlp.down_proj.weight", "BF16", (H, D))]
+        else:
+            t += [(p + "mlp.gate.weight", "BF16", (E, H)), (p + "mlp.gate.e_score_correction_bias", "BF16", (E,))]
+            for n, shp in (("gate_proj", (SI, H)), ("up_proj", (SI, H)), ("down_proj", (H, SI))):
+                t.append((p + f"mlp.shared_experts.{n}.weight", "BF16", shp))
+            for e in range(E):
+                for n, (r, c) in (("gate_proj", (I, H)), ("up_proj", (I, H)), ("down_proj", (H, I))):
+                    t.append((p + f"mlp.experts.{e}.{n}.weight_packed", "I32", (r, c // 8)))
+                    t.append((p + f"mlp.experts.{e}.{n}.weight_scale", "BF16", (r, c // 32)))
+        shards.append(t)
+    root = tempfile.mkdtemp(prefix="kx_load_", dir=args.load_dir)
+    try:
+        for i, tensors in enumerate(shards):
+            header, at = {}, 0
+            for name, dtype, shape in tensors:
+                n = int(np.prod(shape)) * (2 if dtype == "BF16" else 4)
+                header[name] = {"dtype": dtype, "shape": list(shape), "data_offsets": [at, at + n]}
+                at += n
+            body = json.dumps(header, separators=(",", ":")).encode()
+            with open(os.path.join(root, f"model-{i + 1:05d}-of-{len(shards):06d}.safetensors"), "wb") as f:
+                f.write(struct.pack("<Q", len(body)))
+                f.write(body)
+                f.truncate(8 + len(body) + at)
+        report = model_index.materialize(root, os.path.join(root, "meta"))
+        times = []
+        for _ in range(max(1, min(args.steps, 3))):
+            h = C.c_void_p()
+            check(lib.kx_model_load(C.byref(cfg), report["index"].encode(), C.byref(h)))
+            nbytes, secs = C.c_uint64(), C.c_double()
+            check(lib.kx_model_load_info(h, C.byref(nbytes), C.byref(secs)))
+            check(lib.kx_model_destroy(h))
+            times.append(secs.value)
+    finally:
+        import shutil
+        shutil.rmtree(root, ignore_errors=True)
+    best = min(times)
+    print(json.dumps({"metric": "checkpoint load GB/s (sparse shards, no disk reads)", "value": round(nbytes.value / best / 1e9, 2),
+                      "unit": "GB/s", "n_gpus": 1, "steps": len(times), "warmup": 0, "ms_per_step": round(best * 1e3, 1),
+                      "higher_is_better": True, "data": "synthetic",
+                      "config": {"workload": f"kx_model_load, Kimi-K2 shapes, {cfg.n_layers} layers, {report['tensors']} tensors, "
+                                             f"{nbytes.value / 1e9:.2f} GB", "threads": int(os.environ.get("KX_LOAD_THREADS", "8")),
+                                 "direct": os.environ.get("KX_LOAD_DIRECT", "1") != "0", "seconds_each": [round(t, 3) for t in times]}}),
+          flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--workload", default="stack", choices=["stack", "moe_layer", "prefill", "mla", "copy"])
+    ap.add_argument("--workload", default="stack", choices=["stack", "moe_layer", "prefill", "mla", "copy", "load"])
+    ap.add_argument("--load-dir", default=None, help="where the load workload writes its sparse shards (default: the temp dir)")
     ap.add_argument("--context", type=int, default=32768)
     ap.add_argument("--copy-mib", type=int, default=1024)
     ap.add_argument("--batch", type=int, default=1)
@@ -517,6 +590,9 @@ def main():
     build_if_missing()
     if args.workload == "copy":
         run_copy(args)
+        return
+    if args.workload == "load":
+        run_load(args)
         return
     if args.workload == "mla":
         run_mla(args)

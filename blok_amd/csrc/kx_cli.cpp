@@ -5,8 +5,10 @@
 //   --index <file> --prompt-tokens <id,id,...> --tokens <n>
 // reads one JSON line {"status":"ok","token_ids":[...]} from stdout and treats a
 // non-zero exit code as failure, surfacing stderr.  The same contract holds
-// here.  --index is accepted and ignored (weights are seeded random-init, there
-// is no checkpoint); --layers / --seed / --ignore-eos are additions.
+// here.  With --index the weights are read from the checkpoint the index describes
+// (runtime_index() + validate_forward_contract(), :559-585, :736-778): the stack's shapes are taken
+// from the index and --layers truncates it (the full 61 layers do not fit one GPU's HBM).  Without
+// --index the weights are seeded random-init.  --layers / --seed / --topk / --ignore-eos are additions.
 #include <errno.h>
 #include <stdint.h>
 #include <stdio.h>
@@ -30,22 +32,25 @@ static uint64_t u64(const char *s, const char *what) {  // :504-510
 
 int main(int argc, char **argv) {
   std::string prompt_tokens, index;
-  uint64_t tokens = 0, layers = 24, seed = 0;
+  uint64_t tokens = 0, layers = 0, seed = 0, topk = 0;
   int ignore_eos = 0;
   for (int i = 1; i < argc; i += 2) {
     std::string f = argv[i];
     if (f == "--ignore-eos") { ignore_eos = 1; --i; continue; }
-    if (i + 1 >= argc) die("usage: kx-kimi-exec [--index runtime-index.blok] --prompt-tokens ids --tokens n [--layers n] [--seed n] [--ignore-eos]");
+    if (i + 1 >= argc) die("usage: kx-kimi-exec [--index runtime-index.blok] --prompt-tokens ids --tokens n [--layers n] [--seed n] [--topk n] [--ignore-eos]");
     if (f == "--index") index = argv[i + 1];
     else if (f == "--prompt-tokens") prompt_tokens = argv[i + 1];
     else if (f == "--tokens") tokens = u64(argv[i + 1], "tokens");
     else if (f == "--layers") layers = u64(argv[i + 1], "layers");
     else if (f == "--seed") seed = u64(argv[i + 1], "seed");
+    else if (f == "--topk") topk = u64(argv[i + 1], "topk");
     else die("unknown flag: " + f);  // :540
   }
   if (prompt_tokens.empty() || tokens == 0) die("bad args");  // :542
   kx_config cfg;
   if (kx_config_default(&cfg)) die(kx_last_error());
+  if (topk) cfg.topk = (int32_t)topk;
+  if (!index.empty() && kx_index_infer_config(index.c_str(), &cfg)) die(kx_last_error());
   std::vector<uint32_t> ids;  // token_ids(), :546-557
   size_t at = 0;
   while (at <= prompt_tokens.size()) {
@@ -58,7 +63,9 @@ int main(int argc, char **argv) {
     at = comma + 1;
   }
   if (ids.empty()) die("prompt token list is empty");
-  if (layers == 0 || layers > 61) die("bad layers");
+  if (layers > 61) die("bad layers");
+  if (layers == 0) layers = index.empty() || cfg.n_layers > 24 ? 24 : (uint64_t)cfg.n_layers;  // 24 Kimi-K2 layers fill one GPU
+  if (!index.empty() && layers > (uint64_t)cfg.n_layers) die("the checkpoint has fewer layers than --layers");
   const uint64_t max_context = 262144;  // :180
   if (tokens > max_context || ids.size() > max_context - tokens) die("requested sequence exceeds Kimi context");  // :784
   cfg.n_layers = (int32_t)layers;
@@ -66,7 +73,7 @@ int main(int argc, char **argv) {
   cfg.max_batch = 1;
   cfg.max_context = (int32_t)(ids.size() + tokens);
   kx_model *m = nullptr;
-  if (kx_model_create(&cfg, &m)) die(kx_last_error());
+  if (index.empty() ? kx_model_create(&cfg, &m) : kx_model_load(&cfg, index.c_str(), &m)) die(kx_last_error());
   std::vector<uint32_t> out(tokens);
   int32_t count = 0;
   if (kx_generate(m, ids.data(), 1, (int32_t)ids.size(), (int32_t)tokens, ignore_eos, out.data(), &count)) {

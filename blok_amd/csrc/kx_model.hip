@@ -4,7 +4,8 @@
 // reference allocates 19 single-token fp32 scratch buffers (:792-799), streams
 // every weight tile from NVMe inside the layer loop and synchronises with the
 // host once per MoE layer (:844) and twice per vocabulary tile (:728-730).
-// Here one arena in HBM holds the seeded random-init weights, the latent KV
+// Here one arena in HBM holds the weights (seeded random-init, kx_model_create, or
+// copied in from the checkpoint a runtime-index.blok describes, kx_model_load), the latent KV
 // cache and the scratch of a step for `max_batch` sequences; a step enqueues
 // kernels on one stream and never waits for the host.
 //
@@ -22,6 +23,8 @@
 #include <vector>
 #include "kx_common.h"
 #include "kx_dense.h"
+#include "kx_index.h"
+#include "kx_load.h"
 #include "kx_mla.h"
 
 namespace {
@@ -70,6 +73,8 @@ struct kx_model {
   int batch = 0, pos = 0;
   bool sampled = false;
   float ms_prefill = 0, ms_decode = 0;
+  uint64_t load_bytes = 0;  // checkpoint bytes copied in by kx_model_load, and the time that took
+  double load_seconds = 0;
 };
 
 namespace {
@@ -174,6 +179,17 @@ int layout(const kx_config *c, Plan &p, kx_model *m) {
   return KX_OK;
 }
 
+// rope table for every position, computed on the host
+int init_rope(kx_model *m) {
+  const kx_config &c = m->c;
+  std::vector<uint16_t> tab((size_t)c.max_context * c.qk_rope);
+  int rc = kx_rope_table(&c, 0, c.max_context, tab.data());
+  if (rc) return rc;
+  KX_HIP(hipMemcpyAsync(m->rope_tab, tab.data(), tab.size() * 2, hipMemcpyHostToDevice, m->st));
+  KX_HIP(hipStreamSynchronize(m->st));
+  return KX_OK;
+}
+
 int init_weights(kx_model *m) {
   const kx_config &c = m->c;
   const size_t H = c.hidden, V = c.vocab, E = c.experts, I = c.moe_inter, SI = c.shared_inter, D = c.dense_inter;
@@ -217,13 +233,8 @@ int init_weights(kx_model *m) {
       KX_TRY(kx_fill_normal_bf16((void *)w.d_shared_down, H * SI, c.seed, b + TL_SH_DOWN, sg, 0, st));
     }
   }
-  // rope table for every position, computed on the host
-  std::vector<uint16_t> tab((size_t)c.max_context * c.qk_rope);
-  KX_TRY(kx_rope_table(&c, 0, c.max_context, tab.data()));
-  KX_HIP(hipMemcpyAsync(m->rope_tab, tab.data(), tab.size() * 2, hipMemcpyHostToDevice, m->st));
-  KX_HIP(hipStreamSynchronize(m->st));
 #undef KX_TRY
-  return KX_OK;
+  return init_rope(m);
 }
 
 // one run() of the reference for `B` tokens at position m->pos; ids on the device
@@ -324,8 +335,9 @@ extern "C" int kx_model_bytes(const kx_config *cfg, uint64_t *weights, uint64_t 
   return KX_OK;
 }
 
-extern "C" int kx_model_create(const kx_config *cfg, kx_model **out) {
-  KX_REQUIRE(out, "kx_model_create: null out pointer");
+// allocates the arena, lays the model out and creates its stream, events and MoE workspace; weights are not set
+static int model_new(const kx_config *cfg, const char *who, kx_model **out) {
+  KX_REQUIRE(out, "%s: null out pointer", who);
   *out = nullptr;
   int rc = check_model_cfg(cfg);
   if (rc) return rc;
@@ -333,13 +345,13 @@ extern "C" int kx_model_create(const kx_config *cfg, kx_model **out) {
   layout(cfg, p, nullptr);
   size_t free_b = 0, total_b = 0;
   KX_HIP(hipMemGetInfo(&free_b, &total_b));
-  KX_REQUIRE(p.total + ((size_t)1 << 30) <= free_b, "kx_model_create: the model needs %.1f GB of HBM, %.1f GB are free",
+  KX_REQUIRE(p.total + ((size_t)1 << 30) <= free_b, "%s: the model needs %.1f GB of HBM, %.1f GB are free", who,
              p.total / 1e9, free_b / 1e9);
   kx_model *m = new kx_model();
   m->c = *cfg;
   hipError_t e = hipMalloc((void **)&m->arena, p.total);
   if (e != hipSuccess) {
-    kx_set_error("kx_model_create: hipMalloc(%zu): %s", p.total, hipGetErrorString(e));
+    kx_set_error("%s: hipMalloc(%zu): %s", who, p.total, hipGetErrorString(e));
     delete m;
     return KX_ERR_HIP;
   }
@@ -351,13 +363,96 @@ extern "C" int kx_model_create(const kx_config *cfg, kx_model **out) {
   for (auto &ev : m->ev)
     if (!rc && hipEventCreate(&ev) != hipSuccess) rc = KX_ERR_HIP;
   if (!rc && cfg->first_dense < cfg->n_layers) rc = kx_moe_workspace_create(cfg, cfg->max_batch, &m->moe_ws);
-  if (!rc) rc = init_weights(m);
   if (rc) {
-    if (rc == KX_ERR_HIP && !kx_last_error()[0]) kx_set_error("kx_model_create: HIP resource creation failed");
+    if (rc == KX_ERR_HIP && !kx_last_error()[0]) kx_set_error("%s: HIP resource creation failed", who);
     kx_model_destroy(m);
     return rc;
   }
   *out = m;
+  return KX_OK;
+}
+
+extern "C" int kx_model_create(const kx_config *cfg, kx_model **out) {
+  kx_model *m = nullptr;
+  int rc = model_new(cfg, "kx_model_create", &m);
+  if (rc) return rc;
+  if ((rc = init_weights(m))) {
+    kx_model_destroy(m);
+    return rc;
+  }
+  *out = m;
+  return KX_OK;
+}
+
+// where checkpoint tensor `n` lives in the arena
+static char *need_dst(kx_model *m, const KxNeed &n) {
+  const kx_config &c = m->c;
+  const size_t H = c.hidden, I = c.moe_inter, e = n.expert < 0 ? 0 : (size_t)n.expert;
+  if (n.layer < 0) return (char *)(n.slot == KXS_EMBED ? m->embed : n.slot == KXS_FINAL_NORM ? m->final_norm : m->lm_head);
+  Layer &L = m->layers[n.layer];
+  const kx_moe_weights &w = L.moe;
+  switch (n.slot) {
+    case KXS_INPUT_LN: return (char *)L.input_ln;
+    case KXS_QA: return (char *)L.qkv_a;
+    case KXS_KVA: return (char *)(L.qkv_a + (size_t)c.q_rank * H);  // kv_a rows follow the q_a rows: one GEMV reads both
+    case KXS_QA_LN: return (char *)L.qa_ln;
+    case KXS_QB: return (char *)L.qb;
+    case KXS_KV_LN: return (char *)L.kv_ln;
+    case KXS_KVB: return (char *)L.kvb;  // rows h*(nope+v)+d: d < nope is W_UK[h], the rest W_UV[h] (split_kv_k, :364-370)
+    case KXS_O: return (char *)L.o;
+    case KXS_POST_LN: return (char *)L.post_ln;
+    case KXS_DENSE_GATE: return (char *)L.dgate;
+    case KXS_DENSE_UP: return (char *)L.dup;
+    case KXS_DENSE_DOWN: return (char *)L.ddown;
+    case KXS_ROUTER: return (char *)w.d_router_gate;
+    case KXS_ROUTER_BIAS: return (char *)w.d_router_bias;
+    case KXS_GATE_P: return (char *)w.d_gate_packed + e * (I * H / 2);
+    case KXS_GATE_S: return (char *)w.d_gate_scale + e * (I * H / 16);
+    case KXS_UP_P: return (char *)w.d_up_packed + e * (I * H / 2);
+    case KXS_UP_S: return (char *)w.d_up_scale + e * (I * H / 16);
+    case KXS_DOWN_P: return (char *)w.d_down_packed + e * (H * I / 2);
+    case KXS_DOWN_S: return (char *)w.d_down_scale + e * (H * I / 16);
+    case KXS_SH_GATE: return (char *)w.d_shared_gate;
+    case KXS_SH_UP: return (char *)w.d_shared_up;
+    case KXS_SH_DOWN: return (char *)w.d_shared_down;
+    default: return nullptr;
+  }
+}
+
+extern "C" int kx_model_load(const kx_config *cfg, const char *index_path, kx_model **out) {
+  KX_REQUIRE(out, "kx_model_load: null out pointer");
+  *out = nullptr;
+  KX_REQUIRE(cfg, "kx_model_load: null config");
+  KxIndex ix;
+  int rc = kx_index_parse(index_path, ix);
+  if (rc) return rc;
+  std::vector<KxNeed> needs;
+  if ((rc = check_model_cfg(cfg)) || (rc = kx_index_contract(ix, cfg, needs))) return rc;
+  kx_model *m = nullptr;
+  if ((rc = model_new(cfg, "kx_model_load", &m))) return rc;
+  std::vector<KxLoadItem> items;
+  items.reserve(needs.size());
+  for (const KxNeed &n : needs) {
+    KxLoadItem it;
+    it.t = n.t;
+    it.dst = need_dst(m, n);
+    it.widen = n.slot == KXS_ROUTER_BIAS;  // the router keeps the bias in f32; the checkpoint's bf16 widens exactly
+    items.push_back(it);
+  }
+  rc = kx_load_run(items, &m->load_bytes, &m->load_seconds);
+  if (!rc) rc = init_rope(m);
+  if (rc) {
+    kx_model_destroy(m);
+    return rc;
+  }
+  *out = m;
+  return KX_OK;
+}
+
+extern "C" int kx_model_load_info(kx_model *m, uint64_t *bytes, double *seconds) {
+  KX_REQUIRE(m, "kx_model_load_info: null model");
+  if (bytes) *bytes = m->load_bytes;
+  if (seconds) *seconds = m->load_seconds;
   return KX_OK;
 }
 

@@ -314,7 +314,7 @@ __global__ void __launch_bounds__(WAVES * 64, (I4 || WAVES < 8) ? 1 : 2) grouped
             if (po < p_end) {
               const int pr = a.pairs ? a.pairs[po] : po;
               float r = acc[0][t][v];
-              if (DUAL) r = kx_swiglu(kx_bfround(r), kx_bfround(acc[1][t][v]));
+              if (DUAL) r = kx_swiglu(kx_bfround(r), kx_bfround(acc[MATS - 1][t][v]));
               if (DUAL || a.out_mode == KX_GG_BF16) {
                 ((uint16_t *)a.out)[(size_t)pr * a.N + n] = kx_bf16_rne(r);
               } else if (a.out_mode == KX_GG_F32) {

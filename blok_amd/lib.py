@@ -91,6 +91,10 @@ _SIGS = {
     "kx_moe_decode_layer_timed": [C.POINTER(KxConfig), C.POINTER(KxMoeWeights), _P, _P, _P, _I,
                                   C.c_uint32, _P, C.POINTER(C.c_float)],
     "kx_moe_routed_only": [C.POINTER(KxConfig), C.POINTER(KxMoeWeights), _P, _P, _I, _I, _P],
+    "kx_index_check": [C.POINTER(KxConfig), C.c_char_p, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)],
+    "kx_index_infer_config": [C.c_char_p, C.POINTER(KxConfig)],
+    "kx_model_load": [C.POINTER(KxConfig), C.c_char_p, _PP],
+    "kx_model_load_info": [_P, C.POINTER(C.c_uint64), C.POINTER(C.c_double)],
 }
 
 _lib = None

@@ -229,6 +229,30 @@ int kx_decode_step(kx_model *model, const uint32_t *h_ids);
 int kx_greedy_sample(kx_model *model, uint32_t *h_out);
 int kx_generate(kx_model *model, const uint32_t *h_prompt, int32_t batch, int32_t prompt_len,
                 int32_t n_tokens, int ignore_eos, uint32_t *h_out, int32_t *h_counts);
+/* ---- checkpoint: runtime-index.blok -> resident weights ----------------------------------------
+ * The index is the text file scripts/model_fetch.py materialize() writes (:116-131): a header line
+ * `blok-runtime-index-v1`, then one line per checkpoint tensor,
+ *   tensor <name> <role> <layer> <expert> <slot> <dtype> <shape> <off> <bytes> <align> <data> <data_bytes> <file>
+ * with [off, off+bytes) the 4096-aligned extent of <file> that holds the data range
+ * [data, data+data_bytes).  A <file> that is not absolute is taken relative to the index's directory.
+ * kx_index_check       : runtime_index() (:559-585) + validate_forward_contract() (:736-778) with the
+ *                        shapes of *cfg for layers [0, cfg->n_layers): the tensors the forward pass
+ *                        reads and their data bytes.  Needs no GPU.
+ * kx_index_infer_config: overwrites the shape fields of *cfg (vocab, hidden, n_layers, first_dense,
+ *                        q_rank, kv_rank, heads, dense_inter, experts, shared_inter, moe_inter) with what
+ *                        the index's tensor shapes say; head dimensions, topk and the numeric constants
+ *                        are not in a checkpoint's shapes and stay as they are.  Needs no GPU.
+ * kx_model_load        : a kx_model whose weights are read from the index's files instead of being
+ *                        random-init (load_tensor / load_rows, :608-649, which the reference runs per
+ *                        tile per token; here once).  kv_b_proj stays whole: its rows h*256+d are
+ *                        W_UK[h] for d < 128 and W_UV[h] above (split_kv_k, :364-370).  The router bias
+ *                        is widened from bf16 to f32.  KX_LOAD_THREADS (default 8) reader threads;
+ *                        KX_LOAD_DIRECT=0 turns O_DIRECT reads off.
+ * kx_model_load_info   : data bytes copied by kx_model_load and the seconds it took.               */
+int kx_index_check(const kx_config *cfg, const char *index_path, uint64_t *n_tensors, uint64_t *weight_bytes);
+int kx_index_infer_config(const char *index_path, kx_config *cfg);
+int kx_model_load(const kx_config *cfg, const char *index_path, kx_model **model);
+int kx_model_load_info(kx_model *model, uint64_t *bytes, double *seconds);
 /* views for parity checks (synchronise): residual stream bf16 [batch][hidden], logits f32
  * [batch][vocab] of the last sampled step, latent cache rows bf16 [n][kv_rank+qk_rope]         */
 int kx_model_hidden(kx_model *model, uint16_t *h_out);

@@ -624,6 +624,59 @@ ox_model *ox_model_create(const ox_config *cfg, int mode) {
 }
 void ox_model_destroy(ox_model *m) { delete m; }
 
+// Overwrites one weight tensor of the model with `bytes` bytes from `src` (the element type the model keeps:
+// bf16, u32 words, f32 for the router bias).  layer < 0: id is TID_EMBED / TID_FINAL_NORM / TID_LM_HEAD; else a
+// TL_* id; expert >= 0 addresses one expert's part of a routed tensor.  Returns 0, or -1 when the id, the
+// coordinates or the byte count do not fit.  It is how a test hands the oracle the weights of a checkpoint
+// (the reference reads them per tile, load_tensor / load_rows, :608-649).
+int ox_model_set_tensor(ox_model *m, int layer, int id, int expert, const void *src, uint64_t bytes) {
+  void *dst = nullptr;
+  size_t have = 0;
+  auto whole16 = [&](std::vector<uint16_t> &v) { dst = v.data(); have = v.size() * 2; };
+  auto part = [&](auto &v, size_t esz) {
+    const size_t per = v.size() / (size_t)m->c.experts;
+    if (expert < 0 || expert >= m->c.experts) return;
+    dst = v.data() + per * (size_t)expert;
+    have = per * esz;
+  };
+  if (layer < 0) {
+    if (id == TID_EMBED) whole16(m->embed);
+    else if (id == TID_FINAL_NORM) whole16(m->final_norm);
+    else if (id == TID_LM_HEAD) whole16(m->lm_head);
+  } else if (layer < m->c.n_layers) {
+    OxLayer &L = m->layers[layer];
+    switch (id) {
+      case TL_INPUT_LN: whole16(L.input_ln); break;
+      case TL_QA: whole16(L.qa); break;
+      case TL_QA_LN: whole16(L.qa_ln); break;
+      case TL_QB: whole16(L.qb); break;
+      case TL_KVA: whole16(L.kva); break;
+      case TL_KV_LN: whole16(L.kv_ln); break;
+      case TL_KVB: whole16(L.kvb); break;
+      case TL_O: whole16(L.o); break;
+      case TL_POST_LN: whole16(L.post_ln); break;
+      case TL_DENSE_GATE: whole16(L.dgate); break;
+      case TL_DENSE_UP: whole16(L.dup); break;
+      case TL_DENSE_DOWN: whole16(L.ddown); break;
+      case TL_ROUTER: whole16(L.router); break;
+      case TL_ROUTER_BIAS: dst = L.router_bias.data(); have = L.router_bias.size() * 4; break;
+      case TL_GATE_P: part(L.gate_p, 4); break;
+      case TL_GATE_S: part(L.gate_s, 2); break;
+      case TL_UP_P: part(L.up_p, 4); break;
+      case TL_UP_S: part(L.up_s, 2); break;
+      case TL_DOWN_P: part(L.down_p, 4); break;
+      case TL_DOWN_S: part(L.down_s, 2); break;
+      case TL_SH_GATE: whole16(L.sh_gate); break;
+      case TL_SH_UP: whole16(L.sh_up); break;
+      case TL_SH_DOWN: whole16(L.sh_down); break;
+      default: break;
+    }
+  }
+  if (!dst || have == 0 || have != bytes) return -1;
+  memcpy(dst, src, bytes);
+  return 0;
+}
+
 // y = bf(W x) for one token through the selected schedule
 static void mv(const ox_model *m, const std::vector<uint16_t> &w, const uint16_t *x, uint16_t *y, int rows, int cols) {
   ox_gemv_bf16(w.data(), x, y, rows, cols, 1, 0, m->mode);

@@ -46,6 +46,7 @@ _SIGS = {
     "ox_mla_decode": ([_P, _P, C.c_size_t, _P, _P, _I, _I, _I], None),
     "ox_model_create": ([_P, _I], _P),
     "ox_model_destroy": ([_P], None),
+    "ox_model_set_tensor": ([_P, _I, _I, _I, _P, _U64], _I),
     "ox_generate": ([_P, _P, _I, _I, _I, _I, _P, _P], _I),
     "ox_model_logits": ([_P], C.POINTER(C.c_float)),
     "ox_model_hidden": ([_P], C.POINTER(C.c_uint16)),
@@ -146,6 +147,11 @@ class OxModel:
         counts = np.zeros(B, dtype=np.int32)
         rc = self.lib.ox_generate(self.h, ptr(np.ascontiguousarray(prompt)), B, P, n_tokens, int(ignore_eos), ptr(out), ptr(counts))
         return rc, out, counts
+
+    def set_tensor(self, layer, tid, expert, arr):
+        arr = np.ascontiguousarray(arr)
+        if self.lib.ox_model_set_tensor(self.h, layer, tid, expert, ptr(arr), arr.nbytes) != 0:
+            raise ValueError(f"ox_model_set_tensor({layer}, {tid}, {expert}, {arr.nbytes} bytes) does not fit the model")
 
     def logits(self, B):
         p = self.lib.ox_model_logits(self.h)

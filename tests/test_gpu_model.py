@@ -249,7 +249,7 @@ def test_executor_json_line(kxlib):
     import subprocess
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     exe = os.path.join(root, "blok_amd", "kx-kimi-exec")
-    r = subprocess.run([exe, "--index", "ignored", "--prompt-tokens", "11,12,13", "--tokens", "3", "--layers", "2", "--seed", "7",
+    r = subprocess.run([exe, "--prompt-tokens", "11,12,13", "--tokens", "3", "--layers", "2", "--seed", "7",
                         "--ignore-eos"], capture_output=True, text=True, timeout=300)
     assert r.returncode == 0, r.stderr
     doc = json.loads(r.stdout)                       # blok/runtime.py:88-94
