@@ -95,6 +95,13 @@ _SIGS = {
     "kx_index_infer_config": [C.c_char_p, C.POINTER(KxConfig)],
     "kx_model_load": [C.POINTER(KxConfig), C.c_char_p, _PP],
     "kx_model_load_info": [_P, C.POINTER(C.c_uint64), C.POINTER(C.c_double)],
+    "kx_tokenizer_open": [C.c_char_p, _PP],
+    "kx_tokenizer_close": [_P],
+    "kx_tokenizer_info": [_P, C.POINTER(C.c_int32), C.POINTER(C.c_int32), C.POINTER(C.c_int32)],
+    "kx_pretokenize": [C.c_char_p, _SZ, _P, _SZ, C.POINTER(_SZ)],
+    "kx_tokenizer_encode": [_P, C.c_char_p, _SZ, C.c_int, _P, _SZ, C.POINTER(_SZ)],
+    "kx_tokenizer_decode": [_P, _P, _SZ, _P, _SZ, C.POINTER(_SZ)],
+    "kx_encode_prompt": [_P, C.c_char_p, _SZ, _P, _SZ, C.POINTER(_SZ)],
 }
 
 _lib = None

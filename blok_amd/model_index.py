@@ -12,6 +12,7 @@ src/kimi_exec.cu:559-585) finds tensors by (layer, expert, role, slot), never by
 Only the safetensors header is read here: 8 bytes little-endian length, then that many bytes of JSON
 mapping names to {dtype, shape, data_offsets}; offsets count from the end of the header.
 """
+import base64
 import json
 import re
 import struct
@@ -107,14 +108,49 @@ def index_lines(rows, align=ALIGN):
     return lines
 
 
-def materialize(local_dir, meta_dir):
-    """Writes <meta_dir>/runtime-index.blok for the shards in local_dir; returns a small report (:115-131)."""
+TOKENIZER_HEADER = "blok-tokenizer-v2"
+
+
+def tokenizer(local_dir, n_tokens=163584, n_special=256):
+    """Text of tokenizer.blok from the checkpoint's tiktoken.model (`<base64 bytes> <rank>` per line) and the
+    added_tokens_decoder of tokenizer_config.json (:81-97).  Ranks must be exactly 0..n_tokens-1 and the special
+    ids the n_special that follow (Kimi-K2: 163584 + 256 = the 163840-row embedding); None skips that check."""
+    root = Path(local_dir)
+    vocab_file, config_file = root / "tiktoken.model", root / "tokenizer_config.json"
+    if not vocab_file.is_file() or not config_file.is_file():
+        raise SystemExit("pinned checkpoint requires tiktoken.model and tokenizer_config.json")
+    ranks = {}
+    for line in vocab_file.read_bytes().splitlines():
+        if not line.strip():
+            continue
+        encoded, rank = line.split()
+        ranks[int(rank)] = base64.b64decode(encoded)
+    added = json.loads(config_file.read_text()).get("added_tokens_decoder", {})
+    special = {int(i): meta["content"].encode() for i, meta in added.items()}
+    if n_tokens is not None:
+        if sorted(ranks) != list(range(n_tokens)) or sorted(special) != list(range(n_tokens, n_tokens + n_special)):
+            raise SystemExit("unexpected Kimi tokenizer rank contract")
+    rows = [TOKENIZER_HEADER]
+    rows += [f"tok {i} {ranks[i].hex()}" for i in sorted(ranks)]
+    rows += [f"special {i} {special[i].hex()}" for i in sorted(special)]
+    return "\n".join(rows) + "\n"
+
+
+def materialize(local_dir, meta_dir, tokenizer_ranks=(163584, 256)):
+    """Writes <meta_dir>/runtime-index.blok for the shards in local_dir and, when the checkpoint carries
+    tiktoken.model, <meta_dir>/tokenizer.blok; returns a small report (:115-131)."""
     meta = Path(meta_dir)
     meta.mkdir(parents=True, exist_ok=True)
+    report = {}
+    if (Path(local_dir) / "tiktoken.model").is_file():
+        n_tokens, n_special = tokenizer_ranks if tokenizer_ranks else (None, None)
+        (meta / "tokenizer.blok").write_text(tokenizer(local_dir, n_tokens, n_special))
+        report["tokenizer"] = str(meta / "tokenizer.blok")
     lines = index_lines(tensors(local_dir))
     index = meta / "runtime-index.blok"
     index.write_text("\n".join(lines) + "\n")
-    return {"tensors": len(lines) - 1, "index": str(index)}
+    report.update(tensors=len(lines) - 1, index=str(index))
+    return report
 
 
 def main(argv=None):

@@ -253,6 +253,29 @@ int kx_index_check(const kx_config *cfg, const char *index_path, uint64_t *n_ten
 int kx_index_infer_config(const char *index_path, kx_config *cfg);
 int kx_model_load(const kx_config *cfg, const char *index_path, kx_model **model);
 int kx_model_load_info(kx_model *model, uint64_t *bytes, double *seconds);
+/* ---- tokenizer.blok: the encoder on the caller's side of the executor (host only, needs no GPU) ----
+ * The file is written by scripts/model_fetch.py tokenizer() (:81-97): `blok-tokenizer-v2`, then
+ * `tok <id> <hex>` per mergeable byte string and `special <id> <hex>` per special token.
+ * kx_tokenizer_open  : tokenizer_encoding() of blok/runtime.py (:121-134); "bad tokenizer" on a malformed file.
+ * kx_pretokenize     : the split the pattern KIMI_PATTERN (runtime.py:37-48) makes of UTF-8 `text`:
+ *                      h_ends[i] = byte offset where piece i ends.
+ * kx_tokenizer_encode: tiktoken's Encoding.encode: with allow_special every special token's text found in
+ *                      `text` becomes its id (allowed_special="all", runtime.py:140) and the text between
+ *                      is split by the pattern and merged pair by pair, lowest rank first; without it the
+ *                      whole text is ordinary.
+ * kx_tokenizer_decode: the bytes of the ids, concatenated (Encoding.decode before its UTF-8 step).
+ * kx_encode_prompt   : encode_prompt() (runtime.py:137-140): the chat template
+ *                      <|im_user|>user<|im_middle|>{prompt}<|im_end|><|im_assistant|>assistant<|im_middle|><think></think>
+ * Output buffers: *n (or *len) is always set to the size needed; a buffer that is too small is an error. */
+typedef struct kx_tokenizer kx_tokenizer;
+int kx_tokenizer_open(const char *path, kx_tokenizer **tok);
+int kx_tokenizer_close(kx_tokenizer *tok);
+int kx_tokenizer_info(const kx_tokenizer *tok, int32_t *n_tokens, int32_t *n_special, int32_t *max_id);
+int kx_pretokenize(const char *text, size_t len, uint32_t *h_ends, size_t cap, size_t *n);
+int kx_tokenizer_encode(const kx_tokenizer *tok, const char *text, size_t len, int allow_special, uint32_t *h_ids,
+                        size_t cap, size_t *n);
+int kx_tokenizer_decode(const kx_tokenizer *tok, const uint32_t *h_ids, size_t n_ids, char *h_bytes, size_t cap, size_t *len);
+int kx_encode_prompt(const kx_tokenizer *tok, const char *prompt, size_t len, uint32_t *h_ids, size_t cap, size_t *n);
 /* views for parity checks (synchronise): residual stream bf16 [batch][hidden], logits f32
  * [batch][vocab] of the last sampled step, latent cache rows bf16 [n][kv_rank+qk_rope]         */
 int kx_model_hidden(kx_model *model, uint16_t *h_out);
