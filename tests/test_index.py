@@ -136,3 +136,77 @@ def test_reader_rejects_what_the_reference_rejects(tmp_path, edit, msg):
 def test_missing_index_names_the_file(tmp_path):
     rc, _, _, err = _check(O.small_config(), tmp_path / "runtime-index.blok")
     assert rc != 0 and "missing runtime-index.blok" in err   # :561
+
+
+def _kimi_index_lines(layers=61):
+    """Index lines of the full Kimi-K2 checkpoint layout (no files behind them): the shapes of
+    scripts/check_kimi_contract.py:50-73, data packed back to back into one imaginary shard."""
+    H, D, I, E, V = 7168, 18432, 2048, 384, 163840
+    rows, at = [], [8]
+
+    def add(name, dtype, *shape):
+        n = 1
+        for d in shape:
+            n *= d
+        size = n * (2 if dtype == "bf16" else 4)
+        rows.append((name, MI.role(name), dtype, "x".join(map(str, shape)), "/ckpt/model-00001-of-000064.safetensors", at[0], size))
+        at[0] += size
+
+    lm = "language_model."
+    add(lm + "model.embed_tokens.weight", "bf16", V, H)
+    add(lm + "model.norm.weight", "bf16", H)
+    add(lm + "lm_head.weight", "bf16", V, H)
+    for l in range(layers):
+        p = f"{lm}model.layers.{l}."
+        add(p + "input_layernorm.weight", "bf16", H)
+        add(p + "post_attention_layernorm.weight", "bf16", H)
+        for n, shp in (("q_a_proj", (1536, H)), ("q_a_layernorm", (1536,)), ("q_b_proj", (64 * 192, 1536)), ("kv_a_proj_with_mqa", (576, H)),
+                       ("kv_a_layernorm", (512,)), ("kv_b_proj", (64 * 256, 512)), ("o_proj", (H, 64 * 128))):
+            add(p + "self_attn." + n + ".weight", "bf16", *shp)
+        if l == 0:
+            add(p + "mlp.gate_proj.weight", "bf16", D, H)
+            add(p + "mlp.up_proj.weight", "bf16", D, H)
+            add(p + "mlp.down_proj.weight", "bf16", H, D)
+            continue
+        add(p + "mlp.gate.weight", "bf16", E, H)
+        add(p + "mlp.gate.e_score_correction_bias", "bf16", E)
+        for n, shp in (("gate_proj", (I, H)), ("up_proj", (I, H)), ("down_proj", (H, I))):
+            add(p + f"mlp.shared_experts.{n}.weight", "bf16", *shp)
+            for e in range(E):
+                add(p + f"mlp.experts.{e}.{n}.weight_packed", "i32", shp[0], shp[1] // 8)
+                add(p + f"mlp.experts.{e}.{n}.weight_scale", "bf16", shp[0], shp[1] // 32)
+    return MI.index_lines(rows), at[0] - 8
+
+
+def test_full_kimi_k2_contract_and_checker(tmp_path):
+    # all 61 layers x 384 experts at the real shapes, through the writer's naming rules and the C++ contract
+    from blok_amd import check_contract as CC
+    from blok_amd.lib import default_config
+    lines, data_bytes = _kimi_index_lines()
+    index = tmp_path / "runtime-index.blok"
+    index.write_text("\n".join(lines) + "\n")
+    cfg = default_config()
+    cfg.n_layers = 61
+    rc, n, nbytes, err = _check(cfg, index)
+    assert rc == 0, err
+    assert n == len(lines) - 1 == 3 + 61 * 9 + 3 + 60 * (2 + 3 + 384 * 6)
+    assert nbytes == data_bytes
+    cfg.n_layers = 24            # the truncation that fits one GPU reads a prefix
+    rc, n24, b24, err = _check(cfg, index)
+    assert rc == 0 and n24 == 3 + 24 * 9 + 3 + 23 * (2 + 3 + 384 * 6), err
+    assert abs(b24 - 231.29e9) < 0.3e9   # the resident weights of the 24-layer stack
+    # the checker: index ok, tokenizer missing, then present with the real ids of the words involved
+    with pytest.raises(SystemExit, match="missing or bad tokenizer.blok"):
+        CC.check(tmp_path)
+    import test_tokenizer as TT
+    ranks = {bytes([b]): i for i, b in enumerate(TT.byte_order())}
+    ranks.update({b"user": 2482, b"hello": 22931, b"assistant": 69702, b"123": 6694, b"456": 12972, b"789": 16242})
+    special = {"<|im_end|>": 163586, "<|im_user|>": 163587, "<|im_assistant|>": 163588, "<|im_middle|>": 163601, "<think>": 163606, "</think>": 163607}
+    TT.write_blok(tmp_path / "tokenizer.blok", ranks, special)
+    assert CC.check(tmp_path) == (n, nbytes)
+    ranks[b"hello"] = 22930
+    TT.write_blok(tmp_path / "tokenizer.blok", ranks, special)
+    with pytest.raises(SystemExit, match="tokenizer mismatch for 'hello'"):
+        CC.check(tmp_path)
+    with pytest.raises(SystemExit, match="missing runtime-index.blok"):
+        CC.check(tmp_path / "nowhere")
