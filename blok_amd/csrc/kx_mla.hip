@@ -25,6 +25,7 @@
 //              over spans ascending; o_lat = bf(O / Z)
 //   q_lat      eight chains over d = j, j+8, ... then ((0+1)+(2+3))+((4+5)+(6+7))
 #include <math.h>
+#include <type_traits>
 #include "kx_common.h"
 #include "kx_dense.h"
 #include "kx_math.h"
@@ -343,45 +344,73 @@ __global__ void __launch_bounds__(256) mla_partial_k(MlaArgs a) {
 // q_abs and p = bf(exp(s - m)) are bf16-representable and the cache is bf16, so q.c and p.c are exact
 // products summed in fp32: v_mfma_f32_16x16x32_bf16 computes what mla_partial_k computes with another
 // summation order (held to the 1e-2 bar, not bit-exact; the token-identity runs use mla_partial_k).
-// Workgroup = (sequence, span), 8 waves, 32-position tiles; the two products split the work differently and
-// hand p, the running-maximum factor and the row sums over through LDS:
+// Workgroup = (sequence, span), 8 waves, 32-position tiles staged in LDS at their natural layout; the two
+// products split the work differently and hand p, the running-maximum factor and the row sums over through LDS:
 //  * scores: wave (hw, pb) computes heads 16 hw .. +15 against positions 16 pb .. +15 of the tile,
 //    S^T[pos, head] = C[pos, 576] Q^T[576, head] with v_mfma_f32_16x16x32_bf16 (A = cache rows from LDS, B = the
 //    lane's head of q in registers, 18 K steps); the two waves of a head group exchange their maxima, then each
-//    writes p = bf(exp(s - m)) of its 16 positions in the K order of the second product;
+//    writes p = bf(exp(s - m)) of its 16 positions at the K indices the second product reads them from;
 //  * O^T[col, head] += C^T[col, pos] P^T[pos, head]: wave (hb, cq) owns heads 32 hb .. +31 and latent columns
 //    128 cq .. +127 (v_mfma_f32_32x32x16_bf16, two K steps per tile).  The A operand needs 8 positions of one
-//    column, so the 512 latent columns of the tile are transposed once per tile into a second LDS buffer
-//    (LDS -> LDS, lanes = positions, conflict-free both ways), position 16 a + 4 g + v at K index 8 g + 4 a + v --
-//    the order in which the score accumulators hold the positions, so p is stored without any shuffle;
-//  * the 32 cache rows of tile t+2 are copied global -> LDS (no registers) while tile t is computed; rows sit at
-//    their natural pitch of 1152 B with the 16-byte pieces xor-swizzled by the row, so the row-per-lane operand
-//    reads are free of bank conflicts.
+//    column; ds_read_b64_tr_b16 delivers them from the row-major tile: within 16 lanes, lane i points at four
+//    consecutive columns of row i / 4, and lane j receives column j of the four rows;
+//  * the loop is software-pipelined: between two barriers a wave issues the second product of tile t-1 and the
+//    scores of tile t (independent MFMA chains, interleaved), then the maxima are exchanged, and after the
+//    second barrier the exponentials and p of tile t are written.  Two barriers per tile;
+//  * the 32 cache rows of tile t+2 are copied global -> LDS (no registers) while tile t is computed, into a ring
+//    of four buffers (tile t-1 is still read by the second product); rows sit at their natural pitch of 1152 B
+//    with the 16-byte pieces xor-swizzled by the row, so the row-per-lane operand reads of the scores are free
+//    of bank conflicts, and a transposing read touches rows that differ in bit 3 of the position in its two
+//    lane halves, which spreads it over all banks.
 constexpr int MM_T = 32;                      // positions per tile
 constexpr int MM_NAT = MM_T * MLA_KVA * 2;    // bytes of one staged tile
-constexpr int MM_CT_PITCH = 80;               // bytes per transposed column: 32 positions + pad
-constexpr int MM_CT = MLA_R * MM_CT_PITCH;
-constexpr int MM_P_PITCH = 80;                // bytes per head of the staged probabilities: 32 K indices + pad
-constexpr int MM_XCH = 64 * MM_P_PITCH + 5 * 64 * 4;  // p, two maxima, two row sums and the rescale factor per head
+constexpr int MM_RING = 4;
+constexpr int MM_P_PITCH = 80;                // bytes per head of the staged probabilities: 32 positions + pad
+constexpr int MM_LDS = MM_RING * MM_NAT;  // dynamic part: the tile ring
 typedef float kx_f32x16v __attribute__((ext_vector_type(16)));
 typedef __bf16 kx_bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 kx_bf16x2v __attribute__((ext_vector_type(2)));
 typedef float kx_f32x2v __attribute__((ext_vector_type(2)));
 typedef float kx_f32x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 kx_bf16x4t;
 // two f32 -> packed bf16 pair, round to nearest even (v_cvt_pk_bf16_f32; the same values as kx_bf16_rne for finite inputs)
 __device__ __forceinline__ uint32_t mm_pack_bf16(float lo, float hi) {
   kx_f32x2v v = {lo, hi};
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, kx_bf16x2v));
 }
+// ds_read_b64_tr_b16 at LDS byte address `addr`
+__device__ __forceinline__ uint2 mm_read_tr(uint32_t addr) {
+  kx_bf16x4t v = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) kx_bf16x4t *)(uintptr_t)addr);
+  return __builtin_bit_cast(uint2, v);
+}
+// global_load_lds_dwordx4: lane i's 16 bytes at `src` land at LDS byte address lds_base + 16 i (lds_base uniform).
+// Written as asm so that the compiler does not know of the copy: it completes every copy in flight (s_waitcnt
+// vmcnt(0)) in front of each LDS access it cannot tell from the copy's target, and in front of every fenced
+// barrier -- which would make the tiles copied ahead land at once.  This kernel waits for a tile itself, where
+// it needs it (wait_tile below).
+__device__ __forceinline__ void mm_copy16_to_lds(const void *src, uint32_t lds_base) {
+  uint32_t m0_saved;  // the instruction takes the LDS address from m0; m0 is put back, the compiler owns it
+  asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, off\n\ts_mov_b32 m0, %0"
+               : "=&s"(m0_saved)
+               : "s"(lds_base), "v"(src)
+               : "memory");
+}
+
+// Workgroup barrier for this kernel.  __syncthreads() carries a fence, and the compiler completes every memory
+// operation for it -- s_waitcnt vmcnt(0), i.e. the tiles being copied ahead would have to land at every barrier.
+// Here only the wave's LDS operations are completed (what the waves exchange goes through LDS); the landing of
+// a copied tile is waited for explicitly where the tile is needed.
+__device__ __forceinline__ void mm_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 __global__ void __launch_bounds__(512, 1) mla_partial_mfma_k(MlaArgs a) {
-  extern __shared__ __attribute__((aligned(16))) uint8_t mm_lds[];
-  uint8_t *nat = mm_lds;                       // [3][32 rows][72 pieces of 16 B]
-  uint8_t *ct = mm_lds + 3 * MM_NAT;           // [512 columns][MM_CT_PITCH]
-  uint8_t *p_lds = ct + MM_CT;                 // [64 heads][MM_P_PITCH]: bf16 p at K index order
-  float *mx_lds = (float *)(p_lds + 64 * MM_P_PITCH);  // [2][64] tile maxima of the two position halves
-  float *ps_lds = mx_lds + 128;                // [2][64] row sums of the two position halves
-  float *al_lds = ps_lds + 128;                // [64] exp(M_old - M_new)
+  // the tile ring is the dynamic LDS; what the waves exchange lives in separate objects, so that the compiler can
+  // tell a store to them from the global -> LDS copies in flight (it would wait for those before the store)
+  extern __shared__ __attribute__((aligned(128))) uint8_t mm_lds[];
+  uint8_t *nat = mm_lds;                       // [4][32 rows][72 pieces of 16 B]
+  __shared__ __attribute__((aligned(16))) uint8_t p_lds[64 * MM_P_PITCH];  // [64 heads]: bf16 p by position
+  __shared__ float mx_lds[128];                // [2][64] tile maxima of the two position halves
+  __shared__ float ps_lds[128];                // [2][64] row sums of the two position halves
+  __shared__ float al_lds[64];                 // [64] exp(M_old - M_new)
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int span = blockIdx.x, b = blockIdx.z;
@@ -398,6 +427,7 @@ __global__ void __launch_bounds__(512, 1) mla_partial_mfma_k(MlaArgs a) {
   const int n_tiles = (pos_end - pos0 + MM_T - 1) / MM_T;
   const float scale = a.rs * a.mscale * a.mscale;
   constexpr float LOG2E = 1.44269504088896341f;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)nat;  // LDS address of the ring
 
   // q of this lane's head as B operands: K step ks covers columns 32 ks .. +31, lane group g its 8 g .. +7
   kx_bf16x8 qf[18];
@@ -424,13 +454,9 @@ __global__ void __launch_bounds__(512, 1) mla_partial_mfma_k(MlaArgs a) {
         const int p = slot / 72, js = slot - p * 72;
         const int j = (js & ~7) | ((js ^ (p >> 1)) & 7);
         const int row = min(pos0 + t * MM_T + p, a.seq - 1);
-        __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)(cache + (size_t)row * MLA_KVA + j * 8),
-                                         (void __attribute__((address_space(3))) *)(nat + (t % 3) * MM_NAT + ii * 1024), 16, 0, 0);
+        mm_copy16_to_lds(cache + (size_t)row * MLA_KVA + j * 8, lds0 + (t % MM_RING) * MM_NAT + ii * 1024);
       }
     }
-  };
-  auto nat_piece = [&](const uint8_t *st, int p, int j) {  // address of piece j of staged row p
-    return st + p * (MLA_KVA * 2) + (((j & ~7) | ((j ^ (p >> 1)) & 7)) << 4);
   };
   // byte offsets of this lane's A operands of the score product: row 16 pb + c16, piece 4 ks + g = 8 (ks / 2) + (4 (ks % 2) + g)
   int s_off[2];
@@ -439,59 +465,99 @@ __global__ void __launch_bounds__(512, 1) mla_partial_mfma_k(MlaArgs a) {
     const int pr = pb * 16 + c16;
     s_off[o] = pr * (MLA_KVA * 2) + (((4 * o + g) ^ (pr >> 1)) & 7) * 16;
   }
+  // byte offsets of this lane's transposing reads for the PV product.  Position r (0-15 inside the 16 positions of
+  // MFMA step s) sits at K index kk(r) = 4 ((r & 7) >> 1) + 2 (r >> 3) + (r & 1): the four K slots 4 w .. 4 w + 3 of
+  // lane half `half` are then positions a, a+1, a+8, a+9 with a = 16 s + 4 half + 2 w, four rows that fall into
+  // four different quarters of the banks (a row is 1152 B = 4.5 bank lines, and the xor of the 16-byte pieces moves
+  // with bit 3 of the position), so a transposing read of a half-wave is free of bank conflicts.  Lane i of its
+  // group of 16 points at row a + ((i >> 2) & 1) + 8 (i >> 3), columns 128 cq + 32 cbk + 16 (group & 1) + 4 (i & 3) .. +3,
+  // i.e. piece 16 cq + 4 cbk + 2 (group & 1) + ((i >> 1) & 1), low or high half by i & 1.  cbk odd flips bit 2 of the
+  // piece (xor 64 on the swizzled offset), cbk >> 1 adds 128.
+  int t_off[2][2];
+  {
+    const int i = lane & 15, grp = (lane >> 4) & 1;
+#pragma unroll
+    for (int sidx = 0; sidx < 2; ++sidx)
+#pragma unroll
+      for (int w = 0; w < 2; ++w) {
+        const int p = 16 * sidx + 4 * half + 2 * w + ((i >> 2) & 1) + 8 * (i >> 3);
+        const int low3 = 2 * grp + ((i >> 1) & 1);
+        t_off[sidx][w] = p * (MLA_KVA * 2) + (2 * cq) * 128 + ((low3 ^ (p >> 1)) & 7) * 16 + (i & 1) * 8;
+      }
+  }
+  // where this score lane's p values go: positions 16 pb + 4 g + v, v = 0, 1 at K index kk0, kk0 + 1 and v = 2, 3 at
+  // kk0 + 4, kk0 + 5 (r = 4 g + v in the formula above)
+  const int p_off = head * MM_P_PITCH + (16 * pb + 8 * (g & 1) + 2 * (g >> 1)) * 2;
   float M = -__builtin_inff(), Z = 0.0f;  // of `head`; the two waves of a head group keep identical copies
+  float alpha_prev = 1.0f;
   kx_f32x16v O[4];                        // heads 32 hb .. +31 x columns 128 cq + 32 cbk .. +31
 #pragma unroll
   for (int cbk = 0; cbk < 4; ++cbk)
 #pragma unroll
     for (int i = 0; i < 16; ++i) O[cbk][i] = 0.0f;
 
-  // tiles are copied two ahead into a ring of three buffers; loads complete in order, so waiting until only the
-  // copies of the newest tile (5 instructions for waves 0-3, 4 for the others) are outstanding means tile t has landed
-  copy_tile(0);
-  if (n_tiles > 1) copy_tile(1);
-  for (int t = 0; t < n_tiles; ++t) {
+  // tiles are copied two ahead into the ring; loads complete in order, so waiting until only the copies of the
+  // newest tile (5 instructions for waves 0-3, 4 for the others) are outstanding means tile t has landed
+  auto wait_tile = [&](int t) {
     if (t + 1 < n_tiles) {
       if (wave < 4) asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
       else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
     } else {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
-    __syncthreads();  // everybody's share of tile t has landed; the previous tile is done with every buffer
-    if (t + 2 < n_tiles) copy_tile(t + 2);
-    const uint8_t *st = nat + (t % 3) * MM_NAT;
-    // scores of positions 16 pb + 4 g + v for this lane's head
+  };
+  // what follows the first barrier of iteration t for the second product of tile t-1: row sums, p, rescale
+  kx_bf16x8 pf[2];
+  auto pv_begin = [&]() {
+    Z = __builtin_fmaf(Z, alpha_prev, ps_lds[head] + ps_lds[64 + head]);
+    pf[0] = *(const kx_bf16x8 *)(p_lds + head2 * MM_P_PITCH + half * 16);
+    pf[1] = *(const kx_bf16x8 *)(p_lds + head2 * MM_P_PITCH + 32 + half * 16);
+    const float alpha2 = al_lds[head2];
+    if (__builtin_amdgcn_ballot_w64(alpha2 != 1.0f) != 0) {  // the running maximum of some head of the wave moved
+      asm volatile("" ::: "memory");                          // keep this a branch: it is rarely taken after the first tiles
+#pragma unroll
+      for (int cbk = 0; cbk < 4; ++cbk) O[cbk] *= alpha2;
+    }
+  };
+  // the A operands of the second product of the tile staged at LDS byte address sp: for block cbk = m / 2 and
+  // step sidx = m % 2 two transposing reads (K slots 0-3 and 4-7 of the lane's eight)
+  kx_bf16x8 pa[8];
+  auto pv_operands = [&](uint32_t sp) {
+#pragma unroll
+    for (int sidx = 0; sidx < 2; ++sidx) {
+      const uint32_t a0 = sp + t_off[sidx][0], a1 = sp + t_off[sidx][1];              // blocks 0 and 2
+      const uint32_t b0 = sp + (t_off[sidx][0] ^ 64), b1 = sp + (t_off[sidx][1] ^ 64);  // blocks 1 and 3
+      const uint2 l0 = mm_read_tr(a0), h0 = mm_read_tr(a1), l1 = mm_read_tr(b0), h1 = mm_read_tr(b1);
+      const uint2 l2 = mm_read_tr(a0 + 128), h2 = mm_read_tr(a1 + 128), l3 = mm_read_tr(b0 + 128), h3 = mm_read_tr(b1 + 128);
+      pa[0 + sidx] = __builtin_bit_cast(kx_bf16x8, make_uint4(l0.x, l0.y, h0.x, h0.y));
+      pa[2 + sidx] = __builtin_bit_cast(kx_bf16x8, make_uint4(l1.x, l1.y, h1.x, h1.y));
+      pa[4 + sidx] = __builtin_bit_cast(kx_bf16x8, make_uint4(l2.x, l2.y, h2.x, h2.y));
+      pa[6 + sidx] = __builtin_bit_cast(kx_bf16x8, make_uint4(l3.x, l3.y, h3.x, h3.y));
+    }
+  };
+  auto pv_frag = [&](int m) { return pa[m]; };
+  // scores of tile t (staged at st) and, with PV, the second product of tile t-1 (staged at sp), interleaved
+  auto products = [&](auto with_pv, const uint8_t *st, uint32_t sp) {
+    constexpr bool PV = decltype(with_pv)::value;
+    constexpr int AH = 3;  // score operands are read three K steps ahead of the MFMAs that consume them
     kx_f32x4 sacc = kx_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-    {
-      constexpr int AH = 4;  // operands are read four K steps ahead of the MFMAs that consume them
-      kx_bf16x8 av[AH + 1];
+    kx_bf16x8 av[AH + 1];
+    if (PV) pv_operands(sp);
 #pragma unroll
-      for (int ks = 0; ks < AH; ++ks) av[ks] = *(const kx_bf16x8 *)(st + s_off[ks & 1] + (ks >> 1) * 128);
+    for (int ks = 0; ks < AH; ++ks) av[ks] = *(const kx_bf16x8 *)(st + s_off[ks & 1] + (ks >> 1) * 128);
 #pragma unroll
-      for (int ks = 0; ks < 18; ++ks) {
-        if (ks + AH < 18) av[(ks + AH) % (AH + 1)] = *(const kx_bf16x8 *)(st + s_off[(ks + AH) & 1] + ((ks + AH) >> 1) * 128);
-        sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[ks % (AH + 1)], qf[ks], sacc, 0, 0, 0);
+    for (int ks = 0; ks < 18; ++ks) {
+      if (ks + AH < 18) av[(ks + AH) % (AH + 1)] = *(const kx_bf16x8 *)(st + s_off[(ks + AH) & 1] + ((ks + AH) >> 1) * 128);
+      sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[ks % (AH + 1)], qf[ks], sacc, 0, 0, 0);
+      if (PV && (ks & 1) && ks < 16) {  // one MFMA of the second product after every other score step
+        const int m = ks >> 1;
+        O[m >> 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pv_frag(m), pf[m & 1], O[m >> 1], 0, 0, 0);
       }
     }
-    // transpose the latent columns 64 wave .. +63: lanes 0-31 take piece j, lanes 32-63 piece j+1, position = lane % 32
-    {
-      const int p = lane & 31;
-      const int kidx = ((p >> 2) & 3) * 8 + (p >> 4) * 4 + (p & 3);  // position 16 a + 4 g + v -> K index 8 g + 4 a + v
-      uint4 u[4];
-#pragma unroll
-      for (int it = 0; it < 4; ++it) u[it] = *(const uint4 *)nat_piece(st, p, wave * 8 + it * 2 + (lane >> 5));
-#pragma unroll
-      for (int it = 0; it < 4; ++it) {
-        const int j = wave * 8 + it * 2 + (lane >> 5);
-        uint8_t *d = ct + (j * 8) * MM_CT_PITCH + kidx * 2;
-        const uint32_t w[4] = {u[it].x, u[it].y, u[it].z, u[it].w};
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          *(uint16_t *)(d + (2 * e) * MM_CT_PITCH) = (uint16_t)(w[e] & 0xffffu);
-          *(uint16_t *)(d + (2 * e + 1) * MM_CT_PITCH) = (uint16_t)(w[e] >> 16);
-        }
-      }
-    }
+    return sacc;
+  };
+  // maxima, exponentials, p and row sums of tile t from its score accumulators; contains the second barrier
+  auto softmax_tile = [&](int t, kx_f32x4 sacc) {
     float sv[4];
     float mloc = -__builtin_inff();
 #pragma unroll
@@ -506,51 +572,60 @@ __global__ void __launch_bounds__(512, 1) mla_partial_mfma_k(MlaArgs a) {
       sv[v + 1] = s1;
       mloc = fmaxf(mloc, fmaxf(s0, s1));
     }
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 16));
-    mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
+    {  // maximum over the four lane groups of the head: lanes l ^ 16 and l ^ 32
+      float o = mloc;
+      kxw::swap_rows16(mloc, o);
+      mloc = fmaxf(mloc, o);
+      o = mloc;
+      kxw::swap_halves32(mloc, o);
+      mloc = fmaxf(mloc, o);
+    }
     if (g == 0) mx_lds[pb * 64 + head] = mloc;
-    __syncthreads();  // the maxima of both position halves and the transposed tile are complete
+    mm_barrier();  // the maxima of both position halves are complete; every wave is done reading p of tile t-1
     const float Mn = fmaxf(M, fmaxf(mloc, mx_lds[(pb ^ 1) * 64 + head]));
     // exponentials through v_exp_f32: this path is held to a tolerance, not to the bits of kx_expf
     const float alpha = __builtin_amdgcn_exp2f((M - Mn) * LOG2E);
     const float e0 = __builtin_amdgcn_exp2f((sv[0] - Mn) * LOG2E), e1 = __builtin_amdgcn_exp2f((sv[1] - Mn) * LOG2E);
     const float e2 = __builtin_amdgcn_exp2f((sv[2] - Mn) * LOG2E), e3 = __builtin_amdgcn_exp2f((sv[3] - Mn) * LOG2E);
     float ps = (e0 + e1) + (e2 + e3);
-    ps += __shfl_xor(ps, 16);
-    ps += __shfl_xor(ps, 32);
-    // positions 16 pb + 4 g + v sit at K indices 8 g + 4 pb + v
-    *(uint2 *)(p_lds + head * MM_P_PITCH + (8 * g + 4 * pb) * 2) = make_uint2(mm_pack_bf16(e0, e1), mm_pack_bf16(e2, e3));
+    {
+      float o = ps;
+      kxw::swap_rows16(ps, o);
+      ps += o;
+      o = ps;
+      kxw::swap_halves32(ps, o);
+      ps += o;
+    }
+    *(uint32_t *)(p_lds + p_off) = mm_pack_bf16(e0, e1);
+    *(uint32_t *)(p_lds + p_off + 8) = mm_pack_bf16(e2, e3);
     if (g == 0) {
       ps_lds[pb * 64 + head] = ps;
       if (pb == 0) al_lds[head] = alpha;
     }
     M = Mn;
-    __syncthreads();  // p, row sums and rescale factors are complete
-    Z = __builtin_fmaf(Z, alpha, ps_lds[head] + ps_lds[64 + head]);
-    // second product, for heads 32 hb .. +31 and columns 128 cq .. +127
-    const float alpha2 = al_lds[head2];
-    if (__builtin_amdgcn_ballot_w64(alpha2 != 1.0f) != 0) {  // the running maximum of some head of the wave moved
-      asm volatile("" ::: "memory");                          // keep this a branch: it is rarely taken after the first tiles
-#pragma unroll
-      for (int cbk = 0; cbk < 4; ++cbk) O[cbk] *= alpha2;
-    }
-    {
-      const kx_bf16x8 pf0 = *(const kx_bf16x8 *)(p_lds + head2 * MM_P_PITCH + half * 16);
-      const kx_bf16x8 pf1 = *(const kx_bf16x8 *)(p_lds + head2 * MM_P_PITCH + 32 + half * 16);
-      const uint8_t *cbase = ct + (cq * 128 + l32) * MM_CT_PITCH + half * 16;
-      kx_bf16x8 av[4][2];
-#pragma unroll
-      for (int cbk = 0; cbk < 4; ++cbk) {
-        av[cbk][0] = *(const kx_bf16x8 *)(cbase + cbk * 32 * MM_CT_PITCH);
-        av[cbk][1] = *(const kx_bf16x8 *)(cbase + cbk * 32 * MM_CT_PITCH + 32);
-      }
-#pragma unroll
-      for (int cbk = 0; cbk < 4; ++cbk) {
-        O[cbk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[cbk][0], pf0, O[cbk], 0, 0, 0);
-        O[cbk] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[cbk][1], pf1, O[cbk], 0, 0, 0);
-      }
-    }
+    alpha_prev = alpha;
+  };
+
+  copy_tile(0);
+  if (n_tiles > 1) copy_tile(1);
+  // tile 0: scores only
+  wait_tile(0);
+  mm_barrier();
+  if (2 < n_tiles) copy_tile(2);
+  softmax_tile(0, products(std::false_type{}, nat, lds0));
+  for (int t = 1; t < n_tiles; ++t) {
+    wait_tile(t);
+    mm_barrier();  // everybody's share of tile t has landed; p, row sums and rescale factors of tile t-1 are complete
+    if (t + 2 < n_tiles) copy_tile(t + 2);
+    pv_begin();
+    softmax_tile(t, products(std::true_type{}, nat + (t % MM_RING) * MM_NAT, lds0 + ((t - 1) % MM_RING) * MM_NAT));
   }
+  // the second product of the last tile
+  mm_barrier();
+  pv_begin();
+  pv_operands(lds0 + ((n_tiles - 1) % MM_RING) * MM_NAT);
+#pragma unroll
+  for (int m = 0; m < 8; ++m) O[m >> 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pv_frag(m), pf[m & 1], O[m >> 1], 0, 0, 0);
   // partials.  Maxima and sums: the score lanes of the first position half; O: lane = (head, column
   // 128 cq + 32 cbk + 8 q + 4 half + c) for accumulator register 4 q + c
   if (pb == 0 && g == 0) {
@@ -668,10 +743,10 @@ int kx_mla_partials_launch(const kx_config *c, const uint16_t *cache, size_t seq
     KX_REQUIRE(c->heads == 64, "kx_mla: the matrix-core kernel is built for 64 heads (got %d)", c->heads);
     static bool mfma_attr = false;
     if (!mfma_attr) {
-      KX_HIP(hipFuncSetAttribute((const void *)mla_partial_mfma_k, hipFuncAttributeMaxDynamicSharedMemorySize, 3 * MM_NAT + MM_CT + MM_XCH));
+      KX_HIP(hipFuncSetAttribute((const void *)mla_partial_mfma_k, hipFuncAttributeMaxDynamicSharedMemorySize, MM_LDS));
       mfma_attr = true;
     }
-    hipLaunchKernelGGL(mla_partial_mfma_k, dim3(a.spans, 1, batch), dim3(512), 3 * MM_NAT + MM_CT + MM_XCH, st, a);
+    hipLaunchKernelGGL(mla_partial_mfma_k, dim3(a.spans, 1, batch), dim3(512), MM_LDS, st, a);
     KX_LAUNCH_CHECK();
     out->pm = a.pm; out->pz = a.pz; out->po = a.po; out->spans = a.spans;
     return KX_OK;
