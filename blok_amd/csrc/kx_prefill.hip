@@ -75,6 +75,27 @@ __device__ __forceinline__ uint32_t pf_pack(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, kx_bf16x2));
 }
 
+// The INT4 kernels keep copies and loads in flight across barriers and LDS accesses, and say themselves when
+// one has to have landed.  The compiler would not let them: it completes every global -> LDS copy in flight
+// (s_waitcnt vmcnt(0)) in front of an LDS access it cannot tell from the copy's target and in front of every
+// fenced barrier, and loads complete in order, so a wait for a plain load it issued waits for the copies too.
+// Hence: weights and activations both reach LDS by copies issued from inline asm (unknown to the compiler), the
+// barrier has no fence, and the waits are explicit and counted.
+// global_load_lds_dwordx4: lane i's 16 bytes at `src` land at LDS byte address lds_base + 16 i (lds_base uniform)
+__device__ __forceinline__ void pf_copy16_to_lds(const void *src, uint32_t lds_base) {
+  lds_base = __builtin_amdgcn_readfirstlane(lds_base);
+  uint32_t m0_saved;  // the instruction takes the LDS address from m0; m0 is put back, the compiler owns it
+  asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, off\n\ts_mov_b32 m0, %0"
+               : "=&s"(m0_saved)
+               : "s"(lds_base), "v"(src)
+               : "memory");
+}
+// waits until at most N of this wave's copies are in flight (they complete in order)
+template <int N>
+__device__ __forceinline__ void pf_wait_copies() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+// workgroup barrier without a fence: the wave's LDS operations are complete, nothing else is waited for
+__device__ __forceinline__ void pf_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 // dequantize one packed word (8 weights) to 8 bf16, columns ascending
 __device__ __forceinline__ kx_bf16x8 dequant_word(uint32_t w, float sc, float sc16, float c0, float c1, uint32_t magic) {
   const uint32_t w8 = w >> 8;
@@ -99,7 +120,9 @@ __global__ void __launch_bounds__(WAVES * 64, (I4 || WAVES < 8) ? 1 : 2) grouped
   uint16_t *xs_lds = (uint16_t *)pf_lds;                 // two activation tiles
   uint8_t *w_ring = pf_lds + 2 * XT * 2;                 // INT4: [2 stages][MATS][256 rows][4 pieces of 16 B]
   uint8_t *sc_lds = w_ring + 2 * MATS * W_STAGE;         // INT4: [2][256 rows * MATS][SC_STRIDE]
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const uint32_t ring0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)w_ring;  // LDS address of the ring
+  const uint32_t xs0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)pf_lds;    // and of the activation tiles
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lr = lane & 31, lh = lane >> 5;
   const int n0 = blockIdx.x * (WAVES * 32);
   int4 wk = a.work ? a.work[blockIdx.y] : make_int4(0, 0, a.n_pairs, 0);
@@ -131,9 +154,7 @@ __global__ void __launch_bounds__(WAVES * 64, (I4 || WAVES < 8) ? 1 : 2) grouped
     if (I4) {
 #pragma unroll
       for (int u = 0; u < MATS * 2; ++u)
-        __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *)(dma_src[u] + ss * 16),
-                                         (void __attribute__((address_space(3))) *)(w_ring + (ss & 1) * MATS * W_STAGE + dma_dst[u]),
-                                         16, 0, 0);
+        pf_copy16_to_lds(dma_src[u] + ss * 16, ring0 + (ss & 1) * MATS * W_STAGE + dma_dst[u]);
     }
   };
   // scale staging: thread -> (row, matrix), 16 scales = 8 K steps per load
@@ -172,6 +193,25 @@ __global__ void __launch_bounds__(WAVES * 64, (I4 || WAVES < 8) ? 1 : 2) grouped
       xrow[q] = a.x + (size_t)(pair / a.x_div) * a.K + xc;
     }
 
+    // INT4 path: the activation tile goes global -> LDS like the weights.  A row of a K step is 128 B = 8 pieces;
+    // copy instruction ii covers rows 8 ii .. 8 ii + 7, slot (row, p') holding piece p' ^ ((row >> 1) & 7), so that
+    // the row-per-lane operand reads are free of bank conflicts without padding.  Rows past the expert's tokens
+    // read pair 0: they only feed accumulator rows that are never stored.
+    constexpr int XCMAX = 2;  // copy instructions per wave and K step at 128 tokens
+    const uint16_t *xc_src[XCMAX];
+    int xc_dst[XCMAX];
+    if (I4) {
+#pragma unroll
+      for (int q = 0; q < XCMAX; ++q) {
+        const int ii = min(wave + 8 * q, a.nb_max * 4 - 1);
+        const int slot = ii * 64 + lane, row = slot >> 3, piece = (slot & 7) ^ ((row >> 1) & 7);
+        const int pi = m0 + row;
+        const int pair = pi < p_end ? (a.pairs ? a.pairs[pi] : pi) : 0;
+        xc_src[q] = a.x + (size_t)(pair / a.x_div) * a.K + piece * 8;
+        xc_dst[q] = ii * 1024;
+      }
+    }
+
     // the tile with NB token blocks, NB a compile-time constant so that the K loop has no branches
     auto run = [&](auto nb_c) {
       constexpr int NB = decltype(nb_c)::value;
@@ -189,7 +229,7 @@ __global__ void __launch_bounds__(WAVES * 64, (I4 || WAVES < 8) ? 1 : 2) grouped
       };
       constexpr int XQ = (NB * 32 + XROWS - 1) / XROWS;  // staging passes that hold rows of this tile
       uint4 xv[XQ][2];
-      auto load_x = [&](int ks) {
+      auto load_x = [&](int ks) {  // bf16 weights: activations through registers
 #pragma unroll
         for (int q = 0; q < XQ; ++q) {
           xv[q][0] = xv[q][1] = make_uint4(0, 0, 0, 0);
@@ -206,6 +246,11 @@ __global__ void __launch_bounds__(WAVES * 64, (I4 || WAVES < 8) ? 1 : 2) grouped
             *(uint4 *)(st + (q * XROWS + xr) * LDS_STRIDE + xc) = xv[q][0];
             *(uint4 *)(st + (q * XROWS + xr) * LDS_STRIDE + xc + 8) = xv[q][1];
           }
+      };
+      constexpr int XC = (NB * 4 + 7) / 8;  // INT4: activation copies per wave and K step (every wave issues XC)
+      auto copy_x = [&](int ks) {            // activations of K step ks into tile ks % 2
+#pragma unroll
+        for (int q = 0; q < XC; ++q) pf_copy16_to_lds(xc_src[q] + ks * BK, xs0 + (ks & 1) * XT * 2 + xc_dst[q]);
       };
       // this lane's weights of K step ks: INT4 from the LDS ring and the staged scales, bf16 from memory
       auto fetch_w = [&](WRaw &r, int ks) {
@@ -236,9 +281,15 @@ __global__ void __launch_bounds__(WAVES * 64, (I4 || WAVES < 8) ? 1 : 2) grouped
         }
       };
       auto read_a = [&](const uint16_t *xs, int j, kx_bf16x8 (&av)[NB]) {
-        const int kcol = lh * 32 + j * 8;
+        if (I4) {  // 128-byte rows, pieces xor-swizzled by the row
+          const int off = lr * 128 + (((lh * 4 + j) ^ (lr >> 1)) & 7) * 16;
 #pragma unroll
-        for (int t = 0; t < NB; ++t) av[t] = *(const kx_bf16x8 *)(xs + (t * 32 + lr) * LDS_STRIDE + kcol);
+          for (int t = 0; t < NB; ++t) av[t] = *(const kx_bf16x8 *)((const uint8_t *)xs + t * 32 * 128 + off);
+        } else {
+          const int kcol = lh * 32 + j * 8;
+#pragma unroll
+          for (int t = 0; t < NB; ++t) av[t] = *(const kx_bf16x8 *)(xs + (t * 32 + lr) * LDS_STRIDE + kcol);
+        }
       };
       constexpr int VPER = I4 ? (34 * MATS + NB * MATS - 1) / (NB * MATS) : 0;  // VALU instructions per MFMA
       auto mfma_group = [&](const kx_bf16x8 (&av)[NB], const kx_bf16x8 (&b)[MATS], auto with_valu) {
@@ -273,34 +324,57 @@ __global__ void __launch_bounds__(WAVES * 64, (I4 || WAVES < 8) ? 1 : 2) grouped
       };
 
       // prologue: stage 0 of the ring, the first scale block, the first activation tile
+      auto barrier = [&]() {
+        if (I4) pf_barrier();
+        else __syncthreads();
+      };
       WRaw w0, w1;
-      dma_stage(0);
       load_scales(0);
-      load_x(0);
-      if (!I4) fetch_w(w0, 0);
+      if (I4) {
+        copy_x(0);
+        dma_stage(0);
+      } else {
+        load_x(0);
+        fetch_w(w0, 0);
+      }
       store_scales(0);
-      store_x(xs_lds);
+      if (!I4) store_x(xs_lds);
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      __syncthreads();
+      barrier();
       for (int ks = 0; ks < nk; ks += 2) {
-        // even step: the other ring stage was last read two steps ago, behind a barrier
-        if (ks + 2 < nk) dma_stage((ks >> 1) + 1);
+        // even step: the other ring stage and the other activation tile were last read behind a barrier.  Order of
+        // issue: scales, activations of the next step, then the ring copies; the activations have to land by the
+        // end of this step, the ring copies stay in flight until the end of the odd step
         if ((ks & 7) == 0 && ks + 8 < nk) load_scales((ks >> 3) + 1);
-        if (ks + 1 < nk) load_x(ks + 1);
-        if (I4) fetch_w(w0, ks);
-        if (!I4 && ks + 1 < nk) fetch_w(w1, ks + 1);
+        if (I4) {
+          if (ks + 1 < nk) copy_x(ks + 1);
+          if (ks + 2 < nk) dma_stage((ks >> 1) + 1);
+          fetch_w(w0, ks);
+        } else {
+          if (ks + 1 < nk) load_x(ks + 1);
+          if (ks + 1 < nk) fetch_w(w1, ks + 1);
+        }
         step(w0, ks);
-        if (ks + 1 < nk) store_x(xs_lds + XT);
-        __syncthreads();
+        if (I4) {
+          if (ks + 2 < nk) pf_wait_copies<MATS * 2>();
+          else pf_wait_copies<0>();
+        } else if (ks + 1 < nk) {
+          store_x(xs_lds + XT);
+        }
+        barrier();
         if (ks + 1 < nk) {
-          if (ks + 2 < nk) load_x(ks + 2);
-          if (I4) fetch_w(w1, ks + 1);
-          if (!I4 && ks + 2 < nk) fetch_w(w0, ks + 2);
+          if (I4) {
+            if (ks + 2 < nk) copy_x(ks + 2);
+            fetch_w(w1, ks + 1);
+          } else {
+            if (ks + 2 < nk) load_x(ks + 2);
+            if (ks + 2 < nk) fetch_w(w0, ks + 2);
+          }
           step(w1, ks + 1);
-          if (ks + 2 < nk) store_x(xs_lds);
+          if (!I4 && ks + 2 < nk) store_x(xs_lds);
           if ((ks & 7) == 6 && ks + 2 < nk) store_scales((ks >> 3) + 1);
-          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's copies into the ring have landed
-          __syncthreads();
+          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's copies (ring stage, activations) have landed
+          barrier();
         }
       }
       // epilogue: D[i][j], j = lane % 32 (weight row), i = 8*(v/4) + 4*(lane/32) + v%4 (token of the 32-token block)
