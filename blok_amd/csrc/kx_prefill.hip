@@ -23,7 +23,9 @@
 //    for eight K steps at a time (32 bytes per row and matrix, one load per thread);
 //  * bf16 weights (shared expert, router gate) are loaded by the lanes themselves, 64
 //    contiguous bytes per lane and step, one step ahead;
-//  * the gathered activation rows go through a double-buffered LDS tile, one barrier per step.
+//  * the gathered activation rows go through a double-buffered LDS tile, one barrier per step; with INT4
+//    weights they are copied global -> LDS as well (128-byte rows, pieces xor-swizzled by the row), with bf16
+//    weights they pass through registers into rows padded to 144 bytes.
 //
 // Dequant without integer conversion: (w & 0x000F000F) | 0x64006400 is the f16 pair
 // (1024+n0, 1024+n4), (w & 0x00F000F0) | 0x64006400 is (1024+16 n1, 1024+16 n5), w >> 8 gives
