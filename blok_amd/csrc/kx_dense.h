@@ -40,10 +40,16 @@ struct KxGemvArgs {
   int topk;
   uint32_t flags;              // bit 0: MOE_COMBINE overwrites x; KX_GEMV_COHERENT_OUT: see below
 };
-// F32 epilogue: store the outputs with device-scope stores (another workgroup of the launch reads them)
+// F32 and BF16 epilogues: store the outputs with device-scope stores (another workgroup of the launch reads them)
 #define KX_GEMV_COHERENT_OUT 2u
 
 int kx_gemv_launch(int epi, KxGemvArgs a, hipStream_t st);
+// The q_b GEMV (g: rows = heads * (nope + rope), bf16 epilogue) that also finishes the query: the workgroup that
+// completes a head last computes q_abs of that head (W_UK absorb + RoPE, the sums of q_absorb_k), and one extra
+// workgroup norms kv_a, rotates the rope key and writes the cache row.  head_count: one zeroed int per head.
+// Returns KX_OK with *fused = false, having launched nothing, when the shapes do not allow it.
+struct QAbsArgs;
+int kx_gemv_absorb_launch(KxGemvArgs g, const QAbsArgs &q, bool *fused, hipStream_t st);
 int kx_rmsnorm_launch(const uint16_t *x, const uint16_t *w, uint16_t *y, int tokens, int n, int x_stride,
                       int y_stride, float eps, hipStream_t st);
 int kx_argmax_launch(const float *logits, int tokens, int n, int stride, uint32_t *out, float *scratch, hipStream_t st);

@@ -13,6 +13,7 @@
 //   lane partial  p[s][l] = fma chain over e = 0..7 of w[r, 512 s + 8 l + e] * x[t, ...]
 //   slice sum     B[s]    = xor-butterfly over the 64 lanes (32,16,8,4,2,1)
 //   row sum       y       = B[0] + B[1] + ... + B[S-1], left to right
+#include "kx_attn_parts.h"
 #include "kx_common.h"
 #include "kx_dense.h"
 #include "kx_gemv_body.h"
@@ -108,6 +109,37 @@ __global__ void __launch_bounds__(TT > 1 ? 512 : 1024) gemv_pair_k(KxGemvArgs a0
   kxr::route_block_any<true>((const float *)a1.out, r.bias, r.ids, r.weights, a1.tokens, r.experts, r.topk, r.routed_scale,
                        r.counts, r.offsets, r.pairs, r.work, r.n_active, s_ids4, s_cnt, s_act);
   if (threadIdx.x == 0) *r.counter = 0;
+}
+
+// The q_b GEMV that also finishes the query.  Workgroup 0 norms kv_a, rotates the shared rope key and writes the
+// cache row; workgroup 1 + c computes chunk c of q (device-scope stores) and counts itself in on the counter of
+// its head; the one that counts in last has all of the head's q in memory and computes q_abs of the head (W_UK
+// absorb + RoPE) while other heads are still streaming.  Nothing waits for another workgroup.
+template <int RI, int TT>
+__global__ void __launch_bounds__(TT > 1 ? 512 : 1024) gemv_absorb_k(KxGemvArgs a, QAbsArgs q) {
+  extern __shared__ float part[];
+  __shared__ float ab_part[8 * 512];
+  __shared__ float ab_q[256];
+  __shared__ float ab_ws[4];
+  __shared__ int s_last;
+  if (blockIdx.x == 0) {
+    const int kva = q.kv_rank + q.rope;
+    for (int t = 0; t < a.tokens; ++t)
+      kxa::kv_finish_block(q.kva + (size_t)t * q.kva_stride, q.w_kv_ln, q.rope_row,
+                           q.cache + (size_t)t * q.seq_stride + (size_t)q.pos * kva, q.kv_rank, q.rope, q.eps, ab_ws);
+    return;
+  }
+  const int chunk = blockIdx.x - 1;
+  gemv_body<1, RI, TT>(a, chunk, gridDim.x - 1, part);
+  __builtin_amdgcn_s_waitcnt(0);  // this wave's stores of q have been acknowledged
+  __syncthreads();
+  const int h = chunk / q.head_chunks;
+  if (threadIdx.x == 0)
+    s_last = __hip_atomic_fetch_add(q.head_count + h, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == q.head_chunks - 1;
+  __syncthreads();
+  if (!s_last) return;
+  kxa::absorb_head_block(q, h, a.tokens, ab_part, ab_q);
+  if (threadIdx.x == 0) q.head_count[h] = 0;
 }
 
 // lowest-index argmax over bf16-rounded logits (sample_lm_head :718-734, argmax_k :477-493), in two
@@ -283,6 +315,37 @@ int kx_gemv_pair_route_launch(KxGemvArgs a0, KxGemvArgs a1, const float *bias, u
   if (ri0 == 2) { if (tt == 4) KX_PAIR(2, 4); else if (tt == 2) KX_PAIR(2, 2); else KX_PAIR(2, 1); }
   else          { if (tt == 4) KX_PAIR(1, 4); else if (tt == 2) KX_PAIR(1, 2); else KX_PAIR(1, 1); }
 #undef KX_PAIR
+  KX_LAUNCH_CHECK();
+  *fused = true;
+  return KX_OK;
+}
+
+int kx_gemv_absorb_launch(KxGemvArgs g, const QAbsArgs &q0, bool *fused, hipStream_t st) {
+  *fused = false;
+  QAbsArgs q = q0;
+  const int qk = q.nope + q.rope;
+  if (g.tokens > 4 || g.rows != q.heads * qk || q.kv_rank > 512 || q.kv_rank % 8 || qk > 256 || qk % 2 || q.rope % 2 ||
+      !q.head_count || !q.cache)
+    return KX_OK;
+  int ri;
+  const int CR = gemv_plan(KX_EPI_BF16, g, ri, 4);
+  if (CR < 0) return KX_ERR_ARG;
+  const int threads = g.nw * g.rs * 64;
+  if (qk % CR || g.rows / CR + 1 > 4096 || (threads < 256 && q.kv_rank / 8 > threads) || q.rope / 2 > threads) return KX_OK;
+  q.head_chunks = qk / CR;
+  g.flags |= KX_GEMV_COHERENT_OUT;
+  const int S = g.cols / 512;
+  const size_t lds = (size_t)CR * g.tokens * S * sizeof(float);
+  KX_REQUIRE(lds <= 128 * 1024, "kx_gemv: %zu bytes of LDS needed", lds);
+  const int tt = g.tokens >= 4 ? 4 : g.tokens >= 2 ? 2 : 1;
+  dim3 grid(g.rows / CR + 1), blk(threads);
+#define KX_ABS(R, TT_) hipLaunchKernelGGL((gemv_absorb_k<R, TT_>), grid, blk, lds, st, g, q)
+#define KX_ABS_TT(R) do { if (tt == 4) KX_ABS(R, 4); else if (tt == 2) KX_ABS(R, 2); else KX_ABS(R, 1); } while (0)
+  if (ri == 4) KX_ABS_TT(4);
+  else if (ri >= 2) KX_ABS_TT(2);
+  else KX_ABS_TT(1);
+#undef KX_ABS_TT
+#undef KX_ABS
   KX_LAUNCH_CHECK();
   *fused = true;
   return KX_OK;

@@ -26,6 +26,7 @@
 //   q_lat      eight chains over d = j, j+8, ... then ((0+1)+(2+3))+((4+5)+(6+7))
 #include <math.h>
 #include <type_traits>
+#include "kx_attn_parts.h"
 #include "kx_common.h"
 #include "kx_dense.h"
 #include "kx_math.h"
@@ -89,90 +90,16 @@ int kx_mla_span_tiles(int seq) {
 
 namespace {
 
-__device__ __forceinline__ float bf_lo(uint32_t u) { return kx_bits_f32(u << 16); }
-__device__ __forceinline__ float bf_hi(uint32_t u) { return kx_bits_f32(u & 0xffff0000u); }
-__device__ __forceinline__ void unpack8(float (&f)[8], uint4 u) {
-  f[0] = bf_lo(u.x); f[1] = bf_hi(u.x); f[2] = bf_lo(u.y); f[3] = bf_hi(u.y);
-  f[4] = bf_lo(u.z); f[5] = bf_hi(u.z); f[6] = bf_lo(u.w); f[7] = bf_hi(u.w);
-}
-
-// RMSNorm of one row by the first 256 threads of a workgroup; the schedule of rmsnorm_k (kx_dense.hip).
-// Every thread of the workgroup must call it (it contains barriers).  A workgroup of fewer than 256
-// threads must cover the row's n/8 chunks with one chunk per thread (the missing waves add +0).
-__device__ __forceinline__ void rmsnorm_block(const uint16_t *xr, const uint16_t *w, uint16_t *yr, int n, float eps,
-                                              float *ws /* 4 floats of LDS */) {
-  const int chunks = n >> 3;
-  const bool active = threadIdx.x < 256;
-  float v = 0.0f;
-  if (active)
-    for (int c = threadIdx.x; c < chunks; c += 256) {
-      float f[8];
-      unpack8(f, ((const uint4 *)xr)[c]);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) v = __builtin_fmaf(f[e], f[e], v);
-    }
-  float vv[1] = {v};
-  kxw::reduce<1, 64>(vv, threadIdx.x & 63);
-  __syncthreads();  // ws may still be read from a previous call
-  if (threadIdx.x < 4) ws[threadIdx.x] = 0.0f;
-  __syncthreads();
-  if (active && (threadIdx.x & 63) == 0) ws[threadIdx.x >> 6] = vv[0];
-  __syncthreads();
-  const float total = ((ws[0] + ws[1]) + ws[2]) + ws[3];
-  const float scale = kx_rsqrtf(total / (float)n + eps);
-  if (active)
-    for (int c = threadIdx.x; c < chunks; c += 256) {
-      float f[8], g[8];
-      unpack8(f, ((const uint4 *)xr)[c]);
-      unpack8(g, ((const uint4 *)w)[c]);
-      uint32_t o[4];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        uint32_t a = kx_bf16_rne(kx_bfround(f[2 * e] * scale) * g[2 * e]);
-        uint32_t b = kx_bf16_rne(kx_bfround(f[2 * e + 1] * scale) * g[2 * e + 1]);
-        o[e] = a | (b << 16);
-      }
-      ((uint4 *)yr)[c] = make_uint4(o[0], o[1], o[2], o[3]);
-    }
-}
-
-// interleaved-pair rotation of rope_k (:352-356): reads (2p, 2p+1), writes (p, half+p)
-__device__ __forceinline__ void rope_pair(float x0, float x1, float c, float s, float &y_lo, float &y_hi) {
-  y_lo = kx_bfround(kx_bfround(x0 * c) - kx_bfround(x1 * s));
-  y_hi = kx_bfround(kx_bfround(x1 * c) + kx_bfround(x0 * s));
-}
-
-// kv_a RMSNorm on the latent part only (:817), RoPE of the shared rope key (:820-823) and the write of
-// the cache row (:824) for token t; kva bf16 [kv_rank + rope] is the kv_a output of the token.
-__device__ __forceinline__ void kv_finish_block(const uint16_t *kva, const uint16_t *w_kv_ln, const uint16_t *rope_row,
-                                                uint16_t *crow, int kv_rank, int rope, float eps, float *ws) {
-  rmsnorm_block(kva, w_kv_ln, crow, kv_rank, eps, ws);
-  const int half = rope >> 1;
-  if ((int)threadIdx.x < half) {
-    const int p = threadIdx.x;
-    const uint16_t *kr = kva + kv_rank;
-    float lo, hi;
-    rope_pair(kx_bf16_f32(kr[2 * p]), kx_bf16_f32(kr[2 * p + 1]), kx_bf16_f32(rope_row[p]), kx_bf16_f32(rope_row[half + p]),
-              lo, hi);
-    crow[kv_rank + p] = kx_bf16_rne(lo);
-    crow[kv_rank + half + p] = kx_bf16_rne(hi);
-  }
-}
+using kxg::bf_hi;
+using kxg::bf_lo;
+using kxg::unpack8;
+using namespace kxa;
 
 // q_abs[t][h] = (bf(W_UK[h]^T q_nope[h]) | rope(q_rope[h])) as f32.  A workgroup of 128 threads takes
 // 128 latent columns of one head: thread (chain, cl) = (tid / 16, tid % 16) runs the fma chain over
 // d = chain, chain+8, ... for columns 8 cl .. 8 cl + 7; the 8 chains are then summed pairwise.
 // Grid (heads * ceil(kv_rank / 128) + 1, T): the extra workgroup finishes the token's kv_a output and
 // writes its cache row.
-struct QAbsArgs {
-  const uint16_t *q, *kvb, *rope_row;
-  float *qabs;
-  const uint16_t *kva, *w_kv_ln;  // kva: first kv_a output row, kva_stride elements between tokens
-  uint16_t *cache;
-  size_t seq_stride;
-  int heads, nope, rope, v_head, kv_rank, kva_stride, pos;
-  float eps;
-};
 __global__ void __launch_bounds__(128) q_absorb_k(QAbsArgs a) {
   __shared__ float part[8][128];
   __shared__ float ws[4];
@@ -691,7 +618,7 @@ int kx_q_absorb_launch(const uint16_t *q, const uint16_t *kvb, const uint16_t *r
                        int heads, int nope, int rope, int v_head, int kv_rank, const uint16_t *kva, int kva_stride,
                        const uint16_t *w_kv_ln, uint16_t *cache, size_t seq_stride, int pos, float eps, hipStream_t st) {
   KX_REQUIRE(kv_rank % 8 == 0 && kv_rank <= 1024 && rope % 2 == 0 && rope / 2 <= 128, "kx_q_absorb: kv_rank=%d (multiple of 8, at most 1024), rope=%d (even, at most 256)", kv_rank, rope);
-  QAbsArgs a;
+  QAbsArgs a = {};
   a.q = q; a.kvb = kvb; a.rope_row = rope_row; a.qabs = qabs; a.kva = kva; a.w_kv_ln = w_kv_ln; a.cache = cache;
   a.seq_stride = seq_stride; a.heads = heads; a.nope = nope; a.rope = rope; a.v_head = v_head; a.kv_rank = kv_rank;
   a.kva_stride = kva_stride; a.pos = pos; a.eps = eps;

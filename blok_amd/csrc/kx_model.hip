@@ -21,6 +21,7 @@
 #include <math.h>
 #include <string.h>
 #include <vector>
+#include "kx_attn_parts.h"
 #include "kx_common.h"
 #include "kx_dense.h"
 #include "kx_index.h"
@@ -67,6 +68,8 @@ struct kx_model {
   uint16_t *x, *n, *qkv, *qa, *q, *o_lat, *att, *dmid;
   float *qabs, *partial, *logits, *argmax_scratch;
   uint32_t *ids, *next, *history;  // [max_context][B], [B], [max_context][B]
+  int *head_count;                 // [heads] arrival counters of the q_b GEMV that finishes the query; zero between launches
+  uint32_t fusion = KX_FUSE_ALL;
   kx_moe_workspace *moe_ws = nullptr;
   hipStream_t st = nullptr;
   hipEvent_t ev[3] = {nullptr, nullptr, nullptr};
@@ -170,11 +173,13 @@ int layout(const kx_config *c, Plan &p, kx_model *m) {
   auto *ids = KX_AT(uint32_t *, (size_t)c->max_context * B * 4);
   auto *next = KX_AT(uint32_t *, B * 4);
   auto *history = KX_AT(uint32_t *, (size_t)c->max_context * B * 4);
+  auto *head_count = KX_AT(int *, (size_t)c->heads * 4);
 #undef KX_AT
   p.scratch = p.total - p.weights - p.cache;
   if (m) {
     m->x = x; m->n = n; m->qkv = qkv; m->qa = qa; m->q = q; m->o_lat = o_lat; m->att = att; m->dmid = dmid;
     m->qabs = qabs; m->partial = partial; m->logits = logits; m->argmax_scratch = argmax_scratch; m->ids = ids; m->next = next; m->history = history;
+    m->head_count = head_count;
   }
   return KX_OK;
 }
@@ -272,10 +277,22 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample) {
     g.w0 = L.qb; g.x = m->qa; g.x_stride = c.q_rank; g.out = m->q; g.out_stride = KD; g.rows = KD; g.cols = c.q_rank; g.tokens = B;
     if (fuse) { g.x = m->qkv; g.x_stride = QKV; g.norm_w = L.qa_ln; g.norm_eps = c.rms_eps; }
     else KX_TRY(kx_rmsnorm_launch(m->qkv, L.qa_ln, m->qa, B, c.q_rank, QKV, c.q_rank, c.rms_eps, st)); // :814
-    KX_TRY(dense(KX_EPI_BF16, g));                                                                      // :815
-    // W_UK absorb + rope(q); the extra block norms kv_a, rotates the rope key, writes the cache row (:817-824)
-    KX_TRY(kx_q_absorb_launch(m->q, L.kvb, rope_row, m->qabs, B, c.heads, c.qk_nope, c.qk_rope, c.v_head, c.kv_rank,
-                              m->qkv + c.q_rank, QKV, L.kv_ln, L.cache, seq_stride, pos, c.rms_eps, st));
+    // W_UK absorb + rope(q); kv_a norm, rope of the shared key, cache row (:817-824): inside the q_b launch when
+    // the shapes allow, else as a kernel of their own
+    bool absorbed = false;
+    if (fuse && (m->fusion & KX_FUSE_ABSORB)) {
+      QAbsArgs qa = {};
+      qa.q = m->q; qa.kvb = L.kvb; qa.rope_row = rope_row; qa.qabs = m->qabs; qa.kva = m->qkv + c.q_rank; qa.kva_stride = QKV;
+      qa.w_kv_ln = L.kv_ln; qa.cache = L.cache; qa.seq_stride = seq_stride; qa.heads = c.heads; qa.nope = c.qk_nope;
+      qa.rope = c.qk_rope; qa.v_head = c.v_head; qa.kv_rank = c.kv_rank; qa.pos = pos; qa.eps = c.rms_eps;
+      qa.head_count = m->head_count;
+      KX_TRY(kx_gemv_absorb_launch(g, qa, &absorbed, st));                                             // :815
+    }
+    if (!absorbed) {
+      KX_TRY(dense(KX_EPI_BF16, g));                                                                    // :815
+      KX_TRY(kx_q_absorb_launch(m->q, L.kvb, rope_row, m->qabs, B, c.heads, c.qk_nope, c.qk_rope, c.v_head, c.kv_rank,
+                                m->qkv + c.q_rank, QKV, L.kv_ln, L.cache, seq_stride, pos, c.rms_eps, st));
+    }
     g = {};  // W_UV of :818 per head
     g.w0 = L.kvb; g.x = m->o_lat; g.x_stride = c.heads * c.kv_rank; g.out = m->att; g.out_stride = VD; g.rows = VD;
     g.cols = c.kv_rank; g.tokens = B; g.row_block = c.v_head; g.w_block_stride = c.qk_nope + c.v_head;
@@ -363,6 +380,8 @@ static int model_new(const kx_config *cfg, const char *who, kx_model **out) {
   for (auto &ev : m->ev)
     if (!rc && hipEventCreate(&ev) != hipSuccess) rc = KX_ERR_HIP;
   if (!rc && cfg->first_dense < cfg->n_layers) rc = kx_moe_workspace_create(cfg, cfg->max_batch, &m->moe_ws);
+  if (!rc && (hipMemsetAsync(m->head_count, 0, (size_t)cfg->heads * 4, m->st) != hipSuccess || hipStreamSynchronize(m->st) != hipSuccess))
+    rc = KX_ERR_HIP;
   if (rc) {
     if (rc == KX_ERR_HIP && !kx_last_error()[0]) kx_set_error("%s: HIP resource creation failed", who);
     kx_model_destroy(m);
@@ -553,6 +572,13 @@ extern "C" int kx_generate(kx_model *m, const uint32_t *h_prompt, int32_t batch,
     }
     h_counts[b] = n;
   }
+  return KX_OK;
+}
+
+extern "C" int kx_model_set_fusion(kx_model *m, uint32_t mask) {
+  KX_REQUIRE(m, "kx_model_set_fusion: null model");
+  KX_REQUIRE(!(mask & ~(uint32_t)KX_FUSE_ALL), "kx_model_set_fusion: unknown bits in mask 0x%x", mask);
+  m->fusion = mask;
   return KX_OK;
 }
 

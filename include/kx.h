@@ -285,6 +285,13 @@ int kx_model_latent(kx_model *model, int32_t layer, int32_t seq_index, int32_t p
 int kx_model_stream(kx_model *model, void **stream);
 /* ms of GPU time of the last kx_generate: [0] prefill, [1] decode steps                         */
 int kx_model_timing(kx_model *model, float *ms2);
+/* Which steps of a decode layer ride inside the launch of the GEMV before them (up to 4 tokens).
+ * Results do not depend on the mask (same sums, same rounding points); it exists so that a test
+ * can run both forms.  No counterpart in the reference, which launches every step on its own
+ * (src/kimi_exec.cu:812-827).  Default KX_FUSE_ALL.                                            */
+#define KX_FUSE_ABSORB 1u /* W_UK absorb, RoPE of q, kv_a norm + cache row: inside the q_b GEMV */
+#define KX_FUSE_ALL 1u
+int kx_model_set_fusion(kx_model *model, uint32_t mask);
 /* bf(mean + sigma*z) fill used for the norm weights */
 int kx_fill_affine_bf16(void *d_out, uint64_t n, uint64_t seed, uint64_t tensor_id, float mean,
                         float sigma, void *stream);

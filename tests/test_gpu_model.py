@@ -187,6 +187,36 @@ def test_kimi_shape_truncated_stack_tokens_identical(kxlib, ox):
     km.close(); om.close()
 
 
+@pytest.mark.parametrize("shape", ["small-1", "small-3", "kimi"])
+def test_fused_and_separate_launches_agree(kxlib, ox, shape):
+    # the q_b GEMV that finishes the query in its own launch against the same steps as kernels of their own:
+    # cache rows, hidden state, logits and ids to the bit (the oracle comparison above runs the fused form)
+    say(f"fusion on/off {shape}")
+    if shape == "kimi":
+        cfg = default_config()
+        cfg.n_layers, cfg.first_dense, cfg.max_batch, cfg.max_context, cfg.seed = 2, 1, 1, 32, 11
+        batch, prompt_len, n_tokens = 1, 5, 4
+    else:
+        batch = int(shape[-1])
+        cfg = O.small_config(batch=batch, context=64)
+        prompt_len, n_tokens = 11, 9
+    prompt = O.tokens_u32(batch * prompt_len, cfg.seed, 4, cfg.vocab).reshape(batch, prompt_len)
+    got = []
+    for mask in (1, 0):
+        km = KxModel(kxlib, cfg)
+        check(kxlib.kx_model_set_fusion(km.h, mask))
+        rc, out, _ = km.generate(prompt, n_tokens)
+        assert rc == 0, kxlib.kx_last_error()
+        total = prompt_len + n_tokens - 1
+        lat = [km.latent(layer, b, total) for layer in range(cfg.n_layers) for b in range(batch)]
+        got.append((out, km.hidden(batch), km.logits(batch).view(np.uint32), lat))
+        km.close()
+    assert kxlib.kx_model_set_fusion(None, 1) != 0
+    (o1, h1, l1, c1), (o0, h0, l0, c0) = got
+    assert all((a == b).all() for a, b in zip(c1, c0)), "latent cache differs"
+    assert (h1 == h0).all() and (l1 == l0).all() and (o1 == o0).all()
+
+
 @pytest.mark.parametrize("batch,seq", [(1, 1), (1, 100), (2, 700), (1, 5000)])
 def test_mla_decode_operator(kxlib, ox, batch, seq):
     # BASELINE config 3 shapes (64 heads, latent 512+64) at lengths the scalar oracle finishes quickly
