@@ -56,6 +56,27 @@ int kx_argmax_launch(const float *logits, int tokens, int n, int stride, uint32_
 #define KX_ARGMAX_SCRATCH_FLOATS(tokens) ((size_t)(tokens) * 128)
 
 // kx_i4.hip
+// What the routed down launch needs to finish the MoE layer itself (up to 4 tokens): its workgroups and those of the
+// shared expert's down GEMV, which ride in the same launch, count themselves in per block of output rows; whichever
+// completes a block combines it (expert_accum_k / round_bf16_k :399-407, the shared add :684, the residual :877).
+struct KxMoeTail {
+  int *counter;          // one per row block, zero between launches; nullptr: no tail
+  const int *n_active;   // experts with work (device value written by the routing)
+  int shared_chunks;     // chunks of the shared down GEMV per row block
+  const uint16_t *sy;    // bf16 [tokens, rows]: the shared down GEMV's output (device-scope stores)
+  const float *route_w;  // f32 [tokens, topk]
+  uint16_t *x;           // residual rows, updated in place
+  int x_stride, tokens, topk;
+  uint32_t flags;        // bit 0: x = down instead of x += down
+};
+// The routed down GEMV over the work list + the shared expert's down GEMV (shared: weights, activations, rows, cols,
+// tokens; its output goes to tail.sy) + the combine, in one launch.  Returns KX_OK with *fused = false, having
+// launched nothing, when the shapes do not allow it.
+int kx_i4_down_shared_launch(const uint32_t *packed, const uint16_t *scale, const uint16_t *x, uint16_t *out, const int4 *work,
+                             const int *pairs, int rows, int cols, int x_div, size_t expert_words, size_t expert_scales,
+                             int n_slots, KxGemvArgs shared, KxMoeTail tail, bool *fused, hipStream_t st);
+// the launch shape kx_gemv_launch would give a GEMV (fills a.nw, a.rs, a.nt, a.epi); returns rows per chunk or -1
+int kx_gemv_plan(int epi, KxGemvArgs &a, int *ri);
 // cnt_lo..cnt_hi: only the experts of the work list with that many pairs are processed (0, INT_MAX: all)
 int kx_i4_launch(bool dual, const uint32_t *packed0, const uint16_t *scale0, const uint32_t *packed1,
                  const uint16_t *scale1, const uint16_t *x, uint16_t *out, const int4 *work,
@@ -88,5 +109,7 @@ int kx_moe_combine_launch(const uint16_t *eout, const float *rw, const uint16_t 
 // kx_moe.hip: the decode layer with the post-attention RMSNorm fused into the router GEMV.
 // When norm_w is set, d_x is normed on the fly and the normed rows are written to d_n first.
 struct kx_moe_workspace;
+// flag for kx_moe_layer_launch (beside bit 0): keep the shared down GEMV and the combine a launch of their own
+#define KX_MOE_SEPARATE_TAIL 0x100u
 int kx_moe_layer_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_workspace *ws, void *d_n, void *d_x,
                         int tokens, uint32_t flags, const uint16_t *norm_w, hipStream_t st, bool timed);

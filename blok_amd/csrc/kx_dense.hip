@@ -254,6 +254,8 @@ int gemv_plan(int epi, KxGemvArgs &a, int &ri, int ri_max, int target_chunks = 2
 }
 }  // namespace
 
+int kx_gemv_plan(int epi, KxGemvArgs &a, int *ri) { return gemv_plan(epi, a, *ri, 4); }
+
 // Tokens are taken in blocks of at most 32 (LDS holds a partial per token and slice).
 int kx_gemv_launch(int epi, KxGemvArgs a, hipStream_t st) {
   int ri;

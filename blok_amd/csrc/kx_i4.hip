@@ -27,6 +27,8 @@
 // All arithmetic is IEEE binary32 (fma, mul, add), so a scalar host program
 // that follows the same order reproduces the result bit for bit.
 #include "kx_common.h"
+#include "kx_dense.h"
+#include "kx_gemv_body.h"
 #include "kx_math.h"
 #include "kx_wave.h"
 
@@ -147,6 +149,7 @@ struct I4Args {
   int nt;      // tiles per chunk
   size_t expert_words, expert_scales;
   int cnt_lo, cnt_hi;  // only experts with cnt_lo <= pairs <= cnt_hi are processed by this launch
+  KxMoeTail tail;      // tail.counter != nullptr: single-matrix launches finish the MoE layer (see moe_tail_arrive)
 };
 
 constexpr int I4_RI = 2;  // rows per half-wave per tile
@@ -154,6 +157,55 @@ constexpr int I4_RI = 2;  // rows per half-wave per tile
 // Rows of a chunk for tiles of rt rows: 32 for the fused gate/up kernel; for one matrix 112 when rt divides it
 // (7168 rows / 112 = 64 chunks per expert: 8 experts fill the 512 resident workgroups exactly once), else 64.
 __host__ __device__ constexpr int i4_chunk_rows(bool dual, int rt) { return dual ? 32 : (112 % rt == 0 ? 112 : 64); }
+
+// Called by every thread of a workgroup that has finished its contributions to the MoE layer's down projection: a
+// routed expert's chunk inside row block blk_a and/or a chunk of the shared expert's down GEMV inside row block
+// blk_b (-1: none), blocks of `block_rows` rows.  The outputs were stored with device-scope stores; the workgroup
+// counts itself in on the counters of its blocks, and where it completes a block -- n_active experts and
+// shared_chunks shared chunks -- it combines it: down = bf(sum_slot y_slot * w_slot) in slot order,
+// down = bf(down + bf(shared)), x = bf(x + down).  Nothing waits for another workgroup.  Counters are left at zero.
+__device__ __forceinline__ void moe_tail_arrive(const KxMoeTail &t, int blk_a, int blk_b, int block_rows, int rows,
+                                                const uint16_t *eout) {
+  __shared__ int s_last[2];
+  __builtin_amdgcn_s_waitcnt(0);  // this wave's stores have been acknowledged
+  __syncthreads();
+  if (threadIdx.x < 2) {
+    const int blk = threadIdx.x ? blk_b : blk_a;
+    int last = 0;
+    if (blk >= 0) {
+      const int target = *t.n_active + t.shared_chunks;
+      last = __hip_atomic_fetch_add(t.counter + blk, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == target - 1;
+    }
+    s_last[threadIdx.x] = last;
+  }
+  __syncthreads();
+  for (int which = 0; which < 2; ++which) {
+    if (!s_last[which]) continue;
+    const int blk = which ? blk_b : blk_a;
+    const int r0 = blk * block_rows;
+    for (int idx = threadIdx.x; idx < block_rows * t.tokens; idx += blockDim.x) {
+      const int rc = idx % block_rows, tok = idx / block_rows, row = r0 + rc;
+      const uint16_t *y = eout + (size_t)tok * t.topk * rows + row;
+      const float *w = t.route_w + (size_t)tok * t.topk;
+      const uint16_t sh = __hip_atomic_load(t.sy + (size_t)tok * rows + row, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      float acc = 0.0f;
+      int k = 0;
+      for (; k + 8 <= t.topk; k += 8) {  // the loads of eight slots go out together; the sum stays in slot order
+        uint16_t v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = __hip_atomic_load(y + (size_t)(k + j) * rows, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc = __builtin_fmaf(kx_bf16_f32(v[j]), w[k + j], acc);
+      }
+      for (; k < t.topk; ++k)
+        acc = __builtin_fmaf(kx_bf16_f32(__hip_atomic_load(y + (size_t)k * rows, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)), w[k], acc);
+      const float down = kx_bfround(kx_bfround(acc) + kx_bf16_f32(sh));
+      uint16_t *xr = t.x + (size_t)tok * t.x_stride + row;
+      *xr = (t.flags & 1u) ? kx_bf16_rne(down) : kx_bf16_rne(kx_bf16_f32(*xr) + down);
+    }
+    if (threadIdx.x == 0) t.counter[blk] = 0;
+  }
+}
 
 // A workgroup of ks*rs waves takes chunks of nt tiles of RT = rs*4 rows of one expert.
 // Wave (s, rset): slice s of rows rset*4 .. rset*4+3 of each tile; its half-waves take
@@ -167,9 +219,10 @@ __host__ __device__ constexpr int i4_chunk_rows(bool dual, int rt) { return dual
 // with identical results, and written once).
 // KS_T > 0 fixes ks (and rs, nt) at compile time; 0 reads them from the arguments.
 // FILTER: the launch processes only the experts whose pair count lies in [cnt_lo, cnt_hi]
-template <bool DUAL, int TT, int KS_T, int MAXT, int WPE, bool FILTER>
-__global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) i4_gemv_k(I4Args a) {
-  extern __shared__ float lds[];
+// `idle` is called once, where the last chunk's loads have landed and nothing more will be requested: what it
+// requests arrives during the epilogue.
+template <bool DUAL, int TT, int KS_T, bool FILTER, class Idle>
+__device__ __forceinline__ void i4_body(const I4Args &a, const int bid, const int nblocks, float *lds, Idle &&idle) {
   constexpr int MATS = DUAL ? 2 : 1;
   constexpr int RI = I4_RI;
   constexpr int NV = RI * MATS * TT;
@@ -240,20 +293,20 @@ __global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(WPE, 
     }
   };
 
-  // the work of the first chunk at or after c (stride gridDim.x) whose expert this launch processes; e < 0: none
+  // the work of the first chunk at or after c (stride nblocks) whose expert this launch processes; e < 0: none
   auto next_work = [&](int &c) {
     Work w = load_work(c < n_chunks ? c : 0);
     if (c >= n_chunks) w.e = -1;
     if (FILTER) {
       while (w.e >= 0 && (w.p_end - w.p_begin < a.cnt_lo || w.p_end - w.p_begin > a.cnt_hi)) {
-        c += gridDim.x;
+        c += nblocks;
         if (c >= n_chunks) { w.e = -1; break; }
         w = load_work(c);
       }
     }
     return w;  // records with work come first: e < 0 ends the list
   };
-  int chunk = blockIdx.x;
+  int chunk = bid;
   if (chunk >= n_chunks) return;
   Work cur = next_work(chunk);
   if (cur.e < 0) return;
@@ -266,7 +319,7 @@ __global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(WPE, 
   bool fresh = true;  // the scales of `cur` have not been made visible to the workgroup yet
 
   while (true) {
-    int nchunk = chunk + gridDim.x;
+    int nchunk = chunk + nblocks;
     bool more = nchunk < n_chunks;
     Work nxt = cur;
     if (more) {
@@ -330,6 +383,7 @@ __global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(WPE, 
         for (int t = 0; t < TT; ++t)
 #pragma unroll
           for (int q = 0; q < 4; ++q) xraw[t][q] = make_uint4(0, 0, 0, 0);
+        idle();
       }
       __syncthreads();
       // sequential sum over the slices, rounding and epilogue
@@ -347,7 +401,10 @@ __global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(WPE, 
             for (int q = 1; q < ks; ++q) y1 += p1[q];
             res = kx_swiglu(kx_bfround(y0), kx_bfround(y1));
           }
-          a.out[(size_t)pair * a.rows + cur.c0 + rc] = kx_bf16_rne(res);
+          if (!DUAL && a.tail.counter)  // read back by another workgroup of this launch
+            __hip_atomic_store(a.out + (size_t)pair * a.rows + cur.c0 + rc, kx_bf16_rne(res), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          else
+            a.out[(size_t)pair * a.rows + cur.c0 + rc] = kx_bf16_rne(res);
         }
       }
       __syncthreads();  // `part` is free again; the next chunk's scale copies are visible to every wave
@@ -357,6 +414,89 @@ __global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(WPE, 
     chunk = nchunk;
     sb ^= 1;
   }
+}
+
+template <bool DUAL, int TT, int KS_T, int MAXT, int WPE, bool FILTER>
+__global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) i4_gemv_k(I4Args a) {
+  extern __shared__ float lds[];
+  i4_body<DUAL, TT, KS_T, FILTER>(a, blockIdx.x, gridDim.x, lds, [] {});
+}
+
+// The routed down GEMV of one token and the shared expert's down GEMV ([rows, 2048] bf16) in one launch.  Workgroup b
+// takes routed chunk b (112 rows of one expert) and then chunk b of the shared matrix (16 rows), whose weights and
+// first tile and activations it requests where the routed chunk's last loads have landed, so that they arrive during
+// its epilogue.
+// Both chunks finish through moe_tail_arrive: the launch leaves the layer's output in x.
+// The shared chunk is computed as kx_gemv_launch computes it for this shape (4 slice waves x 2 row sets, 4 rows per
+// wave and tile, 2 tiles): lane partials over 8 columns, butterfly over the wave, slices summed left to right.
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) i4_down_shared_k(I4Args a, KxGemvArgs g, int n_i4,
+                                                                                                 int n_g) {
+  extern __shared__ float lds[];
+  constexpr int S = 4, RI = 4, RT = 8, CR = 16;  // two tiles of RT rows per chunk
+  const int bid = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wslot = wave & 3, rset = wave >> 2;
+  const bool has_g = bid < n_g;
+  const uint32_t col = (uint32_t)wslot * 512u + (uint32_t)lane * 8u;
+  uint4 gw0[RI], gx = make_uint4(0, 0, 0, 0);
+  bool loaded = false;
+  auto load_tile = [&](uint4 (&w)[RI], int t) {
+#pragma unroll
+    for (int i = 0; i < RI; ++i) w[i] = kxg::ld_stream16(g.w0 + (size_t)(bid * CR + t * RT + rset * RI + i) * g.cols + col);
+  };
+  auto load_shared = [&]() {  // first tile and the activations
+    if (has_g && !loaded) {
+      load_tile(gw0, 0);
+      gx = *(const uint4 *)(g.x + col);
+    }
+    loaded = true;
+  };
+  // one routed chunk per workgroup (the host launches one workgroup per chunk): its row block, if it has work
+  constexpr int BLOCK = i4_chunk_rows(false, 16);
+  int routed_blk = -1;
+  if (bid < n_i4) {
+    i4_body<false, 1, 2, false>(a, bid, n_i4, lds, load_shared);
+    if (a.work[bid / (a.rows / BLOCK)].x >= 0) routed_blk = bid % (a.rows / BLOCK);
+  }
+  load_shared();  // a workgroup without routed work
+  if (!has_g) {
+    if (routed_blk >= 0) moe_tail_arrive(a.tail, routed_blk, -1, BLOCK, a.rows, a.out);
+    return;
+  }
+  uint4 gw1[RI];
+  load_tile(gw1, 1);
+  float xs[8];
+  kxg::unpack8(xs, gx);
+  auto compute_tile = [&](const uint4 (&w)[RI], int t) {
+    float v[RI];
+#pragma unroll
+    for (int i = 0; i < RI; ++i) {
+      float wf[8];
+      kxg::unpack8(wf, w[i]);
+      float acc = 0.0f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc = __builtin_fmaf(wf[e], xs[e], acc);
+      v[i] = acc;
+    }
+    kxw::reduce<RI, 64>(v, lane);
+    if (kxw::reduce_writer<RI, 64>(lane)) {
+#pragma unroll
+      for (int j = 0; j < kxw::reduce_out<RI, 64>(); ++j) {
+        const int i = kxw::reduce_index<RI, 64>(lane, j);
+        lds[(t * RT + rset * RI + i) * S + wslot] = v[j];
+      }
+    }
+  };
+  compute_tile(gw0, 0);
+  compute_tile(gw1, 1);
+  __syncthreads();
+  if (threadIdx.x < CR) {
+    const float *p = lds + threadIdx.x * S;
+    float y = p[0];
+    for (int q = 1; q < S; ++q) y += p[q];
+    __hip_atomic_store((uint16_t *)g.out + bid * CR + threadIdx.x, kx_bf16_rne(y), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  moe_tail_arrive(a.tail, routed_blk, bid * CR / BLOCK, BLOCK, a.rows, a.out);
 }
 
 struct I4Launch {
@@ -417,6 +557,7 @@ int kx_i4_launch(bool dual, const uint32_t *packed0, const uint16_t *scale0, con
   a.rows = rows; a.cols = cols; a.x_div = x_div; a.ks = pl.ks; a.rs = pl.rs; a.nt = pl.nt;
   a.expert_words = expert_words; a.expert_scales = expert_scales;
   a.cnt_lo = cnt_lo; a.cnt_hi = cnt_hi;
+  a.tail = KxMoeTail{};
   long chunks = (long)n_slots * kx_cdiv(rows, pl.cr);
   dim3 g((unsigned)(chunks < 32768 ? chunks : 32768)), b(pl.threads);
   const bool full = pl.rs == (pl.ks >= 5 ? 1 : 8 / pl.ks) && pl.nt == i4_chunk_rows(dual, pl.rs * 4) / (pl.rs * 4);
@@ -434,6 +575,41 @@ int kx_i4_launch(bool dual, const uint32_t *packed0, const uint16_t *scale0, con
     else launch_tt<false, 0, 1024>(a, tt, g, b, pl.lds, st);
   }
   KX_LAUNCH_CHECK();
+  return KX_OK;
+}
+
+int kx_i4_down_shared_launch(const uint32_t *packed, const uint16_t *scale, const uint16_t *x, uint16_t *out, const int4 *work,
+                             const int *pairs, int rows, int cols, int x_div, size_t expert_words, size_t expert_scales,
+                             int n_slots, KxGemvArgs shared, KxMoeTail tail, bool *fused, hipStream_t st) {
+  *fused = false;
+  if (tail.tokens != 1 || shared.tokens != 1 || !tail.counter || !work || shared.rows != rows) return KX_OK;
+  I4Launch pl;
+  int rc = plan(cols, rows, 1, 1, pl);
+  if (rc) return rc;
+  if (!(pl.ks == 2 && pl.rs == 4 && pl.cr == i4_chunk_rows(false, 16) && rows % pl.cr == 0)) return KX_OK;
+  // the kernel computes the shared chunk with the launch shape kx_gemv_launch gives this matrix
+  int ri;
+  shared.out = (void *)tail.sy;
+  shared.out_stride = rows;
+  if (kx_gemv_plan(KX_EPI_BF16, shared, &ri) < 0) return KX_ERR_ARG;
+  if (!(shared.cols == 2048 && ri == 4 && shared.nw == 4 && shared.rs == 2) || shared.row_block || shared.norm_w) return KX_OK;
+  const int g_cr = 16;
+  if (pl.cr % g_cr || rows % g_cr) return KX_OK;
+  tail.shared_chunks = pl.cr / g_cr;
+  const long n_i4 = (long)n_slots * (rows / pl.cr), n_g = rows / g_cr;
+  if (n_i4 > 32768 || n_g > 32768) return KX_OK;
+  const size_t lds_g = (size_t)g_cr * 4 * sizeof(float);
+  const size_t lds = pl.lds > lds_g ? pl.lds : lds_g;
+  I4Args a;
+  a.packed0 = packed; a.scale0 = scale; a.packed1 = nullptr; a.scale1 = nullptr;
+  a.x = x; a.out = out; a.work = work; a.pairs = pairs; a.n_pairs = 0; a.n_slots = n_slots;
+  a.rows = rows; a.cols = cols; a.x_div = x_div; a.ks = pl.ks; a.rs = pl.rs; a.nt = pl.nt;
+  a.expert_words = expert_words; a.expert_scales = expert_scales;
+  a.cnt_lo = 0; a.cnt_hi = 0x7fffffff;
+  a.tail = tail;
+  hipLaunchKernelGGL(i4_down_shared_k, dim3((unsigned)(n_i4 > n_g ? n_i4 : n_g)), dim3(512), lds, st, a, shared, (int)n_i4, (int)n_g);
+  KX_LAUNCH_CHECK();
+  *fused = true;
   return KX_OK;
 }
 

@@ -18,6 +18,8 @@
 #include "kx_common.h"
 #include "kx_dense.h"
 
+constexpr int KX_TAIL_BLOCKS = 1024;
+
 struct kx_moe_workspace {
   int max_tokens;
   kx_config cfg;
@@ -30,6 +32,7 @@ struct kx_moe_workspace {
   int4 *work;         // [E] {expert, first, last, first pair}
   int *n_active;      // [1]
   int *route_counter; // [1] zero between launches: workgroups of the router GEMV count themselves in
+  int *tail_count;    // [KX_TAIL_BLOCKS] zero between launches: arrivals per block of output rows (routed down + shared down)
   uint16_t *mid;      // [T*topk, moe_inter]
   uint16_t *eout;     // [T*topk, hidden]
   uint16_t *smid;     // [T, shared_inter]
@@ -60,7 +63,7 @@ extern "C" int kx_moe_workspace_create(const kx_config *cfg, int32_t max_tokens,
   struct { void **p; size_t bytes; } allocs[] = {
       {(void **)&ws->logits, T * E * 4}, {(void **)&ws->ids, T * K * 2}, {(void **)&ws->weights, T * K * 4},
       {(void **)&ws->counts, E * 4}, {(void **)&ws->offsets, (E + 1) * 4}, {(void **)&ws->pairs, T * K * 4},
-      {(void **)&ws->work, E * 16}, {(void **)&ws->n_active, 8},
+      {(void **)&ws->work, E * 16}, {(void **)&ws->n_active, 8}, {(void **)&ws->tail_count, KX_TAIL_BLOCKS * 4},
       {(void **)&ws->mid, T * K * (size_t)cfg->moe_inter * 2}, {(void **)&ws->eout, T * K * (size_t)cfg->hidden * 2},
       {(void **)&ws->smid, T * (size_t)cfg->shared_inter * 2}, {(void **)&ws->sy, T * (size_t)cfg->hidden * 2}};
   for (auto &al : allocs) {
@@ -73,6 +76,7 @@ extern "C" int kx_moe_workspace_create(const kx_config *cfg, int32_t max_tokens,
   }
   ws->route_counter = ws->n_active + 1;
   KX_HIP(hipMemset(ws->n_active, 0, 8));
+  KX_HIP(hipMemset(ws->tail_count, 0, KX_TAIL_BLOCKS * 4));
   for (auto &e : ws->ev) KX_HIP(hipEventCreate(&e));
   *out = ws;
   return KX_OK;
@@ -182,8 +186,24 @@ int kx_moe_layer_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_work
   // routed gate/up + SwiGLU
   if ((rc = routed_launch(c, w, ws, n, tokens, 0, st))) return rc;
   if (timed) KX_HIP(hipEventRecord(ws->ev[2], st));
+  // shared down + combine + residual: as the epilogue of a GEMV of its own, or, for one token, inside the routed
+  // down launch (whichever workgroup completes a block of rows combines it)
+  KxGemvArgs d = {};
+  d.w0 = (const uint16_t *)w->d_shared_down; d.x = ws->smid; d.x_stride = c->shared_inter; d.out = d_x;
+  d.out_stride = H; d.rows = H; d.cols = c->shared_inter; d.tokens = tokens; d.expert_out = ws->eout;
+  d.route_w = ws->weights; d.topk = K; d.flags = flags & 1u;
+  bool tailed = false;
+  if (paired && tokens == 1 && !(flags & KX_MOE_SEPARATE_TAIL) && H / 16 <= KX_TAIL_BLOCKS) {
+    KxMoeTail t = {};
+    t.counter = ws->tail_count; t.n_active = ws->n_active; t.sy = ws->sy; t.route_w = ws->weights; t.x = (uint16_t *)d_x;
+    t.x_stride = H; t.tokens = tokens; t.topk = K; t.flags = flags & 1u;
+    const int I = c->moe_inter;
+    if ((rc = kx_i4_down_shared_launch((const uint32_t *)w->d_down_packed, (const uint16_t *)w->d_down_scale, ws->mid, ws->eout,
+                                       ws->work, ws->pairs, H, I, 1, (size_t)H * (I / 8), (size_t)H * (I / 32),
+                                       (long)tokens * K < E ? tokens * K : E, d, t, &tailed, st))) return rc;
+  }
   // routed down
-  if ((rc = routed_launch(c, w, ws, n, tokens, 1, st))) return rc;
+  if (!tailed && (rc = routed_launch(c, w, ws, n, tokens, 1, st))) return rc;
   if (timed) KX_HIP(hipEventRecord(ws->ev[3], st));
   // shared gate/up + SwiGLU when it did not ride with the router
   if (!paired) {
@@ -191,12 +211,7 @@ int kx_moe_layer_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_work
     if ((rc = kx_gemv_launch(KX_EPI_SWIGLU, s, st))) return rc;
   }
   if (timed) KX_HIP(hipEventRecord(ws->ev[4], st));
-  // shared down + combine + residual
-  KxGemvArgs d = {};
-  d.w0 = (const uint16_t *)w->d_shared_down; d.x = ws->smid; d.x_stride = c->shared_inter; d.out = d_x;
-  d.out_stride = H; d.rows = H; d.cols = c->shared_inter; d.tokens = tokens; d.expert_out = ws->eout;
-  d.route_w = ws->weights; d.topk = K; d.flags = flags;
-  if ((rc = kx_gemv_launch(KX_EPI_MOE_COMBINE, d, st))) return rc;
+  if (!tailed && (rc = kx_gemv_launch(KX_EPI_MOE_COMBINE, d, st))) return rc;
   if (timed) KX_HIP(hipEventRecord(ws->ev[5], st));
   return KX_OK;
 }

@@ -159,7 +159,9 @@ int kx_moe_workspace_views(kx_moe_workspace *ws, void **d_logits, void **d_ids, 
 /* d_n   bf16 [T, hidden]: the post-attention RMSNorm output (input of the FFN)
  * d_x   bf16 [T, hidden]: the residual stream; on return x = bf(x + down)
  *       with down = bf(bf(sum_slot y_slot * w_slot) + bf(shared)) (:868-877).
- * flags bit0: skip the residual add and write `down` to d_x instead.        */
+ * flags bit0: skip the residual add and write `down` to d_x instead.
+ *       bit8: run the shared expert's down GEMV and the combine as a launch of their own even
+ *             for one token (by default they ride in the routed down launch; same results). */
 int kx_moe_decode_layer(const kx_config *cfg, const kx_moe_weights *w, kx_moe_workspace *ws,
                         const void *d_n, void *d_x, int32_t tokens, uint32_t flags, void *stream);
 /* The same layer for a prefill chunk of T tokens (BASELINE config 4): the tokens of each expert are
@@ -289,8 +291,9 @@ int kx_model_timing(kx_model *model, float *ms2);
  * Results do not depend on the mask (same sums, same rounding points); it exists so that a test
  * can run both forms.  No counterpart in the reference, which launches every step on its own
  * (src/kimi_exec.cu:812-827).  Default KX_FUSE_ALL.                                            */
-#define KX_FUSE_ABSORB 1u /* W_UK absorb, RoPE of q, kv_a norm + cache row: inside the q_b GEMV */
-#define KX_FUSE_ALL 1u
+#define KX_FUSE_ABSORB 1u   /* W_UK absorb, RoPE of q, kv_a norm + cache row: inside the q_b GEMV */
+#define KX_FUSE_MOE_TAIL 2u /* one token: shared down GEMV + combine + residual inside the routed down launch */
+#define KX_FUSE_ALL 3u
 int kx_model_set_fusion(kx_model *model, uint32_t mask);
 /* bf(mean + sigma*z) fill used for the norm weights */
 int kx_fill_affine_bf16(void *d_out, uint64_t n, uint64_t seed, uint64_t tensor_id, float mean,

@@ -220,8 +220,9 @@ def test_kimi_shape_stack_batch_invariance(kxlib, ox):
 
 @pytest.mark.parametrize("shape", ["small-1", "small-3", "kimi"])
 def test_fused_and_separate_launches_agree(kxlib, ox, shape):
-    # the q_b GEMV that finishes the query in its own launch against the same steps as kernels of their own:
-    # cache rows, hidden state, logits and ids to the bit (the oracle comparison above runs the fused form)
+    # the q_b GEMV that finishes the query in its own launch, and (batch 1) the routed down launch that finishes the
+    # MoE layer, against the same steps as kernels of their own: cache rows, hidden state, logits and ids to the bit
+    # (the oracle comparisons above run the fused forms)
     say(f"fusion on/off {shape}")
     if shape == "kimi":
         cfg = default_config()
@@ -233,7 +234,7 @@ def test_fused_and_separate_launches_agree(kxlib, ox, shape):
         prompt_len, n_tokens = 11, 9
     prompt = O.tokens_u32(batch * prompt_len, cfg.seed, 4, cfg.vocab).reshape(batch, prompt_len)
     got = []
-    for mask in (1, 0):
+    for mask in (3, 0):
         km = KxModel(kxlib, cfg)
         check(kxlib.kx_model_set_fusion(km.h, mask))
         rc, out, _ = km.generate(prompt, n_tokens)
@@ -243,6 +244,9 @@ def test_fused_and_separate_launches_agree(kxlib, ox, shape):
         got.append((out, km.hidden(batch), km.logits(batch).view(np.uint32), lat))
         km.close()
     assert kxlib.kx_model_set_fusion(None, 1) != 0
+    km = KxModel(kxlib, cfg)
+    assert kxlib.kx_model_set_fusion(km.h, 4) != 0 and b"mask" in kxlib.kx_last_error()
+    km.close()
     (o1, h1, l1, c1), (o0, h0, l0, c0) = got
     assert all((a == b).all() for a, b in zip(c1, c0)), "latent cache differs"
     assert (h1 == h0).all() and (l1 == l0).all() and (o1 == o0).all()

@@ -85,14 +85,14 @@ def test_bucket_bit_exact(kxlib, ox, T, E, topk):
     assert (work[na:] == np.array([-1, 0, 0, 0])).all()
 
 
-def _run_layer(kxlib, ox, H, I, SI, E, K, T, seed, flags=0):
+def _run_layer(kxlib, ox, H, I, SI, E, K, T, seed, flags=0, gpu_flags=0):
     host, n, x = moe_case(kxlib, H, I, SI, E, K, T, seed)
     cfg = moe_cfg(H, I, SI, E, K)
     w, bufs = moe_device_weights(host)
     ws = C.c_void_p()
     check(kxlib.kx_moe_workspace_create(C.byref(cfg), T, C.byref(ws)))
     dn, dx = dev(n), dev(x)
-    check(kxlib.kx_moe_decode_layer(C.byref(cfg), C.byref(w), ws, dn.ptr, dx.ptr, T, flags, None))
+    check(kxlib.kx_moe_decode_layer(C.byref(cfg), C.byref(w), ws, dn.ptr, dx.ptr, T, flags | gpu_flags, None))
     check(kxlib.kx_sync(None))
     views = [C.c_void_p() for _ in range(8)]
     check(kxlib.kx_moe_workspace_views(ws, *[C.byref(v) for v in views]))
@@ -152,6 +152,15 @@ def test_moe_layer_kimi_shape(kxlib, ox, T):
     # BASELINE config 2: hidden 7168, 384 experts top-8, moe_inter 2048, shared 2048
     say(f"moe layer kimi shape T={T}")
     got, exp = _run_layer(kxlib, ox, 7168, 2048, 2048, 384, 8, T, 9)
+    _assert_layer(got, exp)
+
+
+@pytest.mark.parametrize("flags,gpu_flags", [(0, 0x100), (1, 0), (1, 0x100)])
+def test_moe_layer_kimi_shape_one_token_tail(kxlib, ox, flags, gpu_flags):
+    # one token: by default the routed down launch also runs the shared expert's down GEMV and combines (bit 8 of
+    # the flags keeps them a launch of their own); both forms, with and without the residual add, against the oracle
+    say(f"moe layer kimi shape T=1 flags={flags} gpu_flags={gpu_flags:#x}")
+    got, exp = _run_layer(kxlib, ox, 7168, 2048, 2048, 384, 8, 1, 10, flags=flags, gpu_flags=gpu_flags)
     _assert_layer(got, exp)
 
 
