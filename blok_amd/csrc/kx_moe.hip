@@ -12,6 +12,8 @@
 //   3 routed down INT4 GEMV                               -> eout [T*topk, hidden]
 //   4 shared down bf16 GEMV; epilogue combines the topk routed outputs in slot
 //     order, adds the shared output and the residual.
+// For one token 3 and 4 are one launch: every workgroup of the routed down GEMV goes on to a chunk
+// of the shared down GEMV, and the workgroup that completes a block of output rows combines it.
 // More tokens: router GEMV, top-k + bucketing, and the shared gate+up GEMV are launches of
 // their own; beyond T*topk = E pairs the routed kernels run as two launches each (experts
 // with one pair, experts with more).
