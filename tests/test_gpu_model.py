@@ -234,7 +234,7 @@ def test_fused_and_separate_launches_agree(kxlib, ox, shape):
         prompt_len, n_tokens = 11, 9
     prompt = O.tokens_u32(batch * prompt_len, cfg.seed, 4, cfg.vocab).reshape(batch, prompt_len)
     got = []
-    for mask in (3, 0):
+    for mask in (3, 0, 1, 2):
         km = KxModel(kxlib, cfg)
         check(kxlib.kx_model_set_fusion(km.h, mask))
         rc, out, _ = km.generate(prompt, n_tokens)
@@ -247,9 +247,10 @@ def test_fused_and_separate_launches_agree(kxlib, ox, shape):
     km = KxModel(kxlib, cfg)
     assert kxlib.kx_model_set_fusion(km.h, 4) != 0 and b"mask" in kxlib.kx_last_error()
     km.close()
-    (o1, h1, l1, c1), (o0, h0, l0, c0) = got
-    assert all((a == b).all() for a, b in zip(c1, c0)), "latent cache differs"
-    assert (h1 == h0).all() and (l1 == l0).all() and (o1 == o0).all()
+    o0, h0, l0, c0 = got[1]   # every launch on its own
+    for (o1, h1, l1, c1) in (got[0], got[2], got[3]):
+        assert all((a == b).all() for a, b in zip(c1, c0)), "latent cache differs"
+        assert (h1 == h0).all() and (l1 == l0).all() and (o1 == o0).all()
 
 
 @pytest.mark.parametrize("batch,seq", [(1, 1), (1, 100), (2, 700), (1, 5000)])
