@@ -231,7 +231,8 @@ def run_moe_layer(args, emit=True):
                              "distinct_experts": U_last, "layer_gbs": round(layer_gbs, 1)},
         "phase_ms": {"shared_gate_up_router_route": round(float(phases[0]), 5), "routed_gate_up": round(float(phases[1]), 5),
                      "routed_down": round(float(phases[2]), 5), "shared_down_combine": round(float(phases[3] + phases[4]), 5),
-                     "note": "events around each launch inside the layer; they include the event commands themselves"},
+                     "note": "events around each launch inside the layer; they include the event commands themselves; "
+                             "for one token the routed down launch also runs the shared down GEMV and the combine"},
         "wall_ms_per_step": round(wall_ms / args.steps, 5),
         "cpu_baseline": cpu,
     }
