@@ -574,7 +574,7 @@ __global__ void __launch_bounds__(64) mla_combine_k(const float *__restrict__ pm
                                                     const float *__restrict__ po, uint16_t *__restrict__ o_lat, int heads,
                                                     int spans) {
   // M = max M_j; w_j = exp(M_j - M); Z = fma(Z_j, w_j, Z); O = fma(O_j, w_j, O) in span order; lane j holds span
-  // j's (M_j, Z_j, w_j) (at most 64 spans), the O_j rows are fetched four spans at a time
+  // j's (M_j, Z_j, w_j) (at most 64 spans), the O_j rows are fetched sixteen spans at a time
   constexpr int R = 512;
   const int h = blockIdx.x, b = blockIdx.y, lane = threadIdx.x;
   const size_t idx0 = (size_t)b * spans * heads + h;
@@ -586,16 +586,16 @@ __global__ void __launch_bounds__(64) mla_combine_k(const float *__restrict__ pm
   for (int j = 0; j < spans; ++j)
     Z = __builtin_fmaf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, zj), j)),
                        __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wj), j)), Z);
-  for (int j0 = 0; j0 < spans; j0 += 4) {
-    float4 o0[4], o1[4];
+  for (int j0 = 0; j0 < spans; j0 += 16) {
+    float4 o0[16], o1[16];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < 16; ++u) {
       const float4 *o = (const float4 *)(po + (idx0 + (size_t)min(j0 + u, spans - 1) * heads) * R + lane * 8);
       o0[u] = o[0];
       o1[u] = o[1];
     }
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < 16; ++u) {
       if (j0 + u < spans) {
         const float w = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wj), j0 + u));
         O[0] = __builtin_fmaf(o0[u].x, w, O[0]); O[1] = __builtin_fmaf(o0[u].y, w, O[1]);
