@@ -88,6 +88,19 @@ int kx_mla_span_tiles(int seq) {
   return st;
 }
 
+// The matrix-core kernel is not tied to that partition (it is held to a tolerance, not to the oracle's sums): few
+// sequences get more, shorter spans so that sequences x spans fills the chip -- up to 256 spans, merged 64 at a time.
+static int mfma_span_cap(int batch) {
+  const int want = 1024 / (batch > 0 ? batch : 1);
+  return want > 256 ? 256 : want < 64 ? 64 : want;
+}
+static int mfma_span_tiles(int seq, int batch) {
+  const int tiles = (seq + 63) / 64, cap = mfma_span_cap(batch);
+  int st = 1;
+  while (tiles > cap * st) st *= 2;
+  return st;
+}
+
 namespace {
 
 using kxg::bf_hi;
@@ -573,35 +586,42 @@ __global__ void __launch_bounds__(512, 1) mla_partial_mfma_k(MlaArgs a) {
 __global__ void __launch_bounds__(64) mla_combine_k(const float *__restrict__ pm, const float *__restrict__ pz,
                                                     const float *__restrict__ po, uint16_t *__restrict__ o_lat, int heads,
                                                     int spans) {
-  // M = max M_j; w_j = exp(M_j - M); Z = fma(Z_j, w_j, Z); O = fma(O_j, w_j, O) in span order; lane j holds span
-  // j's (M_j, Z_j, w_j) (at most 64 spans), the O_j rows are fetched sixteen spans at a time
+  // M = max M_j; w_j = exp(M_j - M); Z = fma(Z_j, w_j, Z); O = fma(O_j, w_j, O) in span order.  Spans are taken in
+  // groups of 64: lane j holds (M_j, Z_j, w_j) of the group's span j; the O_j rows are fetched sixteen at a time.
   constexpr int R = 512;
   const int h = blockIdx.x, b = blockIdx.y, lane = threadIdx.x;
   const size_t idx0 = (size_t)b * spans * heads + h;
-  const size_t my = idx0 + (size_t)min(lane, spans - 1) * heads;
-  const float mj = pm[my], zj = pz[my];
-  const float M = kxw::wave_max_f32(lane < spans ? mj : -__builtin_inff());
-  const float wj = kx_expf(mj - M);
+  float M = -__builtin_inff();
+  for (int g0 = 0; g0 < spans; g0 += 64) {
+    const float mj = g0 + lane < spans ? pm[idx0 + (size_t)(g0 + lane) * heads] : -__builtin_inff();
+    M = fmaxf(M, kxw::wave_max_f32(mj));
+  }
   float Z = 0.0f, O[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-  for (int j = 0; j < spans; ++j)
-    Z = __builtin_fmaf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, zj), j)),
-                       __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wj), j)), Z);
-  for (int j0 = 0; j0 < spans; j0 += 16) {
-    float4 o0[16], o1[16];
+  for (int g0 = 0; g0 < spans; g0 += 64) {
+    const int gn = min(64, spans - g0);
+    const size_t my = idx0 + (size_t)(g0 + min(lane, gn - 1)) * heads;
+    const float mj = pm[my], zj = pz[my];
+    const float wj = kx_expf(mj - M);
+    for (int j = 0; j < gn; ++j)
+      Z = __builtin_fmaf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, zj), j)),
+                         __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wj), j)), Z);
+    for (int j0 = 0; j0 < gn; j0 += 16) {
+      float4 o0[16], o1[16];
 #pragma unroll
-    for (int u = 0; u < 16; ++u) {
-      const float4 *o = (const float4 *)(po + (idx0 + (size_t)min(j0 + u, spans - 1) * heads) * R + lane * 8);
-      o0[u] = o[0];
-      o1[u] = o[1];
-    }
+      for (int u = 0; u < 16; ++u) {
+        const float4 *o = (const float4 *)(po + (idx0 + (size_t)(g0 + min(j0 + u, gn - 1)) * heads) * R + lane * 8);
+        o0[u] = o[0];
+        o1[u] = o[1];
+      }
 #pragma unroll
-    for (int u = 0; u < 16; ++u) {
-      if (j0 + u < spans) {
-        const float w = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wj), j0 + u));
-        O[0] = __builtin_fmaf(o0[u].x, w, O[0]); O[1] = __builtin_fmaf(o0[u].y, w, O[1]);
-        O[2] = __builtin_fmaf(o0[u].z, w, O[2]); O[3] = __builtin_fmaf(o0[u].w, w, O[3]);
-        O[4] = __builtin_fmaf(o1[u].x, w, O[4]); O[5] = __builtin_fmaf(o1[u].y, w, O[5]);
-        O[6] = __builtin_fmaf(o1[u].z, w, O[6]); O[7] = __builtin_fmaf(o1[u].w, w, O[7]);
+      for (int u = 0; u < 16; ++u) {
+        if (j0 + u < gn) {
+          const float w = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wj), j0 + u));
+          O[0] = __builtin_fmaf(o0[u].x, w, O[0]); O[1] = __builtin_fmaf(o0[u].y, w, O[1]);
+          O[2] = __builtin_fmaf(o0[u].z, w, O[2]); O[3] = __builtin_fmaf(o0[u].w, w, O[3]);
+          O[4] = __builtin_fmaf(o1[u].x, w, O[4]); O[5] = __builtin_fmaf(o1[u].y, w, O[5]);
+          O[6] = __builtin_fmaf(o1[u].z, w, O[6]); O[7] = __builtin_fmaf(o1[u].w, w, O[7]);
+        }
       }
     }
   }
@@ -610,6 +630,41 @@ __global__ void __launch_bounds__(64) mla_combine_k(const float *__restrict__ pm
   for (int e = 0; e < 4; ++e)
     r[e] = (uint32_t)kx_bf16_rne(O[2 * e] / Z) | ((uint32_t)kx_bf16_rne(O[2 * e + 1] / Z) << 16);
   *(uint4 *)(o_lat + ((size_t)b * heads + h) * R + lane * 8) = make_uint4(r[0], r[1], r[2], r[3]);
+}
+
+// the same merge for few (sequence, head) pairs: grid (heads, B, 8), one wave per 64 latent columns, lane = one column
+__global__ void __launch_bounds__(64) mla_combine_cols_k(const float *__restrict__ pm, const float *__restrict__ pz,
+                                                    const float *__restrict__ po, uint16_t *__restrict__ o_lat, int heads,
+                                                    int spans) {
+  // M = max M_j; w_j = exp(M_j - M); Z = fma(Z_j, w_j, Z); O = fma(O_j, w_j, O) in span order.  Spans are taken in
+  // groups of 64: lane j holds (M_j, Z_j, w_j) of the group's span j, and the group's 64 values of the lane's
+  // column are requested together.
+  constexpr int R = 512;
+  const int h = blockIdx.x, b = blockIdx.y, lane = threadIdx.x;
+  const int col = blockIdx.z * 64 + lane;
+  const size_t idx0 = (size_t)b * spans * heads + h;
+  float M = -__builtin_inff();
+  for (int g0 = 0; g0 < spans; g0 += 64) {
+    const float mj = g0 + lane < spans ? pm[idx0 + (size_t)(g0 + lane) * heads] : -__builtin_inff();
+    M = fmaxf(M, kxw::wave_max_f32(mj));
+  }
+  float Z = 0.0f, O = 0.0f;
+  for (int g0 = 0; g0 < spans; g0 += 64) {
+    const int gn = min(64, spans - g0);
+    const size_t my = idx0 + (size_t)(g0 + min(lane, gn - 1)) * heads;
+    const float mj = pm[my], zj = pz[my];
+    const float wj = kx_expf(mj - M);
+    for (int j = 0; j < gn; ++j)
+      Z = __builtin_fmaf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, zj), j)),
+                         __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wj), j)), Z);
+    float o[64];
+#pragma unroll
+    for (int u = 0; u < 64; ++u) o[u] = po[(idx0 + (size_t)(g0 + min(u, gn - 1)) * heads) * R + col];
+#pragma unroll
+    for (int u = 0; u < 64; ++u)
+      if (u < gn) O = __builtin_fmaf(o[u], __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wj), u)), O);
+  }
+  o_lat[((size_t)b * heads + h) * R + col] = kx_bf16_rne(O / Z);
 }
 
 }  // namespace
@@ -631,7 +686,13 @@ size_t kx_mla_partial_floats(int batch, int heads, int kv_rank, int max_seq) {
   const int tiles = (max_seq + 63) / 64, st = kx_mla_span_tiles(max_seq);
   int spans = (tiles + st - 1) / st;
   if (spans < 64) spans = tiles < 64 ? tiles : 64;  // shorter sequences use up to 64 spans
-  return (size_t)batch * spans * heads * (kv_rank + 2);
+  size_t rows = (size_t)batch * spans;              // (sequence, span) pairs of the fixed partition
+  for (int b = 1; b <= batch; ++b) {                // and of the matrix-core kernel's, for every batch up to this one
+    const int cap = mfma_span_cap(b);
+    const size_t r = (size_t)b * (tiles < cap ? tiles : cap);
+    if (r > rows) rows = r;
+  }
+  return rows * heads * (kv_rank + 2);
 }
 
 int kx_mla_partials_launch(const kx_config *c, const uint16_t *cache, size_t seq_stride, const float *qabs, float *partial,
@@ -640,9 +701,11 @@ int kx_mla_partials_launch(const kx_config *c, const uint16_t *cache, size_t seq
              c->kv_rank, c->qk_rope);
   KX_REQUIRE(c->heads % 4 == 0, "kx_mla: heads=%d must be a multiple of 4", c->heads);
   KX_REQUIRE(batch > 0 && seq > 0, "kx_mla: batch=%d seq=%d must be positive", batch, seq);
+  // automatic choice: the matrix-core kernel from 2048 positions on, where it is built for the shape (64 heads)
+  const bool use_mfma = g_mla_kernel == 2 || (g_mla_kernel == 0 && seq >= 2048 && c->heads == 64);
   MlaArgs a;
   a.cache = cache; a.qabs = qabs; a.heads = c->heads; a.seq = seq; a.seq_stride = seq_stride;
-  a.span_tiles = kx_mla_span_tiles(seq);
+  a.span_tiles = use_mfma ? mfma_span_tiles(seq, batch) : kx_mla_span_tiles(seq);
   const int tiles = (seq + 63) / 64;
   a.spans = (tiles + a.span_tiles - 1) / a.span_tiles;
   const size_t n = (size_t)batch * a.spans * c->heads;
@@ -664,8 +727,6 @@ int kx_mla_partials_launch(const kx_config *c, const uint16_t *cache, size_t seq
     KX_HIP(hipFuncSetAttribute((const void *)mla_partial_k<8>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
     attr_set = true;
   }
-  // automatic choice: the matrix-core kernel from 2048 positions on, where it is built for the shape (64 heads)
-  const bool use_mfma = g_mla_kernel == 2 || (g_mla_kernel == 0 && seq >= 2048 && c->heads == 64);
   if (use_mfma) {
     KX_REQUIRE(c->heads == 64, "kx_mla: the matrix-core kernel is built for 64 heads (got %d)", c->heads);
     static bool mfma_attr = false;
@@ -687,14 +748,21 @@ int kx_mla_partials_launch(const kx_config *c, const uint16_t *cache, size_t seq
   return KX_OK;
 }
 
+int kx_mla_combine_launch(const KxMlaPartials &p, uint16_t *o_lat, int batch, int heads, hipStream_t st) {
+  if ((long)heads * batch < 512)  // few waves: a wave per 64 columns, all of a group's rows in flight
+    hipLaunchKernelGGL(mla_combine_cols_k, dim3(heads, batch, 8), dim3(64), 0, st, p.pm, p.pz, p.po, o_lat, heads, p.spans);
+  else
+    hipLaunchKernelGGL(mla_combine_k, dim3(heads, batch), dim3(64), 0, st, p.pm, p.pz, p.po, o_lat, heads, p.spans);
+  KX_LAUNCH_CHECK();
+  return KX_OK;
+}
+
 int kx_mla_attend_launch(const kx_config *c, const uint16_t *cache, size_t seq_stride, const float *qabs, float *partial,
                          uint16_t *o_lat, int batch, int seq, hipStream_t st) {
   KxMlaPartials p;
   int rc = kx_mla_partials_launch(c, cache, seq_stride, qabs, partial, batch, seq, &p, st);
   if (rc) return rc;
-  hipLaunchKernelGGL(mla_combine_k, dim3(c->heads, batch), dim3(64), 0, st, p.pm, p.pz, p.po, o_lat, c->heads, p.spans);
-  KX_LAUNCH_CHECK();
-  return KX_OK;
+  return kx_mla_combine_launch(p, o_lat, batch, c->heads, st);
 }
 
 // ---- C ABI: BASELINE config 3 as an operator -------------------------------------------

@@ -297,10 +297,14 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample) {
     g.w0 = L.kvb; g.x = m->o_lat; g.x_stride = c.heads * c.kv_rank; g.out = m->att; g.out_stride = VD; g.rows = VD;
     g.cols = c.kv_rank; g.tokens = B; g.row_block = c.v_head; g.w_block_stride = c.qk_nope + c.v_head;
     g.w_block_off = c.qk_nope; g.x_block_stride = c.kv_rank;
-    if (fuse) {  // its activations are the attention partials, merged as they are loaded      // :825
+    if (fuse) {                                                                                 // :825
       KxMlaPartials mp;
       KX_TRY(kx_mla_partials_launch(&c, L.cache, seq_stride, m->qabs, m->partial, B, pos + 1, &mp, st));
-      g.mla_pm = mp.pm; g.mla_pz = mp.pz; g.mla_po = mp.po; g.mla_spans = mp.spans; g.mla_heads = c.heads;
+      if (mp.spans <= 64) {  // the GEMV's activations are the attention partials, merged as they are loaded
+        g.mla_pm = mp.pm; g.mla_pz = mp.pz; g.mla_po = mp.po; g.mla_spans = mp.spans; g.mla_heads = c.heads;
+      } else {               // long context, few sequences: more spans than the GEMV's merge takes
+        KX_TRY(kx_mla_combine_launch(mp, m->o_lat, B, c.heads, st));
+      }
     } else {
       KX_TRY(kx_mla_attend_launch(&c, L.cache, seq_stride, m->qabs, m->partial, m->o_lat, B, pos + 1, st));
     }

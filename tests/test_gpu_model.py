@@ -280,9 +280,10 @@ def test_mla_decode_operator(kxlib, ox, batch, seq):
         assert (got == cache[:, 0:1, :R]).all()   # one position: the latent itself
 
 
-@pytest.mark.parametrize("batch,seq", [(1, 1), (1, 31), (1, 100), (2, 700), (1, 4133), (1, 5000)])
+@pytest.mark.parametrize("batch,seq", [(1, 1), (1, 31), (1, 100), (2, 700), (1, 4133), (1, 5000), (8, 4200)])
 def test_mla_decode_matrix_core_kernel(kxlib, ox, batch, seq):
-    # the MFMA variant sums in another order: max-rel 1e-2 against both oracle schedules, and against the VALU kernel
+    # the MFMA variant sums in another order: max-rel 1e-2 against both oracle schedules, and against the VALU kernel.
+    # From 4097 positions on, one to eight sequences are cut into more than 64 spans (both merge kernels, in groups)
     say(f"mla decode (matrix cores) batch={batch} seq={seq}")
     cfg = default_config()
     H, KVA, R = cfg.heads, 576, 512
@@ -307,6 +308,30 @@ def test_mla_decode_matrix_core_kernel(kxlib, ox, batch, seq):
     e1, e0 = O.max_rel(outs[2], O.bf16_to_f32(exp1)), O.max_rel(outs[2], O.bf16_to_f32(exp0))
     print(f"matrix-core MLA seq={seq}: max-rel {e_valu:.2e} vs VALU kernel, {e1:.2e} vs mode 1, {e0:.2e} vs mode 0", flush=True)
     assert e_valu < 1e-2 and e1 < 1e-2 and e0 < 1e-2
+
+
+def test_kimi_shape_long_context_stack_attention_paths(kxlib, ox):
+    # batch 1 past 4096 positions: the matrix-core attention kernel cuts the sequence into more than 64 spans, which
+    # the stack merges with a kernel of its own instead of inside the W_UV GEMV.  Held against the same stack with the
+    # VALU kernel forced (the bit-exact path): logits of the first sampled step within the stack-level 3e-2, same id.
+    say("kimi shape 2-layer stack, 4200-token prompt, attention paths")
+    cfg = default_config()
+    cfg.n_layers, cfg.first_dense, cfg.max_batch, cfg.max_context, cfg.seed = 2, 1, 1, 4300, 3
+    prompt = O.tokens_u32(4200, cfg.seed, 4, cfg.vocab).reshape(1, 4200)
+    got = {}
+    try:
+        for mode in (0, 1):
+            check(kxlib.kx_mla_set_kernel(mode))
+            km = KxModel(kxlib, cfg)
+            rc, out, _ = km.generate(prompt, 1)
+            assert rc == 0, kxlib.kx_last_error()
+            got[mode] = (out.copy(), km.logits(1))
+            km.close()
+    finally:
+        check(kxlib.kx_mla_set_kernel(0))
+    err = O.max_rel(got[0][1], got[1][1])
+    print(f"long-context stack, matrix-core vs VALU attention: logits max-rel {err:.3e}", flush=True)
+    assert err < 3e-2 and (got[0][0] == got[1][0]).all()
 
 
 def test_executor_json_line(kxlib):
