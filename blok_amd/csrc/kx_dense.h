@@ -103,6 +103,10 @@ int kx_grouped_gemm_launch(bool dual, bool i4, const void *w0, const uint16_t *s
                            const uint16_t *x, void *out, int out_mode, const int4 *work, const int *pairs, int n_pairs,
                            int n_slots, int N, int K, int x_div, size_t expert_w, size_t expert_s, int n_pairs_max,
                            hipStream_t st);
+// kx_skinny.hip: one tile of up to 32 tokens against a bf16 matrix (two for SwiGLU) on the matrix cores, out_mode as
+// above.  *done = false (nothing launched) when the shape is not the kernel's.
+int kx_skinny_gemm_launch(bool dual, const uint16_t *w0, const uint16_t *w1, const uint16_t *x, int x_stride, void *out,
+                          int out_stride, int out_mode, int tokens, int rows, int cols, bool *done, hipStream_t st);
 int kx_moe_combine_launch(const uint16_t *eout, const float *rw, const uint16_t *sy, uint16_t *x, int tokens, int hidden,
                           int topk, uint32_t flags, hipStream_t st);
 

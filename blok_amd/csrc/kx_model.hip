@@ -263,6 +263,12 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample) {
     if (!mm) return kx_gemv_launch(epi, g, st);
     const bool dual = epi == KX_EPI_SWIGLU;
     const int mode = epi == KX_EPI_RESID ? KX_GG_RESID : epi == KX_EPI_ARGMAX ? KX_GG_F32_OF_BF16 : epi == KX_EPI_F32 ? KX_GG_F32 : KX_GG_BF16;
+    if (g.tokens <= 32) {  // one tile: the kernel built for it
+      bool done = false;
+      int rc2 = kx_skinny_gemm_launch(dual, g.w0, dual ? g.w1 : nullptr, g.x, g.x_stride, g.out, g.out_stride, mode, g.tokens, g.rows,
+                                      g.cols, &done, st);
+      if (rc2 || done) return rc2;
+    }
     return kx_grouped_gemm_launch(dual, false, g.w0, nullptr, dual ? g.w1 : nullptr, nullptr, g.x, g.out, mode, nullptr, nullptr,
                                   g.tokens, 1, g.rows, g.cols, 1, 0, 0, g.tokens, st);
   };
