@@ -6,13 +6,23 @@
 //
 // A GEMV kernel is bound by its fma count from about 16 tokens on (every weight meets every token on the VALU), and
 // the grouped prefill GEMM of kx_prefill.hip, built for 128-token tiles of many experts, leaves most of the chip idle
-// on one 32-token tile.  Here a workgroup of 8 waves owns 32 weight rows and walks the columns in steps of 512; in step
-// j wave w takes columns 512 j + 64 w .. + 63, so that the eight waves read 1 KB of every row together (a wave on its
-// own would touch 128 bytes of 32 rows, a new DRAM page with every access).  Load m of a step takes, for lane
-// (r, h) = (lane % 32, lane / 32), the 16 bytes of row r at columns 512 j + 64 w + 16 m + 8 h, and the same bytes of
-// token r's activations (from L2: the activations are small and shared by every workgroup).  Load m feeds
-// v_mfma_f32_32x32x16_bf16 number m: its 16 contraction indices are those 16 columns, the same for both operands.  Two steps are in flight while one is multiplied.  The eight partial
-// 32 x 32 tiles are summed through LDS in wave order and the epilogue runs on the sum.
+// on one 32-token tile.  Here a workgroup of 8 waves owns 32 weight rows and all (up to 32) tokens, the eight waves
+// split the columns, and their partial 32 x 32 tiles (v_mfma_f32_32x32x16_bf16) are summed through LDS in wave
+// order before the epilogue.
+//
+// Both operands are staged through LDS.  The operand layout of the matrix cores is one row per lane: loading the
+// operands straight from memory makes every load instruction touch 32 rows with 32 bytes each, and that streams at
+// 2.3-3 TB/s whatever the number of waves (measured; the lm_head then takes 1.0 ms).  So the columns are walked in
+// blocks of 256: a copy instruction (global_load_lds_dwordx4, no registers) moves 512 contiguous bytes of two rows,
+// lane (l / 32, l % 32) = (row of the pair, 16-byte slot); the lane fetches piece slot ^ (row % 16) of its row, so
+// that the operand reads -- lane (r, h) wants piece p of row r and finds it in slot p ^ (r % 16) -- fall into different
+// banks.  Blocks go through a ring of 4 stages (3 for two matrices), three (two) blocks in flight behind the one being
+// multiplied; each wave issues its share of a block's copies, waits for its own by count (they complete in order),
+// and one barrier per block makes every wave's copies visible and the stage that is overwritten next free.  Wave w
+// multiplies pieces 4w .. 4w+3 of the block (two products per matrix).  The lm_head takes 0.43 ms this way (5.5 TB/s).
+// The copies are issued from inline asm and the barrier carries no fence: a copy the compiler knows of makes it
+// complete everything in flight before every LDS access it cannot tell from the copy's target.
+//
 // Sums are fp32 over exact bf16 products in another order than the GEMV's: this path is held to the 1e-2 bar, like the
 // other matrix-core paths, and serves batches the token-identity checks do not run on.
 #include "kx_common.h"
@@ -23,7 +33,6 @@ namespace {
 
 typedef __bf16 kx_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float kx_f32x16 __attribute__((ext_vector_type(16)));
-typedef unsigned int kx_u32x4 __attribute__((ext_vector_type(4)));
 
 struct SkinnyArgs {
   const uint16_t *w0, *w1;  // bf16 [rows, cols]; w1 for the two-matrix SwiGLU form
@@ -32,80 +41,90 @@ struct SkinnyArgs {
   int rows, cols, tokens, x_stride, out_stride, mode;
 };
 
-__device__ __forceinline__ kx_u32x4 ld_w(const uint16_t *p) { return __builtin_nontemporal_load((const kx_u32x4 *)p); }
+// global_load_lds_dwordx4: lane i's 16 bytes at `src` land at LDS byte address lds_base + 16 i (lds_base uniform)
+__device__ __forceinline__ void sk_copy16_to_lds(const void *src, uint32_t lds_base) {
+  lds_base = __builtin_amdgcn_readfirstlane(lds_base);
+  uint32_t m0_saved;  // the instruction takes the LDS address from m0; m0 is put back, the compiler owns it
+  asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, off\n\ts_mov_b32 m0, %0"
+               : "=&s"(m0_saved)
+               : "s"(lds_base), "v"(src)
+               : "memory");
+}
+template <int N>
+__device__ __forceinline__ void sk_wait_copies() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+__device__ __forceinline__ void sk_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-// NW waves per workgroup
-template <bool DUAL, int NW>
-__global__ void __launch_bounds__(NW * 64) skinny_gemm_k(SkinnyArgs a) {
+template <bool DUAL>
+__global__ void __launch_bounds__(512) skinny_staged_k(SkinnyArgs a) {
   constexpr int MATS = DUAL ? 2 : 1;
-  __shared__ float part[MATS][NW][32][32];  // [matrix][wave][token][row]
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  constexpr int TILES = MATS + 1;            // weight tiles and the activation tile of a stage, 16 KB each
+  constexpr int NS = DUAL ? 3 : 4;           // stages
+  constexpr int CPW = TILES * 2;             // copy instructions per wave and block (16 per tile over 8 waves)
+  constexpr uint32_t TILE = 32 * 512, STAGE = TILES * TILE;
+  extern __shared__ __attribute__((aligned(16))) uint8_t sk_lds[];
+  const uint32_t lds0 = (uint32_t)(uintptr_t)sk_lds;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int r = lane & 31, h = lane >> 5;
   const int row0 = blockIdx.x * 32;
-  const int steps = a.cols / (NW * 64);  // steps of NW * 64 columns (the host checks that they divide cols)
-  const int wrow = min(row0 + r, a.rows - 1), tok = min(r, a.tokens - 1);
-  const uint16_t *wp[MATS];
-  wp[0] = a.w0 + (size_t)wrow * a.cols + wave * 64 + 8 * h;
-  if (DUAL) wp[MATS - 1] = a.w1 + (size_t)wrow * a.cols + wave * 64 + 8 * h;
-  const uint16_t *xp = a.x + (size_t)tok * a.x_stride + wave * 64 + 8 * h;
+  const int nb = a.cols >> 8;  // blocks of 256 columns
+  // this wave's copies of a block: instruction u moves rows 2 i, 2 i + 1 of tile t, (t, i) = ((8 u + wave) / 16, .. % 16)
+  const uint16_t *csrc[CPW];
+  uint32_t cdst[CPW];
+#pragma unroll
+  for (int u = 0; u < CPW; ++u) {
+    const int idx = u * 8 + wave, t = idx >> 4, i = idx & 15;
+    const int row = 2 * i + h, piece = r ^ (row & 15);
+    const uint16_t *base = t == MATS ? a.x + (size_t)min(row, a.tokens - 1) * a.x_stride
+                                     : (t == 0 ? a.w0 : a.w1) + (size_t)min(row0 + row, a.rows - 1) * a.cols;
+    csrc[u] = base + piece * 8;
+    cdst[u] = t * TILE + i * 1024;
+  }
+  auto copy_block = [&](int b) {
+    const uint32_t st = lds0 + (uint32_t)(b % NS) * STAGE;
+#pragma unroll
+    for (int u = 0; u < CPW; ++u) sk_copy16_to_lds(csrc[u] + b * 256, st + cdst[u]);
+  };
   kx_f32x16 acc[MATS];
 #pragma unroll
   for (int m = 0; m < MATS; ++m)
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[m][v] = 0.0f;
+  // operand reads of this lane: piece 4 wave + 2 q + h of row r sits in slot piece ^ (r % 16)
+  uint32_t roff[2];
+#pragma unroll
+  for (int q = 0; q < 2; ++q) roff[q] = (uint32_t)r * 512 + (uint32_t)((4 * wave + 2 * q + h) ^ (r & 15)) * 16;
 
-  struct Step { kx_u32x4 w[MATS][4], x[4]; };
-  auto load = [&](Step &s, int j) {
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
+  for (int b = 0; b < NS - 1; ++b)
+    if (b < nb) copy_block(b);
+  for (int b = 0; b < nb; ++b) {
+    // this wave's copies of block b have landed when at most those of the blocks behind it are in flight
+    const int behind = min(nb - 1 - b, NS - 2);
+    if (behind >= 2) sk_wait_copies<2 * CPW>();
+    else if (behind == 1) sk_wait_copies<CPW>();
+    else sk_wait_copies<0>();
+    sk_barrier();  // every wave's copies of block b are in LDS; every wave is done with block b - 1
+    if (b + NS - 1 < nb) copy_block(b + NS - 1);  // into the stage block b - 1 was read from
+    const uint8_t *st = sk_lds + (uint32_t)(b % NS) * STAGE;
 #pragma unroll
-      for (int m = 0; m < MATS; ++m) s.w[m][q] = ld_w(wp[m] + j * (NW * 64) + q * 16);
-      s.x[q] = *(const kx_u32x4 *)(xp + j * (NW * 64) + q * 16);
+    for (int q = 0; q < 2; ++q) {
+      const kx_bf16x8 xv = *(const kx_bf16x8 *)(st + MATS * TILE + roff[q]);
+#pragma unroll
+      for (int m = 0; m < MATS; ++m) {
+        const kx_bf16x8 wv = *(const kx_bf16x8 *)(st + m * TILE + roff[q]);
+        acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xv, wv, acc[m], 0, 0, 0);
+      }
     }
-  };
-  auto mul = [&](const Step &s) {
-#pragma unroll
-    for (int q = 0; q < 4; ++q)
-#pragma unroll
-      for (int m = 0; m < MATS; ++m)
-        acc[m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(kx_bf16x8, s.x[q]), __builtin_bit_cast(kx_bf16x8, s.w[m][q]),
-                                                         acc[m], 0, 0, 0);
-  };
-  // Three buffers: two steps in flight while one is multiplied.  Every load is unconditional (past the end the last
-  // step is requested again and never used), so that the waits in front of the products count exactly the loads
-  // behind them: after a load under a condition the compiler would wait for everything in flight.
-  // The scheduler is kept from moving a step's loads behind the products in front of them (it would, to save
-  // registers, and the kernel would wait for every step it is about to multiply).
-  const int last = steps - 1;
-  Step s0, s1, s2;
-  load(s0, 0);
-  load(s1, min(1, last));
-  __builtin_amdgcn_sched_barrier(0);
-  for (int j = 0;; j += 3) {
-    load(s2, min(j + 2, last));
-    __builtin_amdgcn_sched_barrier(0);
-    mul(s0);
-    __builtin_amdgcn_sched_barrier(0);
-    if (j + 1 >= steps) break;
-    load(s0, min(j + 3, last));
-    __builtin_amdgcn_sched_barrier(0);
-    mul(s1);
-    __builtin_amdgcn_sched_barrier(0);
-    if (j + 2 >= steps) break;
-    load(s1, min(j + 4, last));
-    __builtin_amdgcn_sched_barrier(0);
-    mul(s2);
-    __builtin_amdgcn_sched_barrier(0);
-    if (j + 3 >= steps) break;
   }
-  // D[i][jj]: jj = lane % 32 (weight row), i = 8 (v / 4) + 4 (lane / 32) + v % 4 (token)
+  sk_barrier();  // the ring is free: it takes the partial tiles
+  float(*part)[8][32][32] = (float(*)[8][32][32])sk_lds;
 #pragma unroll
   for (int m = 0; m < MATS; ++m)
 #pragma unroll
     for (int v = 0; v < 16; ++v) part[m][wave][8 * (v >> 2) + 4 * h + (v & 3)][r] = acc[m][v];
   __syncthreads();
-  for (int idx = threadIdx.x; idx < 32 * 32; idx += NW * 64) {
-    const int rr = idx & 31, t = idx >> 5;  // consecutive threads: consecutive rows of one token
+  for (int idx = threadIdx.x; idx < 32 * 32; idx += 512) {
+    const int rr = idx & 31, t = idx >> 5;
     const int row = row0 + rr;
     if (row >= a.rows || t >= a.tokens) continue;
     float y[MATS];
@@ -113,7 +132,7 @@ __global__ void __launch_bounds__(NW * 64) skinny_gemm_k(SkinnyArgs a) {
     for (int m = 0; m < MATS; ++m) {
       float sum = part[m][0][t][rr];
 #pragma unroll
-      for (int w = 1; w < NW; ++w) sum += part[m][w][t][rr];
+      for (int w = 1; w < 8; ++w) sum += part[m][w][t][rr];
       y[m] = sum;
     }
     const size_t o = (size_t)t * a.out_stride + row;
@@ -139,15 +158,21 @@ __global__ void __launch_bounds__(NW * 64) skinny_gemm_k(SkinnyArgs a) {
 int kx_skinny_gemm_launch(bool dual, const uint16_t *w0, const uint16_t *w1, const uint16_t *x, int x_stride, void *out,
                           int out_stride, int out_mode, int tokens, int rows, int cols, bool *done, hipStream_t st) {
   *done = false;
-  if (tokens < 1 || tokens > 32 || rows < 1 || cols < 512 || cols % 512 || x_stride % 8 || (dual && !w1)) return KX_OK;
+  if (tokens < 1 || tokens > 32 || rows < 1 || cols < 512 || cols % 512 || x_stride % 8 || x_stride < cols || (dual && !w1)) return KX_OK;
   KX_REQUIRE(out_mode >= KX_GG_BF16 && out_mode <= KX_GG_RESID && !(dual && out_mode != KX_GG_BF16), "kx_skinny_gemm: out_mode=%d", out_mode);
   SkinnyArgs a;
   a.w0 = w0; a.w1 = w1; a.x = x; a.out = out; a.rows = rows; a.cols = cols; a.tokens = tokens; a.x_stride = x_stride;
   a.out_stride = out_stride; a.mode = out_mode;
   const dim3 g((unsigned)kx_cdiv(rows, 32));
-  // eight waves: with 12 or 16 (where they divide the columns) the same matrices take 1.2-1.4 times as long
-  if (dual) hipLaunchKernelGGL((skinny_gemm_k<true, 8>), g, dim3(512), 0, st, a);
-  else hipLaunchKernelGGL((skinny_gemm_k<false, 8>), g, dim3(512), 0, st, a);
+  const size_t lds = (size_t)(dual ? 3 * 3 : 4 * 2) * 32 * 512;  // the ring: stages x tiles x 16 KB
+  static bool attr = false;
+  if (!attr) {
+    KX_HIP(hipFuncSetAttribute((const void *)skinny_staged_k<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 4 * 2 * 32 * 512));
+    KX_HIP(hipFuncSetAttribute((const void *)skinny_staged_k<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 3 * 3 * 32 * 512));
+    attr = true;
+  }
+  if (dual) hipLaunchKernelGGL(skinny_staged_k<true>, g, dim3(512), lds, st, a);
+  else hipLaunchKernelGGL(skinny_staged_k<false>, g, dim3(512), lds, st, a);
   KX_LAUNCH_CHECK();
   *done = true;
   return KX_OK;
