@@ -331,7 +331,7 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample) {
       KX_TRY(dense(KX_EPI_RESID, g));                                                                   // :684, :877
     } else {
       if (!fuse) KX_TRY(kx_rmsnorm_launch(m->x, L.post_ln, m->n, B, H, H, H, c.rms_eps, st));          // :829
-      KX_TRY(kx_moe_layer_launch(&c, &L.moe, m->moe_ws, m->n, m->x, B, (m->fusion & KX_FUSE_MOE_TAIL) ? 0u : KX_MOE_SEPARATE_TAIL,
+      KX_TRY(kx_moe_layer_launch(&c, &L.moe, m->moe_ws, m->n, m->x, B, ((m->fusion & KX_FUSE_MOE_TAIL) ? 0u : KX_MOE_SEPARATE_TAIL) | (mm ? KX_MOE_SHARED_MATRIX_CORES : 0u),
                                  fuse ? L.post_ln : nullptr, st, false));  // :835-877
     }
   }

@@ -208,26 +208,40 @@ int kx_moe_layer_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_work
   if (!tailed && (rc = routed_launch(c, w, ws, n, tokens, 1, st))) return rc;
   if (timed) KX_HIP(hipEventRecord(ws->ev[3], st));
   // shared gate/up + SwiGLU when it did not ride with the router
+  // From 16 tokens on a caller may ask for the shared expert on the matrix cores (another summation order, held to
+  // the 1e-2 bar; the router and the routed experts stay as they are, so the routing does not change)
+  const bool mm = (flags & KX_MOE_SHARED_MATRIX_CORES) && tokens >= 16 && tokens <= 32;
   if (!paired) {
     if (norm_w) { s.x = n; s.norm_w = nullptr; }  // d_n holds the normed rows by now
-    if ((rc = kx_gemv_launch(KX_EPI_SWIGLU, s, st))) return rc;
+    bool done = false;
+    if (mm && !s.norm_w &&
+        (rc = kx_skinny_gemm_launch(true, s.w0, s.w1, s.x, s.x_stride, s.out, s.out_stride, KX_GG_BF16, tokens, s.rows, s.cols, &done, st)))
+      return rc;
+    if (!done && (rc = kx_gemv_launch(KX_EPI_SWIGLU, s, st))) return rc;
   }
   if (timed) KX_HIP(hipEventRecord(ws->ev[4], st));
-  if (!tailed && (rc = kx_gemv_launch(KX_EPI_MOE_COMBINE, d, st))) return rc;
+  if (!tailed) {
+    bool done = false;
+    if (mm) {  // shared down into sy, then the combine as a kernel of its own
+      if ((rc = kx_skinny_gemm_launch(false, d.w0, nullptr, d.x, d.x_stride, ws->sy, H, KX_GG_BF16, tokens, d.rows, d.cols, &done, st))) return rc;
+      if (done && (rc = kx_moe_combine_launch(ws->eout, ws->weights, ws->sy, (uint16_t *)d_x, tokens, H, K, flags & 1u, st))) return rc;
+    }
+    if (!done && (rc = kx_gemv_launch(KX_EPI_MOE_COMBINE, d, st))) return rc;
+  }
   if (timed) KX_HIP(hipEventRecord(ws->ev[5], st));
   return KX_OK;
 }
 
 extern "C" int kx_moe_decode_layer(const kx_config *cfg, const kx_moe_weights *w, kx_moe_workspace *ws, const void *d_n,
                                    void *d_x, int32_t tokens, uint32_t flags, void *stream) {
-  return kx_moe_layer_launch(cfg, w, ws, (void *)d_n, d_x, tokens, flags, nullptr, kx_stream(stream), false);
+  return kx_moe_layer_launch(cfg, w, ws, (void *)d_n, d_x, tokens, flags & (1u | KX_MOE_SEPARATE_TAIL), nullptr, kx_stream(stream), false);
 }
 
 extern "C" int kx_moe_decode_layer_timed(const kx_config *cfg, const kx_moe_weights *w, kx_moe_workspace *ws,
                                          const void *d_n, void *d_x, int32_t tokens, uint32_t flags, void *stream,
                                          float *ms5) {
   KX_REQUIRE(ms5, "kx_moe_decode_layer_timed: null output");
-  int rc = kx_moe_layer_launch(cfg, w, ws, (void *)d_n, d_x, tokens, flags, nullptr, kx_stream(stream), true);
+  int rc = kx_moe_layer_launch(cfg, w, ws, (void *)d_n, d_x, tokens, flags & (1u | KX_MOE_SEPARATE_TAIL), nullptr, kx_stream(stream), true);
   if (rc) return rc;
   KX_HIP(hipEventSynchronize(ws->ev[5]));
   for (int i = 0; i < 5; ++i) KX_HIP(hipEventElapsedTime(&ms5[i], ws->ev[i], ws->ev[i + 1]));
