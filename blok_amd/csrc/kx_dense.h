@@ -115,7 +115,7 @@ int kx_moe_combine_launch(const uint16_t *eout, const float *rw, const uint16_t 
 struct kx_moe_workspace;
 // flag for kx_moe_layer_launch (beside bit 0): keep the shared down GEMV and the combine a launch of their own
 #define KX_MOE_SEPARATE_TAIL 0x100u
-// 16 to 32 tokens: the shared expert's GEMVs on the matrix cores (kx_skinny.hip; tolerance instead of bit parity)
+// 5 to 32 tokens: the shared expert's GEMVs on the matrix cores (kx_skinny.hip; tolerance instead of bit parity)
 #define KX_MOE_SHARED_MATRIX_CORES 0x200u
 int kx_moe_layer_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_workspace *ws, void *d_n, void *d_x,
                         int tokens, uint32_t flags, const uint16_t *norm_w, hipStream_t st, bool timed);

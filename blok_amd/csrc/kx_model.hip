@@ -17,7 +17,7 @@
 //   them) -> o_proj GEMV with the residual add
 //   -> dense SwiGLU MLP (layers < first_dense) or the routed MoE layer (post-attention norm
 //   in their first GEMV).
-// From 16 sequences on the dense projections run as GEMMs on the matrix cores.
+// From 5 sequences on the dense projections run as GEMMs on the matrix cores.
 #include <math.h>
 #include <string.h>
 #include <vector>
@@ -256,9 +256,9 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample) {
   const uint16_t *rope_row = m->rope_tab + (size_t)pos * c.qk_rope;
   const size_t seq_stride = (size_t)c.max_context * KVA;
   const bool fuse = B <= 4;  // RMSNorms ride in the prologue of the GEMV that consumes them
-  // From 16 sequences on, the dense projections run as GEMMs on the matrix cores (one group of B rows): the
+  // From 5 sequences on (the fused prologues cover up to 4), the dense projections run as GEMMs on the matrix cores: the
   // GEMV is bound by its fma count there.  Same values, another summation order (the bf16 rounding points stay).
-  const bool mm = B >= 16;
+  const bool mm = B >= 5;
   auto dense = [&](int epi, const KxGemvArgs &g) -> int {
     if (!mm) return kx_gemv_launch(epi, g, st);
     const bool dual = epi == KX_EPI_SWIGLU;

@@ -208,9 +208,9 @@ int kx_moe_layer_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_work
   if (!tailed && (rc = routed_launch(c, w, ws, n, tokens, 1, st))) return rc;
   if (timed) KX_HIP(hipEventRecord(ws->ev[3], st));
   // shared gate/up + SwiGLU when it did not ride with the router
-  // From 16 tokens on a caller may ask for the shared expert on the matrix cores (another summation order, held to
+  // From 5 tokens on a caller may ask for the shared expert on the matrix cores (another summation order, held to
   // the 1e-2 bar; the router and the routed experts stay as they are, so the routing does not change)
-  const bool mm = (flags & KX_MOE_SHARED_MATRIX_CORES) && tokens >= 16 && tokens <= 32;
+  const bool mm = (flags & KX_MOE_SHARED_MATRIX_CORES) && tokens >= 5 && tokens <= 32;
   if (!paired) {
     if (norm_w) { s.x = n; s.norm_w = nullptr; }  // d_n holds the normed rows by now
     bool done = false;

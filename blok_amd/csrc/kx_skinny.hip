@@ -1,10 +1,11 @@
-// kx_skinny.hip -- dense projections for decode batches of 16 to 32 sequences: y[t, r] = sum_k x[t, k] w[r, k] with
+// kx_skinny.hip -- dense projections for decode batches of 5 to 32 sequences: y[t, r] = sum_k x[t, k] w[r, k] with
 // bf16 weights [rows, cols] streamed once and the tokens as the other side of a matrix-core product.
 //
 // Reference: matvec_bf16_k / matvec_bf16_f32_k (src/kimi_exec.cu:272-298) called once per token; the epilogues are
 // add_k (:248-251), silu_mul_k (:253-256) and the bf16 rounding of the logits (:718-734).
 //
-// A GEMV kernel is bound by its fma count from about 16 tokens on (every weight meets every token on the VALU), and
+// A GEMV kernel streams the weights once per block of four tokens and is bound by its fma count from about 16 tokens
+// on (every weight meets every token on the VALU), and
 // the grouped prefill GEMM of kx_prefill.hip, built for 128-token tiles of many experts, leaves most of the chip idle
 // on one 32-token tile.  Here a workgroup of 8 waves owns 32 weight rows and all (up to 32) tokens, the eight waves
 // split the columns, and their partial 32 x 32 tiles (v_mfma_f32_32x32x16_bf16) are summed through LDS in wave
