@@ -74,7 +74,7 @@ extern "C" int kx_softmax_scale(const kx_config *cfg, float *rs, float *mscale) 
   return KX_OK;
 }
 
-// 0: matrix-core kernel from 2048 positions on, 1: VALU kernel always, 2: matrix-core kernel always
+// 0: matrix-core kernel from 2048 positions on (128 for 5 sequences and more), 1: VALU kernel always, 2: matrix-core kernel always
 static int g_mla_kernel = 0;
 extern "C" int kx_mla_set_kernel(int32_t mode) {
   KX_REQUIRE(mode >= 0 && mode <= 2, "kx_mla_set_kernel: mode=%d outside [0, 2]", mode);
@@ -701,8 +701,10 @@ int kx_mla_partials_launch(const kx_config *c, const uint16_t *cache, size_t seq
              c->kv_rank, c->qk_rope);
   KX_REQUIRE(c->heads % 4 == 0, "kx_mla: heads=%d must be a multiple of 4", c->heads);
   KX_REQUIRE(batch > 0 && seq > 0, "kx_mla: batch=%d seq=%d must be positive", batch, seq);
-  // automatic choice: the matrix-core kernel from 2048 positions on, where it is built for the shape (64 heads)
-  const bool use_mfma = g_mla_kernel == 2 || (g_mla_kernel == 0 && seq >= 2048 && c->heads == 64);
+  // automatic choice, where the matrix-core kernel is built for the shape (64 heads): from 2048 positions on, and from
+  // 128 positions on for 5 sequences and more (batches the stack runs on the matrix cores anyway; the VALU kernel
+  // takes 190-360 us per layer at 32 sequences of 1100 positions)
+  const bool use_mfma = g_mla_kernel == 2 || (g_mla_kernel == 0 && c->heads == 64 && (seq >= 2048 || (batch >= 5 && seq >= 128)));
   MlaArgs a;
   a.cache = cache; a.qabs = qabs; a.heads = c->heads; a.seq = seq; a.seq_stride = seq_stride;
   a.span_tiles = use_mfma ? mfma_span_tiles(seq, batch) : kx_mla_span_tiles(seq);

@@ -202,7 +202,7 @@ int kx_q_absorb(const kx_config *cfg, const void *d_q, const void *d_kvb, const 
                 void *d_qabs, int32_t tokens, void *stream);
 int kx_mla_workspace_bytes(const kx_config *cfg, int32_t batch, int32_t max_seq, size_t *bytes);
 /* Which kernel computes the attention partials, process-wide: 0 (default) the matrix-core kernel from 2048
- * cached positions on and the VALU kernel below, 1 the VALU kernel always (fixed summation order, the one
+ * cached positions on (from 128 for five sequences and more) and the VALU kernel below, 1 the VALU kernel always (fixed summation order, the one
  * the token-identity checks rest on), 2 the matrix-core kernel always (same values, another summation
  * order; 64 heads).  No counterpart in the reference.                                              */
 int kx_mla_set_kernel(int32_t mode);
