@@ -335,6 +335,32 @@ def test_kimi_shape_long_context_stack_attention_paths(kxlib, ox):
     assert err < 3e-2 and (got[0][0] == got[1][0]).all()
 
 
+def test_kimi_shape_batched_stack_attention_paths(kxlib, ox):
+    # five sequences and more take the matrix-core attention kernel from 128 cached positions on (their projections run
+    # on the matrix cores as well).  Held against the same stack with the VALU attention kernel forced: logits of the
+    # first sampled step within the stack-level 3e-2, the same first id for at least three quarters of the sequences.
+    say("kimi shape 2-layer stack, batch 8, 160-token prompts, attention paths")
+    cfg = default_config()
+    batch, plen = 8, 160
+    cfg.n_layers, cfg.first_dense, cfg.max_batch, cfg.max_context, cfg.seed = 2, 1, batch, 192, 5
+    prompt = O.tokens_u32(batch * plen, cfg.seed, 4, cfg.vocab).reshape(batch, plen)
+    got = {}
+    try:
+        for mode in (0, 1):
+            check(kxlib.kx_mla_set_kernel(mode))
+            km = KxModel(kxlib, cfg)
+            rc, out, _ = km.generate(prompt, 1)
+            assert rc == 0, kxlib.kx_last_error()
+            got[mode] = (out.copy(), km.logits(batch))
+            km.close()
+    finally:
+        check(kxlib.kx_mla_set_kernel(0))
+    err = O.max_rel(got[0][1], got[1][1])
+    agree = float(np.mean(got[0][0] == got[1][0]))
+    print(f"batch-8 stack, matrix-core vs VALU attention: logits max-rel {err:.3e}, first ids equal for {agree:.0%}", flush=True)
+    assert err < 3e-2 and agree >= 0.75
+
+
 def test_executor_json_line(kxlib):
     import json
     import os
