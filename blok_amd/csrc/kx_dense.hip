@@ -68,6 +68,20 @@ __global__ void __launch_bounds__(TT > 1 ? 512 : 1024) gemv_bf16_k(KxGemvArgs a)
   gemv_body<MATS, RI, TT>(a, blockIdx.x, gridDim.x, part);
 }
 
+// The same GEMV with the tokens spread over the grid: workgroup (c, y) takes chunk c for tokens 4 y .. 4 y + 3.  For
+// many tokens against a small matrix (router logits, the per-head W_UV blocks): one workgroup going over the token
+// blocks one after the other spends its time waiting for each block's activations, while the weights all these
+// workgroups read again come from L2.  The sums are those of gemv_bf16_k (they do not depend on the launch shape).
+template <int RI>
+__global__ void __launch_bounds__(512) gemv_tokblk_k(KxGemvArgs a) {
+  extern __shared__ float part[];
+  const int t0 = blockIdx.y * 4;
+  a.x += (size_t)t0 * a.x_stride;
+  a.out = (char *)a.out + (size_t)t0 * a.out_stride * (a.epi == KX_EPI_F32 ? 4 : 2);
+  a.tokens = min(4, a.tokens - t0);
+  gemv_body<1, RI, 4>(a, blockIdx.x, gridDim.x, part);
+}
+
 // Two GEMVs over the same activations in one launch: the first gridDim.x - n0 workgroups run the
 // second problem (the router gate, f32 logits), the other n0 the first (two matrices, SwiGLU:
 // the shared expert's gate and up).  The router workgroup that finishes last routes the tokens: top-k and
@@ -277,9 +291,27 @@ int kx_gemv_launch(int epi, KxGemvArgs a, hipStream_t st) {
       b.route_w = a.route_w + (size_t)t0 * a.topk;
     }
     const int tt = b.tokens >= 4 ? 4 : b.tokens >= 2 ? 2 : 1;
+    const int chunks = kx_cdiv(a.rows, CR);
+    // 8 tokens and more against a matrix that stays in L2: the token blocks side by side (gemv_tokblk_k)
+    if (b.tokens >= 8 && (epi == KX_EPI_BF16 || epi == KX_EPI_F32) && !b.norm_w && !b.mla_po && chunks <= 4096 &&
+        (size_t)a.rows * a.cols * 2 <= (16u << 20)) {
+      // longer chunks, about 512 workgroups in all: a chunk's activations are read once, so rows per chunk divide the
+      // L2 traffic of the activations (one row per chunk: 57 KB of them against 14 KB of weights for the router)
+      const int blocks = kx_cdiv(b.tokens, 4);
+      int ri4;
+      const int CR4 = gemv_plan(epi, b, ri4, 4, 512 / blocks > 32 ? 512 / blocks : 32);
+      if (CR4 < 0) return KX_ERR_ARG;
+      ri = ri4;
+      const size_t lds4 = (size_t)CR4 * 4 * S * sizeof(float);
+      const dim3 g(kx_cdiv(a.rows, CR4), blocks), blk(b.nw * b.rs * 64);
+      if (ri == 4) hipLaunchKernelGGL(gemv_tokblk_k<4>, g, blk, lds4, st, b);
+      else if (ri == 2) hipLaunchKernelGGL(gemv_tokblk_k<2>, g, blk, lds4, st, b);
+      else hipLaunchKernelGGL(gemv_tokblk_k<1>, g, blk, lds4, st, b);
+      KX_LAUNCH_CHECK();
+      continue;
+    }
     const size_t lds = (size_t)mats * CR * b.tokens * S * sizeof(float);
     KX_REQUIRE(lds <= 160 * 1024, "kx_gemv: %zu bytes of LDS needed", lds);
-    const int chunks = kx_cdiv(a.rows, CR);
     dim3 g(chunks < 4096 ? chunks : 4096), blk(a.nw * a.rs * 64);
     if (mats == 2) launch_ri<2>(b, ri, tt, g, blk, lds, st);
     else launch_ri<1>(b, ri, tt, g, blk, lds, st);

@@ -36,6 +36,9 @@ def test_rmsnorm_parity(kxlib, ox, n, tokens):
     (64, 8192, 1, 0),       # o_proj width
     (40, 18432, 2, 0),      # dense down width (three slices per wave)
     (96, 2048, 5, 0),
+    (384, 7168, 32, 1),     # 8 tokens and more against a small matrix: token blocks side by side in the grid
+    (1000, 1536, 13, 0),    # the same, ragged rows and a ragged last token block
+    (2048, 512, 9, 0),
 ])
 def test_gemv_bf16_parity(kxlib, ox, rows, cols, tokens, f32):
     say(f"gemv_bf16 rows={rows} cols={cols} tokens={tokens} f32={f32}")
