@@ -113,54 +113,74 @@ using namespace kxa;
 // d = chain, chain+8, ... for columns 8 cl .. 8 cl + 7; the 8 chains are then summed pairwise.
 // Grid (heads * ceil(kv_rank / 128) + 1, T): the extra workgroup finishes the token's kv_a output and
 // writes its cache row.
-__global__ void __launch_bounds__(128) q_absorb_k(QAbsArgs a) {
-  __shared__ float part[8][128];
+// TB tokens per workgroup (blockIdx.y = block of TB tokens): a weight is loaded once for all of them, and each token's
+// sums are those of one token alone.  One token per workgroup reads the head's W_UK from L2 once per token, which
+// bounds the kernel from about 8 tokens on.
+template <int TB>
+__global__ void __launch_bounds__(128) q_absorb_k(QAbsArgs a, int tokens) {
+  __shared__ float part[TB][8][128];
   __shared__ float ws[4];
-  const int t = blockIdx.y;
+  const int t0 = blockIdx.y * TB;
   const int nope = a.nope, rope = a.rope, kv_rank = a.kv_rank;
   const int qk = nope + rope, kva = kv_rank + rope;
   const int cq_n = (kv_rank + 127) >> 7;
   if ((int)blockIdx.x == a.heads * cq_n) {
     if (a.cache)
-      kv_finish_block(a.kva + (size_t)t * a.kva_stride, a.w_kv_ln, a.rope_row, a.cache + (size_t)t * a.seq_stride + (size_t)a.pos * kva,
-                      kv_rank, rope, a.eps, ws);
+      for (int t = t0; t < min(t0 + TB, tokens); ++t) {
+        kv_finish_block(a.kva + (size_t)t * a.kva_stride, a.w_kv_ln, a.rope_row, a.cache + (size_t)t * a.seq_stride + (size_t)a.pos * kva,
+                        kv_rank, rope, a.eps, ws);
+        __syncthreads();  // ws is reused by the next token
+      }
     return;
   }
   const int h = blockIdx.x / cq_n, cq = blockIdx.x - h * cq_n;
   const int cl = threadIdx.x & 15, chain = threadIdx.x >> 4;
-  const uint16_t *qh = a.q + ((size_t)t * a.heads + h) * qk;
+  const uint16_t *qh[TB];
+#pragma unroll
+  for (int i = 0; i < TB; ++i) qh[i] = a.q + ((size_t)min(t0 + i, tokens - 1) * a.heads + h) * qk;
   const uint16_t *wuk = a.kvb + (size_t)h * (nope + a.v_head) * kv_rank;
-  float *out = a.qabs + ((size_t)t * a.heads + h) * kva;
   const int c0 = cq * 128 + cl * 8;
   if (c0 < kv_rank) {
-    float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll 16
+    float acc[TB][8];
+#pragma unroll
+    for (int i = 0; i < TB; ++i)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[i][e] = 0.0f;
+#pragma unroll(TB == 1 ? 16 : 4)
     for (int d = chain; d < nope; d += 8) {
       float wf[8];
       unpack8(wf, *(const uint4 *)(wuk + (size_t)d * kv_rank + c0));
-      const float qd = kx_bf16_f32(qh[d]);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(wf[e], qd, acc[e]);
+      for (int i = 0; i < TB; ++i) {
+        const float qd = kx_bf16_f32(qh[i][d]);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[i][e] = __builtin_fmaf(wf[e], qd, acc[i][e]);
+      }
     }
 #pragma unroll
-    for (int e = 0; e < 8; ++e) part[chain][cl * 8 + e] = acc[e];
+    for (int i = 0; i < TB; ++i)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) part[i][chain][cl * 8 + e] = acc[i][e];
   }
   __syncthreads();
-  {
+  const int half = rope >> 1;
+#pragma unroll
+  for (int i = 0; i < TB; ++i) {
+    if (t0 + i >= tokens) break;
+    float *out = a.qabs + ((size_t)(t0 + i) * a.heads + h) * kva;
     const int c = threadIdx.x;
     if (cq * 128 + c < kv_rank) {
-      const float s = ((part[0][c] + part[1][c]) + (part[2][c] + part[3][c])) + ((part[4][c] + part[5][c]) + (part[6][c] + part[7][c]));
+      const float s = ((part[i][0][c] + part[i][1][c]) + (part[i][2][c] + part[i][3][c])) + ((part[i][4][c] + part[i][5][c]) + (part[i][6][c] + part[i][7][c]));
       out[cq * 128 + c] = kx_bfround(s);
     }
-  }
-  const int half = rope >> 1;
-  if (cq == 0 && (int)threadIdx.x < half) {
-    const int p = threadIdx.x;
-    float lo, hi;
-    rope_pair(kx_bf16_f32(qh[nope + 2 * p]), kx_bf16_f32(qh[nope + 2 * p + 1]), kx_bf16_f32(a.rope_row[p]),
-              kx_bf16_f32(a.rope_row[half + p]), lo, hi);
-    out[kv_rank + p] = lo;
-    out[kv_rank + half + p] = hi;
+    if (cq == 0 && (int)threadIdx.x < half) {
+      const int p = threadIdx.x;
+      float lo, hi;
+      rope_pair(kx_bf16_f32(qh[i][nope + 2 * p]), kx_bf16_f32(qh[i][nope + 2 * p + 1]), kx_bf16_f32(a.rope_row[p]),
+                kx_bf16_f32(a.rope_row[half + p]), lo, hi);
+      out[kv_rank + p] = lo;
+      out[kv_rank + half + p] = hi;
+    }
   }
 }
 
@@ -677,7 +697,9 @@ int kx_q_absorb_launch(const uint16_t *q, const uint16_t *kvb, const uint16_t *r
   a.q = q; a.kvb = kvb; a.rope_row = rope_row; a.qabs = qabs; a.kva = kva; a.w_kv_ln = w_kv_ln; a.cache = cache;
   a.seq_stride = seq_stride; a.heads = heads; a.nope = nope; a.rope = rope; a.v_head = v_head; a.kv_rank = kv_rank;
   a.kva_stride = kva_stride; a.pos = pos; a.eps = eps;
-  hipLaunchKernelGGL(q_absorb_k, dim3(heads * ((kv_rank + 127) / 128) + (cache ? 1 : 0), tokens), dim3(128), 0, st, a);
+  const dim3 g1(heads * ((kv_rank + 127) / 128) + (cache ? 1 : 0), tokens);
+  if (tokens >= 8) hipLaunchKernelGGL(q_absorb_k<4>, dim3(g1.x, (tokens + 3) / 4), dim3(128), 0, st, a, tokens);
+  else hipLaunchKernelGGL(q_absorb_k<1>, g1, dim3(128), 0, st, a, tokens);
   KX_LAUNCH_CHECK();
   return KX_OK;
 }

@@ -254,6 +254,38 @@ def test_fused_and_separate_launches_agree(kxlib, ox, shape):
         assert (h1 == h0).all() and (l1 == l0).all() and (o1 == o0).all()
 
 
+@pytest.mark.parametrize("tokens", [1, 3, 9, 32])
+def test_q_absorb_operator(kxlib, ox, tokens):
+    # bf(W_UK^T q_nope): eight fp32 chains over d = j, j+8, ... summed ((0+1)+(2+3))+((4+5)+(6+7)) (bf16 products are
+    # exact in fp32, so numpy's add of the product is the fma).  From 8 tokens on a workgroup takes four tokens: every
+    # row, rope part included, must equal the row the one-token launch gives, to the bit.
+    say(f"q_absorb tokens={tokens}")
+    cfg = default_config()
+    Hd, nope, rope, vh, R = cfg.heads, cfg.qk_nope, cfg.qk_rope, cfg.v_head, cfg.kv_rank
+    q = O.normal_bf16(tokens * Hd * (nope + rope), 9, 1, 1.0).reshape(tokens, Hd, nope + rope)
+    kvb = O.normal_bf16(Hd * (nope + vh) * R, 9, 2, 0.05).reshape(Hd, nope + vh, R)
+    tab = np.empty((1, rope), dtype=np.uint16)
+    check(kxlib.kx_rope_table(C.byref(cfg), 77, 1, ptr(tab)))
+    dq, dk, dr = dev(q), dev(kvb), dev(tab)
+    do = DevBuf(tokens * Hd * (R + rope) * 4)
+    check(kxlib.kx_q_absorb(C.byref(cfg), dq.ptr, dk.ptr, dr.ptr, do.ptr, tokens, None))
+    check(kxlib.kx_sync(None))
+    got = do.to_numpy(np.float32, (tokens, Hd, R + rope))
+    d1 = DevBuf(Hd * (R + rope) * 4)
+    for t in range(tokens):
+        check(kxlib.kx_q_absorb(C.byref(cfg), dq.ptr + t * Hd * (nope + rope) * 2, dk.ptr, dr.ptr, d1.ptr, 1, None))
+        check(kxlib.kx_sync(None))
+        one = d1.to_numpy(np.float32, (Hd, R + rope))
+        assert (one.view(np.uint32) == got[t].view(np.uint32)).all(), f"token {t} differs from the one-token launch"
+    qf, wf = O.bf16_to_f32(q), O.bf16_to_f32(kvb)
+    acc = np.zeros((8, tokens, Hd, R), dtype=np.float32)
+    for d in range(nope):
+        acc[d % 8] = acc[d % 8] + wf[None, :, d, :] * qf[:, :, d, None]
+    tot = ((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7]))
+    exp = O.bf16_to_f32(O.f32_to_bf16(tot))
+    assert (exp.view(np.uint32) == got[:, :, :R].view(np.uint32)).all()
+
+
 @pytest.mark.parametrize("batch,seq", [(1, 1), (1, 100), (2, 700), (1, 5000)])
 def test_mla_decode_operator(kxlib, ox, batch, seq):
     # BASELINE config 3 shapes (64 heads, latent 512+64) at lengths the scalar oracle finishes quickly
