@@ -412,6 +412,19 @@ extern "C" int kx_rmsnorm(const void *d_x, const void *d_w, void *d_y, int32_t t
                            kx_stream(stream));
 }
 
+// sample_lm_head (:718-734) as an operator: bf16-rounded logits of the normed rows, then argmax_k's choice (:477-493)
+extern "C" int kx_lm_head_argmax(const void *d_w, const void *d_n, void *d_logits, void *d_ids, int32_t vocab,
+                                 int32_t hidden, int32_t tokens, void *d_scratch, void *stream) {
+  KX_REQUIRE(d_w && d_n && d_logits && d_ids && d_scratch, "kx_lm_head_argmax: null pointer");
+  KX_REQUIRE(vocab > 0 && tokens > 0, "kx_lm_head_argmax: vocab=%d tokens=%d must be positive", vocab, tokens);
+  KxGemvArgs a = {};
+  a.w0 = (const uint16_t *)d_w; a.x = (const uint16_t *)d_n; a.x_stride = hidden;
+  a.out = d_logits; a.out_stride = vocab; a.rows = vocab; a.cols = hidden; a.tokens = tokens;
+  int rc = kx_gemv_launch(KX_EPI_ARGMAX, a, kx_stream(stream));
+  if (rc) return rc;
+  return kx_argmax_launch((const float *)d_logits, tokens, vocab, vocab, (uint32_t *)d_ids, (float *)d_scratch, kx_stream(stream));
+}
+
 extern "C" int kx_gemv_bf16(const void *d_w, const void *d_x, void *d_y, int32_t rows, int32_t cols,
                             int32_t tokens, int out_f32, void *stream) {
   KX_REQUIRE(d_w && d_x && d_y, "kx_gemv_bf16: null pointer");

@@ -109,11 +109,18 @@ int kx_i4_gemv(const void *d_packed, const void *d_scale, const void *d_x, void 
  * kx_rmsnorm  : rmsnorm_k (:258-270); x, y bf16 [T, n], w bf16 [n].
  * kx_gemv_bf16: matvec_bf16_k (:272-284) when out_f32 == 0 (y bf16 [T, rows],
  *               rounded) and matvec_bf16_f32_k (:286-298) when out_f32 != 0
- *               (y f32 [T, rows], unrounded).  cols multiple of 512.         */
+ *               (y f32 [T, rows], unrounded).  cols multiple of 512.
+ * kx_lm_head_argmax: sample_lm_head (:718-734) + argmax_k (:477-493) on rows that
+ *               are already normed (:880): d_logits f32 [T, vocab] receives the
+ *               bf16-rounded logits bf(W n), d_ids u32 [T] the index of the
+ *               largest one, the lowest index on ties, 0 when no logit compares
+ *               greater than -inf.  d_scratch: T * 512 bytes.  hidden multiple of 512. */
 int kx_rmsnorm(const void *d_x, const void *d_w, void *d_y, int32_t tokens, int32_t n, float eps,
                void *stream);
 int kx_gemv_bf16(const void *d_w, const void *d_x, void *d_y, int32_t rows, int32_t cols,
                  int32_t tokens, int out_f32, void *stream);
+int kx_lm_head_argmax(const void *d_w, const void *d_n, void *d_logits, void *d_ids, int32_t vocab,
+                      int32_t hidden, int32_t tokens, void *d_scratch, void *stream);
 
 /* ---- router --------------------------------------------------------------
  * kx_router_topk: sigmoid_k + add_bf16_k + router_topk_k (:372-397) on fp32

@@ -58,6 +58,31 @@ def test_gemv_bf16_parity(kxlib, ox, rows, cols, tokens, f32):
     assert O.max_rel(to_f(y), to_f(y0)) < 1e-2
 
 
+@pytest.mark.parametrize("vocab,hidden,tokens", [(5000, 1024, 1), (5000, 1024, 3), (777, 512, 9)])
+def test_lm_head_argmax_parity(kxlib, ox, vocab, hidden, tokens):
+    # logits = bf(W n) to the bit against the oracle's GEMV; the id is the lowest index of the largest rounded logit:
+    # the winning row of token 0 is copied to a later row, so that token has an exact tie
+    say(f"lm_head_argmax vocab={vocab} hidden={hidden} tokens={tokens}")
+    w = O.normal_bf16(vocab * hidden, 6, 1, 0.02).reshape(vocab, hidden)
+    x = O.normal_bf16(tokens * hidden, 6, 2, 1.0).reshape(tokens, hidden)
+    y1 = np.empty((tokens, vocab), dtype=np.uint16)
+    ox.ox_gemv_bf16(ptr(w), ptr(x), ptr(y1), vocab, hidden, tokens, 0, 1)
+    first = int(np.argmax(O.bf16_to_f32(y1)[0]))
+    later = vocab - 1 if first != vocab - 1 else vocab - 2
+    w[max(first, later)] = w[min(first, later)]
+    ox.ox_gemv_bf16(ptr(w), ptr(x), ptr(y1), vocab, hidden, tokens, 0, 1)
+    exp = O.bf16_to_f32(y1)
+    dw, dx = dev(w), dev(x)
+    dl, di, ds = DevBuf(tokens * vocab * 4), DevBuf(tokens * 4), DevBuf(tokens * 512)
+    check(kxlib.kx_lm_head_argmax(dw.ptr, dx.ptr, dl.ptr, di.ptr, vocab, hidden, tokens, ds.ptr, None))
+    check(kxlib.kx_sync(None))
+    got = dl.to_numpy(np.float32, (tokens, vocab))
+    ids = di.to_numpy(np.uint32, (tokens,))
+    assert (got.view(np.uint32) == exp.view(np.uint32)).all()
+    assert (ids == np.argmax(exp, axis=1)).all()
+    assert ids[0] == min(first, later)
+
+
 def test_shape_errors(kxlib):
     b = DevBuf(4096)
     assert kxlib.kx_gemv_bf16(b.ptr, b.ptr, b.ptr, 4, 500, 1, 0, None) != 0
