@@ -92,9 +92,9 @@ int kx_gemv_pair_route_launch(KxGemvArgs shared_gate_up, KxGemvArgs router, cons
                               int *n_active, int *counter, bool *fused, hipStream_t st);
 int kx_route_launch(const float *logits, const float *bias, uint16_t *ids, float *weights, int tokens, int experts,
                     int topk, float routed_scale, int *counts, int *offsets, int *pairs, int4 *work, int *n_active,
-                    hipStream_t st);
+                    hipStream_t st, int4 *pair_work = nullptr);
 int kx_bucket_launch(const uint16_t *ids, int tokens, int experts, int topk, int *counts, int *offsets,
-                     int *pairs, int4 *work, int *n_active, hipStream_t st);
+                     int *pairs, int4 *work, int *n_active, hipStream_t st, int4 *pair_work = nullptr);
 
 // kx_prefill.hip
 // outputs of the grouped GEMM: bf16; fp32 unrounded; fp32 holding the bf16-rounded value; bf16 residual add into out

@@ -53,13 +53,17 @@ __device__ __forceinline__ void topk_token(const float *lg, const float *__restr
 }
 
 // one workgroup, thread e owns expert e: count, exclusive scan, stable placement.
+// pair_work, if set, receives a second work list with one record per pair, {expert, q, q + 1, pairs[q]} for sorted
+// pair q: the routed kernels then give every (chunk, pair) a workgroup of its own, and the workgroups of one chunk
+// (an expert's pairs are neighbours in the list, so they are `chunks per expert` apart in the grid) stream it at the
+// same time instead of one workgroup streaming it once per pair.
 // The ids are staged in LDS (padded with 0xffff to a multiple of 8) and scanned 8 at a time;
 // `staged` says the caller has already put them there.
 __device__ __forceinline__ void bucket_block(const uint16_t *__restrict__ ids, int n_pairs, int E,
                                              int *__restrict__ counts, int *__restrict__ offsets,
                                              int *__restrict__ pairs, int4 *__restrict__ work,
                                              int *__restrict__ n_active, uint4 *s_ids4, int *s_cnt, int *s_act,
-                                             bool staged = false) {
+                                             bool staged = false, int4 *__restrict__ pair_work = nullptr) {
   const int e = threadIdx.x, n = blockDim.x;
   const int n8 = (n_pairs + 7) >> 3;
   uint16_t *s_ids = (uint16_t *)s_ids4;
@@ -100,6 +104,7 @@ __device__ __forceinline__ void bucket_block(const uint16_t *__restrict__ ids, i
           const uint32_t h = (j & 1) ? (w[j >> 1] >> 16) : (w[j >> 1] & 0xffffu);
           if (h == 0) {
             if (pos == off) first = q * 8 + j;
+            if (pair_work) pair_work[pos] = make_int4(e, pos, pos + 1, q * 8 + j);
             pairs[pos++] = q * 8 + j;
           }
         }
@@ -120,7 +125,8 @@ __device__ __forceinline__ void route_block(const float *__restrict__ logits, co
                                             uint16_t *__restrict__ ids, float *__restrict__ weights, int tokens, int E,
                                             int topk, float routed_scale, int *__restrict__ counts,
                                             int *__restrict__ offsets, int *__restrict__ pairs, int4 *__restrict__ work,
-                                            int *__restrict__ n_active, uint4 *s_ids4, int *s_cnt, int *s_act) {
+                                            int *__restrict__ n_active, uint4 *s_ids4, int *s_cnt, int *s_act,
+                                            int4 *__restrict__ pair_work = nullptr) {
   uint16_t *s_ids = (uint16_t *)s_ids4;
   const int n_pairs = tokens * topk, n8 = (n_pairs + 7) >> 3;
   for (int p = n_pairs + threadIdx.x; p < n8 * 8; p += blockDim.x) s_ids[p] = (uint16_t)0xffff;
@@ -129,7 +135,7 @@ __device__ __forceinline__ void route_block(const float *__restrict__ logits, co
     topk_token<EPL, COHERENT>(logits + (size_t)t * E, bias, ids + (size_t)t * topk, weights + (size_t)t * topk, E, topk,
                               routed_scale, threadIdx.x & 63, s_ids + t * topk);
   __syncthreads();
-  bucket_block(ids, n_pairs, E, counts, offsets, pairs, work, n_active, s_ids4, s_cnt, s_act, true);
+  bucket_block(ids, n_pairs, E, counts, offsets, pairs, work, n_active, s_ids4, s_cnt, s_act, true, pair_work);
 }
 
 // route_block with the per-lane expert count chosen at run time; COHERENT: the logits were written by other

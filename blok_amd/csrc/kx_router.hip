@@ -35,11 +35,11 @@ __global__ void __launch_bounds__(64) router_topk_k(const float *__restrict__ lo
 __global__ void __launch_bounds__(1024) bucket_k(const uint16_t *__restrict__ ids, int n_pairs, int E,
                                                  int *__restrict__ counts, int *__restrict__ offsets,
                                                  int *__restrict__ pairs, int4 *__restrict__ work,
-                                                 int *__restrict__ n_active) {
+                                                 int *__restrict__ n_active, int4 *__restrict__ pair_work) {
   extern __shared__ uint4 s_ids4[];  // ceil(n_pairs / 8) pieces
   __shared__ int s_cnt[1024];
   __shared__ int s_act[1024];
-  bucket_block(ids, n_pairs, E, counts, offsets, pairs, work, n_active, s_ids4, s_cnt, s_act);
+  bucket_block(ids, n_pairs, E, counts, offsets, pairs, work, n_active, s_ids4, s_cnt, s_act, false, pair_work);
 }
 
 // top-k of the tokens (one wave each, in turns), then the bucketing, in one workgroup
@@ -48,12 +48,13 @@ __global__ void __launch_bounds__(1024) topk_bucket_k(const float *__restrict__ 
                                                       uint16_t *__restrict__ ids, float *__restrict__ weights, int tokens,
                                                       int E, int topk, float routed_scale, int *__restrict__ counts,
                                                       int *__restrict__ offsets, int *__restrict__ pairs,
-                                                      int4 *__restrict__ work, int *__restrict__ n_active) {
+                                                      int4 *__restrict__ work, int *__restrict__ n_active,
+                                                      int4 *__restrict__ pair_work) {
   extern __shared__ uint4 s_ids4[];
   __shared__ int s_cnt[1024];
   __shared__ int s_act[1024];
   kxr::route_block<EPL>(logits, bias, ids, weights, tokens, E, topk, routed_scale, counts, offsets, pairs, work, n_active,
-                        s_ids4, s_cnt, s_act);
+                        s_ids4, s_cnt, s_act, pair_work);
 }
 
 // ---- bucketing of a prefill chunk: one workgroup per expert instead of one per launch ------------
@@ -184,12 +185,13 @@ int kx_router_topk_launch(const float *logits, const float *bias, uint16_t *ids,
 }
 
 int kx_bucket_launch(const uint16_t *ids, int tokens, int experts, int topk, int *counts, int *offsets, int *pairs,
-                     int4 *work, int *n_active, hipStream_t st) {
+                     int4 *work, int *n_active, hipStream_t st, int4 *pair_work) {
   KX_REQUIRE(tokens > 0 && topk > 0, "kx_bucket: tokens=%d topk=%d must be positive", tokens, topk);
   KX_REQUIRE(experts > 0 && experts <= 1024, "kx_bucket: experts=%d outside [1, 1024]", experts);
   int threads = kx_cdiv(experts, 64) * 64;
   const long n_pairs = (long)tokens * topk;
   KX_REQUIRE(n_pairs < (1L << 30), "kx_bucket: %ld pairs", n_pairs);
+  KX_REQUIRE(!pair_work || n_pairs <= 1024, "kx_bucket: the per-pair work list is written for up to 1024 pairs (got %ld)", n_pairs);
   if (n_pairs > 1024) {  // a chunk: one workgroup per expert counts, one scans, one per expert places
     hipLaunchKernelGGL(bucket_count_k, dim3(experts), dim3(256), 0, st, ids, (int)n_pairs, counts);
     KX_LAUNCH_CHECK();
@@ -201,7 +203,7 @@ int kx_bucket_launch(const uint16_t *ids, int tokens, int experts, int topk, int
   }
   const size_t lds = (size_t)kx_cdiv((int)n_pairs, 8) * 16;
   hipLaunchKernelGGL(bucket_k, dim3(1), dim3(threads), lds, st, ids, (int)n_pairs, experts, counts, offsets, pairs,
-                     work, n_active);
+                     work, n_active, pair_work);
   KX_LAUNCH_CHECK();
   return KX_OK;
 }
@@ -217,24 +219,24 @@ extern "C" int kx_bucket(const void *d_ids, int32_t tokens, int32_t experts, int
                          void *d_offsets, void *d_pairs, void *d_work, void *d_n_active, void *stream) {
   KX_REQUIRE(d_ids && d_counts && d_offsets && d_pairs && d_work && d_n_active, "kx_bucket: null pointer");
   return kx_bucket_launch((const uint16_t *)d_ids, tokens, experts, topk, (int *)d_counts, (int *)d_offsets,
-                          (int *)d_pairs, (int4 *)d_work, (int *)d_n_active, kx_stream(stream));
+                          (int *)d_pairs, (int4 *)d_work, (int *)d_n_active, kx_stream(stream), nullptr);
 }
 
 // top-k and bucketing; one launch when the tokens fit one workgroup (16 waves), two otherwise
 int kx_route_launch(const float *logits, const float *bias, uint16_t *ids, float *weights, int tokens, int experts,
                     int topk, float routed_scale, int *counts, int *offsets, int *pairs, int4 *work, int *n_active,
-                    hipStream_t st) {
+                    hipStream_t st, int4 *pair_work) {
   if (tokens > 16 || experts > 1024) {
     int rc = kx_router_topk_launch(logits, bias, ids, weights, tokens, experts, topk, routed_scale, st);
     if (rc) return rc;
-    return kx_bucket_launch(ids, tokens, experts, topk, counts, offsets, pairs, work, n_active, st);
+    return kx_bucket_launch(ids, tokens, experts, topk, counts, offsets, pairs, work, n_active, st, pair_work);
   }
   KX_REQUIRE(tokens > 0 && experts > 0 && topk > 0 && topk <= 64 && topk <= experts, "kx_route: tokens=%d experts=%d topk=%d", tokens, experts, topk);
   int threads = kx_cdiv(experts, 64) * 64;
   if (threads < tokens * 64) threads = tokens * 64;
   const size_t lds = (size_t)kx_cdiv(tokens * topk, 8) * 16;
   const int epl = kx_cdiv(experts, 64);
-#define KX_TB(N) hipLaunchKernelGGL(topk_bucket_k<N>, dim3(1), dim3(threads), lds, st, logits, bias, ids, weights, tokens, experts, topk, routed_scale, counts, offsets, pairs, work, n_active)
+#define KX_TB(N) hipLaunchKernelGGL(topk_bucket_k<N>, dim3(1), dim3(threads), lds, st, logits, bias, ids, weights, tokens, experts, topk, routed_scale, counts, offsets, pairs, work, n_active, pair_work)
   if (epl <= 1) KX_TB(1);
   else if (epl <= 2) KX_TB(2);
   else if (epl <= 4) KX_TB(4);
