@@ -89,7 +89,7 @@ int kx_router_topk_launch(const float *logits, const float *bias, uint16_t *ids,
                           int experts, int topk, float routed_scale, hipStream_t st);
 int kx_gemv_pair_route_launch(KxGemvArgs shared_gate_up, KxGemvArgs router, const float *bias, uint16_t *ids, float *weights,
                               int experts, int topk, float routed_scale, int *counts, int *offsets, int *pairs, int4 *work,
-                              int *n_active, int *counter, bool *fused, hipStream_t st);
+                              int *n_active, int *counter, bool *fused, hipStream_t st, int4 *pair_work = nullptr);
 int kx_route_launch(const float *logits, const float *bias, uint16_t *ids, float *weights, int tokens, int experts,
                     int topk, float routed_scale, int *counts, int *offsets, int *pairs, int4 *work, int *n_active,
                     hipStream_t st, int4 *pair_work = nullptr);

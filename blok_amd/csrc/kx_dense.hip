@@ -96,6 +96,7 @@ struct KxRouteArgs {
   int *counts, *offsets, *pairs;
   int4 *work;
   int *n_active;
+  int4 *pair_work;  // optional second work list, one record per pair
 };
 template <int RI0, int TT>
 __global__ void __launch_bounds__(TT > 1 ? 512 : 1024) gemv_pair_k(KxGemvArgs a0, KxGemvArgs a1, int n0, KxRouteArgs r) {
@@ -121,7 +122,7 @@ __global__ void __launch_bounds__(TT > 1 ? 512 : 1024) gemv_pair_k(KxGemvArgs a0
   __syncthreads();
   if (!s_last) return;
   kxr::route_block_any<true>((const float *)a1.out, r.bias, r.ids, r.weights, a1.tokens, r.experts, r.topk, r.routed_scale,
-                       r.counts, r.offsets, r.pairs, r.work, r.n_active, s_ids4, s_cnt, s_act);
+                       r.counts, r.offsets, r.pairs, r.work, r.n_active, s_ids4, s_cnt, s_act, r.pair_work);
   if (threadIdx.x == 0) *r.counter = 0;
 }
 
@@ -325,7 +326,7 @@ int kx_gemv_launch(int epi, KxGemvArgs a, hipStream_t st) {
 // *fused = false, having launched nothing, when the shapes do not allow the combination.
 int kx_gemv_pair_route_launch(KxGemvArgs a0, KxGemvArgs a1, const float *bias, uint16_t *ids, float *weights, int experts,
                               int topk, float routed_scale, int *counts, int *offsets, int *pairs, int4 *work,
-                              int *n_active, int *counter, bool *fused, hipStream_t st) {
+                              int *n_active, int *counter, bool *fused, hipStream_t st, int4 *pair_work) {
   *fused = false;
   if (a0.tokens != a1.tokens || a0.tokens > 4 || a0.tokens * topk > 32 || a0.cols != a1.cols || topk > 64 || topk > experts) return KX_OK;
   int ri0, ri1;
@@ -342,7 +343,7 @@ int kx_gemv_pair_route_launch(KxGemvArgs a0, KxGemvArgs a1, const float *bias, u
   KxRouteArgs r;
   r.counter = counter; r.bias = bias; r.ids = ids; r.weights = weights; r.experts = experts; r.topk = topk;
   a1.flags |= KX_GEMV_COHERENT_OUT;
-  r.routed_scale = routed_scale; r.counts = counts; r.offsets = offsets; r.pairs = pairs; r.work = work; r.n_active = n_active;
+  r.routed_scale = routed_scale; r.counts = counts; r.offsets = offsets; r.pairs = pairs; r.work = work; r.n_active = n_active; r.pair_work = pair_work;
   const int tt = T >= 4 ? 4 : T >= 2 ? 2 : 1;
   dim3 g(n0 + n1), blk(threads);
 #define KX_PAIR(R, TT_) hipLaunchKernelGGL((gemv_pair_k<R, TT_>), g, blk, lds, st, a0, a1, n0, r)

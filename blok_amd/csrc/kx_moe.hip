@@ -132,13 +132,13 @@ static RoutedPlan routed_plan(int tokens, int topk, int experts) {
   return p;
 }
 
-// From 5 tokens on (below, the launches that finish the layer want the per-expert list) and while one launch with one
-// token per pass is the plan, the routed kernels go over the per-pair work list: one workgroup per (chunk, pair).
+// From 2 tokens on (the launch that finishes the layer for one token wants the per-expert list) and while one launch
+// with one token per pass is the plan, the routed kernels go over the per-pair work list: one workgroup per (chunk, pair).
 // A chunk's workgroups run at the same time on the same L2 (their ids differ by multiples of the chunks per expert,
 // a multiple of 8 at Kimi shapes), where one workgroup doing the expert's pairs one after the other streams the chunk
 // from memory once per pair (the chunks in flight, 29 MB, do not stay in L2) and is the launch's tail when an expert
 // has many pairs.  Batch 32 in the stack: gate/up 670 -> 544 us, down 385 -> 330 us per layer.
-static bool routed_per_pair(int tokens, int topk, int experts) { return tokens >= 5 && (long)tokens * topk <= experts; }
+static bool routed_per_pair(int tokens, int topk, int experts) { return tokens >= 2 && (long)tokens * topk <= experts; }
 
 // the routed gate/up (which = 0) or down (which = 1) kernel(s) over the work list in the workspace
 static int routed_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_workspace *ws, const uint16_t *n, int tokens,
@@ -197,7 +197,7 @@ int kx_moe_layer_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_work
   bool paired = false;
   if ((rc = kx_gemv_pair_route_launch(s, g, (const float *)w->d_router_bias, ws->ids, ws->weights, E, K, c->routed_scale,
                                       ws->counts, ws->offsets, ws->pairs, ws->work, ws->n_active, ws->route_counter, &paired,
-                                      st))) return rc;
+                                      st, routed_per_pair(tokens, K, E) ? ws->pair_work : nullptr))) return rc;
   if (!paired) {
     if ((rc = kx_gemv_launch(KX_EPI_F32, g, st))) return rc;
     if ((rc = kx_route_launch(ws->logits, (const float *)w->d_router_bias, ws->ids, ws->weights, tokens, E, K, c->routed_scale,

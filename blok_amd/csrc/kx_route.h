@@ -143,9 +143,10 @@ __device__ __forceinline__ void route_block(const float *__restrict__ logits, co
 template <bool COHERENT = false>
 __device__ __forceinline__ void route_block_any(const float *logits, const float *bias, uint16_t *ids, float *weights,
                                                 int tokens, int E, int topk, float routed_scale, int *counts, int *offsets,
-                                                int *pairs, int4 *work, int *n_active, uint4 *s_ids4, int *s_cnt, int *s_act) {
+                                                int *pairs, int4 *work, int *n_active, uint4 *s_ids4, int *s_cnt, int *s_act,
+                                                int4 *pair_work = nullptr) {
   const int epl = (E + 63) >> 6;
-#define KX_RB(N) route_block<N, COHERENT>(logits, bias, ids, weights, tokens, E, topk, routed_scale, counts, offsets, pairs, work, n_active, s_ids4, s_cnt, s_act)
+#define KX_RB(N) route_block<N, COHERENT>(logits, bias, ids, weights, tokens, E, topk, routed_scale, counts, offsets, pairs, work, n_active, s_ids4, s_cnt, s_act, pair_work)
   if (epl <= 1) KX_RB(1);
   else if (epl <= 2) KX_RB(2);
   else if (epl <= 4) KX_RB(4);
