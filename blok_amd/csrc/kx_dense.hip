@@ -304,6 +304,7 @@ int kx_gemv_launch(int epi, KxGemvArgs a, hipStream_t st) {
       if (CR4 < 0) return KX_ERR_ARG;
       ri = ri4;
       const size_t lds4 = (size_t)CR4 * 4 * S * sizeof(float);
+      KX_REQUIRE(lds4 <= 64 * 1024, "kx_gemv: %zu bytes of LDS needed", lds4);
       const dim3 g(kx_cdiv(a.rows, CR4), blocks), blk(b.nw * b.rs * 64);
       if (ri == 4) hipLaunchKernelGGL(gemv_tokblk_k<4>, g, blk, lds4, st, b);
       else if (ri == 2) hipLaunchKernelGGL(gemv_tokblk_k<2>, g, blk, lds4, st, b);
