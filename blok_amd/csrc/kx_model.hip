@@ -74,6 +74,8 @@ struct kx_model {
   hipStream_t st = nullptr;
   hipEvent_t ev[3] = {nullptr, nullptr, nullptr};
   int batch = 0, pos = 0;
+  int prefill_chunk = 1;  // prompt positions per prefill step (kx_model_set_prefill_chunk)
+  int x_row0 = 0;         // first row of x that belongs to the last position of the last step
   bool sampled = false;
   float ms_prefill = 0, ms_decode = 0;
   uint64_t load_bytes = 0;  // checkpoint bytes copied in by kx_model_load, and the time that took
@@ -81,6 +83,10 @@ struct kx_model {
 };
 
 namespace {
+
+// tokens a step may carry: a decode step has one per sequence, a prefill step up to this many (positions x sequences)
+constexpr int STEP_TOKENS = 32;
+inline int step_tokens(const kx_config *c) { return c->max_batch > STEP_TOKENS ? c->max_batch : STEP_TOKENS; }
 
 struct Plan {  // byte offsets of everything in the arena
   size_t total = 0, weights = 0, cache = 0, scratch = 0;
@@ -158,15 +164,16 @@ int layout(const kx_config *c, Plan &p, kx_model *m) {
   }
   p.cache = p.total - p.weights;
   const size_t inter = D > KD ? D : KD;
-  auto *x = KX_AT(uint16_t *, B * H * 2);
-  auto *n = KX_AT(uint16_t *, B * H * 2);
-  auto *qkv = KX_AT(uint16_t *, B * ((size_t)c->q_rank + KVA) * 2);
-  auto *qa = KX_AT(uint16_t *, B * (size_t)c->q_rank * 2);
-  auto *q = KX_AT(uint16_t *, B * KD * 2);
-  auto *o_lat = KX_AT(uint16_t *, B * (size_t)c->heads * c->kv_rank * 2);
-  auto *att = KX_AT(uint16_t *, B * VD * 2);
-  auto *dmid = KX_AT(uint16_t *, B * inter * 2);
-  auto *qabs = KX_AT(float *, B * (size_t)c->heads * KVA * 4);
+  const size_t BT = step_tokens(c);  // rows of the per-token scratch
+  auto *x = KX_AT(uint16_t *, BT * H * 2);
+  auto *n = KX_AT(uint16_t *, BT * H * 2);
+  auto *qkv = KX_AT(uint16_t *, BT * ((size_t)c->q_rank + KVA) * 2);
+  auto *qa = KX_AT(uint16_t *, BT * (size_t)c->q_rank * 2);
+  auto *q = KX_AT(uint16_t *, BT * KD * 2);
+  auto *o_lat = KX_AT(uint16_t *, BT * (size_t)c->heads * c->kv_rank * 2);
+  auto *att = KX_AT(uint16_t *, BT * VD * 2);
+  auto *dmid = KX_AT(uint16_t *, BT * inter * 2);
+  auto *qabs = KX_AT(float *, BT * (size_t)c->heads * KVA * 4);
   auto *partial = KX_AT(float *, kx_mla_partial_floats(c->max_batch, c->heads, c->kv_rank, c->max_context) * 4);
   auto *logits = KX_AT(float *, B * V * 4);
   auto *argmax_scratch = KX_AT(float *, KX_ARGMAX_SCRATCH_FLOATS(B) * 4);
@@ -242,10 +249,14 @@ int init_weights(kx_model *m) {
   return init_rope(m);
 }
 
-// one run() of the reference for `B` tokens at position m->pos; ids on the device
-int step(kx_model *m, const uint32_t *d_ids, bool sample) {
+// one run() of the reference for `B` tokens at position m->pos; ids on the device.
+// C > 1 (prefill): C consecutive positions of every sequence in one step, tokens position-major (token i * B + b is
+// position pos + i of sequence b).  Everything but the attention is per token, so the step runs as a batch of B * C
+// tokens; the cache rows of all C positions are written first, then position i attends to rows 0 .. pos + i.  Only the
+// last position is sampled.
+int step(kx_model *m, const uint32_t *d_ids, bool sample, int C = 1) {
   const kx_config &c = m->c;
-  const int B = m->batch, H = c.hidden, pos = m->pos;
+  const int NB = m->batch, B = NB * C, H = c.hidden, pos = m->pos;
   const int KD = c.heads * (c.qk_nope + c.qk_rope), VD = c.heads * c.v_head, KVA = c.kv_rank + c.qk_rope;
   const int QKV = c.q_rank + KVA;
   hipStream_t st = m->st;
@@ -255,7 +266,7 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample) {
   KX_LAUNCH_CHECK();
   const uint16_t *rope_row = m->rope_tab + (size_t)pos * c.qk_rope;
   const size_t seq_stride = (size_t)c.max_context * KVA;
-  const bool fuse = B <= 4;  // RMSNorms ride in the prologue of the GEMV that consumes them
+  const bool fuse = B <= 4 && C == 1;  // RMSNorms ride in the prologue of the GEMV that consumes them
   // From 5 sequences on (the fused prologues cover up to 4), the dense projections run as GEMMs on the matrix cores: the
   // GEMV is bound by its fma count there.  Same values, another summation order (the bf16 rounding points stay).
   const bool mm = B >= 5;
@@ -296,8 +307,11 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample) {
     }
     if (!absorbed) {
       KX_TRY(dense(KX_EPI_BF16, g));                                                                    // :815
-      KX_TRY(kx_q_absorb_launch(m->q, L.kvb, rope_row, m->qabs, B, c.heads, c.qk_nope, c.qk_rope, c.v_head, c.kv_rank,
-                                m->qkv + c.q_rank, QKV, L.kv_ln, L.cache, seq_stride, pos, c.rms_eps, st));
+      for (int i = 0; i < C; ++i)
+        KX_TRY(kx_q_absorb_launch(m->q + (size_t)i * NB * KD, L.kvb, rope_row + (size_t)i * c.qk_rope,
+                                  m->qabs + (size_t)i * NB * c.heads * KVA, NB, c.heads, c.qk_nope, c.qk_rope, c.v_head,
+                                  c.kv_rank, m->qkv + c.q_rank + (size_t)i * NB * QKV, QKV, L.kv_ln, L.cache, seq_stride,
+                                  pos + i, c.rms_eps, st));
     }
     g = {};  // W_UV of :818 per head
     g.w0 = L.kvb; g.x = m->o_lat; g.x_stride = c.heads * c.kv_rank; g.out = m->att; g.out_stride = VD; g.rows = VD;
@@ -312,7 +326,9 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample) {
         KX_TRY(kx_mla_combine_launch(mp, m->o_lat, B, c.heads, st));
       }
     } else {
-      KX_TRY(kx_mla_attend_launch(&c, L.cache, seq_stride, m->qabs, m->partial, m->o_lat, B, pos + 1, st));
+      for (int i = 0; i < C; ++i)
+        KX_TRY(kx_mla_attend_launch(&c, L.cache, seq_stride, m->qabs + (size_t)i * NB * c.heads * KVA, m->partial,
+                                    m->o_lat + (size_t)i * NB * c.heads * c.kv_rank, NB, pos + i + 1, st));
     }
     KX_TRY(kx_gemv_launch(KX_EPI_BF16, g, st));
     g = {};
@@ -335,18 +351,20 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample) {
                                  fuse ? L.post_ln : nullptr, st, false));  // :835-877
     }
   }
+  const uint16_t *x_last = m->x + (size_t)(C - 1) * NB * H;  // rows of the last position
   if (sample) {                                                                                          // :880-881
     KxGemvArgs g = {};
     g.w0 = m->lm_head; g.x = m->n; g.x_stride = H; g.out = m->logits; g.out_stride = c.vocab; g.rows = c.vocab; g.cols = H;
-    g.tokens = B;
+    g.tokens = NB;
     if (fuse) { g.x = m->x; g.norm_w = m->final_norm; g.norm_eps = c.rms_eps; }
-    else KX_TRY(kx_rmsnorm_launch(m->x, m->final_norm, m->n, B, H, H, H, c.rms_eps, st));
+    else KX_TRY(kx_rmsnorm_launch(x_last, m->final_norm, m->n, NB, H, H, H, c.rms_eps, st));
     KX_TRY(dense(KX_EPI_ARGMAX, g));
-    KX_TRY(kx_argmax_launch(m->logits, B, c.vocab, c.vocab, m->next, m->argmax_scratch, st));
+    KX_TRY(kx_argmax_launch(m->logits, NB, c.vocab, c.vocab, m->next, m->argmax_scratch, st));
   }
 #undef KX_TRY
   m->sampled = sample;
-  m->pos = pos + 1;
+  m->pos = pos + C;
+  m->x_row0 = (C - 1) * NB;
   return KX_OK;
 }
 
@@ -390,7 +408,7 @@ static int model_new(const kx_config *cfg, const char *who, kx_model **out) {
   if (hipStreamCreate(&m->st) != hipSuccess) rc = KX_ERR_HIP;
   for (auto &ev : m->ev)
     if (!rc && hipEventCreate(&ev) != hipSuccess) rc = KX_ERR_HIP;
-  if (!rc && cfg->first_dense < cfg->n_layers) rc = kx_moe_workspace_create(cfg, cfg->max_batch, &m->moe_ws);
+  if (!rc && cfg->first_dense < cfg->n_layers) rc = kx_moe_workspace_create(cfg, step_tokens(cfg), &m->moe_ws);
   if (!rc && (hipMemsetAsync(m->head_count, 0, (size_t)cfg->heads * 4, m->st) != hipSuccess || hipStreamSynchronize(m->st) != hipSuccess))
     rc = KX_ERR_HIP;
   if (rc) {
@@ -517,8 +535,13 @@ extern "C" int kx_prefill(kx_model *m, const uint32_t *h_ids, int32_t batch, int
   KX_HIP(hipStreamSynchronize(m->st));  // pm goes out of scope
   m->batch = batch;
   m->pos = 0;
-  for (int i = 0; i < prompt_len; ++i)  // :886: one run() per prompt token, sampling on the last
-    if ((rc = step(m, m->ids + (size_t)i * batch, i + 1 == prompt_len))) return rc;
+  // :886: one run() per prompt token, sampling on the last; with a prefill chunk set, up to that many positions per step
+  int chunk = m->prefill_chunk < STEP_TOKENS / batch ? m->prefill_chunk : STEP_TOKENS / batch;
+  if (chunk < 1) chunk = 1;
+  for (int i = 0; i < prompt_len; i += chunk) {
+    const int n = prompt_len - i < chunk ? prompt_len - i : chunk;
+    if ((rc = step(m, m->ids + (size_t)i * batch, i + n == prompt_len, n))) return rc;
+  }
   return KX_OK;
 }
 
@@ -586,6 +609,13 @@ extern "C" int kx_generate(kx_model *m, const uint32_t *h_prompt, int32_t batch,
   return KX_OK;
 }
 
+extern "C" int kx_model_set_prefill_chunk(kx_model *m, int32_t positions) {
+  KX_REQUIRE(m, "kx_model_set_prefill_chunk: null model");
+  KX_REQUIRE(positions >= 1 && positions <= STEP_TOKENS, "kx_model_set_prefill_chunk: positions=%d outside [1, %d]", positions, STEP_TOKENS);
+  m->prefill_chunk = positions;
+  return KX_OK;
+}
+
 extern "C" int kx_model_set_fusion(kx_model *m, uint32_t mask) {
   KX_REQUIRE(m, "kx_model_set_fusion: null model");
   KX_REQUIRE(!(mask & ~(uint32_t)KX_FUSE_ALL), "kx_model_set_fusion: unknown bits in mask 0x%x", mask);
@@ -602,7 +632,7 @@ extern "C" int kx_model_timing(kx_model *m, float *ms2) {
 
 extern "C" int kx_model_hidden(kx_model *m, uint16_t *h_out) {
   KX_REQUIRE(m && h_out && m->batch > 0, "kx_model_hidden: null argument or no step has run");
-  KX_HIP(hipMemcpyAsync(h_out, m->x, (size_t)m->batch * m->c.hidden * 2, hipMemcpyDeviceToHost, m->st));
+  KX_HIP(hipMemcpyAsync(h_out, m->x + (size_t)m->x_row0 * m->c.hidden, (size_t)m->batch * m->c.hidden * 2, hipMemcpyDeviceToHost, m->st));
   KX_HIP(hipStreamSynchronize(m->st));
   return KX_OK;
 }

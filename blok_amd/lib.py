@@ -88,6 +88,7 @@ _SIGS = {
     "kx_model_latent": [_P, _I, _I, _I, _I, _P],
     "kx_model_timing": [_P, C.POINTER(C.c_float)],
     "kx_model_set_fusion": [_P, C.c_uint32],
+    "kx_model_set_prefill_chunk": [_P, _I],
     "kx_model_stream": [_P, _PP],
     "kx_moe_prefill_layer": [C.POINTER(KxConfig), C.POINTER(KxMoeWeights), _P, _P, _P, _I, C.c_uint32, _P],
     "kx_moe_decode_layer_timed": [C.POINTER(KxConfig), C.POINTER(KxMoeWeights), _P, _P, _P, _I,

@@ -302,6 +302,13 @@ int kx_model_timing(kx_model *model, float *ms2);
 #define KX_FUSE_MOE_TAIL 2u /* one token: shared down GEMV + combine + residual inside the routed down launch */
 #define KX_FUSE_ALL 3u
 int kx_model_set_fusion(kx_model *model, uint32_t mask);
+/* Prompt positions per prefill step.  1 (default) is the reference's prefill, one run() per prompt token (:886),
+ * and the bit-reproducible path.  With n > 1, kx_prefill and kx_generate take up to n consecutive positions of
+ * every sequence in one step (at most 32 tokens a step, so min(n, 32 / batch) positions): the projections, the
+ * shared expert and the attention then run on the matrix cores as they do for a batch of that many sequences
+ * (same values, another summation order: logits within the stack-level tolerance of the token-by-token prefill),
+ * each position attends to the cache rows up to its own, and only the last position is sampled. 1 <= n <= 32. */
+int kx_model_set_prefill_chunk(kx_model *model, int32_t positions);
 /* bf(mean + sigma*z) fill used for the norm weights */
 int kx_fill_affine_bf16(void *d_out, uint64_t n, uint64_t seed, uint64_t tensor_id, float mean,
                         float sigma, void *stream);

@@ -393,6 +393,55 @@ def test_kimi_shape_batched_stack_attention_paths(kxlib, ox):
     assert err < 3e-2 and agree >= 0.75
 
 
+@pytest.mark.parametrize("shape,batch,prompt_len,chunk", [
+    ("small", 1, 21, 8), ("small", 3, 23, 32), ("small", 1, 3, 2), ("kimi", 1, 150, 32), ("kimi", 4, 40, 8)])
+def test_chunked_prefill_against_token_by_token(kxlib, ox, shape, batch, prompt_len, chunk):
+    # several prompt positions per prefill step: the step runs as a batch of positions x sequences tokens (matrix-core
+    # projections from 5 tokens on, so another summation order).  Held against the token-by-token prefill of the same
+    # model (the reference's loop, the path the token-identity checks pin to the oracle): every cache row within
+    # 1e-2, logits of the first sampled step within the stack-level 3e-2, the same first id for at least three
+    # quarters of the sequences; the decode steps that follow run from the chunk-filled cache.  Chunks that leave at
+    # most 4 tokens a step take the same GEMV kernels as the token-by-token path and must match it to the bit.
+    say(f"chunked prefill shape={shape} batch={batch} prompt={prompt_len} chunk={chunk}")
+    if shape == "small":
+        cfg = O.small_config(batch=batch, context=prompt_len + 8)
+    else:
+        cfg = default_config()
+        cfg.n_layers, cfg.first_dense, cfg.max_batch, cfg.max_context, cfg.seed = 2, 1, batch, prompt_len + 8, 7
+    prompt = O.tokens_u32(batch * prompt_len, cfg.seed, 4, cfg.vocab).reshape(batch, prompt_len)
+    got = {}
+    for c in (1, chunk):
+        km = KxModel(kxlib, cfg)
+        check(kxlib.kx_model_set_prefill_chunk(km.h, c))
+        rc, out, _ = km.generate(prompt, 4)
+        assert rc == 0, kxlib.kx_last_error()
+        rc, out1, _ = km.generate(prompt, 1)
+        assert rc == 0, kxlib.kx_last_error()
+        rows = np.stack([km.latent(cfg.n_layers - 1, b, prompt_len) for b in range(batch)])
+        got[c] = (out.copy(), km.logits(batch), rows)
+        km.close()
+    (ids1, log1, rows1), (idsc, logc, rowsc) = got[1], got[chunk]
+    tokens_per_step = min(chunk, 32 // batch) * batch
+    if tokens_per_step <= 4:
+        assert (rows1 == rowsc).all() and (log1.view(np.uint32) == logc.view(np.uint32)).all() and (ids1 == idsc).all()
+        return
+    e_rows = O.max_rel(O.bf16_to_f32(rowsc), O.bf16_to_f32(rows1))
+    e_log = O.max_rel(logc, log1)
+    agree = float(np.mean(ids1[:, 0] == idsc[:, 0]))
+    print(f"chunked prefill: cache rows max-rel {e_rows:.3e}, logits max-rel {e_log:.3e}, first ids equal for {agree:.0%}", flush=True)
+    assert e_rows < 1e-2 and e_log < 3e-2 and agree >= 0.75
+
+
+def test_prefill_chunk_errors(kxlib):
+    cfg = O.small_config(batch=1, context=16)
+    km = KxModel(kxlib, cfg)
+    assert kxlib.kx_model_set_prefill_chunk(km.h, 0) != 0
+    assert kxlib.kx_model_set_prefill_chunk(km.h, 33) != 0
+    assert kxlib.kx_model_set_prefill_chunk(None, 4) != 0
+    assert kxlib.kx_model_set_prefill_chunk(km.h, 32) == 0
+    km.close()
+
+
 def test_executor_json_line(kxlib):
     import json
     import os
