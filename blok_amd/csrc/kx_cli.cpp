@@ -32,18 +32,19 @@ static uint64_t u64(const char *s, const char *what) {  // :504-510
 
 int main(int argc, char **argv) {
   std::string prompt_tokens, index;
-  uint64_t tokens = 0, layers = 0, seed = 0, topk = 0;
+  uint64_t tokens = 0, layers = 0, seed = 0, topk = 0, prefill_chunk = 1;
   int ignore_eos = 0;
   for (int i = 1; i < argc; i += 2) {
     std::string f = argv[i];
     if (f == "--ignore-eos") { ignore_eos = 1; --i; continue; }
-    if (i + 1 >= argc) die("usage: kx-kimi-exec [--index runtime-index.blok] --prompt-tokens ids --tokens n [--layers n] [--seed n] [--topk n] [--ignore-eos]");
+    if (i + 1 >= argc) die("usage: kx-kimi-exec [--index runtime-index.blok] --prompt-tokens ids --tokens n [--layers n] [--seed n] [--topk n] [--prefill-chunk n] [--ignore-eos]");
     if (f == "--index") index = argv[i + 1];
     else if (f == "--prompt-tokens") prompt_tokens = argv[i + 1];
     else if (f == "--tokens") tokens = u64(argv[i + 1], "tokens");
     else if (f == "--layers") layers = u64(argv[i + 1], "layers");
     else if (f == "--seed") seed = u64(argv[i + 1], "seed");
     else if (f == "--topk") topk = u64(argv[i + 1], "topk");
+    else if (f == "--prefill-chunk") prefill_chunk = u64(argv[i + 1], "prefill chunk");  // not in the reference: prompt positions per prefill step
     else die("unknown flag: " + f);  // :540
   }
   if (prompt_tokens.empty() || tokens == 0) die("bad args");  // :542
@@ -74,6 +75,11 @@ int main(int argc, char **argv) {
   cfg.max_context = (int32_t)(ids.size() + tokens);
   kx_model *m = nullptr;
   if (index.empty() ? kx_model_create(&cfg, &m) : kx_model_load(&cfg, index.c_str(), &m)) die(kx_last_error());
+  if (prefill_chunk != 1 && kx_model_set_prefill_chunk(m, prefill_chunk > 1000 ? 1000 : (int32_t)prefill_chunk)) {
+    std::string msg = kx_last_error();
+    kx_model_destroy(m);
+    die(msg);
+  }
   std::vector<uint32_t> out(tokens);
   int32_t count = 0;
   if (kx_generate(m, ids.data(), 1, (int32_t)ids.size(), (int32_t)tokens, ignore_eos, out.data(), &count)) {
