@@ -10,6 +10,9 @@
 #include "kx_math.h"
 #include "kx_wave.h"
 
+// seqs (stand-alone q absorb kernel only): 0: token t is sequence t at position pos.  n > 0 (a prefill step of several
+// positions of n sequences): token t = i * n + b is position pos + i of sequence b; rope_row then points at the row of
+// position pos, the rows of the following positions behind it.
 struct QAbsArgs {
   const uint16_t *q, *kvb, *rope_row;
   float *qabs;
@@ -20,6 +23,7 @@ struct QAbsArgs {
   float eps;
   int *head_count;  // gemv_absorb_k only: one counter per head, zero before the launch and left at zero
   int head_chunks;  // gemv_absorb_k only: workgroups per head
+  int seqs;         // q_absorb_k only, see above
 };
 
 namespace kxa {

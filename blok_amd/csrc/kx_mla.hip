@@ -127,8 +127,9 @@ __global__ void __launch_bounds__(128) q_absorb_k(QAbsArgs a, int tokens) {
   if ((int)blockIdx.x == a.heads * cq_n) {
     if (a.cache)
       for (int t = t0; t < min(t0 + TB, tokens); ++t) {
-        kv_finish_block(a.kva + (size_t)t * a.kva_stride, a.w_kv_ln, a.rope_row, a.cache + (size_t)t * a.seq_stride + (size_t)a.pos * kva,
-                        kv_rank, rope, a.eps, ws);
+        const int sb = a.seqs ? t % a.seqs : t, i = a.seqs ? t / a.seqs : 0;
+        kv_finish_block(a.kva + (size_t)t * a.kva_stride, a.w_kv_ln, a.rope_row + (size_t)i * rope,
+                        a.cache + (size_t)sb * a.seq_stride + (size_t)(a.pos + i) * kva, kv_rank, rope, a.eps, ws);
         __syncthreads();  // ws is reused by the next token
       }
     return;
@@ -175,9 +176,10 @@ __global__ void __launch_bounds__(128) q_absorb_k(QAbsArgs a, int tokens) {
     }
     if (cq == 0 && (int)threadIdx.x < half) {
       const int p = threadIdx.x;
+      const uint16_t *rr = a.rope_row + (size_t)(a.seqs ? (t0 + i) / a.seqs : 0) * rope;
       float lo, hi;
-      rope_pair(kx_bf16_f32(qh[i][nope + 2 * p]), kx_bf16_f32(qh[i][nope + 2 * p + 1]), kx_bf16_f32(a.rope_row[p]),
-                kx_bf16_f32(a.rope_row[half + p]), lo, hi);
+      rope_pair(kx_bf16_f32(qh[i][nope + 2 * p]), kx_bf16_f32(qh[i][nope + 2 * p + 1]), kx_bf16_f32(rr[p]),
+                kx_bf16_f32(rr[half + p]), lo, hi);
       out[kv_rank + p] = lo;
       out[kv_rank + half + p] = hi;
     }
@@ -189,6 +191,9 @@ struct MlaArgs {
   const float *qabs;      // f32 [B][heads][kva]
   float *pm, *pz, *po;    // partials [B][spans][heads], same, [B][spans][heads][kv_rank]
   int heads, seq, span_tiles, spans;
+  int seqs;               // 0: grid index z is sequence z, which attends `seq` positions.  n > 0 (a prefill step of
+                          // several positions of n sequences): z = i * n + b is position i of sequence b; it reads
+                          // cache block b and attends seq - (grid z / n - 1) + i positions, the last position all `seq`
   size_t seq_stride;      // elements between sequences in the cache
   float rs, mscale;
 };
@@ -208,9 +213,10 @@ __global__ void __launch_bounds__(256) mla_partial_k(MlaArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: q is then read through the scalar path
   const int span = blockIdx.x, b = blockIdx.z;
   const int h0 = (blockIdx.y * 4 + wave) * HG;
-  const uint16_t *cache = a.cache + (size_t)b * a.seq_stride;
+  const int seq = a.seqs ? a.seq - (int)(gridDim.z / a.seqs) + 1 + b / a.seqs : a.seq;
+  const uint16_t *cache = a.cache + (size_t)(a.seqs ? b % a.seqs : b) * a.seq_stride;
   const float *q = a.qabs + ((size_t)b * a.heads + h0) * KVA;
-  const int tiles = (a.seq + 63) >> 6;
+  const int tiles = (seq + 63) >> 6;  // a span past them leaves M = -inf, Z = 0, O = 0, which the merge weighs with 0
   const int tile_end = min(tiles, (span + 1) * a.span_tiles);
   float M[HG], Z[HG], O[HG][8];
 #pragma unroll
@@ -221,7 +227,7 @@ __global__ void __launch_bounds__(256) mla_partial_k(MlaArgs a) {
     for (int e = 0; e < 8; ++e) O[h][e] = 0.0f;
   }
   for (int tile = span * a.span_tiles; tile < tile_end; ++tile) {
-    const int t0 = tile << 6, n = min(64, a.seq - t0);
+    const int t0 = tile << 6, n = min(64, seq - t0);
     // stage rows t0 .. t0+n-1: 72 pieces of 16 bytes per row, 18 per thread
     {
       const uint4 *src = (const uint4 *)(cache + (size_t)t0 * KVA);
@@ -382,8 +388,15 @@ __global__ void __launch_bounds__(512, 1) mla_partial_mfma_k(MlaArgs a) {
   const int hb = wave & 1, cq = wave >> 1;
   const int l32 = lane & 31, half = lane >> 5;
   const int head2 = hb * 32 + l32;
-  const uint16_t *cache = a.cache + (size_t)b * a.seq_stride;
-  const int pos0 = span * a.span_tiles * 64, pos_end = min(a.seq, (span + 1) * a.span_tiles * 64);
+  const int seq = a.seqs ? a.seq - (int)(gridDim.z / a.seqs) + 1 + b / a.seqs : a.seq;
+  const uint16_t *cache = a.cache + (size_t)(a.seqs ? b % a.seqs : b) * a.seq_stride;
+  const int pos0 = span * a.span_tiles * 64, pos_end = min(seq, (span + 1) * a.span_tiles * 64);
+  if (pos0 >= seq) {  // a span past this position's rows (prefill steps only): partials the merge weighs with 0
+    const size_t base = ((size_t)b * a.spans + span) * a.heads;
+    if (threadIdx.x < (unsigned)a.heads) { a.pm[base + threadIdx.x] = -__builtin_inff(); a.pz[base + threadIdx.x] = 0.0f; }
+    for (int i = threadIdx.x; i < a.heads * 512; i += 512) a.po[base * 512 + i] = 0.0f;
+    return;
+  }
   const int n_tiles = (pos_end - pos0 + MM_T - 1) / MM_T;
   const float scale = a.rs * a.mscale * a.mscale;
   constexpr float LOG2E = 1.44269504088896341f;
@@ -413,7 +426,7 @@ __global__ void __launch_bounds__(512, 1) mla_partial_mfma_k(MlaArgs a) {
         const int slot = ii * 64 + lane;
         const int p = slot / 72, js = slot - p * 72;
         const int j = (js & ~7) | ((js ^ (p >> 1)) & 7);
-        const int row = min(pos0 + t * MM_T + p, a.seq - 1);
+        const int row = min(pos0 + t * MM_T + p, seq - 1);
         mm_copy16_to_lds(cache + (size_t)row * MLA_KVA + j * 8, lds0 + (t % MM_RING) * MM_NAT + ii * 1024);
       }
     }
@@ -691,12 +704,13 @@ __global__ void __launch_bounds__(64) mla_combine_cols_k(const float *__restrict
 
 int kx_q_absorb_launch(const uint16_t *q, const uint16_t *kvb, const uint16_t *rope_row, float *qabs, int tokens,
                        int heads, int nope, int rope, int v_head, int kv_rank, const uint16_t *kva, int kva_stride,
-                       const uint16_t *w_kv_ln, uint16_t *cache, size_t seq_stride, int pos, float eps, hipStream_t st) {
+                       const uint16_t *w_kv_ln, uint16_t *cache, size_t seq_stride, int pos, float eps, hipStream_t st, int seqs) {
   KX_REQUIRE(kv_rank % 8 == 0 && kv_rank <= 1024 && rope % 2 == 0 && rope / 2 <= 128, "kx_q_absorb: kv_rank=%d (multiple of 8, at most 1024), rope=%d (even, at most 256)", kv_rank, rope);
   QAbsArgs a = {};
   a.q = q; a.kvb = kvb; a.rope_row = rope_row; a.qabs = qabs; a.kva = kva; a.w_kv_ln = w_kv_ln; a.cache = cache;
   a.seq_stride = seq_stride; a.heads = heads; a.nope = nope; a.rope = rope; a.v_head = v_head; a.kv_rank = kv_rank;
-  a.kva_stride = kva_stride; a.pos = pos; a.eps = eps;
+  a.kva_stride = kva_stride; a.pos = pos; a.eps = eps; a.seqs = seqs;
+  KX_REQUIRE(seqs == 0 || (seqs > 0 && tokens % seqs == 0), "kx_q_absorb: %d tokens do not split into %d sequences", tokens, seqs);
   const dim3 g1(heads * ((kv_rank + 127) / 128) + (cache ? 1 : 0), tokens);
   if (tokens >= 8) hipLaunchKernelGGL(q_absorb_k<4>, dim3(g1.x, (tokens + 3) / 4), dim3(128), 0, st, a, tokens);
   else hipLaunchKernelGGL(q_absorb_k<1>, g1, dim3(128), 0, st, a, tokens);
@@ -718,17 +732,18 @@ size_t kx_mla_partial_floats(int batch, int heads, int kv_rank, int max_seq) {
 }
 
 int kx_mla_partials_launch(const kx_config *c, const uint16_t *cache, size_t seq_stride, const float *qabs, float *partial,
-                           int batch, int seq, KxMlaPartials *out, hipStream_t st) {
+                           int batch, int seq, KxMlaPartials *out, hipStream_t st, int seqs) {
   KX_REQUIRE(c->kv_rank == 512 && c->qk_rope == 64, "kx_mla: the attention kernel is built for kv_rank 512, qk_rope 64 (got %d, %d)",
              c->kv_rank, c->qk_rope);
   KX_REQUIRE(c->heads % 4 == 0, "kx_mla: heads=%d must be a multiple of 4", c->heads);
   KX_REQUIRE(batch > 0 && seq > 0, "kx_mla: batch=%d seq=%d must be positive", batch, seq);
+  KX_REQUIRE(seqs == 0 || (seqs > 0 && batch % seqs == 0 && seq >= batch / seqs), "kx_mla: %d positions x sequences do not split into %d sequences of at least %d positions", batch, seqs, seq);
   // automatic choice, where the matrix-core kernel is built for the shape (64 heads): from 2048 positions on, and from
   // 128 positions on for 5 sequences and more (batches the stack runs on the matrix cores anyway; the VALU kernel
   // takes 190-360 us per layer at 32 sequences of 1100 positions)
   const bool use_mfma = g_mla_kernel == 2 || (g_mla_kernel == 0 && c->heads == 64 && (seq >= 2048 || (batch >= 5 && seq >= 128)));
   MlaArgs a;
-  a.cache = cache; a.qabs = qabs; a.heads = c->heads; a.seq = seq; a.seq_stride = seq_stride;
+  a.cache = cache; a.qabs = qabs; a.heads = c->heads; a.seq = seq; a.seq_stride = seq_stride; a.seqs = seqs;
   a.span_tiles = use_mfma ? mfma_span_tiles(seq, batch) : kx_mla_span_tiles(seq);
   const int tiles = (seq + 63) / 64;
   a.spans = (tiles + a.span_tiles - 1) / a.span_tiles;
@@ -782,9 +797,9 @@ int kx_mla_combine_launch(const KxMlaPartials &p, uint16_t *o_lat, int batch, in
 }
 
 int kx_mla_attend_launch(const kx_config *c, const uint16_t *cache, size_t seq_stride, const float *qabs, float *partial,
-                         uint16_t *o_lat, int batch, int seq, hipStream_t st) {
+                         uint16_t *o_lat, int batch, int seq, hipStream_t st, int seqs) {
   KxMlaPartials p;
-  int rc = kx_mla_partials_launch(c, cache, seq_stride, qabs, partial, batch, seq, &p, st);
+  int rc = kx_mla_partials_launch(c, cache, seq_stride, qabs, partial, batch, seq, &p, st, seqs);
   if (rc) return rc;
   return kx_mla_combine_launch(p, o_lat, batch, c->heads, st);
 }

