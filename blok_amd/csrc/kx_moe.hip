@@ -78,6 +78,10 @@ extern "C" int kx_moe_workspace_create(const kx_config *cfg, int32_t max_tokens,
     }
   }
   ws->route_counter = ws->n_active + 1;
+  // work records nobody has written yet say "no expert" (-1): kx_moe_routed_only before any layer call, or with more
+  // tokens than the last one had, then does nothing instead of following uninitialised records
+  KX_HIP(hipMemset(ws->work, 0xff, E * 16));
+  KX_HIP(hipMemset(ws->pair_work, 0xff, T * K * 16));
   KX_HIP(hipMemset(ws->n_active, 0, 8));
   KX_HIP(hipMemset(ws->tail_count, 0, KX_TAIL_BLOCKS * 4));
   for (auto &e : ws->ev) KX_HIP(hipEventCreate(&e));
