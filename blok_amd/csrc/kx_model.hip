@@ -85,7 +85,7 @@ struct kx_model {
 namespace {
 
 // tokens a step may carry: a decode step has one per sequence, a prefill step up to this many (positions x sequences)
-constexpr int STEP_TOKENS = 32;
+constexpr int STEP_TOKENS = 256;
 inline int step_tokens(const kx_config *c) { return c->max_batch > STEP_TOKENS ? c->max_batch : STEP_TOKENS; }
 
 struct Plan {  // byte offsets of everything in the arena
@@ -342,8 +342,12 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample, int C = 1) {
       KX_TRY(dense(KX_EPI_RESID, g));                                                                   // :684, :877
     } else {
       if (!fuse) KX_TRY(kx_rmsnorm_launch(m->x, L.post_ln, m->n, B, H, H, H, c.rms_eps, st));          // :829
-      KX_TRY(kx_moe_layer_launch(&c, &L.moe, m->moe_ws, m->n, m->x, B, ((m->fusion & KX_FUSE_MOE_TAIL) ? 0u : KX_MOE_SEPARATE_TAIL) | (mm ? KX_MOE_SHARED_MATRIX_CORES : 0u),
-                                 fuse ? L.post_ln : nullptr, st, false));  // :835-877
+      if (C > 1 && B > 32) {  // a prefill step of more than 32 tokens: the grouped GEMMs of the prefill layer
+        KX_TRY(kx_moe_prefill_layer(&c, &L.moe, m->moe_ws, m->n, m->x, B, 0, st));
+      } else {
+        const uint32_t flags = ((m->fusion & KX_FUSE_MOE_TAIL) ? 0u : KX_MOE_SEPARATE_TAIL) | (mm ? KX_MOE_SHARED_MATRIX_CORES : 0u);
+        KX_TRY(kx_moe_layer_launch(&c, &L.moe, m->moe_ws, m->n, m->x, B, flags, fuse ? L.post_ln : nullptr, st, false));  // :835-877
+      }
     }
   }
   const uint16_t *x_last = m->x + (size_t)(C - 1) * NB * H;  // rows of the last position
