@@ -282,6 +282,25 @@ int kx_gemv_launch(int epi, KxGemvArgs a, hipStream_t st) {
   const uint16_t *x0 = a.x;
   char *out0 = (char *)a.out;
   const size_t out_elem = (epi == KX_EPI_F32 || epi == KX_EPI_ARGMAX) ? 4 : 2;
+  // 8 tokens and more against a matrix that stays in L2: the token blocks side by side (gemv_tokblk_k), all in one launch
+  if (all_tokens >= 8 && all_tokens <= 4 * 65535 && (epi == KX_EPI_BF16 || epi == KX_EPI_F32) && !a.norm_w && !a.mla_po &&
+      kx_cdiv(a.rows, CR) <= 4096 && (size_t)a.rows * a.cols * 2 <= (16u << 20)) {
+    // longer chunks, about 512 workgroups in all: a chunk's activations are read once, so rows per chunk divide the
+    // L2 traffic of the activations (one row per chunk: 57 KB of them against 14 KB of weights for the router)
+    const int blocks = kx_cdiv(all_tokens, 4);
+    KxGemvArgs b = a;
+    int ri4;
+    const int CR4 = gemv_plan(epi, b, ri4, 4, 512 / blocks > 32 ? 512 / blocks : 32);
+    if (CR4 < 0) return KX_ERR_ARG;
+    const size_t lds4 = (size_t)CR4 * 4 * S * sizeof(float);
+    KX_REQUIRE(lds4 <= 64 * 1024, "kx_gemv: %zu bytes of LDS needed", lds4);
+    const dim3 g(kx_cdiv(a.rows, CR4), blocks), blk(b.nw * b.rs * 64);
+    if (ri4 == 4) hipLaunchKernelGGL(gemv_tokblk_k<4>, g, blk, lds4, st, b);
+    else if (ri4 == 2) hipLaunchKernelGGL(gemv_tokblk_k<2>, g, blk, lds4, st, b);
+    else hipLaunchKernelGGL(gemv_tokblk_k<1>, g, blk, lds4, st, b);
+    KX_LAUNCH_CHECK();
+    return KX_OK;
+  }
   for (int t0 = 0; t0 < all_tokens; t0 += 32) {
     a.tokens = all_tokens - t0 < 32 ? all_tokens - t0 : 32;
     a.x = x0 + (size_t)t0 * a.x_stride;
@@ -293,25 +312,6 @@ int kx_gemv_launch(int epi, KxGemvArgs a, hipStream_t st) {
     }
     const int tt = b.tokens >= 4 ? 4 : b.tokens >= 2 ? 2 : 1;
     const int chunks = kx_cdiv(a.rows, CR);
-    // 8 tokens and more against a matrix that stays in L2: the token blocks side by side (gemv_tokblk_k)
-    if (b.tokens >= 8 && (epi == KX_EPI_BF16 || epi == KX_EPI_F32) && !b.norm_w && !b.mla_po && chunks <= 4096 &&
-        (size_t)a.rows * a.cols * 2 <= (16u << 20)) {
-      // longer chunks, about 512 workgroups in all: a chunk's activations are read once, so rows per chunk divide the
-      // L2 traffic of the activations (one row per chunk: 57 KB of them against 14 KB of weights for the router)
-      const int blocks = kx_cdiv(b.tokens, 4);
-      int ri4;
-      const int CR4 = gemv_plan(epi, b, ri4, 4, 512 / blocks > 32 ? 512 / blocks : 32);
-      if (CR4 < 0) return KX_ERR_ARG;
-      ri = ri4;
-      const size_t lds4 = (size_t)CR4 * 4 * S * sizeof(float);
-      KX_REQUIRE(lds4 <= 64 * 1024, "kx_gemv: %zu bytes of LDS needed", lds4);
-      const dim3 g(kx_cdiv(a.rows, CR4), blocks), blk(b.nw * b.rs * 64);
-      if (ri == 4) hipLaunchKernelGGL(gemv_tokblk_k<4>, g, blk, lds4, st, b);
-      else if (ri == 2) hipLaunchKernelGGL(gemv_tokblk_k<2>, g, blk, lds4, st, b);
-      else hipLaunchKernelGGL(gemv_tokblk_k<1>, g, blk, lds4, st, b);
-      KX_LAUNCH_CHECK();
-      continue;
-    }
     const size_t lds = (size_t)mats * CR * b.tokens * S * sizeof(float);
     KX_REQUIRE(lds <= 160 * 1024, "kx_gemv: %zu bytes of LDS needed", lds);
     dim3 g(chunks < 4096 ? chunks : 4096), blk(a.nw * a.rs * 64);

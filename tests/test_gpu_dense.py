@@ -39,6 +39,7 @@ def test_rmsnorm_parity(kxlib, ox, n, tokens):
     (384, 7168, 32, 1),     # 8 tokens and more against a small matrix: token blocks side by side in the grid
     (1000, 1536, 13, 0),    # the same, ragged rows and a ragged last token block
     (2048, 512, 9, 0),
+    (384, 1024, 70, 1),     # more than 32 tokens: still one launch
 ])
 def test_gemv_bf16_parity(kxlib, ox, rows, cols, tokens, f32):
     say(f"gemv_bf16 rows={rows} cols={cols} tokens={tokens} f32={f32}")
