@@ -25,6 +25,7 @@
 //              over spans ascending; o_lat = bf(O / Z)
 //   q_lat      eight chains over d = j, j+8, ... then ((0+1)+(2+3))+((4+5)+(6+7))
 #include <math.h>
+#include <atomic>
 #include <type_traits>
 #include "kx_attn_parts.h"
 #include "kx_common.h"
@@ -758,7 +759,7 @@ int kx_mla_partials_launch(const kx_config *c, const uint16_t *cache, size_t seq
   while (hg < 8 && c->heads % (4 * hg * 2) == 0 && waves1 / (hg * 2) >= 4096) hg *= 2;
   dim3 g(a.spans, c->heads / (4 * hg), batch), b(256);
   const size_t lds = (size_t)64 * MLA_PITCH * 2 + (size_t)4 * hg * 64 * sizeof(float);
-  static bool attr_set = false;
+  static std::atomic<bool> attr_set{false};  // setting it twice from two threads is harmless
   if (!attr_set) {  // more than 64 KB of dynamic LDS has to be allowed per kernel
     KX_HIP(hipFuncSetAttribute((const void *)mla_partial_k<1>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
     KX_HIP(hipFuncSetAttribute((const void *)mla_partial_k<2>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
@@ -768,7 +769,7 @@ int kx_mla_partials_launch(const kx_config *c, const uint16_t *cache, size_t seq
   }
   if (use_mfma) {
     KX_REQUIRE(c->heads == 64, "kx_mla: the matrix-core kernel is built for 64 heads (got %d)", c->heads);
-    static bool mfma_attr = false;
+    static std::atomic<bool> mfma_attr{false};
     if (!mfma_attr) {
       KX_HIP(hipFuncSetAttribute((const void *)mla_partial_mfma_k, hipFuncAttributeMaxDynamicSharedMemorySize, MM_LDS));
       mfma_attr = true;

@@ -35,6 +35,7 @@
 //
 // MFMA's internal summation order is not documented, so this path is held to the
 // max-rel 1e-2 bar and is never used for the token-identity runs.
+#include <atomic>
 #include "kx_common.h"
 #include "kx_dense.h"
 #include "kx_math.h"
@@ -454,7 +455,7 @@ int kx_grouped_gemm_launch(bool dual, bool i4, const void *w0, const uint16_t *s
   dim3 g(kx_cdiv(N, waves * 32), work ? n_slots : 1, mz), b(waves * 64);
   const int mats = dual ? 2 : 1;
   const size_t lds = (size_t)2 * BM * LDS_STRIDE * 2 + (i4 ? (size_t)2 * mats * W_STAGE + (size_t)2 * BN * mats * SC_STRIDE : 0);
-  static bool attr_set = false;
+  static std::atomic<bool> attr_set{false};  // setting it twice from two threads is harmless
   if (!attr_set) {  // more than 64 KB of dynamic LDS has to be allowed per kernel
     KX_HIP(hipFuncSetAttribute((const void *)grouped_gemm_k<true, true, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     KX_HIP(hipFuncSetAttribute((const void *)grouped_gemm_k<false, true, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));

@@ -26,6 +26,7 @@
 //
 // Sums are fp32 over exact bf16 products in another order than the GEMV's: this path is held to the 1e-2 bar, like the
 // other matrix-core paths, and serves batches the token-identity checks do not run on.
+#include <atomic>
 #include "kx_common.h"
 #include "kx_dense.h"
 #include "kx_math.h"
@@ -166,7 +167,7 @@ int kx_skinny_gemm_launch(bool dual, const uint16_t *w0, const uint16_t *w1, con
   a.out_stride = out_stride; a.mode = out_mode;
   const dim3 g((unsigned)kx_cdiv(rows, 32));
   const size_t lds = (size_t)(dual ? 3 * 3 : 4 * 2) * 32 * 512;  // the ring: stages x tiles x 16 KB
-  static bool attr = false;
+  static std::atomic<bool> attr{false};  // setting it twice from two threads is harmless
   if (!attr) {
     KX_HIP(hipFuncSetAttribute((const void *)skinny_staged_k<false>, hipFuncAttributeMaxDynamicSharedMemorySize, 4 * 2 * 32 * 512));
     KX_HIP(hipFuncSetAttribute((const void *)skinny_staged_k<true>, hipFuncAttributeMaxDynamicSharedMemorySize, 3 * 3 * 32 * 512));
