@@ -307,7 +307,7 @@ def run_stack(args):
         "prefill_ms_per_token": round(ms_pre.value / P, 5),
         "workload": f"truncated Kimi-K2 stack (BASELINE config 5): {cfg.n_layers} layers (1 dense + {cfg.n_layers - 1} MoE), "
                     f"vocab {cfg.vocab}, batch {B}, {P}-token uniform-random prompt prefilled "
-                    + ("token by token" if args.prefill_chunk <= 1 else f"{min(args.prefill_chunk, max(1, 256 // B))} positions per step") + ", then "
+                    + ("token by token" if args.prefill_chunk <= 1 else f"{min(args.prefill_chunk, max(1, 2048 // B))} positions per step") + ", then "
                     f"{W} warm-up and {K} timed greedy decode steps; seeded random-init weights resident in HBM",
         "resident_gb": {"weights": round(wb.value / 1e9, 2), "kv_cache": round(cb.value / 1e9, 3), "scratch": round(sb.value / 1e9, 3)},
         "model_create_s": round(t_create, 2), "device": name.value.decode(), "compute_units": cus.value,

@@ -85,8 +85,11 @@ struct kx_model {
 namespace {
 
 // tokens a step may carry: a decode step has one per sequence, a prefill step up to this many (positions x sequences)
-constexpr int STEP_TOKENS = 256;
+constexpr int STEP_TOKENS = 2048;
 inline int step_tokens(const kx_config *c) { return c->max_batch > STEP_TOKENS ? c->max_batch : STEP_TOKENS; }
+// entries (position x sequence) one attention launch of a prefill step takes; the partials are laid out for these
+constexpr int ATT_ENTRIES = 256;
+inline int att_entries(const kx_config *c) { return c->max_batch > ATT_ENTRIES ? c->max_batch : ATT_ENTRIES; }
 
 struct Plan {  // byte offsets of everything in the arena
   size_t total = 0, weights = 0, cache = 0, scratch = 0;
@@ -174,7 +177,7 @@ int layout(const kx_config *c, Plan &p, kx_model *m) {
   auto *att = KX_AT(uint16_t *, BT * VD * 2);
   auto *dmid = KX_AT(uint16_t *, BT * inter * 2);
   auto *qabs = KX_AT(float *, BT * (size_t)c->heads * KVA * 4);
-  auto *partial = KX_AT(float *, kx_mla_partial_floats((int)BT, c->heads, c->kv_rank, c->max_context) * 4);
+  auto *partial = KX_AT(float *, kx_mla_partial_floats(att_entries(c), c->heads, c->kv_rank, c->max_context) * 4);
   auto *logits = KX_AT(float *, B * V * 4);
   auto *argmax_scratch = KX_AT(float *, KX_ARGMAX_SCRATCH_FLOATS(B) * 4);
   auto *ids = KX_AT(uint32_t *, (size_t)c->max_context * B * 4);
@@ -323,7 +326,13 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample, int C = 1) {
         KX_TRY(kx_mla_combine_launch(mp, m->o_lat, B, c.heads, st));
       }
     } else {
-      KX_TRY(kx_mla_attend_launch(&c, L.cache, seq_stride, m->qabs, m->partial, m->o_lat, B, pos + C, st, C > 1 ? NB : 0));
+      // at most ATT_ENTRIES entries a launch: whole positions, in order
+      const int cs = NB >= ATT_ENTRIES ? 1 : ATT_ENTRIES / NB;
+      for (int i0 = 0; i0 < C; i0 += cs) {
+        const int np = C - i0 < cs ? C - i0 : cs;
+        KX_TRY(kx_mla_attend_launch(&c, L.cache, seq_stride, m->qabs + (size_t)i0 * NB * c.heads * KVA, m->partial,
+                                    m->o_lat + (size_t)i0 * NB * c.heads * c.kv_rank, np * NB, pos + i0 + np, st, C > 1 ? NB : 0));
+      }
     }
     KX_TRY(kx_gemv_launch(KX_EPI_BF16, g, st));
     g = {};

