@@ -91,7 +91,10 @@ int kx_mla_span_tiles(int seq) {
 
 // The matrix-core kernel is not tied to that partition (it is held to a tolerance, not to the oracle's sums): few
 // sequences get more, shorter spans so that sequences x spans fills the chip -- up to 256 spans, merged 64 at a time.
+// Beyond 32 entries (the launches of a prefill step) the entries alone fill the chip and every span costs a row of
+// partials that is written and read back: down to 4 spans.
 static int mfma_span_cap(int batch) {
+  if (batch > 32) return 2048 / batch < 4 ? 4 : 2048 / batch;
   const int want = 1024 / (batch > 0 ? batch : 1);
   return want > 256 ? 256 : want < 64 ? 64 : want;
 }
