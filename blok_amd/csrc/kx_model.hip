@@ -51,6 +51,15 @@ __global__ void embed_k(const uint16_t *__restrict__ embed, const uint32_t *__re
   uint4 *dst = (uint4 *)(x + (size_t)blockIdx.x * hidden);
   for (int i = threadIdx.x; i < hidden / 8; i += blockDim.x) dst[i] = src[i];
 }
+// the per-head W_UV products of a long prefill step as one grouped GEMM: group h = the rows t * heads + h of the
+// [tokens * heads, kv_rank] view of the attention output, in token order
+__global__ void head_groups_k(int tokens, int heads, int4 *__restrict__ work, int *__restrict__ pairs) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= tokens * heads) return;
+  const int h = idx / tokens, t = idx - h * tokens;
+  pairs[idx] = t * heads + h;
+  if (t == 0) work[h] = make_int4(h, h * tokens, (h + 1) * tokens, h);
+}
 __global__ void copy_ids_k(const uint32_t *__restrict__ src, uint32_t *__restrict__ dst, int n) {
   int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) dst[i] = src[i];
@@ -69,6 +78,8 @@ struct kx_model {
   float *qabs, *partial, *logits, *argmax_scratch;
   uint32_t *ids, *next, *history;  // [max_context][B], [B], [max_context][B]
   int *head_count;                 // [heads] arrival counters of the q_b GEMV that finishes the query; zero between launches
+  int4 *head_work;                 // [heads], [step tokens * heads]: the groups of head_groups_k
+  int *head_pairs;
   uint32_t fusion = KX_FUSE_ALL;
   kx_moe_workspace *moe_ws = nullptr;
   hipStream_t st = nullptr;
@@ -184,12 +195,14 @@ int layout(const kx_config *c, Plan &p, kx_model *m) {
   auto *next = KX_AT(uint32_t *, B * 4);
   auto *history = KX_AT(uint32_t *, (size_t)c->max_context * B * 4);
   auto *head_count = KX_AT(int *, (size_t)c->heads * 4);
+  auto *head_work = KX_AT(int4 *, (size_t)c->heads * 16);
+  auto *head_pairs = KX_AT(int *, BT * c->heads * 4);
 #undef KX_AT
   p.scratch = p.total - p.weights - p.cache;
   if (m) {
     m->x = x; m->n = n; m->qkv = qkv; m->qa = qa; m->q = q; m->o_lat = o_lat; m->att = att; m->dmid = dmid;
     m->qabs = qabs; m->partial = partial; m->logits = logits; m->argmax_scratch = argmax_scratch; m->ids = ids; m->next = next; m->history = history;
-    m->head_count = head_count;
+    m->head_count = head_count; m->head_work = head_work; m->head_pairs = head_pairs;
   }
   return KX_OK;
 }
@@ -334,7 +347,17 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample, int C = 1) {
                                     m->o_lat + (size_t)i0 * NB * c.heads * c.kv_rank, np * NB, pos + i0 + np, st, C > 1 ? NB : 0));
       }
     }
-    KX_TRY(kx_gemv_launch(KX_EPI_BF16, g, st));
+    if (C > 1 && B > 32 && c.kv_rank % 128 == 0) {  // a long prefill step: one grouped GEMM over the heads
+      if (l == 0) {
+        hipLaunchKernelGGL(head_groups_k, dim3(kx_cdiv(B * c.heads, 256)), dim3(256), 0, st, B, c.heads, m->head_work, m->head_pairs);
+        KX_LAUNCH_CHECK();
+      }
+      KX_TRY(kx_grouped_gemm_launch(false, false, L.kvb + (size_t)c.qk_nope * c.kv_rank, nullptr, nullptr, nullptr, m->o_lat, m->att,
+                                    KX_GG_BF16, m->head_work, m->head_pairs, 0, c.heads, c.v_head, c.kv_rank, 1,
+                                    (size_t)(c.qk_nope + c.v_head) * c.kv_rank, 0, B, st));
+    } else {
+      KX_TRY(kx_gemv_launch(KX_EPI_BF16, g, st));
+    }
     g = {};
     g.w0 = L.o; g.x = m->att; g.x_stride = VD; g.out = m->x; g.out_stride = H; g.rows = H; g.cols = VD; g.tokens = B;
     KX_TRY(dense(KX_EPI_RESID, g));                                                                     // :826-827
