@@ -101,10 +101,11 @@ def test_small_stack_tokens_identical(kxlib, ox, batch, prompt_len, n_tokens):
         m.close()
 
 
-@pytest.mark.parametrize("batch", [16, 8, 5])
+@pytest.mark.parametrize("batch", [16, 8, 5, 40])
 def test_small_stack_matrix_core_projections(kxlib, ox, batch):
     # from 5 sequences on the dense projections and the shared expert run as MFMA GEMMs (another summation order): the logits of the first
-    # sampled step are held to the stack-level 3e-2 against both oracle schedules, not to the bits
+    # sampled step are held to the stack-level 3e-2 against both oracle schedules, not to the bits (batch 40: beyond
+    # one 32-token tile the projections take the prefill GEMM kernel)
     say(f"small stack batch={batch} (dense projections on the matrix cores)")
     prompt_len = 5
     cfg = O.small_config(batch=batch, context=32)
