@@ -296,6 +296,7 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample, int C = 1) {
                                       g.cols, &done, st);
       if (rc2 || done) return rc2;
     }
+    KX_REQUIRE(g.x_stride == g.cols && g.out_stride == g.rows, "kx_model: the GEMM kernel takes dense activation and output rows");
     return kx_grouped_gemm_launch(dual, false, g.w0, nullptr, dual ? g.w1 : nullptr, nullptr, g.x, g.out, mode, nullptr, nullptr,
                                   g.tokens, 1, g.rows, g.cols, 1, 0, 0, g.tokens, st);
   };
