@@ -716,7 +716,8 @@ int kx_q_absorb_launch(const uint16_t *q, const uint16_t *kvb, const uint16_t *r
   a.kva_stride = kva_stride; a.pos = pos; a.eps = eps; a.seqs = seqs;
   KX_REQUIRE(seqs == 0 || (seqs > 0 && tokens % seqs == 0), "kx_q_absorb: %d tokens do not split into %d sequences", tokens, seqs);
   const dim3 g1(heads * ((kv_rank + 127) / 128) + (cache ? 1 : 0), tokens);
-  if (tokens >= 8) hipLaunchKernelGGL(q_absorb_k<4>, dim3(g1.x, (tokens + 3) / 4), dim3(128), 0, st, a, tokens);
+  if (tokens >= 64) hipLaunchKernelGGL(q_absorb_k<8>, dim3(g1.x, (tokens + 7) / 8), dim3(128), 0, st, a, tokens);
+  else if (tokens >= 8) hipLaunchKernelGGL(q_absorb_k<4>, dim3(g1.x, (tokens + 3) / 4), dim3(128), 0, st, a, tokens);
   else hipLaunchKernelGGL(q_absorb_k<1>, g1, dim3(128), 0, st, a, tokens);
   KX_LAUNCH_CHECK();
   return KX_OK;

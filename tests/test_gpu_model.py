@@ -255,7 +255,7 @@ def test_fused_and_separate_launches_agree(kxlib, ox, shape):
         assert (h1 == h0).all() and (l1 == l0).all() and (o1 == o0).all()
 
 
-@pytest.mark.parametrize("tokens", [1, 3, 9, 32])
+@pytest.mark.parametrize("tokens", [1, 3, 9, 32, 70])
 def test_q_absorb_operator(kxlib, ox, tokens):
     # bf(W_UK^T q_nope): eight fp32 chains over d = j, j+8, ... summed ((0+1)+(2+3))+((4+5)+(6+7)) (bf16 products are
     # exact in fp32, so numpy's add of the product is the fma).  From 8 tokens on a workgroup takes four tokens: every
