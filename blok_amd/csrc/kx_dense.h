@@ -82,7 +82,7 @@ int kx_i4_launch(bool dual, const uint32_t *packed0, const uint16_t *scale0, con
                  const uint16_t *scale1, const uint16_t *x, uint16_t *out, const int4 *work,
                  const int *pairs, int n_pairs, int rows,
                  int cols, int x_div, size_t expert_words, size_t expert_scales, int tt, int n_slots,
-                 int cnt_lo, int cnt_hi, hipStream_t st);
+                 int cnt_lo, int cnt_hi, hipStream_t st, int chunk_mult = 1);
 
 // kx_router.hip
 int kx_router_topk_launch(const float *logits, const float *bias, uint16_t *ids, float *weights, int tokens,

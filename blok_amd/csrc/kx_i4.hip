@@ -221,7 +221,7 @@ __device__ __forceinline__ void moe_tail_arrive(const KxMoeTail &t, int blk_a, i
 // FILTER: the launch processes only the experts whose pair count lies in [cnt_lo, cnt_hi]
 // `idle` is called once, where the last chunk's loads have landed and nothing more will be requested: what it
 // requests arrives during the epilogue.
-template <bool DUAL, int TT, int KS_T, bool FILTER, class Idle>
+template <bool DUAL, int TT, int KS_T, bool FILTER, int CM = 1, class Idle>
 __device__ __forceinline__ void i4_body(const I4Args &a, const int bid, const int nblocks, float *lds, Idle &&idle) {
   constexpr int MATS = DUAL ? 2 : 1;
   constexpr int RI = I4_RI;
@@ -230,7 +230,7 @@ __device__ __forceinline__ void i4_body(const I4Args &a, const int bid, const in
   const int ks = KS_T ? KS_T : a.ks;
   const int rs = KS_T ? (KS_T >= 5 ? 1 : 8 / KS_T) : a.rs;
   const int RT = rs * 2 * RI;
-  const int nt = KS_T ? i4_chunk_rows(DUAL, KS_T >= 5 ? 4 : 32 / KS_T) / (KS_T >= 5 ? 4 : 32 / KS_T) : a.nt;
+  const int nt = KS_T ? CM * (i4_chunk_rows(DUAL, KS_T >= 5 ? 4 : 32 / KS_T) / (KS_T >= 5 ? 4 : 32 / KS_T)) : a.nt;  // CM: chunks of CM times the rows
   const int CR = RT * nt;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int l = lane & 31, h = lane >> 5;
@@ -416,10 +416,10 @@ __device__ __forceinline__ void i4_body(const I4Args &a, const int bid, const in
   }
 }
 
-template <bool DUAL, int TT, int KS_T, int MAXT, int WPE, bool FILTER>
+template <bool DUAL, int TT, int KS_T, int MAXT, int WPE, bool FILTER, int CM = 1>
 __global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) i4_gemv_k(I4Args a) {
   extern __shared__ float lds[];
-  i4_body<DUAL, TT, KS_T, FILTER>(a, blockIdx.x, gridDim.x, lds, [] {});
+  i4_body<DUAL, TT, KS_T, FILTER, CM>(a, blockIdx.x, gridDim.x, lds, [] {});
 }
 
 // The routed down GEMV of one token and the shared expert's down GEMV ([rows, 2048] bf16) in one launch.  Workgroup b
@@ -504,7 +504,7 @@ struct I4Launch {
   size_t lds;
 };
 
-int plan(int cols, int rows, int mats, int tt, I4Launch &pl) {
+int plan(int cols, int rows, int mats, int tt, I4Launch &pl, int chunk_mult = 1) {
   KX_REQUIRE(cols > 0 && cols % 1024 == 0, "kx_i4: cols=%d must be a positive multiple of 1024", cols);
   KX_REQUIRE(rows >= 4, "kx_i4: rows=%d must be at least 4", rows);
   pl.ks = cols / 1024;
@@ -516,6 +516,7 @@ int plan(int cols, int rows, int mats, int tt, I4Launch &pl) {
   // chunk: 32 rows of both matrices (gate/up) or 64 rows of one
   int nt = i4_chunk_rows(mats == 2, rt) / rt;
   nt = nt < 1 ? 1 : nt;
+  if (chunk_mult > 1 && rows % (rt * nt * chunk_mult) == 0) nt *= chunk_mult;
   while (nt > 1 && rt * nt > rows) --nt;
   pl.nt = nt;
   pl.cr = rt * nt;
@@ -547,9 +548,13 @@ void launch_tt(const I4Args &a, int tt, dim3 g, dim3 b, size_t lds, hipStream_t 
 int kx_i4_launch(bool dual, const uint32_t *packed0, const uint16_t *scale0, const uint32_t *packed1,
                  const uint16_t *scale1, const uint16_t *x, uint16_t *out, const int4 *work,
                  const int *pairs, int n_pairs, int rows, int cols, int x_div, size_t expert_words,
-                 size_t expert_scales, int tt, int n_slots, int cnt_lo, int cnt_hi, hipStream_t st) {
+                 size_t expert_scales, int tt, int n_slots, int cnt_lo, int cnt_hi, hipStream_t st, int chunk_mult) {
   I4Launch pl;
-  int rc = plan(cols, rows, dual ? 2 : 1, tt, pl);
+  // chunks of twice the rows: for the one-matrix kernel over many work records, where a 112-row chunk (114 KB at
+  // K = 2048) is over before the workgroup's start-up is paid for (routed down at 32 tokens: 0.367 -> 0.33 ms)
+  const bool filter = cnt_lo > 0 || cnt_hi != 0x7fffffff;
+  const int cm = (chunk_mult == 2 && !dual && work && tt == 1 && !filter && cols == 2048) ? 2 : 1;
+  int rc = plan(cols, rows, dual ? 2 : 1, tt, pl, cm);
   if (rc) return rc;
   I4Args a;
   a.packed0 = packed0; a.scale0 = scale0; a.packed1 = packed1; a.scale1 = scale1;
@@ -561,7 +566,10 @@ int kx_i4_launch(bool dual, const uint32_t *packed0, const uint16_t *scale0, con
   long chunks = (long)n_slots * kx_cdiv(rows, pl.cr);
   dim3 g((unsigned)(chunks < 32768 ? chunks : 32768)), b(pl.threads);
   const bool full = pl.rs == (pl.ks >= 5 ? 1 : 8 / pl.ks) && pl.nt == i4_chunk_rows(dual, pl.rs * 4) / (pl.rs * 4);
-  if (full && pl.ks == 7) {        // Kimi-K2 gate/up: K = 7168
+  const bool full2 = cm == 2 && pl.ks == 2 && pl.rs == 4 && pl.nt == 2 * (i4_chunk_rows(false, 16) / 16);
+  if (full2) {                     // Kimi-K2 down over a per-pair list: 224-row chunks
+    hipLaunchKernelGGL((i4_gemv_k<false, 1, 2, 512, 4, false, 2>), g, b, pl.lds, st, a);
+  } else if (full && pl.ks == 7) {        // Kimi-K2 gate/up: K = 7168
     if (dual) launch_tt<true, 7, 448>(a, tt, g, b, pl.lds, st);
     else launch_tt<false, 7, 448>(a, tt, g, b, pl.lds, st);
   } else if (full && pl.ks == 2) {  // Kimi-K2 down: K = 2048

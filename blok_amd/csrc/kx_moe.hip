@@ -158,7 +158,7 @@ static int routed_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_wor
     }
     return kx_i4_launch(false, (const uint32_t *)w->d_down_packed, (const uint16_t *)w->d_down_scale, nullptr, nullptr,
                         ws->mid, ws->eout, ws->pair_work, ws->pairs, 0, H, I, 1, (size_t)H * (I / 8), (size_t)H * (I / 32),
-                        1, tokens * K, 0, 0x7fffffff, st);
+                        1, tokens * K, 0, 0x7fffffff, st, tokens * K >= 32 ? 2 : 1);
   }
   for (int i = 0; i < p.n; ++i) {
     int rc;
