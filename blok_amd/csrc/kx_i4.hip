@@ -553,7 +553,7 @@ int kx_i4_launch(bool dual, const uint32_t *packed0, const uint16_t *scale0, con
   // chunks of twice the rows: for the one-matrix kernel over many work records, where a 112-row chunk (114 KB at
   // K = 2048) is over before the workgroup's start-up is paid for (routed down at 32 tokens: 0.367 -> 0.33 ms)
   const bool filter = cnt_lo > 0 || cnt_hi != 0x7fffffff;
-  const int cm = (chunk_mult == 2 && !dual && work && tt == 1 && !filter && cols == 2048) ? 2 : 1;
+  const int cm = (chunk_mult == 2 && !dual && work && tt <= 2 && cols == 2048) ? 2 : 1;
   int rc = plan(cols, rows, dual ? 2 : 1, tt, pl, cm);
   if (rc) return rc;
   I4Args a;
@@ -567,8 +567,10 @@ int kx_i4_launch(bool dual, const uint32_t *packed0, const uint16_t *scale0, con
   dim3 g((unsigned)(chunks < 32768 ? chunks : 32768)), b(pl.threads);
   const bool full = pl.rs == (pl.ks >= 5 ? 1 : 8 / pl.ks) && pl.nt == i4_chunk_rows(dual, pl.rs * 4) / (pl.rs * 4);
   const bool full2 = cm == 2 && pl.ks == 2 && pl.rs == 4 && pl.nt == 2 * (i4_chunk_rows(false, 16) / 16);
-  if (full2) {                     // Kimi-K2 down over a per-pair list: 224-row chunks
-    hipLaunchKernelGGL((i4_gemv_k<false, 1, 2, 512, 4, false, 2>), g, b, pl.lds, st, a);
+  if (full2) {                     // Kimi-K2 down over many records: 224-row chunks
+    if (tt == 2) hipLaunchKernelGGL((i4_gemv_k<false, 2, 2, 512, 4, true, 2>), g, b, pl.lds, st, a);
+    else if (filter) hipLaunchKernelGGL((i4_gemv_k<false, 1, 2, 512, 4, true, 2>), g, b, pl.lds, st, a);
+    else hipLaunchKernelGGL((i4_gemv_k<false, 1, 2, 512, 4, false, 2>), g, b, pl.lds, st, a);
   } else if (full && pl.ks == 7) {        // Kimi-K2 gate/up: K = 7168
     if (dual) launch_tt<true, 7, 448>(a, tt, g, b, pl.lds, st);
     else launch_tt<false, 7, 448>(a, tt, g, b, pl.lds, st);

@@ -169,7 +169,7 @@ static int routed_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_wor
     else
       rc = kx_i4_launch(false, (const uint32_t *)w->d_down_packed, (const uint16_t *)w->d_down_scale, nullptr, nullptr,
                         ws->mid, ws->eout, ws->work, ws->pairs, 0, H, I, 1, (size_t)H * (I / 8), (size_t)H * (I / 32),
-                        p.tt[i], max_active, p.lo[i], p.hi[i], st);
+                        p.tt[i], max_active, p.lo[i], p.hi[i], st, tokens * K >= 32 ? 2 : 1);
     if (rc) return rc;
   }
   return KX_OK;
