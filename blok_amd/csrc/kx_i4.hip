@@ -504,7 +504,9 @@ struct I4Launch {
   size_t lds;
 };
 
-int plan(int cols, int rows, int mats, int tt, I4Launch &pl, int chunk_mult = 1) {
+// one_chunk: every workgroup has one chunk (the grid is the chunk list), so the second scale buffer, which holds the
+// next chunk's scales, is left out
+int plan(int cols, int rows, int mats, int tt, I4Launch &pl, int chunk_mult = 1, bool one_chunk = false) {
   KX_REQUIRE(cols > 0 && cols % 1024 == 0, "kx_i4: cols=%d must be a positive multiple of 1024", cols);
   KX_REQUIRE(rows >= 4, "kx_i4: rows=%d must be at least 4", rows);
   pl.ks = cols / 1024;
@@ -521,7 +523,7 @@ int plan(int cols, int rows, int mats, int tt, I4Launch &pl, int chunk_mult = 1)
   pl.nt = nt;
   pl.cr = rt * nt;
   const size_t sc_pieces = ((size_t)mats * pl.cr * (cols / 32) / 8 + 63) & ~(size_t)63;  // 16-byte pieces per scale buffer
-  pl.lds = (((size_t)mats * pl.cr * tt * pl.ks + 3) & ~(size_t)3) * sizeof(float) + 2 * sc_pieces * 16;
+  pl.lds = (((size_t)mats * pl.cr * tt * pl.ks + 3) & ~(size_t)3) * sizeof(float) + (one_chunk ? 1 : 2) * sc_pieces * 16;
   KX_REQUIRE(pl.lds <= 160 * 1024, "kx_i4: cols=%d needs %zu bytes of LDS", cols, pl.lds);
   return KX_OK;
 }
@@ -553,8 +555,12 @@ int kx_i4_launch(bool dual, const uint32_t *packed0, const uint16_t *scale0, con
   // chunks of twice the rows: for the one-matrix kernel over many work records, where a 112-row chunk (114 KB at
   // K = 2048) is over before the workgroup's start-up is paid for (routed down at 32 tokens: 0.367 -> 0.33 ms)
   const bool filter = cnt_lo > 0 || cnt_hi != 0x7fffffff;
-  const int cm = (chunk_mult == 2 && !dual && work && tt <= 2 && cols == 2048) ? 2 : 1;
-  int rc = plan(cols, rows, dual ? 2 : 1, tt, pl, cm);
+  int cm = (chunk_mult == 2 && !dual && work && tt <= 2 && cols == 2048) ? 2 : 1;
+  // the gate/up kernel over a per-pair list: 64-row chunks (458 KB) with one scale buffer, when the grid holds them all
+  const bool dual2 = chunk_mult == 2 && dual && work && tt == 1 && !filter && cols == 7168 && rows % 64 == 0 &&
+                     (long)n_slots * (rows / 64) <= 32768;
+  if (dual2) cm = 2;
+  int rc = plan(cols, rows, dual ? 2 : 1, tt, pl, cm, dual2);
   if (rc) return rc;
   I4Args a;
   a.packed0 = packed0; a.scale0 = scale0; a.packed1 = packed1; a.scale1 = scale1;
@@ -567,7 +573,9 @@ int kx_i4_launch(bool dual, const uint32_t *packed0, const uint16_t *scale0, con
   dim3 g((unsigned)(chunks < 32768 ? chunks : 32768)), b(pl.threads);
   const bool full = pl.rs == (pl.ks >= 5 ? 1 : 8 / pl.ks) && pl.nt == i4_chunk_rows(dual, pl.rs * 4) / (pl.rs * 4);
   const bool full2 = cm == 2 && pl.ks == 2 && pl.rs == 4 && pl.nt == 2 * (i4_chunk_rows(false, 16) / 16);
-  if (full2) {                     // Kimi-K2 down over many records: 224-row chunks
+  if (dual2 && pl.ks == 7 && pl.rs == 1 && pl.nt == 16) {
+    hipLaunchKernelGGL((i4_gemv_k<true, 1, 7, 448, 4, false, 2>), g, b, pl.lds, st, a);
+  } else if (full2) {              // Kimi-K2 down over many records: 224-row chunks
     if (tt == 2) hipLaunchKernelGGL((i4_gemv_k<false, 2, 2, 512, 4, true, 2>), g, b, pl.lds, st, a);
     else if (filter) hipLaunchKernelGGL((i4_gemv_k<false, 1, 2, 512, 4, true, 2>), g, b, pl.lds, st, a);
     else hipLaunchKernelGGL((i4_gemv_k<false, 1, 2, 512, 4, false, 2>), g, b, pl.lds, st, a);

@@ -154,7 +154,8 @@ static int routed_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_wor
     if (which == 0) {
       return kx_i4_launch(true, (const uint32_t *)w->d_gate_packed, (const uint16_t *)w->d_gate_scale,
                           (const uint32_t *)w->d_up_packed, (const uint16_t *)w->d_up_scale, n, ws->mid, ws->pair_work, ws->pairs, 0, I,
-                          H, K, (size_t)I * (H / 8), (size_t)I * (H / 32), 1, tokens * K, 0, 0x7fffffff, st);
+                          H, K, (size_t)I * (H / 8), (size_t)I * (H / 32), 1, tokens * K, 0, 0x7fffffff, st,
+                          tokens * K >= 128 ? 2 : 1);  // 64-row chunks from 128 pairs on (3 % at 256 pairs, none at 64)
     }
     return kx_i4_launch(false, (const uint32_t *)w->d_down_packed, (const uint16_t *)w->d_down_scale, nullptr, nullptr,
                         ws->mid, ws->eout, ws->pair_work, ws->pairs, 0, H, I, 1, (size_t)H * (I / 8), (size_t)H * (I / 32),
