@@ -117,5 +117,8 @@ struct kx_moe_workspace;
 #define KX_MOE_SEPARATE_TAIL 0x100u
 // 5 to 32 tokens: the shared expert's GEMVs on the matrix cores (kx_skinny.hip; tolerance instead of bit parity)
 #define KX_MOE_SHARED_MATRIX_CORES 0x200u
+// 5 tokens and more: the routed experts as W4A16 grouped GEMMs on the matrix cores (kx_prefill.hip) instead of the GEMV
+// kernels: an expert's weights are streamed and dequantised once for all its tokens (tolerance instead of bit parity)
+#define KX_MOE_ROUTED_MATRIX_CORES 0x400u
 int kx_moe_layer_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_workspace *ws, void *d_n, void *d_x,
                         int tokens, uint32_t flags, const uint16_t *norm_w, hipStream_t st, bool timed);

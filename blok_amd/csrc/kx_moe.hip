@@ -211,7 +211,14 @@ int kx_moe_layer_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_work
   }
   if (timed) KX_HIP(hipEventRecord(ws->ev[1], st));
   // routed gate/up + SwiGLU
-  if ((rc = routed_launch(c, w, ws, n, tokens, 0, st))) return rc;
+  const bool rmm = (flags & KX_MOE_ROUTED_MATRIX_CORES) && tokens >= 5;
+  const int n_slots = (long)tokens * K < E ? tokens * K : E;
+  if (rmm) {
+    const int I = c->moe_inter;
+    if ((rc = kx_grouped_gemm_launch(true, true, w->d_gate_packed, (const uint16_t *)w->d_gate_scale, w->d_up_packed,
+                                     (const uint16_t *)w->d_up_scale, n, ws->mid, KX_GG_BF16, ws->work, ws->pairs, 0, n_slots, I, H,
+                                     K, (size_t)I * (H / 8), (size_t)I * (H / 32), tokens, st))) return rc;
+  } else if ((rc = routed_launch(c, w, ws, n, tokens, 0, st))) return rc;
   if (timed) KX_HIP(hipEventRecord(ws->ev[2], st));
   // shared down + combine + residual: as the epilogue of a GEMV of its own, or, for one token, inside the routed
   // down launch (whichever workgroup completes a block of rows combines it)
@@ -230,7 +237,12 @@ int kx_moe_layer_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_work
                                        (long)tokens * K < E ? tokens * K : E, d, t, &tailed, st))) return rc;
   }
   // routed down
-  if (!tailed && (rc = routed_launch(c, w, ws, n, tokens, 1, st))) return rc;
+  if (rmm) {
+    const int I = c->moe_inter;
+    if ((rc = kx_grouped_gemm_launch(false, true, w->d_down_packed, (const uint16_t *)w->d_down_scale, nullptr, nullptr,
+                                     ws->mid, ws->eout, KX_GG_BF16, ws->work, ws->pairs, 0, n_slots, H, I, 1, (size_t)H * (I / 8),
+                                     (size_t)H * (I / 32), tokens, st))) return rc;
+  } else if (!tailed && (rc = routed_launch(c, w, ws, n, tokens, 1, st))) return rc;
   if (timed) KX_HIP(hipEventRecord(ws->ev[3], st));
   // shared gate/up + SwiGLU when it did not ride with the router
   // From 5 tokens on a caller may ask for the shared expert on the matrix cores (another summation order, held to
