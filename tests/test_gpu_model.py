@@ -466,6 +466,37 @@ def test_prefill_chunk_errors(kxlib):
     km.close()
 
 
+def test_kimi_shape_batch16_against_single_sequences(kxlib, ox):
+    # 16 sequences: projections, shared expert and (from 16 tokens on) the routed experts run on the matrix cores.
+    # Sequences do not interact, so each must come out as it does alone at batch 1 (the bit-exact path), within the
+    # stack-level tolerance: logits of the first sampled step within 3e-2 for at least three of the four sequences
+    # checked (a router near-tie can move one to another expert), last-layer cache rows within 2e-2.
+    say("kimi shape 2-layer stack, batch 16 against the same sequences alone")
+    cfg = default_config()
+    batch, plen = 16, 24
+    cfg.n_layers, cfg.first_dense, cfg.max_batch, cfg.max_context, cfg.seed = 2, 1, batch, plen + 4, 11
+    prompt = O.tokens_u32(batch * plen, cfg.seed, 4, cfg.vocab).reshape(batch, plen)
+    km = KxModel(kxlib, cfg)
+    rc, out, _ = km.generate(prompt, 1)
+    assert rc == 0, kxlib.kx_last_error()
+    logits = km.logits(batch)
+    rows = {b: O.bf16_to_f32(km.latent(1, b, plen)) for b in (0, 5, 10, 15)}
+    km.close()
+    cfg.max_batch = 1
+    ok = 0
+    for b in (0, 5, 10, 15):
+        k1 = KxModel(kxlib, cfg)
+        rc, o1, _ = k1.generate(prompt[b:b + 1], 1)
+        assert rc == 0, kxlib.kx_last_error()
+        e_log = O.max_rel(logits[b], k1.logits(1)[0])
+        e_rows = O.max_rel(rows[b], O.bf16_to_f32(k1.latent(1, 0, plen)))
+        print(f"sequence {b}: logits max-rel {e_log:.3e}, cache rows max-rel {e_rows:.3e}, id {out[b, 0]} / {o1[0, 0]}", flush=True)
+        assert e_rows < 2e-2
+        ok += e_log < 3e-2
+        k1.close()
+    assert ok >= 3
+
+
 def test_executor_json_line(kxlib):
     import json
     import os
