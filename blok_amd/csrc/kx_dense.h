@@ -102,7 +102,7 @@ enum { KX_GG_BF16 = 0, KX_GG_F32 = 1, KX_GG_F32_OF_BF16 = 2, KX_GG_RESID = 3 };
 int kx_grouped_gemm_launch(bool dual, bool i4, const void *w0, const uint16_t *s0, const void *w1, const uint16_t *s1,
                            const uint16_t *x, void *out, int out_mode, const int4 *work, const int *pairs, int n_pairs,
                            int n_slots, int N, int K, int x_div, size_t expert_w, size_t expert_s, int n_pairs_max,
-                           hipStream_t st);
+                           hipStream_t st, int cnt_lo = 0);
 // kx_skinny.hip: one tile of up to 32 tokens against a bf16 matrix (two for SwiGLU) on the matrix cores, out_mode as
 // above.  *done = false (nothing launched) when the shape is not the kernel's.
 int kx_skinny_gemm_launch(bool dual, const uint16_t *w0, const uint16_t *w1, const uint16_t *x, int x_stride, void *out,
@@ -117,8 +117,9 @@ struct kx_moe_workspace;
 #define KX_MOE_SEPARATE_TAIL 0x100u
 // 5 to 32 tokens: the shared expert's GEMVs on the matrix cores (kx_skinny.hip; tolerance instead of bit parity)
 #define KX_MOE_SHARED_MATRIX_CORES 0x200u
-// 5 tokens and more: the routed experts as W4A16 grouped GEMMs on the matrix cores (kx_prefill.hip) instead of the GEMV
-// kernels: an expert's weights are streamed and dequantised once for all its tokens (tolerance instead of bit parity)
+// 5 tokens and more: the routed experts with more than one pair as W4A16 grouped GEMMs on the matrix cores
+// (kx_prefill.hip) instead of the GEMV kernels: such an expert's weights are streamed and dequantised once for all its
+// tokens (tolerance instead of bit parity); the experts with one pair keep the GEMV kernel
 #define KX_MOE_ROUTED_MATRIX_CORES 0x400u
 int kx_moe_layer_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_workspace *ws, void *d_n, void *d_x,
                         int tokens, uint32_t flags, const uint16_t *norm_w, hipStream_t st, bool timed);

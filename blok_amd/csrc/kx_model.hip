@@ -378,13 +378,14 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample, int C = 1) {
       if (C > 1 && B > 32) {  // a prefill step of more than 32 tokens: the grouped GEMMs of the prefill layer
         KX_TRY(kx_moe_prefill_layer(&c, &L.moe, m->moe_ws, m->n, m->x, B, 0, st));
       } else {
-        // From 16 tokens on the routed experts run as grouped GEMMs: an expert's weights are streamed and dequantised
-        // once for all its tokens, where the GEMV kernels go over them once per token (from L2, but at one fma per
-        // weight and token on the VALU).  With the tokens spread over many experts the two are equal (both stream the
-        // experts once); with 32 sequences that decode alike (70-100 distinct experts for 256 pairs, up to 23 pairs on
-        // one expert) the step goes from 24.5 to 18.6 ms.  At 8 tokens the GEMV kernels are faster (9.8 against 11.4 ms).
+        // From 12 tokens on the routed experts with several pairs run as grouped GEMMs: such an expert's weights are
+        // streamed and dequantised once for all its tokens, where the GEMV kernels go over them once per token (from
+        // L2, but at one fma per weight and token on the VALU); the experts with one pair keep the GEMV kernel, which
+        // streams them faster than the GEMM kernel does at one token.  With 32 sequences that decode alike (70-100
+        // distinct experts for 256 pairs, up to 23 pairs on one expert) the step goes from 24.5 to 18.1 ms; at 12
+        // sequences the two forms are level (12.1 against 12.4 ms), at 8 the GEMV kernels win (9.8 against 10.9 ms).
         const uint32_t flags = ((m->fusion & KX_FUSE_MOE_TAIL) ? 0u : KX_MOE_SEPARATE_TAIL) | (mm ? KX_MOE_SHARED_MATRIX_CORES : 0u) |
-                               (B >= 16 ? KX_MOE_ROUTED_MATRIX_CORES : 0u);
+                               (B >= 12 ? KX_MOE_ROUTED_MATRIX_CORES : 0u);
         KX_TRY(kx_moe_layer_launch(&c, &L.moe, m->moe_ws, m->n, m->x, B, flags, fuse ? L.post_ln : nullptr, st, false));  // :835-877
       }
     }

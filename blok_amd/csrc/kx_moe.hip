@@ -213,11 +213,14 @@ int kx_moe_layer_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_work
   // routed gate/up + SwiGLU
   const bool rmm = (flags & KX_MOE_ROUTED_MATRIX_CORES) && tokens >= 5;
   const int n_slots = (long)tokens * K < E ? tokens * K : E;
-  if (rmm) {
+  if (rmm) {  // experts with one pair: the GEMV kernel (it streams them at its rate); the others: the grouped GEMM
     const int I = c->moe_inter;
+    if ((rc = kx_i4_launch(true, (const uint32_t *)w->d_gate_packed, (const uint16_t *)w->d_gate_scale,
+                           (const uint32_t *)w->d_up_packed, (const uint16_t *)w->d_up_scale, n, ws->mid, ws->work, ws->pairs, 0, I,
+                           H, K, (size_t)I * (H / 8), (size_t)I * (H / 32), 1, n_slots, 1, 1, st))) return rc;
     if ((rc = kx_grouped_gemm_launch(true, true, w->d_gate_packed, (const uint16_t *)w->d_gate_scale, w->d_up_packed,
                                      (const uint16_t *)w->d_up_scale, n, ws->mid, KX_GG_BF16, ws->work, ws->pairs, 0, n_slots, I, H,
-                                     K, (size_t)I * (H / 8), (size_t)I * (H / 32), tokens, st))) return rc;
+                                     K, (size_t)I * (H / 8), (size_t)I * (H / 32), tokens, st, 2))) return rc;
   } else if ((rc = routed_launch(c, w, ws, n, tokens, 0, st))) return rc;
   if (timed) KX_HIP(hipEventRecord(ws->ev[2], st));
   // shared down + combine + residual: as the epilogue of a GEMV of its own, or, for one token, inside the routed
@@ -239,9 +242,12 @@ int kx_moe_layer_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_work
   // routed down
   if (rmm) {
     const int I = c->moe_inter;
+    if ((rc = kx_i4_launch(false, (const uint32_t *)w->d_down_packed, (const uint16_t *)w->d_down_scale, nullptr, nullptr,
+                           ws->mid, ws->eout, ws->work, ws->pairs, 0, H, I, 1, (size_t)H * (I / 8), (size_t)H * (I / 32),
+                           1, n_slots, 1, 1, st, 2))) return rc;
     if ((rc = kx_grouped_gemm_launch(false, true, w->d_down_packed, (const uint16_t *)w->d_down_scale, nullptr, nullptr,
                                      ws->mid, ws->eout, KX_GG_BF16, ws->work, ws->pairs, 0, n_slots, H, I, 1, (size_t)H * (I / 8),
-                                     (size_t)H * (I / 32), tokens, st))) return rc;
+                                     (size_t)H * (I / 32), tokens, st, 2))) return rc;
   } else if (!tailed && (rc = routed_launch(c, w, ws, n, tokens, 1, st))) return rc;
   if (timed) KX_HIP(hipEventRecord(ws->ev[3], st));
   // shared gate/up + SwiGLU when it did not ride with the router

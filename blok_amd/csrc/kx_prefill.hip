@@ -66,6 +66,7 @@ struct PfArgs {
   size_t expert_w, expert_s;    // elements between experts (words or bf16; scales)
   int out_mode;                 // single matrix only: KX_GG_BF16, KX_GG_F32, KX_GG_F32_OF_BF16 or KX_GG_RESID
   int nb_max;                   // 32-token blocks per token tile (1..4): sizes the activation tiles in LDS
+  int cnt_lo;                   // groups with fewer pairs are left to another launch
 };
 
 __device__ __forceinline__ uint32_t pf_and_or(uint32_t a, uint32_t mask, uint32_t magic) {
@@ -132,6 +133,7 @@ __global__ void __launch_bounds__(WAVES * 64, (I4 || WAVES < 8) ? 1 : 2) grouped
   const int e = __builtin_amdgcn_readfirstlane(wk.x);
   if (e < 0) return;
   const int p_begin = __builtin_amdgcn_readfirstlane(wk.y), p_end = __builtin_amdgcn_readfirstlane(wk.z);
+  if (p_end - p_begin < a.cnt_lo) return;
   uint32_t magic;
   asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(magic));
   const int nk = a.K / BK;
@@ -433,7 +435,7 @@ __global__ void __launch_bounds__(256) moe_combine_k(const uint16_t *__restrict_
 int kx_grouped_gemm_launch(bool dual, bool i4, const void *w0, const uint16_t *s0, const void *w1, const uint16_t *s1,
                            const uint16_t *x, void *out, int out_mode, const int4 *work, const int *pairs, int n_pairs,
                            int n_slots, int N, int K, int x_div, size_t expert_w, size_t expert_s, int n_pairs_max,
-                           hipStream_t st) {
+                           hipStream_t st, int cnt_lo) {
   KX_REQUIRE(K > 0 && K % 128 == 0 && (!i4 || K % 512 == 0), "kx_grouped_gemm: K=%d must be a positive multiple of %d", K, i4 ? 512 : 128);
   KX_REQUIRE(N > 0, "kx_grouped_gemm: N=%d must be positive", N);
   KX_REQUIRE(out_mode >= KX_GG_BF16 && out_mode <= KX_GG_RESID && !(dual && out_mode != KX_GG_BF16), "kx_grouped_gemm: out_mode=%d", out_mode);
@@ -441,6 +443,7 @@ int kx_grouped_gemm_launch(bool dual, bool i4, const void *w0, const uint16_t *s
   a.w0 = w0; a.w1 = w1; a.s0 = s0; a.s1 = s1; a.x = x; a.out = out; a.work = work; a.pairs = pairs;
   a.n_pairs = n_pairs; a.N = N; a.K = K; a.x_div = x_div; a.expert_w = expert_w; a.expert_s = expert_s;
   a.out_mode = out_mode;
+  a.cnt_lo = cnt_lo;
   // token tile: 128 tokens for the INT4 kernels, whose dequant work per weight tile is amortised over the tokens;
   // 64 for the bf16 ones (more workgroups for the one-group GEMMs of the shared expert and the router)
   a.nb_max = i4 ? 4 : 2;
