@@ -28,6 +28,15 @@
 //   rmsnorm: float64 textbook; router: sort-based top-k incl. constructed ties,
 //     sum of weights == routed scale; bucket: counting-sort invariants;
 //   exp (mode 1): against libm within 2 ulp over a dense sweep.
+//   rope_apply: position 0 is the (2p, 2p+1) -> (p, half+p) permutation, per-pair norms are kept,
+//     q.k of two rotated vectors depends on the distance of their positions only, and a float64
+//     rotation in the half-split convention of the DeepSeek-V3 model code agrees.
+//   model_step (the wiring of run(), :801-884): a float64 numpy forward pass of the same stack written
+//     from the textbook formulation (tests/witness.py: full causal attention over the prompt, expanded
+//     K/V, no cache) agrees on cache rows, hidden state and logits, and stops agreeing when a norm
+//     weight is swapped, a residual add dropped, the rope dims normed, W_UK/W_UV swapped, the sine sign
+//     or the pair layout changed; the DeepseekV3 model of the transformers library, given the same
+//     weights, agrees as well (tests/test_oracle_wiring.py).
 // No function of the hot path is pinned by a golden vector of the reference:
 // the reference holds none for arithmetic (its only test, scripts/test_host.py,
 // pins the argv/JSON boundary).
@@ -518,6 +527,8 @@ static void rope_apply(const float *x, float *y, const uint16_t *tab, int rotary
     y[half + p] = bf(bf(x1 * c) + bf(x0 * s));
   }
 }
+// rope_apply for the tests: x, y f32 [rotary] (bf16 values), tab = one row of ox_rope_table
+void ox_rope_apply(const float *x, float *y, const uint16_t *tab, int rotary) { rope_apply(x, y, tab, rotary); }
 
 // ---------------------------------------------------------------------------------
 // The decoder stack: run() / generate() (:780-893)

@@ -41,6 +41,7 @@ _SIGS = {
     "ox_fill_tokens_u32": ([_P, _U64, _U64, _U64, C.c_uint32], None),
     "ox_yarn_inv_freq": ([_P, _I], _F),
     "ox_rope_table": ([_P, _I, _I, _P], None),
+    "ox_rope_apply": ([_P, _P, _P, _I], None),
     "ox_softmax_scale": ([_P, C.POINTER(C.c_float), C.POINTER(C.c_float)], None),
     "ox_mla_span_tiles": ([_I], _I),
     "ox_mla_decode": ([_P, _P, C.c_size_t, _P, _P, _I, _I, _I], None),
