@@ -151,7 +151,7 @@ __global__ void __launch_bounds__(128) q_absorb_k(QAbsArgs a, int tokens) {
     for (int i = 0; i < TB; ++i)
 #pragma unroll
       for (int e = 0; e < 8; ++e) acc[i][e] = 0.0f;
-#pragma unroll(TB == 1 ? 16 : 4)
+#pragma unroll TB == 1 ? 16 : 4
     for (int d = chain; d < nope; d += 8) {
       float wf[8];
       unpack8(wf, *(const uint4 *)(wuk + (size_t)d * kv_rank + c0));
