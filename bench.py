@@ -441,11 +441,11 @@ def run_mla(args):
     check(lib.kx_event_create(C.byref(e1)))
     steps = args.steps if args.steps != 256 else 20
     for _ in range(min(args.warmup, 3)):
-        check(lib.kx_mla_decode(C.byref(cfg), cache, L * kva, qabs, wsp, o_lat, B, L, None))
+        check(lib.kx_mla_decode(C.byref(cfg), cache, L * kva, qabs, wsp, o_lat, B, L, 0, None))
     check(lib.kx_sync(None))
     check(lib.kx_event_record(e0, None))
     for _ in range(steps):
-        check(lib.kx_mla_decode(C.byref(cfg), cache, L * kva, qabs, wsp, o_lat, B, L, None))
+        check(lib.kx_mla_decode(C.byref(cfg), cache, L * kva, qabs, wsp, o_lat, B, L, 0, None))
     check(lib.kx_event_record(e1, None))
     check(lib.kx_sync(None))
     ms = C.c_float()

@@ -121,5 +121,8 @@ struct kx_moe_workspace;
 // (kx_prefill.hip) instead of the GEMV kernels: such an expert's weights are streamed and dequantised once for all its
 // tokens (tolerance instead of bit parity); the experts with one pair keep the GEMV kernel
 #define KX_MOE_ROUTED_MATRIX_CORES 0x400u
+int *kx_moe_workspace_n_active(kx_moe_workspace *ws);  // device address of the count of distinct experts of the last call
+// the flags a caller of kx_moe_decode_layer may pass (include/kx.h documents them)
+#define KX_MOE_PUBLIC_FLAGS (1u | KX_MOE_SEPARATE_TAIL | KX_MOE_SHARED_MATRIX_CORES | KX_MOE_ROUTED_MATRIX_CORES)
 int kx_moe_layer_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_workspace *ws, void *d_n, void *d_x,
                         int tokens, uint32_t flags, const uint16_t *norm_w, hipStream_t st, bool timed);

@@ -27,8 +27,8 @@ struct KxMlaPartials {
 // scores + online softmax + PV per span; the merge is left to the caller (kx_mla_combine_launch, or the W_UV GEMV
 // when there are at most 64 spans)
 int kx_mla_partials_launch(const kx_config *c, const uint16_t *cache, size_t seq_stride, const float *qabs, float *partial,
-                           int batch, int seq, KxMlaPartials *out, hipStream_t st, int seqs = 0);
+                           int batch, int seq, KxMlaPartials *out, hipStream_t st, int seqs = 0, int kernel = KX_MLA_AUTO);
 // the merge of the span partials as a kernel of its own: o_lat bf16 [batch][heads][kv_rank] (any number of spans)
 int kx_mla_combine_launch(const KxMlaPartials &p, uint16_t *o_lat, int batch, int heads, hipStream_t st);
 int kx_mla_attend_launch(const kx_config *c, const uint16_t *cache, size_t seq_stride, const float *qabs, float *partial,
-                         uint16_t *o_lat, int batch, int seq, hipStream_t st, int seqs = 0);
+                         uint16_t *o_lat, int batch, int seq, hipStream_t st, int seqs = 0, int kernel = KX_MLA_AUTO);

@@ -75,13 +75,6 @@ extern "C" int kx_softmax_scale(const kx_config *cfg, float *rs, float *mscale) 
   return KX_OK;
 }
 
-// 0: matrix-core kernel from 2048 positions on (128 for 5 sequences and more), 1: VALU kernel always, 2: matrix-core kernel always
-static int g_mla_kernel = 0;
-extern "C" int kx_mla_set_kernel(int32_t mode) {
-  KX_REQUIRE(mode >= 0 && mode <= 2, "kx_mla_set_kernel: mode=%d outside [0, 2]", mode);
-  g_mla_kernel = mode;
-  return KX_OK;
-}
 
 int kx_mla_span_tiles(int seq) {
   int tiles = (seq + 63) / 64, st = 1;
@@ -737,7 +730,8 @@ size_t kx_mla_partial_floats(int batch, int heads, int kv_rank, int max_seq) {
 }
 
 int kx_mla_partials_launch(const kx_config *c, const uint16_t *cache, size_t seq_stride, const float *qabs, float *partial,
-                           int batch, int seq, KxMlaPartials *out, hipStream_t st, int seqs) {
+                           int batch, int seq, KxMlaPartials *out, hipStream_t st, int seqs, int kernel) {
+  KX_REQUIRE(kernel >= KX_MLA_AUTO && kernel <= KX_MLA_MATRIX_CORES, "kx_mla: kernel=%d outside [0, 2]", kernel);
   KX_REQUIRE(c->kv_rank == 512 && c->qk_rope == 64, "kx_mla: the attention kernel is built for kv_rank 512, qk_rope 64 (got %d, %d)",
              c->kv_rank, c->qk_rope);
   KX_REQUIRE(c->heads % 4 == 0, "kx_mla: heads=%d must be a multiple of 4", c->heads);
@@ -746,7 +740,7 @@ int kx_mla_partials_launch(const kx_config *c, const uint16_t *cache, size_t seq
   // automatic choice, where the matrix-core kernel is built for the shape (64 heads): from 2048 positions on, and from
   // 128 positions on for 5 sequences and more (batches the stack runs on the matrix cores anyway; the VALU kernel
   // takes 190-360 us per layer at 32 sequences of 1100 positions)
-  const bool use_mfma = g_mla_kernel == 2 || (g_mla_kernel == 0 && c->heads == 64 && (seq >= 2048 || (batch >= 5 && seq >= 128)));
+  const bool use_mfma = kernel == KX_MLA_MATRIX_CORES || (kernel == KX_MLA_AUTO && c->heads == 64 && (seq >= 2048 || (batch >= 5 && seq >= 128)));
   MlaArgs a;
   a.cache = cache; a.qabs = qabs; a.heads = c->heads; a.seq = seq; a.seq_stride = seq_stride; a.seqs = seqs;
   a.span_tiles = use_mfma ? mfma_span_tiles(seq, batch) : kx_mla_span_tiles(seq);
@@ -802,9 +796,9 @@ int kx_mla_combine_launch(const KxMlaPartials &p, uint16_t *o_lat, int batch, in
 }
 
 int kx_mla_attend_launch(const kx_config *c, const uint16_t *cache, size_t seq_stride, const float *qabs, float *partial,
-                         uint16_t *o_lat, int batch, int seq, hipStream_t st, int seqs) {
+                         uint16_t *o_lat, int batch, int seq, hipStream_t st, int seqs, int kernel) {
   KxMlaPartials p;
-  int rc = kx_mla_partials_launch(c, cache, seq_stride, qabs, partial, batch, seq, &p, st, seqs);
+  int rc = kx_mla_partials_launch(c, cache, seq_stride, qabs, partial, batch, seq, &p, st, seqs, kernel);
   if (rc) return rc;
   return kx_mla_combine_launch(p, o_lat, batch, c->heads, st);
 }
@@ -818,11 +812,11 @@ extern "C" int kx_mla_workspace_bytes(const kx_config *cfg, int32_t batch, int32
 }
 
 extern "C" int kx_mla_decode(const kx_config *cfg, const void *d_cache, size_t seq_stride, const void *d_qabs,
-                             void *d_workspace, void *d_o_lat, int32_t batch, int32_t seq, void *stream) {
+                             void *d_workspace, void *d_o_lat, int32_t batch, int32_t seq, int32_t kernel, void *stream) {
   KX_REQUIRE(cfg && d_cache && d_qabs && d_workspace && d_o_lat, "kx_mla_decode: null argument");
   KX_REQUIRE(seq_stride >= (size_t)seq * (cfg->kv_rank + cfg->qk_rope), "kx_mla_decode: seq_stride shorter than the sequence");
   return kx_mla_attend_launch(cfg, (const uint16_t *)d_cache, seq_stride, (const float *)d_qabs, (float *)d_workspace,
-                              (uint16_t *)d_o_lat, batch, seq, kx_stream(stream));
+                              (uint16_t *)d_o_lat, batch, seq, kx_stream(stream), 0, kernel);
 }
 
 extern "C" int kx_q_absorb(const kx_config *cfg, const void *d_q, const void *d_kvb, const void *d_rope_row, void *d_qabs,

@@ -81,6 +81,9 @@ struct kx_model {
   int4 *head_work;                 // [heads], [step tokens * heads]: the groups of head_groups_k
   int *head_pairs;
   uint32_t fusion = KX_FUSE_ALL;
+  int mla_kernel = KX_MLA_AUTO;    // kx_model_set_attention_kernel
+  float *route_logits = nullptr;   // routing record (kx_model_set_routing_record): [n_layers][max_batch][experts]
+  int *route_distinct = nullptr;   // [n_layers] distinct experts of the last step
   kx_moe_workspace *moe_ws = nullptr;
   hipStream_t st = nullptr;
   hipEvent_t ev[3] = {nullptr, nullptr, nullptr};
@@ -333,7 +336,7 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample, int C = 1) {
     g.w_block_off = c.qk_nope; g.x_block_stride = c.kv_rank;
     if (fuse) {                                                                                 // :825
       KxMlaPartials mp;
-      KX_TRY(kx_mla_partials_launch(&c, L.cache, seq_stride, m->qabs, m->partial, B, pos + 1, &mp, st));
+      KX_TRY(kx_mla_partials_launch(&c, L.cache, seq_stride, m->qabs, m->partial, B, pos + 1, &mp, st, 0, m->mla_kernel));
       if (mp.spans <= 64) {  // the GEMV's activations are the attention partials, merged as they are loaded
         g.mla_pm = mp.pm; g.mla_pz = mp.pz; g.mla_po = mp.po; g.mla_spans = mp.spans; g.mla_heads = c.heads;
       } else {               // long context, few sequences: more spans than the GEMV's merge takes
@@ -345,7 +348,7 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample, int C = 1) {
       for (int i0 = 0; i0 < C; i0 += cs) {
         const int np = C - i0 < cs ? C - i0 : cs;
         KX_TRY(kx_mla_attend_launch(&c, L.cache, seq_stride, m->qabs + (size_t)i0 * NB * c.heads * KVA, m->partial,
-                                    m->o_lat + (size_t)i0 * NB * c.heads * c.kv_rank, np * NB, pos + i0 + np, st, C > 1 ? NB : 0));
+                                    m->o_lat + (size_t)i0 * NB * c.heads * c.kv_rank, np * NB, pos + i0 + np, st, C > 1 ? NB : 0, m->mla_kernel));
       }
     }
     if (C > 1 && B > 32 && c.kv_rank % 128 == 0) {  // a long prefill step: one grouped GEMM over the heads
@@ -387,6 +390,14 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample, int C = 1) {
         const uint32_t flags = ((m->fusion & KX_FUSE_MOE_TAIL) ? 0u : KX_MOE_SEPARATE_TAIL) | (mm ? KX_MOE_SHARED_MATRIX_CORES : 0u) |
                                (B >= 12 ? KX_MOE_ROUTED_MATRIX_CORES : 0u);
         KX_TRY(kx_moe_layer_launch(&c, &L.moe, m->moe_ws, m->n, m->x, B, flags, fuse ? L.post_ln : nullptr, st, false));  // :835-877
+      }
+      if (m->route_logits) {  // the routing record: logits of the first rows and the number of distinct experts
+        const int rows = B < c.max_batch ? B : c.max_batch;
+        void *d_logits = nullptr;
+        KX_TRY(kx_moe_workspace_views(m->moe_ws, &d_logits, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr));
+        KX_HIP(hipMemcpyAsync(m->route_logits + (size_t)l * c.max_batch * c.experts, d_logits, (size_t)rows * c.experts * 4,
+                              hipMemcpyDeviceToDevice, st));
+        KX_HIP(hipMemcpyAsync(m->route_distinct + l, kx_moe_workspace_n_active(m->moe_ws), 4, hipMemcpyDeviceToDevice, st));
       }
     }
   }
@@ -551,6 +562,8 @@ extern "C" int kx_model_destroy(kx_model *m) {
     if (ev) (void)hipEventDestroy(ev);
   if (m->st) (void)hipStreamDestroy(m->st);
   if (m->arena) (void)hipFree(m->arena);
+  if (m->route_logits) (void)hipFree(m->route_logits);
+  if (m->route_distinct) (void)hipFree(m->route_distinct);
   delete m;
   return KX_OK;
 }
@@ -655,6 +668,49 @@ extern "C" int kx_model_set_prefill_chunk(kx_model *m, int32_t positions) {
   return KX_OK;
 }
 
+extern "C" int kx_model_set_attention_kernel(kx_model *m, int32_t kernel) {
+  KX_REQUIRE(m, "kx_model_set_attention_kernel: null model");
+  KX_REQUIRE(kernel >= KX_MLA_AUTO && kernel <= KX_MLA_MATRIX_CORES, "kx_model_set_attention_kernel: kernel=%d outside [0, 2]", kernel);
+  KX_REQUIRE(kernel != KX_MLA_MATRIX_CORES || m->c.heads == 64, "kx_model_set_attention_kernel: the matrix-core kernel is built for 64 heads (model: %d)", m->c.heads);
+  m->mla_kernel = kernel;
+  return KX_OK;
+}
+extern "C" int kx_model_set_routing_record(kx_model *m, int on) {
+  KX_REQUIRE(m, "kx_model_set_routing_record: null model");
+  KX_REQUIRE(m->c.first_dense < m->c.n_layers, "kx_model_set_routing_record: the model has no MoE layer");
+  KX_HIP(hipStreamSynchronize(m->st));
+  if (!on) {
+    if (m->route_logits) (void)hipFree(m->route_logits);
+    if (m->route_distinct) (void)hipFree(m->route_distinct);
+    m->route_logits = nullptr; m->route_distinct = nullptr;
+    return KX_OK;
+  }
+  if (m->route_logits) return KX_OK;
+  const size_t nl = (size_t)m->c.n_layers;
+  float *lg = nullptr;
+  int *di = nullptr;
+  KX_HIP(hipMalloc((void **)&lg, nl * m->c.max_batch * m->c.experts * 4));
+  if (hipMalloc((void **)&di, nl * 4) != hipSuccess || hipMemset(di, 0, nl * 4) != hipSuccess ||
+      hipMemset(lg, 0, nl * m->c.max_batch * m->c.experts * 4) != hipSuccess) {
+    (void)hipFree(lg);
+    if (di) (void)hipFree(di);
+    kx_set_error("kx_model_set_routing_record: no memory for the record");
+    return KX_ERR_HIP;
+  }
+  m->route_logits = lg; m->route_distinct = di;
+  return KX_OK;
+}
+extern "C" int kx_model_routing(kx_model *m, int32_t layer, float *h_logits, int32_t *h_distinct) {
+  KX_REQUIRE(m && m->route_logits, "kx_model_routing: null model, or kx_model_set_routing_record was not switched on");
+  KX_REQUIRE(layer >= m->c.first_dense && layer < m->c.n_layers, "kx_model_routing: layer %d is not a MoE layer of this model", layer);
+  KX_REQUIRE(m->batch > 0, "kx_model_routing: no step has run");
+  if (h_logits)
+    KX_HIP(hipMemcpyAsync(h_logits, m->route_logits + (size_t)layer * m->c.max_batch * m->c.experts, (size_t)m->batch * m->c.experts * 4,
+                          hipMemcpyDeviceToHost, m->st));
+  if (h_distinct) KX_HIP(hipMemcpyAsync(h_distinct, m->route_distinct + layer, 4, hipMemcpyDeviceToHost, m->st));
+  KX_HIP(hipStreamSynchronize(m->st));
+  return KX_OK;
+}
 extern "C" int kx_model_set_fusion(kx_model *m, uint32_t mask) {
   KX_REQUIRE(m, "kx_model_set_fusion: null model");
   KX_REQUIRE(!(mask & ~(uint32_t)KX_FUSE_ALL), "kx_model_set_fusion: unknown bits in mask 0x%x", mask);

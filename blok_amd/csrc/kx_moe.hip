@@ -80,11 +80,17 @@ extern "C" int kx_moe_workspace_create(const kx_config *cfg, int32_t max_tokens,
   ws->route_counter = ws->n_active + 1;
   // work records nobody has written yet say "no expert" (-1): kx_moe_routed_only before any layer call, or with more
   // tokens than the last one had, then does nothing instead of following uninitialised records
-  KX_HIP(hipMemset(ws->work, 0xff, E * 16));
-  KX_HIP(hipMemset(ws->pair_work, 0xff, T * K * 16));
-  KX_HIP(hipMemset(ws->n_active, 0, 8));
-  KX_HIP(hipMemset(ws->tail_count, 0, KX_TAIL_BLOCKS * 4));
-  for (auto &e : ws->ev) KX_HIP(hipEventCreate(&e));
+  hipError_t e = hipMemset(ws->work, 0xff, E * 16);
+  if (e == hipSuccess) e = hipMemset(ws->pair_work, 0xff, T * K * 16);
+  if (e == hipSuccess) e = hipMemset(ws->n_active, 0, 8);
+  if (e == hipSuccess) e = hipMemset(ws->tail_count, 0, KX_TAIL_BLOCKS * 4);
+  for (auto &ev : ws->ev)
+    if (e == hipSuccess) e = hipEventCreate(&ev);
+  if (e != hipSuccess) {
+    kx_set_error("kx_moe_workspace_create: %s", hipGetErrorString(e));
+    kx_moe_workspace_destroy(ws);
+    return KX_ERR_HIP;
+  }
   *out = ws;
   return KX_OK;
 }
@@ -92,7 +98,7 @@ extern "C" int kx_moe_workspace_create(const kx_config *cfg, int32_t max_tokens,
 extern "C" int kx_moe_workspace_destroy(kx_moe_workspace *ws) {
   if (!ws) return KX_OK;
   void *ptrs[] = {ws->logits, ws->ids, ws->weights, ws->counts, ws->offsets, ws->pairs,
-                  ws->work, ws->pair_work, ws->n_active, ws->mid, ws->eout, ws->smid, ws->sy};
+                  ws->work, ws->pair_work, ws->n_active, ws->tail_count, ws->mid, ws->eout, ws->smid, ws->sy};
   for (void *p : ptrs)
     if (p) (void)hipFree(p);
   for (auto &e : ws->ev)
@@ -100,6 +106,8 @@ extern "C" int kx_moe_workspace_destroy(kx_moe_workspace *ws) {
   delete ws;
   return KX_OK;
 }
+
+int *kx_moe_workspace_n_active(kx_moe_workspace *ws) { return ws->n_active; }
 
 extern "C" int kx_moe_workspace_views(kx_moe_workspace *ws, void **d_logits, void **d_ids, void **d_weights,
                                       void **d_counts, void **d_offsets, void **d_pairs, void **d_mid,
@@ -277,14 +285,14 @@ int kx_moe_layer_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_work
 
 extern "C" int kx_moe_decode_layer(const kx_config *cfg, const kx_moe_weights *w, kx_moe_workspace *ws, const void *d_n,
                                    void *d_x, int32_t tokens, uint32_t flags, void *stream) {
-  return kx_moe_layer_launch(cfg, w, ws, (void *)d_n, d_x, tokens, flags & (1u | KX_MOE_SEPARATE_TAIL), nullptr, kx_stream(stream), false);
+  return kx_moe_layer_launch(cfg, w, ws, (void *)d_n, d_x, tokens, flags & KX_MOE_PUBLIC_FLAGS, nullptr, kx_stream(stream), false);
 }
 
 extern "C" int kx_moe_decode_layer_timed(const kx_config *cfg, const kx_moe_weights *w, kx_moe_workspace *ws,
                                          const void *d_n, void *d_x, int32_t tokens, uint32_t flags, void *stream,
                                          float *ms5) {
   KX_REQUIRE(ms5, "kx_moe_decode_layer_timed: null output");
-  int rc = kx_moe_layer_launch(cfg, w, ws, (void *)d_n, d_x, tokens, flags & (1u | KX_MOE_SEPARATE_TAIL), nullptr, kx_stream(stream), true);
+  int rc = kx_moe_layer_launch(cfg, w, ws, (void *)d_n, d_x, tokens, flags & KX_MOE_PUBLIC_FLAGS, nullptr, kx_stream(stream), true);
   if (rc) return rc;
   KX_HIP(hipEventSynchronize(ws->ev[5]));
   for (int i = 0; i < 5; ++i) KX_HIP(hipEventElapsedTime(&ms5[i], ws->ev[i], ws->ev[i + 1]));

@@ -73,9 +73,8 @@ _SIGS = {
     "kx_rope_table": [C.POINTER(KxConfig), _I, _I, _P],
     "kx_softmax_scale": [C.POINTER(KxConfig), C.POINTER(C.c_float), C.POINTER(C.c_float)],
     "kx_q_absorb": [C.POINTER(KxConfig), _P, _P, _P, _P, _I, _P],
-    "kx_mla_set_kernel": [_I],
     "kx_mla_workspace_bytes": [C.POINTER(KxConfig), _I, _I, C.POINTER(_SZ)],
-    "kx_mla_decode": [C.POINTER(KxConfig), _P, _SZ, _P, _P, _P, _I, _I, _P],
+    "kx_mla_decode": [C.POINTER(KxConfig), _P, _SZ, _P, _P, _P, _I, _I, _I, _P],
     "kx_model_bytes": [C.POINTER(KxConfig), C.POINTER(C.c_uint64), C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)],
     "kx_model_create": [C.POINTER(KxConfig), _PP],
     "kx_model_destroy": [_P],
@@ -88,6 +87,9 @@ _SIGS = {
     "kx_model_latent": [_P, _I, _I, _I, _I, _P],
     "kx_model_timing": [_P, C.POINTER(C.c_float)],
     "kx_model_set_fusion": [_P, C.c_uint32],
+    "kx_model_set_attention_kernel": [_P, _I],
+    "kx_model_set_routing_record": [_P, C.c_int],
+    "kx_model_routing": [_P, _I, _P, _P],
     "kx_model_set_prefill_chunk": [_P, _I],
     "kx_model_stream": [_P, _PP],
     "kx_moe_prefill_layer": [C.POINTER(KxConfig), C.POINTER(KxMoeWeights), _P, _P, _P, _I, C.c_uint32, _P],

@@ -168,7 +168,13 @@ int kx_moe_workspace_views(kx_moe_workspace *ws, void **d_logits, void **d_ids, 
  *       with down = bf(bf(sum_slot y_slot * w_slot) + bf(shared)) (:868-877).
  * flags bit0: skip the residual add and write `down` to d_x instead.
  *       bit8: run the shared expert's down GEMV and the combine as a launch of their own even
- *             for one token (by default they ride in the routed down launch; same results). */
+ *             for one token (by default they ride in the routed down launch; same results).
+ *       bit9: 5 to 32 tokens: the shared expert's two GEMVs as bf16 matrix-core products (another
+ *             summation order: within max-rel 1e-2 of the default instead of equal to the bit).
+ *       bit10: 5 tokens and more: the routed experts that have more than one (token, slot) pair as W4A16
+ *             grouped GEMMs on the matrix cores, the experts with one pair through the GEMV kernel (same
+ *             tolerance).  The router is not affected by either bit, so the routing stays the default's.
+ *             The decoder stack sets bit9 from 5 sequences on and bit10 from 12. */
 int kx_moe_decode_layer(const kx_config *cfg, const kx_moe_weights *w, kx_moe_workspace *ws,
                         const void *d_n, void *d_x, int32_t tokens, uint32_t flags, void *stream);
 /* The same layer for a prefill chunk of T tokens (BASELINE config 4): the tokens of each expert are
@@ -208,13 +214,15 @@ int kx_softmax_scale(const kx_config *cfg, float *rsqrt_head, float *mscale);
 int kx_q_absorb(const kx_config *cfg, const void *d_q, const void *d_kvb, const void *d_rope_row,
                 void *d_qabs, int32_t tokens, void *stream);
 int kx_mla_workspace_bytes(const kx_config *cfg, int32_t batch, int32_t max_seq, size_t *bytes);
-/* Which kernel computes the attention partials, process-wide: 0 (default) the matrix-core kernel from 2048
- * cached positions on (from 128 for five sequences and more) and the VALU kernel below, 1 the VALU kernel always (fixed summation order, the one
- * the token-identity checks rest on), 2 the matrix-core kernel always (same values, another summation
- * order; 64 heads).  No counterpart in the reference.                                              */
-int kx_mla_set_kernel(int32_t mode);
+/* `kernel`: which kernel computes the attention partials.  KX_MLA_AUTO: the matrix-core kernel from 2048 cached
+ * positions on (from 128 for five sequences and more) and the VALU kernel below; KX_MLA_VALU: the VALU kernel
+ * always (fixed summation order, the one the token-identity checks rest on); KX_MLA_MATRIX_CORES: the matrix-core
+ * kernel always (same values, another summation order; 64 heads).  No counterpart in the reference.        */
+#define KX_MLA_AUTO 0
+#define KX_MLA_VALU 1
+#define KX_MLA_MATRIX_CORES 2
 int kx_mla_decode(const kx_config *cfg, const void *d_cache, size_t seq_stride, const void *d_qabs,
-                  void *d_workspace, void *d_o_lat, int32_t batch, int32_t seq, void *stream);
+                  void *d_workspace, void *d_o_lat, int32_t batch, int32_t seq, int32_t kernel, void *stream);
 
 /* ---- the decoder stack: generate() / run() (:780-893) ------------------------------------
  * A kx_model owns one HBM arena: seeded random-init weights of cfg->n_layers layers (layer
@@ -302,6 +310,18 @@ int kx_model_timing(kx_model *model, float *ms2);
 #define KX_FUSE_MOE_TAIL 2u /* one token: shared down GEMV + combine + residual inside the routed down launch */
 #define KX_FUSE_ALL 3u
 int kx_model_set_fusion(kx_model *model, uint32_t mask);
+/* The attention kernel this model's steps use: KX_MLA_AUTO (default), KX_MLA_VALU or KX_MLA_MATRIX_CORES, as for
+ * kx_mla_decode.  A property of the model: other models of the process keep theirs.                          */
+int kx_model_set_attention_kernel(kx_model *model, int32_t kernel);
+/* A record of the routing for tests and measurement.  The reference's host knows the expert ids of every layer
+ * (it copies them back, src/kimi_exec.cu:844); here they stay on the device, and this is the way to look at them.
+ * kx_model_set_routing_record(model, 1): from now on every step also keeps, per MoE layer, the router logits of its
+ * first min(tokens, max_batch) tokens and the number of distinct experts its tokens selected (two small device
+ * copies per layer; off by default).
+ * kx_model_routing: the record of the last step for `layer`: h_logits f32 [batch][experts] (or NULL), h_distinct
+ * i32 [1] (or NULL).  Synchronises.  A dense layer is an error.                                              */
+int kx_model_set_routing_record(kx_model *model, int on);
+int kx_model_routing(kx_model *model, int32_t layer, float *h_logits, int32_t *h_distinct);
 /* Prompt positions per prefill step.  1 (default) is the reference's prefill, one run() per prompt token (:886),
  * and the bit-reproducible path.  With n > 1, kx_prefill and kx_generate take up to n consecutive positions of
  * every sequence in one step (at most 2048 tokens a step, so min(n, 2048 / batch) positions): the projections, the

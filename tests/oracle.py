@@ -115,6 +115,16 @@ def max_rel(a, b):
     return float(np.max(np.abs(a - b)) / max(np.max(np.abs(b)), 1e-30))
 
 
+def elem_err(a, b):
+    """Element-wise criterion beside max_rel: max over elements of |a-b| / (|b| + rms(b)).  An element is held to
+    its own magnitude once that is above the tensor's RMS, and to the RMS below it (an fp32-accumulated dot product
+    that cancels to near zero has no relative accuracy of its own)."""
+    a = np.asarray(a, dtype=np.float64)
+    b = np.asarray(b, dtype=np.float64)
+    rms = max(float(np.sqrt(np.mean(b * b))), 1e-30)
+    return float(np.max(np.abs(a - b) / (np.abs(b) + rms)))
+
+
 def tokens_u32(n, seed, tid, vocab):
     out = np.empty(n, dtype=np.uint32)
     load().ox_fill_tokens_u32(ptr(out), n, seed, tid, vocab)

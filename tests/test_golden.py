@@ -54,7 +54,7 @@ def test_gpu_reproduces_the_fixtures(kxlib):
     nbytes = C.c_size_t()
     check(kxlib.kx_mla_workspace_bytes(C.byref(cfg), 1, 8, C.byref(nbytes)))
     dc, dqa, dws, do = dev(GOLD["mla_cache"]), dev(GOLD["mla_qabs"]), DevBuf(nbytes.value), DevBuf(4 * 512 * 2)
-    check(kxlib.kx_mla_decode(C.byref(cfg), dc.ptr, 8 * 576, dqa.ptr, dws.ptr, do.ptr, 1, 8, None))
+    check(kxlib.kx_mla_decode(C.byref(cfg), dc.ptr, 8 * 576, dqa.ptr, dws.ptr, do.ptr, 1, 8, 0, None))
     check(kxlib.kx_sync(None))
     assert (do.to_numpy(np.uint16, (1, 4, 512))[:, :, :64] == GOLD["mla_o_mode1"]).all()
     cfg = O.small_config(batch=2)

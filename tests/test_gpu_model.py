@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 
 import oracle as O
-from kxt import check, dev, say
+from kxt import check, dev, judge_sequences, routing_of, say
 from oracle import ptr
 
 pytestmark = pytest.mark.gpu
@@ -107,24 +107,39 @@ def test_small_stack_matrix_core_projections(kxlib, ox, batch):
     # sampled step are held to the stack-level 3e-2 against both oracle schedules, not to the bits (batch 40: beyond
     # one 32-token tile the projections take the prefill GEMM kernel)
     say(f"small stack batch={batch} (dense projections on the matrix cores)")
+    # Per sequence: logits within 3e-2 and the same first id.  The only excuses are the two a tolerance path has in a
+    # MoE stack, and each is checked and named: the sequence's expert set differs from the bit-exact path's because
+    # that path's own selection was a near-tie there, or the two largest logits lie closer than the tolerance.  The
+    # routing of the bit-exact path comes from the same sequences run four at a time (GEMV kernels, equal to the
+    # oracle's kx schedule to the bit, as the tests above establish).
     prompt_len = 5
     cfg = O.small_config(batch=batch, context=32)
     prompt = O.tokens_u32(batch * prompt_len, cfg.seed, 4, cfg.vocab).reshape(batch, prompt_len)
     km = KxModel(kxlib, cfg)
+    check(kxlib.kx_model_set_routing_record(km.h, 1))
     rc, out, _ = km.generate(prompt, 1)
     assert rc == 0, kxlib.kx_last_error()
-    got = km.logits(batch)
+    got, routes = km.logits(batch), routing_of(kxlib, km.h, cfg, batch)
+    ref_routes = {l: ([], []) for l in routes}
+    for b0 in range(0, batch, 4):
+        nb = min(4, batch - b0)
+        rc, _, _ = km.generate(prompt[b0:b0 + nb], 1)
+        assert rc == 0, kxlib.kx_last_error()
+        for l, (sets, gaps) in routing_of(kxlib, km.h, cfg, nb).items():
+            ref_routes[l][0].extend(sets)
+            ref_routes[l][1].extend(gaps.tolist())
+    km.close()
+    names = [f"sequence {b}" for b in range(batch)]
     for mode in (1, 0):
         om = O.OxModel(cfg, mode)
         rc, out_o, _ = om.generate(prompt, 1)
         assert rc == 0
-        err = O.max_rel(got, om.logits(batch))
-        agree = float(np.mean(out == out_o))
-        print(f"batch-{batch} stack logits vs oracle mode {mode}: max-rel {err:.3e}, first ids equal for {agree:.0%} of the sequences")
-        assert err < 3e-2
-        assert agree >= 0.75
+        ref = om.logits(batch)
+        errs = [O.max_rel(got[b], ref[b]) for b in range(batch)]
+        excused = judge_sequences(names, errs, 3e-2, routes, ref_routes, out[:, 0], out_o[:, 0], ref)
+        print(f"batch-{batch} stack vs oracle mode {mode}: worst logits max-rel {max(errs):.3e}; excused: {excused or 'none'}", flush=True)
+        assert len(excused) <= batch // 4
         om.close()
-    km.close()
 
 
 def test_prefill_decode_sample_entry_points(kxlib, ox):
@@ -298,12 +313,9 @@ def test_mla_decode_operator(kxlib, ox, batch, seq):
     nbytes = C.c_size_t()
     check(kxlib.kx_mla_workspace_bytes(C.byref(cfg), batch, seq, C.byref(nbytes)))
     dc, dq, dw, do = dev(cache), dev(qabs), DevBuf(nbytes.value), DevBuf(batch * H * R * 2)
-    check(kxlib.kx_mla_set_kernel(1))   # the VALU kernel, whose summation order the oracle's mode 1 restates
-    try:
-        check(kxlib.kx_mla_decode(C.byref(cfg), dc.ptr, seq * KVA, dq.ptr, dw.ptr, do.ptr, batch, seq, None))
-        check(kxlib.kx_sync(None))
-    finally:
-        check(kxlib.kx_mla_set_kernel(0))
+    # kernel 1: the VALU kernel, whose summation order the oracle's mode 1 restates
+    check(kxlib.kx_mla_decode(C.byref(cfg), dc.ptr, seq * KVA, dq.ptr, dw.ptr, do.ptr, batch, seq, 1, None))
+    check(kxlib.kx_sync(None))
     got = do.to_numpy(np.uint16, (batch, H, R))
     exp1, exp0 = np.empty_like(got), np.empty_like(got)
     ox.ox_mla_decode(C.byref(cfg), ptr(cache), seq * KVA, ptr(qabs), ptr(exp1), batch, seq, 1)
@@ -327,14 +339,10 @@ def test_mla_decode_matrix_core_kernel(kxlib, ox, batch, seq):
     check(kxlib.kx_mla_workspace_bytes(C.byref(cfg), batch, seq, C.byref(nbytes)))
     dc, dq, dw, do = dev(cache), dev(qabs), DevBuf(nbytes.value), DevBuf(batch * H * R * 2)
     outs = {}
-    try:
-        for mode in (2, 1):
-            check(kxlib.kx_mla_set_kernel(mode))
-            check(kxlib.kx_mla_decode(C.byref(cfg), dc.ptr, seq * KVA, dq.ptr, dw.ptr, do.ptr, batch, seq, None))
-            check(kxlib.kx_sync(None))
-            outs[mode] = O.bf16_to_f32(do.to_numpy(np.uint16, (batch, H, R)))
-    finally:
-        check(kxlib.kx_mla_set_kernel(0))
+    for mode in (2, 1):
+        check(kxlib.kx_mla_decode(C.byref(cfg), dc.ptr, seq * KVA, dq.ptr, dw.ptr, do.ptr, batch, seq, mode, None))
+        check(kxlib.kx_sync(None))
+        outs[mode] = O.bf16_to_f32(do.to_numpy(np.uint16, (batch, H, R)))
     exp1, exp0 = np.empty((batch, H, R), dtype=np.uint16), np.empty((batch, H, R), dtype=np.uint16)
     ox.ox_mla_decode(C.byref(cfg), ptr(cache), seq * KVA, ptr(qabs), ptr(exp1), batch, seq, 1)
     ox.ox_mla_decode(C.byref(cfg), ptr(cache), seq * KVA, ptr(qabs), ptr(exp0), batch, seq, 0)
@@ -342,6 +350,91 @@ def test_mla_decode_matrix_core_kernel(kxlib, ox, batch, seq):
     e1, e0 = O.max_rel(outs[2], O.bf16_to_f32(exp1)), O.max_rel(outs[2], O.bf16_to_f32(exp0))
     print(f"matrix-core MLA seq={seq}: max-rel {e_valu:.2e} vs VALU kernel, {e1:.2e} vs mode 1, {e0:.2e} vs mode 0", flush=True)
     assert e_valu < 1e-2 and e1 < 1e-2 and e0 < 1e-2
+
+
+@pytest.mark.parametrize("batch,seq", [(1, 4096), (1, 32768), (1, 131072), (16, 4096), (16, 32768), (16, 131072)])
+def test_mla_decode_baseline_sizes(kxlib, ox, batch, seq):
+    # BASELINE config 3 at its own sizes.  The cache is generated on the device, sequence b from tensor id b, so the
+    # host can regenerate single sequences.  The scalar oracle runs on a sample -- the first and the last sequence,
+    # eight of the 64 heads (heads do not interact: a config with heads = 8 on that slice of q) -- in both schedules;
+    # the matrix-core kernel (the one these sizes take) is held to 1e-2 on it, normalised maximum and element-wise,
+    # and the VALU kernel to the kx schedule's bits.  On the full output: finite, every element inside the range of
+    # its cache column (a softmax-weighted mean cannot leave it), and matrix-core against VALU kernel within 1e-2.
+    # The element-wise figure is held to 2e-2: a score is rounded to bf16 twice (:429), so another summation order
+    # flips the rounding of a few scores by one bf16 step, 2^-8 |s|, which moves that position's probability by
+    # percents; over half a million outputs the largest such move reaches 1.2e-2 of an output's own size.
+    say(f"mla decode at BASELINE size batch={batch} seq={seq}")
+    cfg = default_config()
+    H, KVA, R = cfg.heads, 576, 512
+    dc = DevBuf(batch * seq * KVA * 2)
+    for b in range(batch):
+        check(kxlib.kx_fill_normal_bf16(dc.ptr + b * seq * KVA * 2, seq * KVA, 77, b, 1.0, 0, None))
+    qabs = O.bf16_to_f32(O.normal_bf16(batch * H * KVA, 77, 1000, 0.5)).reshape(batch, H, KVA)
+    nbytes = C.c_size_t()
+    check(kxlib.kx_mla_workspace_bytes(C.byref(cfg), batch, seq, C.byref(nbytes)))
+    dq, dw, do = dev(qabs), DevBuf(nbytes.value), DevBuf(batch * H * R * 2)
+    outs = {}
+    for kernel in (2, 1, 0):
+        check(kxlib.kx_dev_memset(do.ptr, 0xFF, batch * H * R * 2, None))
+        check(kxlib.kx_mla_decode(C.byref(cfg), dc.ptr, seq * KVA, dq.ptr, dw.ptr, do.ptr, batch, seq, kernel, None))
+        check(kxlib.kx_sync(None))
+        outs[kernel] = do.to_numpy(np.uint16, (batch, H, R))
+    assert (outs[0] == outs[2]).all()          # these sizes take the matrix-core kernel by default
+    f2, f1 = O.bf16_to_f32(outs[2]), O.bf16_to_f32(outs[1])
+    assert np.isfinite(f2).all() and np.isfinite(f1).all()
+    e_k, e_k_el = O.max_rel(f2, f1), O.elem_err(f2, f1)
+    cfg8 = default_config()
+    cfg8.heads = 8
+    for b in sorted({0, batch - 1}):
+        cache = O.normal_bf16(seq * KVA, 77, b, 1.0).reshape(1, seq, KVA)
+        cf = O.bf16_to_f32(cache[0, :, :R])
+        lo, hi = cf.min(axis=0), cf.max(axis=0)
+        for f in (f2, f1):
+            assert (f[b] >= lo - 1e-6).all() and (f[b] <= hi + 1e-6).all(), "an output lies outside the range of its cache column"
+        for h0 in (0, 40):
+            q8 = np.ascontiguousarray(qabs[b:b + 1, h0:h0 + 8])
+            exp1, exp0 = np.empty((1, 8, R), dtype=np.uint16), np.empty((1, 8, R), dtype=np.uint16)
+            ox.ox_mla_decode(C.byref(cfg8), ptr(cache), seq * KVA, ptr(q8), ptr(exp1), 1, seq, 1)
+            ox.ox_mla_decode(C.byref(cfg8), ptr(cache), seq * KVA, ptr(q8), ptr(exp0), 1, seq, 0)
+            assert (outs[1][b, h0:h0 + 8] == exp1[0]).all(), f"VALU kernel differs from the kx schedule (sequence {b}, heads {h0}..)"
+            g = f2[b, h0:h0 + 8]
+            e1 = (O.max_rel(g, O.bf16_to_f32(exp1[0])), O.elem_err(g, O.bf16_to_f32(exp1[0])))
+            e0 = (O.max_rel(g, O.bf16_to_f32(exp0[0])), O.elem_err(g, O.bf16_to_f32(exp0[0])))
+            print(f"sequence {b} heads {h0}-{h0 + 7}: matrix-core kernel vs kx schedule max-rel {e1[0]:.2e} elem {e1[1]:.2e}, "
+                  f"vs reference schedule max-rel {e0[0]:.2e} elem {e0[1]:.2e}", flush=True)
+            assert max(e1[0], e0[0]) < 1e-2 and max(e1[1], e0[1]) < 2e-2
+    print(f"matrix-core vs VALU kernel, all {batch} x 64 heads: max-rel {e_k:.2e}, element-wise {e_k_el:.2e}", flush=True)
+    assert e_k < 1e-2 and e_k_el < 2e-2
+
+
+def test_config5_full_stack_batch_invariance_and_prefix(kxlib, ox):
+    # BASELINE config 5 at full size: 24 layers (231 GB resident), 1024-token uniform-random prompts, 256 greedy tokens.
+    # The scalar oracle cannot walk 24 layers x 1280 positions (the oracle comparisons run on the truncated stacks
+    # above); what holds at any size is checked here: three different sequences decoded together come out, each of
+    # them, exactly as that sequence decoded alone -- ids, final hidden state and logits to the bit -- (the batch-1
+    # run is the driver-timed benchmark path), a rerun reproduces itself, ids stay inside the vocabulary and a shorter
+    # generation is a prefix of the longer one.
+    say("config 5: 24 layers, prompt 1024, 256 tokens, batch 3 against batch 1")
+    cfg = default_config()
+    plen, n_tokens = 1024, 256
+    cfg.max_batch, cfg.max_context, cfg.seed = 3, plen + n_tokens, 0
+    assert cfg.n_layers == 24 and cfg.first_dense == 1 and cfg.vocab == 163840
+    prompt = O.tokens_u32(3 * plen, cfg.seed, 4, cfg.vocab).reshape(3, plen)
+    km = KxModel(kxlib, cfg)
+    rc, out3, counts = km.generate(prompt, n_tokens)
+    assert rc == 0, kxlib.kx_last_error()
+    assert (counts == n_tokens).all() and (out3 < cfg.vocab).all()
+    h3, l3 = km.hidden(3), km.logits(3).view(np.uint32)
+    print(f"batch 3 decoded; first ids {out3[:, :6].tolist()}", flush=True)
+    for b in (1, 2):
+        rc, out1, _ = km.generate(prompt[b:b + 1], n_tokens)
+        assert rc == 0, kxlib.kx_last_error()
+        same = int(np.argmax(np.append(out1[0] != out3[b], True)))
+        assert (out1[0] == out3[b]).all(), f"sequence {b}: ids differ from position {same} on"
+        assert (km.hidden(1)[0] == h3[b]).all() and (km.logits(1).view(np.uint32)[0] == l3[b]).all()
+    rc, short, _ = km.generate(prompt[2:3], 40)
+    assert rc == 0 and (short[0] == out3[2, :40]).all()
+    km.close()
 
 
 def test_kimi_shape_long_context_stack_attention_paths(kxlib, ox):
@@ -353,16 +446,13 @@ def test_kimi_shape_long_context_stack_attention_paths(kxlib, ox):
     cfg.n_layers, cfg.first_dense, cfg.max_batch, cfg.max_context, cfg.seed = 2, 1, 1, 4300, 3
     prompt = O.tokens_u32(4200, cfg.seed, 4, cfg.vocab).reshape(1, 4200)
     got = {}
-    try:
-        for mode in (0, 1):
-            check(kxlib.kx_mla_set_kernel(mode))
-            km = KxModel(kxlib, cfg)
-            rc, out, _ = km.generate(prompt, 1)
-            assert rc == 0, kxlib.kx_last_error()
-            got[mode] = (out.copy(), km.logits(1))
-            km.close()
-    finally:
-        check(kxlib.kx_mla_set_kernel(0))
+    for mode in (0, 1):
+        km = KxModel(kxlib, cfg)
+        check(kxlib.kx_model_set_attention_kernel(km.h, mode))
+        rc, out, _ = km.generate(prompt, 1)
+        assert rc == 0, kxlib.kx_last_error()
+        got[mode] = (out.copy(), km.logits(1))
+        km.close()
     err = O.max_rel(got[0][1], got[1][1])
     print(f"long-context stack, matrix-core vs VALU attention: logits max-rel {err:.3e}", flush=True)
     assert err < 3e-2 and (got[0][0] == got[1][0]).all()
@@ -370,28 +460,28 @@ def test_kimi_shape_long_context_stack_attention_paths(kxlib, ox):
 
 def test_kimi_shape_batched_stack_attention_paths(kxlib, ox):
     # five sequences and more take the matrix-core attention kernel from 128 cached positions on (their projections run
-    # on the matrix cores as well).  Held against the same stack with the VALU attention kernel forced: logits of the
-    # first sampled step within the stack-level 3e-2, the same first id for at least three quarters of the sequences.
+    # on the matrix cores as well).  Held against the same stack with the VALU attention kernel forced, sequence by
+    # sequence: logits of the first sampled step within the stack-level 3e-2 and the same first id, unless the
+    # sequence sits on a router or argmax near-tie, which is then named.
     say("kimi shape 2-layer stack, batch 8, 160-token prompts, attention paths")
     cfg = default_config()
     batch, plen = 8, 160
     cfg.n_layers, cfg.first_dense, cfg.max_batch, cfg.max_context, cfg.seed = 2, 1, batch, 192, 5
     prompt = O.tokens_u32(batch * plen, cfg.seed, 4, cfg.vocab).reshape(batch, plen)
     got = {}
-    try:
-        for mode in (0, 1):
-            check(kxlib.kx_mla_set_kernel(mode))
-            km = KxModel(kxlib, cfg)
-            rc, out, _ = km.generate(prompt, 1)
-            assert rc == 0, kxlib.kx_last_error()
-            got[mode] = (out.copy(), km.logits(batch))
-            km.close()
-    finally:
-        check(kxlib.kx_mla_set_kernel(0))
-    err = O.max_rel(got[0][1], got[1][1])
-    agree = float(np.mean(got[0][0] == got[1][0]))
-    print(f"batch-8 stack, matrix-core vs VALU attention: logits max-rel {err:.3e}, first ids equal for {agree:.0%}", flush=True)
-    assert err < 3e-2 and agree >= 0.75
+    for mode in (0, 1):
+        km = KxModel(kxlib, cfg)
+        check(kxlib.kx_model_set_attention_kernel(km.h, mode))
+        check(kxlib.kx_model_set_routing_record(km.h, 1))
+        rc, out, _ = km.generate(prompt, 1)
+        assert rc == 0, kxlib.kx_last_error()
+        got[mode] = (out.copy(), km.logits(batch), routing_of(kxlib, km.h, cfg, batch))
+        km.close()
+    errs = [O.max_rel(got[0][1][b], got[1][1][b]) for b in range(batch)]
+    excused = judge_sequences([f"sequence {b}" for b in range(batch)], errs, 3e-2, got[0][2], got[1][2], got[0][0][:, 0],
+                              got[1][0][:, 0], got[1][1])
+    print(f"batch-8 stack, matrix-core vs VALU attention: worst logits max-rel {max(errs):.3e}; excused: {excused or 'none'}", flush=True)
+    assert len(excused) <= 2
 
 
 @pytest.mark.parametrize("shape,batch,prompt_len,chunk", [
@@ -466,35 +556,43 @@ def test_prefill_chunk_errors(kxlib):
     km.close()
 
 
-def test_kimi_shape_batch16_against_single_sequences(kxlib, ox):
-    # 16 sequences: projections, shared expert and (from 16 tokens on) the routed experts run on the matrix cores.
-    # Sequences do not interact, so each must come out as it does alone at batch 1 (the bit-exact path), within the
-    # stack-level tolerance: logits of the first sampled step within 3e-2 for at least three of the four sequences
-    # checked (a router near-tie can move one to another expert), last-layer cache rows within 2e-2.
-    say("kimi shape 2-layer stack, batch 16 against the same sequences alone")
+@pytest.mark.parametrize("batch", [16, 32])
+def test_kimi_shape_batched_stack_against_single_sequences(kxlib, ox, batch):
+    # BASELINE config 5's batch 32 (and 16) at Kimi shapes, 2 layers: projections, shared expert, attention (from 128
+    # positions) and the routed experts with several pairs run on the matrix cores.  Sequences do not interact, so each
+    # must come out as it does alone at batch 1 -- the bit-exact path that the tests above hold to the oracle -- within
+    # the stack-level tolerance: last-layer cache rows within 2e-2, logits of the first sampled step within 3e-2 and
+    # the same first id.  Every sequence is checked; one that sits on a router near-tie of the batch-1 run (another
+    # expert is then legitimately picked) or an argmax near-tie is excused by name.
+    say(f"kimi shape 2-layer stack, batch {batch} against the same sequences alone")
     cfg = default_config()
-    batch, plen = 16, 24
+    plen = 140
     cfg.n_layers, cfg.first_dense, cfg.max_batch, cfg.max_context, cfg.seed = 2, 1, batch, plen + 4, 11
     prompt = O.tokens_u32(batch * plen, cfg.seed, 4, cfg.vocab).reshape(batch, plen)
     km = KxModel(kxlib, cfg)
+    check(kxlib.kx_model_set_routing_record(km.h, 1))
     rc, out, _ = km.generate(prompt, 1)
     assert rc == 0, kxlib.kx_last_error()
-    logits = km.logits(batch)
-    rows = {b: O.bf16_to_f32(km.latent(1, b, plen)) for b in (0, 5, 10, 15)}
-    km.close()
-    cfg.max_batch = 1
-    ok = 0
-    for b in (0, 5, 10, 15):
-        k1 = KxModel(kxlib, cfg)
-        rc, o1, _ = k1.generate(prompt[b:b + 1], 1)
+    logits, routes = km.logits(batch), routing_of(kxlib, km.h, cfg, batch)
+    rows = [O.bf16_to_f32(km.latent(1, b, plen)) for b in range(batch)]
+    ref_routes = {l: ([], []) for l in routes}
+    ref_logits, ref_ids, errs = [], [], []
+    for b in range(batch):
+        rc, o1, _ = km.generate(prompt[b:b + 1], 1)      # the same model, one sequence: GEMV kernels, VALU attention
         assert rc == 0, kxlib.kx_last_error()
-        e_log = O.max_rel(logits[b], k1.logits(1)[0])
-        e_rows = O.max_rel(rows[b], O.bf16_to_f32(k1.latent(1, 0, plen)))
-        print(f"sequence {b}: logits max-rel {e_log:.3e}, cache rows max-rel {e_rows:.3e}, id {out[b, 0]} / {o1[0, 0]}", flush=True)
-        assert e_rows < 2e-2
-        ok += e_log < 3e-2
-        k1.close()
-    assert ok >= 3
+        for l, (sets, gaps) in routing_of(kxlib, km.h, cfg, 1).items():
+            ref_routes[l][0].extend(sets)
+            ref_routes[l][1].extend(gaps.tolist())
+        ref_logits.append(km.logits(1)[0])
+        ref_ids.append(int(o1[0, 0]))
+        errs.append(O.max_rel(logits[b], ref_logits[-1]))
+        e_rows = O.max_rel(rows[b], O.bf16_to_f32(km.latent(1, 0, plen)))
+        assert e_rows < 2e-2, f"sequence {b}: cache rows max-rel {e_rows:.3e}"
+    km.close()
+    excused = judge_sequences([f"sequence {b}" for b in range(batch)], errs, 3e-2, routes, ref_routes, out[:, 0], ref_ids,
+                              np.stack(ref_logits))
+    print(f"batch {batch}: logits max-rel per sequence: median {np.median(errs):.2e}, worst {max(errs):.2e}; excused: {excused or 'none'}", flush=True)
+    assert len(excused) <= batch // 4
 
 
 def test_executor_json_line(kxlib):

@@ -85,7 +85,9 @@ def test_bucket_bit_exact(kxlib, ox, T, E, topk):
     assert (work[na:] == np.array([-1, 0, 0, 0])).all()
 
 
-def _run_layer(kxlib, ox, H, I, SI, E, K, T, seed, flags=0, gpu_flags=0):
+def _run_layer(kxlib, ox, H, I, SI, E, K, T, seed, flags=0, gpu_flags=0, mode0_tokens=None):
+    """One layer on the GPU and through both oracle schedules.  mode0_tokens: run the (slower) reference schedule on
+    these token rows only (tokens do not interact); its tensors then hold those rows."""
     host, n, x = moe_case(kxlib, H, I, SI, E, K, T, seed)
     cfg = moe_cfg(H, I, SI, E, K)
     w, bufs = moe_device_weights(host)
@@ -110,14 +112,16 @@ def _run_layer(kxlib, ox, H, I, SI, E, K, T, seed, flags=0, gpu_flags=0):
     check(kxlib.kx_moe_workspace_destroy(ws))
     exp = {}
     for mode in (1, 0):
-        xo = x.copy()
-        o = {"logits": np.empty((T, E), np.float32), "ids": np.empty((T, K), np.uint16),
-             "weights": np.empty((T, K), np.float32), "mid": np.empty((T * K, I), np.uint16),
-             "eout": np.empty((T * K, H), np.uint16)}
+        rows = np.arange(T) if (mode == 1 or mode0_tokens is None) else np.asarray(mode0_tokens)
+        Tm = len(rows)
+        xo, nm = np.ascontiguousarray(x[rows]), np.ascontiguousarray(n[rows])
+        o = {"logits": np.empty((Tm, E), np.float32), "ids": np.empty((Tm, K), np.uint16),
+             "weights": np.empty((Tm, K), np.float32), "mid": np.empty((Tm * K, I), np.uint16),
+             "eout": np.empty((Tm * K, H), np.uint16)}
         wo = moe_oracle_weights(host)
-        ox.ox_moe_layer(C.byref(wo), ptr(n), ptr(xo), T, H, I, SI, E, K, 2.827, flags, mode,
+        ox.ox_moe_layer(C.byref(wo), ptr(nm), ptr(xo), Tm, H, I, SI, E, K, 2.827, flags, mode,
                         ptr(o["logits"]), ptr(o["ids"]), ptr(o["weights"]), ptr(o["mid"]), ptr(o["eout"]))
-        o["x"] = xo
+        o["x"], o["rows"] = xo, rows
         exp[mode] = o
     return got, exp
 
@@ -130,9 +134,18 @@ def _assert_layer(got, exp):
     assert (got["mid"] == e1["mid"]).all(), f"{np.count_nonzero(got['mid'] != e1['mid'])} mid values differ"
     assert (got["eout"] == e1["eout"]).all()
     assert (got["x"] == e1["x"]).all()
-    if (e0["ids"] == e1["ids"]).all():   # same experts under both schedules: compare values
-        assert O.max_rel(O.bf16_to_f32(got["x"]), O.bf16_to_f32(e0["x"])) < 1e-2
-        assert O.max_rel(O.bf16_to_f32(got["mid"]), O.bf16_to_f32(e0["mid"])) < 1e-2
+    rows = e0["rows"]
+    K, I = got["ids"].shape[1], got["mid"].shape[1]
+    same = (e0["ids"] == e1["ids"][rows]).all(axis=1)   # tokens with the same experts under both schedules: compare values
+    assert same.mean() >= 0.9, f"only {same.mean():.0%} of the tokens route alike under the two oracle schedules"
+    gx, gm = O.bf16_to_f32(got["x"][rows][same]), O.bf16_to_f32(got["mid"].reshape(-1, K, I)[rows][same])
+    rx, rm = O.bf16_to_f32(e0["x"][same]), O.bf16_to_f32(e0["mid"].reshape(-1, K, I)[same])
+    errs = (O.max_rel(gx, rx), O.elem_err(gx, rx), O.max_rel(gm, rm), O.elem_err(gm, rm))
+    print("vs reference schedule: x max-rel %.2e elem %.2e, mid max-rel %.2e elem %.2e" % errs, flush=True)
+    # 1e-2 on the normalised maximum (the bar BASELINE states); the element-wise figure is held to 2e-2: one bf16
+    # step is up to 2^-7 of a value's own size, and mid = bf(bf(silu(g)) * u) passes three roundings whose boundary
+    # cases fall differently under another summation order
+    assert max(errs[0], errs[2]) < 1e-2 and max(errs[1], errs[3]) < 2e-2
 
 
 @pytest.mark.parametrize("T", [1, 8, 64])
@@ -147,12 +160,64 @@ def test_moe_layer_flags_write_down_only(kxlib, ox):
     _assert_layer(got, exp)
 
 
-@pytest.mark.parametrize("T", [1, 8])
+@pytest.mark.parametrize("T", [1, 8, 64])
 def test_moe_layer_kimi_shape(kxlib, ox, T):
-    # BASELINE config 2: hidden 7168, 384 experts top-8, moe_inter 2048, shared 2048
+    # BASELINE config 2: hidden 7168, 384 experts top-8, moe_inter 2048, shared 2048.  T = 64 (512 pairs on 384
+    # experts) takes the two-launch plan: experts with one pair through the one-token kernel, the others two tokens
+    # per pass.  Every tensor to the bit against the kx schedule for all tokens; the reference schedule (about four
+    # times the CPU time) on eight of the 64 tokens.
     say(f"moe layer kimi shape T={T}")
-    got, exp = _run_layer(kxlib, ox, 7168, 2048, 2048, 384, 8, T, 9)
+    got, exp = _run_layer(kxlib, ox, 7168, 2048, 2048, 384, 8, T, 9, mode0_tokens=None if T <= 8 else range(3, 64, 8))
     _assert_layer(got, exp)
+
+
+@pytest.mark.parametrize("T,bits", [(16, 0x600), (32, 0x600), (32, 0x200), (32, 0x400), (7, 0x600)])
+def test_moe_layer_kimi_shape_matrix_core_forms(kxlib, ox, T, bits):
+    # What the stack runs from 5 (bit 9: shared expert as bf16 matrix-core products) and 12 sequences on (bit 10:
+    # routed experts with several pairs as W4A16 grouped GEMMs, the others through the one-token GEMV kernel), reached
+    # through the C ABI.  The layer output `down` (flag bit 0: no residual, so the bar is on the layer's own result):
+    # within 1e-2 as normalised maximum (2e-2 element-wise: see _assert_layer) of the default GEMV form for every token, and of the
+    # oracle's reference schedule given the GPU's routing on a sample of tokens; the routing itself must be the
+    # default's to the bit (neither bit touches the router).
+    say(f"moe layer kimi shape T={T} flags={bits:#x}")
+    H, I, SI, E, K = 7168, 2048, 2048, 384, 8
+    host, n, x = moe_case(kxlib, H, I, SI, E, K, T, 9)
+    cfg = moe_cfg(H, I, SI, E, K)
+    w, bufs = moe_device_weights(host)
+    ws = C.c_void_p()
+    check(kxlib.kx_moe_workspace_create(C.byref(cfg), T, C.byref(ws)))
+    dn = dev(n)
+    res = {}
+    for flags in (1, 1 | bits):
+        dx = dev(x)
+        check(kxlib.kx_moe_decode_layer(C.byref(cfg), C.byref(w), ws, dn.ptr, dx.ptr, T, flags, None))
+        check(kxlib.kx_sync(None))
+        views = [C.c_void_p() for _ in range(8)]
+        check(kxlib.kx_moe_workspace_views(ws, *[C.byref(v) for v in views]))
+        tmp = DevBuf.__new__(DevBuf)
+        tmp.ptr, tmp.nbytes = views[1].value, T * K * 2
+        ids = tmp.to_numpy(np.uint16, (T, K))
+        tmp.ptr, tmp.nbytes = views[2].value, T * K * 4
+        wts = tmp.to_numpy(np.float32, (T, K))
+        tmp.ptr = None
+        res[flags] = (O.bf16_to_f32(dx.to_numpy(np.uint16, (T, H))), ids, wts)
+    check(kxlib.kx_moe_workspace_destroy(ws))
+    (d0, ids0, w0), (d1, ids1, w1) = res[1], res[1 | bits]
+    assert (ids0 == ids1).all() and (w0.view(np.uint32) == w1.view(np.uint32)).all()
+    pairs = np.bincount(ids0.ravel(), minlength=E)
+    e_max, e_el = O.max_rel(d1, d0), O.elem_err(d1, d0)
+    print(f"{(pairs > 0).sum()} experts, {(pairs > 1).sum()} with several pairs (most: {pairs.max()}); "
+          f"vs the GEMV form: max-rel {e_max:.2e}, element-wise {e_el:.2e}", flush=True)
+    assert e_max < 1e-2 and e_el < 2e-2
+    rows = np.arange(T)[:: max(1, T // 6)]
+    xo, no = np.ascontiguousarray(x[rows]), np.ascontiguousarray(n[rows])
+    io, wr = np.ascontiguousarray(ids1[rows]), np.ascontiguousarray(w1[rows])
+    wo = moe_oracle_weights(host)
+    ox.ox_moe_layer_routed(C.byref(wo), ptr(no), ptr(xo), len(rows), H, I, SI, E, K, 1, 0, ptr(io), ptr(wr))
+    ref = O.bf16_to_f32(xo)
+    r_max, r_el = O.max_rel(d1[rows], ref), O.elem_err(d1[rows], ref)
+    print(f"vs the reference schedule on tokens {rows.tolist()}: max-rel {r_max:.2e}, element-wise {r_el:.2e}", flush=True)
+    assert r_max < 1e-2 and r_el < 2e-2
 
 
 @pytest.mark.parametrize("flags,gpu_flags", [(0, 0x100), (1, 0), (1, 0x100)])
