@@ -13,6 +13,7 @@
 //   lane partial  p[s][l] = fma chain over e = 0..7 of w[r, 512 s + 8 l + e] * x[t, ...]
 //   slice sum     B[s]    = xor-butterfly over the 64 lanes (32,16,8,4,2,1)
 //   row sum       y       = B[0] + B[1] + ... + B[S-1], left to right
+#include <mutex>
 #include "kx_attn_parts.h"
 #include "kx_common.h"
 #include "kx_dense.h"
@@ -425,6 +426,51 @@ extern "C" int kx_lm_head_argmax(const void *d_w, const void *d_n, void *d_logit
   int rc = kx_gemv_launch(KX_EPI_ARGMAX, a, kx_stream(stream));
   if (rc) return rc;
   return kx_argmax_launch((const float *)d_logits, tokens, vocab, vocab, (uint32_t *)d_ids, (float *)d_scratch, kx_stream(stream));
+}
+
+// ---- the same operator for callers that may not allocate ---------------------------------------
+// The per-token argmax partials (ARGMAX_PARTS values and indices per token) live in a file-scope device
+// array instead of a caller's buffer.  Every GPU holds its own copy of the array at its own address, so
+// the address is looked up once per device, with that device current, and kept.
+constexpr int KX_STATIC_ARGMAX_TOKENS = 256;
+constexpr int KX_STATIC_MAX_DEVICES = 64;
+static __device__ __align__(256) unsigned char g_argmax_scratch[KX_STATIC_ARGMAX_TOKENS * ARGMAX_PARTS * 8];
+static std::mutex g_argmax_scratch_mu;
+static void *g_argmax_scratch_ptr[KX_STATIC_MAX_DEVICES];
+
+static int argmax_scratch_for_current_device(void **out) {
+  int dev = -1;
+  KX_HIP(hipGetDevice(&dev));
+  KX_REQUIRE(dev >= 0 && dev < KX_STATIC_MAX_DEVICES, "kx_lm_head_argmax_static: device %d is beyond the %d this library keeps an address for",
+             dev, KX_STATIC_MAX_DEVICES);
+  std::lock_guard<std::mutex> lock(g_argmax_scratch_mu);
+  if (!g_argmax_scratch_ptr[dev]) {
+    void *p = nullptr;
+    KX_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(g_argmax_scratch)));
+    KX_REQUIRE(p != nullptr, "kx_lm_head_argmax_static: hipGetSymbolAddress gave no address on device %d", dev);
+    g_argmax_scratch_ptr[dev] = p;
+  }
+  *out = g_argmax_scratch_ptr[dev];
+  return KX_OK;
+}
+
+extern "C" int kx_static_scratch_init(void) {
+  void *p = nullptr;
+  return argmax_scratch_for_current_device(&p);
+}
+
+extern "C" int kx_lm_head_argmax_static(const void *d_w, const void *d_n, void *d_logits, void *d_ids, int32_t vocab,
+                                        int32_t hidden, int32_t tokens, void *stream) {
+  KX_REQUIRE(d_w && d_n && d_logits && d_ids, "kx_lm_head_argmax_static: null pointer");
+  KX_REQUIRE(vocab > 0 && tokens > 0, "kx_lm_head_argmax_static: vocab=%d tokens=%d must be positive", vocab, tokens);
+  KX_REQUIRE(tokens <= KX_STATIC_ARGMAX_TOKENS,
+             "kx_lm_head_argmax_static: tokens=%d is more than the %d rows the built-in scratch holds; use kx_lm_head_argmax with a buffer of your own",
+             tokens, KX_STATIC_ARGMAX_TOKENS);
+  void *scratch = nullptr;
+  int rc = argmax_scratch_for_current_device(&scratch);
+  if (rc) return rc;
+  // every partial of rows [0, tokens) is written by the first argmax kernel before the second reads it: nothing to clear
+  return kx_lm_head_argmax(d_w, d_n, d_logits, d_ids, vocab, hidden, tokens, scratch, stream);
 }
 
 extern "C" int kx_gemv_bf16(const void *d_w, const void *d_x, void *d_y, int32_t rows, int32_t cols,

@@ -63,6 +63,8 @@ _SIGS = {
     "kx_rmsnorm": [_P, _P, _P, _I, _I, _F, _P],
     "kx_gemv_bf16": [_P, _P, _P, _I, _I, _I, C.c_int, _P],
     "kx_lm_head_argmax": [_P, _P, _P, _P, _I, _I, _I, _P, _P],
+    "kx_static_scratch_init": [],
+    "kx_lm_head_argmax_static": [_P, _P, _P, _P, _I, _I, _I, _P],
     "kx_router_topk": [_P, _P, _P, _P, _I, _I, _I, _F, _P],
     "kx_bucket": [_P, _I, _I, _I, _P, _P, _P, _P, _P, _P],
     "kx_moe_workspace_create": [C.POINTER(KxConfig), _I, _PP],

@@ -122,6 +122,19 @@ int kx_gemv_bf16(const void *d_w, const void *d_x, void *d_y, int32_t rows, int3
 int kx_lm_head_argmax(const void *d_w, const void *d_n, void *d_logits, void *d_ids, int32_t vocab,
                       int32_t hidden, int32_t tokens, void *d_scratch, void *stream);
 
+/* kx_lm_head_argmax for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same operands and
+ * results as kx_lm_head_argmax, without d_scratch: the argmax partials go to a device array that is part of
+ * the library (128 KiB, held by every GPU the library runs on until the process ends), so tokens <= 256; more
+ * is an error.  The call allocates nothing and frees nothing.  Every call on a GPU shares that GPU's array:
+ * calls that overlap on one GPU (two streams, two threads) race; calls on one stream do not.  Nothing in the
+ * array has to be cleared between calls.  The array's address on a GPU is looked up on the first call there;
+ * kx_static_scratch_init() does that look-up for the current device ahead of time (call it before a graph
+ * capture begins).                                                                                        */
+int kx_static_scratch_init(void);
+int kx_lm_head_argmax_static(const void *d_w, const void *d_n, void *d_logits, void *d_ids, int32_t vocab,
+                             int32_t hidden, int32_t tokens, void *stream);
+
 /* ---- router --------------------------------------------------------------
  * kx_router_topk: sigmoid_k + add_bf16_k + router_topk_k (:372-397) on fp32
  *                 logits [T, E]: ids u16 [T, topk] in descending select
