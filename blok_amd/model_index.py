@@ -111,29 +111,42 @@ def index_lines(rows, align=ALIGN):
 TOKENIZER_HEADER = "blok-tokenizer-v2"
 
 
-def tokenizer(local_dir, n_tokens=163584, n_special=256):
-    """Text of tokenizer.blok from the checkpoint's tiktoken.model (`<base64 bytes> <rank>` per line) and the
-    added_tokens_decoder of tokenizer_config.json (:81-97).  Ranks must be exactly 0..n_tokens-1 and the special
-    ids the n_special that follow (Kimi-K2: 163584 + 256 = the 163840-row embedding); None skips that check."""
-    root = Path(local_dir)
-    vocab_file, config_file = root / "tiktoken.model", root / "tokenizer_config.json"
-    if not vocab_file.is_file() or not config_file.is_file():
-        raise SystemExit("pinned checkpoint requires tiktoken.model and tokenizer_config.json")
-    ranks = {}
-    for line in vocab_file.read_bytes().splitlines():
-        if not line.strip():
+def _tiktoken_ranks(path):
+    """{rank: bytes} of a tiktoken.model file: one `<base64 of the byte string> <rank>` per non-empty line."""
+    table = {}
+    for number, raw in enumerate(path.read_bytes().split(b"\n"), 1):
+        fields = raw.split()
+        if not fields:
             continue
-        encoded, rank = line.split()
-        ranks[int(rank)] = base64.b64decode(encoded)
-    added = json.loads(config_file.read_text()).get("added_tokens_decoder", {})
-    special = {int(i): meta["content"].encode() for i, meta in added.items()}
+        if len(fields) != 2:
+            raise SystemExit(f"{path.name}:{number}: expected '<base64> <rank>'")
+        table[int(fields[1])] = base64.b64decode(fields[0])
+    return table
+
+
+def _special_tokens(path):
+    """{id: utf-8 bytes} from the added_tokens_decoder map of tokenizer_config.json."""
+    decoder = json.loads(path.read_text()).get("added_tokens_decoder") or {}
+    return {int(token_id): entry["content"].encode() for token_id, entry in decoder.items()}
+
+
+def tokenizer(local_dir, n_tokens=163584, n_special=256):
+    """Text of tokenizer.blok (scripts/model_fetch.py:81-97 writes the same file): the header, `tok <id> <hex>` for every
+    mergeable byte string in rank order, `special <id> <hex>` for every added token in id order.  The ranks must be
+    exactly 0..n_tokens-1 and the special ids the n_special that follow (Kimi-K2: 163584 + 256 = the 163840-row
+    embedding); n_tokens=None skips that check."""
+    sources = [Path(local_dir) / name for name in ("tiktoken.model", "tokenizer_config.json")]
+    if not all(p.is_file() for p in sources):
+        raise SystemExit("pinned checkpoint requires tiktoken.model and tokenizer_config.json")
+    sections = (("tok", _tiktoken_ranks(sources[0])), ("special", _special_tokens(sources[1])))
     if n_tokens is not None:
-        if sorted(ranks) != list(range(n_tokens)) or sorted(special) != list(range(n_tokens, n_tokens + n_special)):
+        expected = (range(n_tokens), range(n_tokens, n_tokens + n_special))
+        if any(sorted(table) != list(ids) for (_, table), ids in zip(sections, expected)):
             raise SystemExit("unexpected Kimi tokenizer rank contract")
-    rows = [TOKENIZER_HEADER]
-    rows += [f"tok {i} {ranks[i].hex()}" for i in sorted(ranks)]
-    rows += [f"special {i} {special[i].hex()}" for i in sorted(special)]
-    return "\n".join(rows) + "\n"
+    out = [TOKENIZER_HEADER]
+    for tag, table in sections:
+        out.extend(f"{tag} {token_id} {table[token_id].hex()}" for token_id in sorted(table))
+    return "\n".join(out) + "\n"
 
 
 def materialize(local_dir, meta_dir, tokenizer_ranks=(163584, 256)):

@@ -95,63 +95,92 @@ def encode_prompt(tokenizer, prompt, encoding=None):
     return encoding.encode(CHAT_HEAD + prompt + CHAT_TAIL, allowed_special="all")  # any object with tiktoken's interface
 
 
+PLACEHOLDER_MODELS = ("<kimi k2 model directory", "<kimi k2 model directory>")
+INDEX_NAME = "runtime-index.blok"
+
+
+def _check_kimi_config(directory):
+    """A checkpoint directory's config.json, when there is one, must describe Kimi-K2 (KIMI_TEXT)."""
+    config = directory / "config.json"
+    if not config.is_file():
+        return
+    fields = json.loads(config.read_text())
+    fields = fields.get("text_config", fields)
+    wrong = [name for name in KIMI_TEXT if fields.get(name) != KIMI_TEXT[name]]
+    if wrong:
+        raise BlokRuntimeError("unsupported Kimi config fields: " + ", ".join(wrong))
+
+
+def default_index():
+    """Where the index of the pinned model lives when no model argument names one: BLOK_META_ROOT, else
+    $BLOK_HOME/metadata, else ~/.blok/metadata."""
+    meta_root = os.getenv("BLOK_META_ROOT")
+    if meta_root is None:
+        meta_root = Path(os.getenv("BLOK_HOME", Path.home() / ".blok")) / "metadata"
+    return Path(meta_root) / "moonshotai/Kimi-K2.6" / INDEX_NAME
+
+
 def runtime_index(model):
-    """Path of runtime-index.blok for a model argument: the file, its directory, a checkpoint directory whose
-    config.json must describe Kimi-K2, or the default metadata directory (runtime.py:98-118)."""
-    value = str(model)
-    if value in ("<kimi k2 model directory", "<kimi k2 model directory>"):
-        value = os.getenv("BLOK_MODEL", "")
-    tried = []
-    if value:
-        base = Path(value).expanduser().resolve()
-        tried += [base, base / "runtime-index.blok"]
-        config = base / "config.json"
-        if config.is_file():
-            raw = json.loads(config.read_text())
-            text = raw.get("text_config", raw)
-            wrong = [k for k, v in KIMI_TEXT.items() if text.get(k) != v]
-            if wrong:
-                raise BlokRuntimeError("unsupported Kimi config fields: " + ", ".join(wrong))
-    home = Path(os.getenv("BLOK_HOME", Path.home() / ".blok"))
-    tried.append(Path(os.getenv("BLOK_META_ROOT", home / "metadata")) / "moonshotai/Kimi-K2.6/runtime-index.blok")
-    for path in tried:
-        if path.name == "runtime-index.blok" and path.is_file():
-            return path
-    raise BlokRuntimeError("runtime-index.blok not found; run python -m blok_amd.model_index <checkpoint-dir> <metadata-dir>")
+    """Path of runtime-index.blok for a model argument (blok/runtime.py:98-118 resolves it the same way): the index
+    file itself, a directory holding it (a checkpoint directory's config.json must then describe Kimi-K2), the
+    BLOK_MODEL environment variable when the argument is the command line's placeholder, and last the default
+    metadata directory."""
+    named = os.getenv("BLOK_MODEL", "") if str(model) in PLACEHOLDER_MODELS else str(model)
+    places = []
+    if named:
+        base = Path(named).expanduser().resolve()
+        places = [base, base / INDEX_NAME]
+        _check_kimi_config(base)
+    places.append(default_index())
+    found = next((p for p in places if p.name == INDEX_NAME and p.is_file()), None)
+    if found is None:
+        raise BlokRuntimeError("runtime-index.blok not found; run python -m blok_amd.model_index <checkpoint-dir> <metadata-dir>")
+    return found
 
 
 def executor_path():
     return Path(os.getenv("BLOK_KIMI_EXEC_BIN", Path(__file__).parent / "kx-kimi-exec"))
 
 
+def _run_executor(argv, max_time):
+    """The executor's token ids: one JSON line on stdout, a non-zero exit code means failure with the reason on
+    stderr (src/kimi_exec.cu:495-498, :901-903)."""
+    try:
+        done = subprocess.run(argv, text=True, capture_output=True, timeout=max_time)
+    except subprocess.TimeoutExpired as error:
+        raise BlokRuntimeError(f"generation exceeded {max_time:g} seconds") from error
+    if done.returncode != 0:
+        raise BlokRuntimeError(done.stderr.strip() or done.stdout.strip())
+    try:
+        report = json.loads(done.stdout)
+    except json.JSONDecodeError as error:
+        raise BlokRuntimeError(f"executor returned invalid JSON: {done.stdout!r}") from error
+    ids = report.get("token_ids") if report.get("status") == "ok" else None
+    vocab = KIMI_TEXT["vocab_size"]
+    if not isinstance(ids, list) or any(type(i) is not int or not 0 <= i < vocab for i in ids):
+        raise BlokRuntimeError(f"executor failed: {report}")
+    return ids
+
+
 def generate(*, model_dir, prompt, max_tokens, max_time):
-    """Text generated for `prompt` by the executor (runtime.py:51-95): at most max_tokens ids, max_time seconds."""
+    """Text generated for `prompt` by the executor (blok/runtime.py:51-95): at most max_tokens ids, max_time seconds.
+    The executor computes with the reference's constants for a checkpoint (YaRN factor 64) and refuses a checkpoint
+    that does not fit one GPU; BLOK_KIMI_LAYERS=n runs the first n layers of it (a truncation: not the full model's
+    output)."""
     if not prompt or max_tokens <= 0 or max_time <= 0:
         raise BlokRuntimeError("prompt must be non-empty and limits must be positive")
     index = runtime_index(model_dir)
-    tokenizer = index.parent / "tokenizer.blok"
-    executor = executor_path()
-    missing = [str(p) for p in (index, tokenizer, executor) if not p.is_file()]
-    if missing:
-        raise BlokRuntimeError("missing required file(s): " + ", ".join(missing))
-    encoding = tokenizer_encoding(tokenizer)
-    ids = encode_prompt(tokenizer, prompt, encoding)
-    argv = [str(executor), "--index", str(index), "--prompt-tokens", ",".join(str(i) for i in ids), "--tokens", str(max_tokens)]
-    try:
-        result = subprocess.run(argv, text=True, capture_output=True, timeout=max_time)
-    except subprocess.TimeoutExpired as error:
-        raise BlokRuntimeError(f"generation exceeded {max_time:g} seconds") from error
-    if result.returncode:
-        raise BlokRuntimeError(result.stderr.strip() or result.stdout.strip())
-    try:
-        report = json.loads(result.stdout)
-    except json.JSONDecodeError as error:
-        raise BlokRuntimeError(f"executor returned invalid JSON: {result.stdout!r}") from error
-    out = report.get("token_ids")
-    good = report.get("status") == "ok" and isinstance(out, list) and all(type(i) is int and 0 <= i < KIMI_TEXT["vocab_size"] for i in out)
-    if not good:
-        raise BlokRuntimeError(f"executor failed: {report}")
-    return encoding.decode(out)
+    needed = {"index": index, "tokenizer": index.parent / "tokenizer.blok", "executor": executor_path()}
+    absent = [str(p) for p in needed.values() if not p.is_file()]
+    if absent:
+        raise BlokRuntimeError("missing required file(s): " + ", ".join(absent))
+    encoding = tokenizer_encoding(needed["tokenizer"])
+    ids = encode_prompt(needed["tokenizer"], prompt, encoding)
+    argv = [str(needed["executor"]), "--index", str(index), "--prompt-tokens", ",".join(map(str, ids)), "--tokens", str(max_tokens)]
+    layers = os.getenv("BLOK_KIMI_LAYERS")
+    if layers:
+        argv += ["--layers", layers]
+    return encoding.decode(_run_executor(argv, max_time))
 
 
 def answer(text):

@@ -2,6 +2,7 @@
 entry point include/kx.h declares; the executor keeps the reference's argv / JSON / exit-code contract
 (reference: src/kimi_exec.cu:532-557, :895-904; scripts/test_host.py:43-54 pins the same boundary)."""
 import ctypes as C
+import json
 import os
 import re
 import subprocess
@@ -28,6 +29,38 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), f"{name} is declared in include/kx.h but not exported by libkx.so"
     missing = [n for n in names if n not in _SIGS and n != "kx_last_error"]
     assert not missing, f"no ctypes signature for {missing}"
+
+
+def _print_config(*argv):
+    r = subprocess.run([EXEC, "--prompt-tokens", "1,2,3", "--tokens", "5", "--print-config", *argv], capture_output=True, text=True, timeout=60)
+    return r.returncode, (json.loads(r.stdout) if r.returncode == 0 else None), r.stderr
+
+
+def test_executor_config_for_a_checkpoint_is_the_reference_constants(tmp_path):
+    # src/kimi_exec.cu:176-186: with --index the executor must compute with the reference's constants, YARN_FACTOR 64
+    # (:184) among them; the seeded random-init run (the synthetic benchmark configurations) keeps factor 32.
+    # A checkpoint that does not fit one GPU is not truncated silently.
+    import test_index as TI
+    rc, doc, err = _print_config()
+    assert rc == 0 and doc["yarn_factor"] == 32.0 and doc["n_layers"] == 24 and doc["layers_in_checkpoint"] == 0
+    lines, _ = TI._kimi_index_lines()
+    index = tmp_path / "runtime-index.blok"
+    index.write_text("\n".join(lines) + "\n")
+    rc, doc, err = _print_config("--index", str(index))
+    assert rc == 1 and "61 layers" in err and "--layers" in err
+    rc, doc, err = _print_config("--index", str(index), "--layers", "24")
+    assert rc == 0, err
+    assert (doc["hidden"], doc["vocab"], doc["q_rank"], doc["kv_rank"], doc["heads"]) == (7168, 163840, 1536, 512, 64)   # :176-178
+    assert (doc["qk_nope"], doc["qk_rope"], doc["v_head"]) == (128, 64, 128)                                             # :178
+    assert (doc["experts"], doc["topk"], doc["moe_inter"], doc["dense_inter"]) == (384, 8, 2048, 18432)                  # :179
+    assert doc["first_dense"] == 1 and doc["n_layers"] == 24 and doc["layers_in_checkpoint"] == 61
+    assert abs(doc["rms_eps"] - 1e-5) < 1e-12 and doc["rope_theta"] == 50000.0 and abs(doc["routed_scale"] - 2.827) < 1e-6   # :181-183
+    assert (doc["yarn_factor"], doc["yarn_beta_fast"], doc["yarn_beta_slow"], doc["yarn_orig_ctx"]) == (64.0, 32.0, 1.0, 4096.0)  # :184-185
+    assert doc["eos_id"] == 163586                                                                                       # :186
+    rc, doc, err = _print_config("--index", str(index), "--layers", "24", "--yarn-factor", "32")
+    assert rc == 0 and doc["yarn_factor"] == 32.0
+    rc, doc, err = _print_config("--prefill-chunk", "4096")
+    assert rc == 1 and "prefill chunk" in err
 
 
 def test_config_default_is_kimi_k2():

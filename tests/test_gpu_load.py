@@ -116,6 +116,7 @@ def test_executor_reads_the_index(kxlib, ox, tmp_path):
     assert r.returncode == 0, r.stderr
     doc = json.loads(r.stdout)
     cfg.max_context = 9
+    cfg.yarn_factor = 64.0      # a checkpoint run uses the reference's YARN_FACTOR (src/kimi_exec.cu:184)
     om = _oracle_with(cfg, keyed)
     rc, out1, _ = om.generate(prompt, 4)
     assert doc["status"] == "ok" and doc["token_ids"] == [int(t) for t in out1[0]]
