@@ -33,5 +33,25 @@ void kx_set_error(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
 
 #define KX_LAUNCH_CHECK() KX_HIP(hipGetLastError())
 
+// No exception may cross the C ABI: the host-side entry points that parse files or grow containers run their
+// bodies under this guard (std::bad_alloc from a hostile size, std::out_of_range from a lookup).
+#ifdef __cplusplus
+#include <exception>
+#include <new>
+template <class F>
+static inline int kx_guard(const char *who, F &&body) {
+  try {
+    return body();
+  } catch (const std::bad_alloc &) {
+    kx_set_error("%s: out of memory", who);
+  } catch (const std::exception &e) {
+    kx_set_error("%s: %s", who, e.what());
+  } catch (...) {
+    kx_set_error("%s: unknown exception", who);
+  }
+  return KX_ERR_STATE;
+}
+#endif
+
 static inline hipStream_t kx_stream(void *s) { return (hipStream_t)s; }
 static inline int kx_cdiv(int a, int b) { return (a + b - 1) / b; }

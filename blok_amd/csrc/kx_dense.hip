@@ -14,6 +14,7 @@
 //   slice sum     B[s]    = xor-butterfly over the 64 lanes (32,16,8,4,2,1)
 //   row sum       y       = B[0] + B[1] + ... + B[S-1], left to right
 #include <mutex>
+#include "kx_arrive.h"
 #include "kx_attn_parts.h"
 #include "kx_common.h"
 #include "kx_dense.h"
@@ -113,18 +114,15 @@ __global__ void __launch_bounds__(TT > 1 ? 512 : 1024) gemv_pair_k(KxGemvArgs a0
   __shared__ int s_cnt[1024];
   __shared__ int s_act[1024];
   __shared__ uint4 s_ids4[4];
-  // The logits were stored through to memory (device-scope stores).  Every wave waits for its stores
-  // to be acknowledged; after the barrier one thread counts the workgroup in.  The workgroup that
-  // counts in last reads all logits with device-scope loads, so no cache has to be flushed.
-  __builtin_amdgcn_s_waitcnt(0);
+  // The logits were stored with device-scope stores; after the barrier one thread counts the workgroup in
+  // (release).  The workgroup that counts in last (acquire) reads all logits with device-scope loads.
   __syncthreads();
-  if (threadIdx.x == 0)
-    s_last = __hip_atomic_fetch_add(r.counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == n1 - 1;
+  if (threadIdx.x == 0) s_last = kx_arrive_is_last(r.counter, n1);
   __syncthreads();
   if (!s_last) return;
   kxr::route_block_any<true>((const float *)a1.out, r.bias, r.ids, r.weights, a1.tokens, r.experts, r.topk, r.routed_scale,
                        r.counts, r.offsets, r.pairs, r.work, r.n_active, s_ids4, s_cnt, s_act, r.pair_work);
-  if (threadIdx.x == 0) *r.counter = 0;
+  if (threadIdx.x == 0) kx_arrive_reset(r.counter);
 }
 
 // The q_b GEMV that also finishes the query.  Workgroup 0 norms kv_a, rotates the shared rope key and writes the
@@ -147,15 +145,13 @@ __global__ void __launch_bounds__(TT > 1 ? 512 : 1024) gemv_absorb_k(KxGemvArgs 
   }
   const int chunk = blockIdx.x - 1;
   gemv_body<1, RI, TT>(a, chunk, gridDim.x - 1, part);
-  __builtin_amdgcn_s_waitcnt(0);  // this wave's stores of q have been acknowledged
-  __syncthreads();
+  __syncthreads();  // every lane's stores of q lie before the counting lane's release (kx_arrive.h)
   const int h = chunk / q.head_chunks;
-  if (threadIdx.x == 0)
-    s_last = __hip_atomic_fetch_add(q.head_count + h, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == q.head_chunks - 1;
+  if (threadIdx.x == 0) s_last = kx_arrive_is_last(q.head_count + h, q.head_chunks);
   __syncthreads();
   if (!s_last) return;
   kxa::absorb_head_block(q, h, a.tokens, ab_part, ab_q);
-  if (threadIdx.x == 0) q.head_count[h] = 0;
+  if (threadIdx.x == 0) kx_arrive_reset(q.head_count + h);
 }
 
 // lowest-index argmax over bf16-rounded logits (sample_lm_head :718-734, argmax_k :477-493), in two

@@ -26,6 +26,7 @@
 //
 // All arithmetic is IEEE binary32 (fma, mul, add), so a scalar host program
 // that follows the same order reproduces the result bit for bit.
+#include "kx_arrive.h"
 #include "kx_common.h"
 #include "kx_dense.h"
 #include "kx_gemv_body.h"
@@ -167,15 +168,11 @@ __host__ __device__ constexpr int i4_chunk_rows(bool dual, int rt) { return dual
 __device__ __forceinline__ void moe_tail_arrive(const KxMoeTail &t, int blk_a, int blk_b, int block_rows, int rows,
                                                 const uint16_t *eout) {
   __shared__ int s_last[2];
-  __builtin_amdgcn_s_waitcnt(0);  // this wave's stores have been acknowledged
-  __syncthreads();
+  __syncthreads();  // every lane's outputs lie before the counting lanes' release (kx_arrive.h)
   if (threadIdx.x < 2) {
     const int blk = threadIdx.x ? blk_b : blk_a;
     int last = 0;
-    if (blk >= 0) {
-      const int target = *t.n_active + t.shared_chunks;
-      last = __hip_atomic_fetch_add(t.counter + blk, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == target - 1;
-    }
+    if (blk >= 0) last = kx_arrive_is_last(t.counter + blk, *t.n_active + t.shared_chunks);
     s_last[threadIdx.x] = last;
   }
   __syncthreads();
@@ -203,7 +200,7 @@ __device__ __forceinline__ void moe_tail_arrive(const KxMoeTail &t, int blk_a, i
       uint16_t *xr = t.x + (size_t)tok * t.x_stride + row;
       *xr = (t.flags & 1u) ? kx_bf16_rne(down) : kx_bf16_rne(kx_bf16_f32(*xr) + down);
     }
-    if (threadIdx.x == 0) t.counter[blk] = 0;
+    if (threadIdx.x == 0) kx_arrive_reset(t.counter + blk);
   }
 }
 

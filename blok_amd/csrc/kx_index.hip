@@ -142,6 +142,7 @@ int kx_index_contract(const KxIndex &ix, const kx_config *c, std::vector<KxNeed>
     const KxTensorRec &t = kv.second;
     KX_REQUIRE(!t.slot.empty() && !t.dtype.empty() && !t.shape.empty(), "runtime index has incomplete tensor metadata: %s", t.name.c_str());
     KX_REQUIRE(t.layer >= -1 && t.expert >= -1 && t.expert < c->experts, "runtime index has out-of-range Kimi coordinates: %s", t.name.c_str());
+    KX_REQUIRE(t.off <= UINT64_MAX - t.bytes && t.data <= UINT64_MAX - t.data_bytes, "runtime index has invalid tensor extent: %s", t.name.c_str());
     KX_REQUIRE(t.align == 4096 && t.off % t.align == 0 && t.bytes % t.align == 0 && t.data >= t.off &&
                    t.data_bytes <= t.bytes && t.data - t.off <= t.bytes - t.data_bytes,
                "runtime index has invalid tensor extent: %s", t.name.c_str());
@@ -188,7 +189,7 @@ int kx_index_contract(const KxIndex &ix, const kx_config *c, std::vector<KxNeed>
 }
 
 // ---- C ABI ---------------------------------------------------------------------------------
-extern "C" int kx_index_check(const kx_config *cfg, const char *index_path, uint64_t *n_tensors, uint64_t *weight_bytes) {
+static int kx_index_check_body(const kx_config *cfg, const char *index_path, uint64_t *n_tensors, uint64_t *weight_bytes) {
   KX_REQUIRE(cfg, "kx_index_check: null config");
   KxIndex ix;
   int rc = kx_index_parse(index_path, ix);
@@ -203,7 +204,7 @@ extern "C" int kx_index_check(const kx_config *cfg, const char *index_path, uint
 }
 
 // Shapes of the checkpoint an index describes, written over the matching fields of *cfg.
-extern "C" int kx_index_infer_config(const char *index_path, kx_config *cfg) {
+static int kx_index_infer_config_body(const char *index_path, kx_config *cfg) {
   KX_REQUIRE(cfg, "kx_index_infer_config: null config");
   KxIndex ix;
   int rc = kx_index_parse(index_path, ix);
@@ -240,4 +241,12 @@ extern "C" int kx_index_infer_config(const char *index_path, kx_config *cfg) {
     if ((t = ix.find(first_dense, "routed_expert", "gate_proj.weight_scale", 0)) && dims(t, r, c2)) cfg->moe_inter = (int32_t)r;
   }
   return KX_OK;
+}
+
+// ---- the C ABI: every body above runs under kx_guard, so that no exception leaves the library ----
+extern "C" int kx_index_check(const kx_config *cfg, const char *index_path, uint64_t *n_tensors, uint64_t *weight_bytes) {
+  return kx_guard("kx_index_check", [&] { return kx_index_check_body(cfg, index_path, n_tensors, weight_bytes); });
+}
+extern "C" int kx_index_infer_config(const char *index_path, kx_config *cfg) {
+  return kx_guard("kx_index_infer_config", [&] { return kx_index_infer_config_body(index_path, cfg); });
 }

@@ -29,6 +29,7 @@
 #include <type_traits>
 #include "kx_attn_parts.h"
 #include "kx_common.h"
+#include "kx_lds_copy.h"
 #include "kx_dense.h"
 #include "kx_math.h"
 #include "kx_mla.h"
@@ -346,24 +347,10 @@ __device__ __forceinline__ uint2 mm_read_tr(uint32_t addr) {
   kx_bf16x4t v = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) kx_bf16x4t *)(uintptr_t)addr);
   return __builtin_bit_cast(uint2, v);
 }
-// global_load_lds_dwordx4: lane i's 16 bytes at `src` land at LDS byte address lds_base + 16 i (lds_base uniform).
-// Written as asm so that the compiler does not know of the copy: it completes every copy in flight (s_waitcnt
-// vmcnt(0)) in front of each LDS access it cannot tell from the copy's target, and in front of every fenced
-// barrier -- which would make the tiles copied ahead land at once.  This kernel waits for a tile itself, where
-// it needs it (wait_tile below).
-__device__ __forceinline__ void mm_copy16_to_lds(const void *src, uint32_t lds_base) {
-  uint32_t m0_saved;  // the instruction takes the LDS address from m0; m0 is put back, the compiler owns it
-  asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, off\n\ts_mov_b32 m0, %0"
-               : "=&s"(m0_saved)
-               : "s"(lds_base), "v"(src)
-               : "memory");
-}
-
-// Workgroup barrier for this kernel.  __syncthreads() carries a fence, and the compiler completes every memory
-// operation for it -- s_waitcnt vmcnt(0), i.e. the tiles being copied ahead would have to land at every barrier.
-// Here only the wave's LDS operations are completed (what the waves exchange goes through LDS); the landing of
-// a copied tile is waited for explicitly where the tile is needed.
-__device__ __forceinline__ void mm_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+// the copies into the tile ring and the fence-free barrier: kx_lds_copy.h (this kernel waits for a tile itself,
+// where it needs it: wait_tile below)
+__device__ __forceinline__ void mm_copy16_to_lds(const void *src, uint32_t lds_base) { kx_copy16_to_lds(src, lds_base); }
+__device__ __forceinline__ void mm_barrier() { kx_lds_barrier(); }
 
 __global__ void __launch_bounds__(512, 1) mla_partial_mfma_k(MlaArgs a) {
   // the tile ring is the dynamic LDS; what the waves exchange lives in separate objects, so that the compiler can

@@ -37,6 +37,7 @@
 // max-rel 1e-2 bar and is never used for the token-identity runs.
 #include <atomic>
 #include "kx_common.h"
+#include "kx_lds_copy.h"
 #include "kx_dense.h"
 #include "kx_math.h"
 
@@ -85,20 +86,12 @@ __device__ __forceinline__ uint32_t pf_pack(float lo, float hi) {
 // fenced barrier, and loads complete in order, so a wait for a plain load it issued waits for the copies too.
 // Hence: weights and activations both reach LDS by copies issued from inline asm (unknown to the compiler), the
 // barrier has no fence, and the waits are explicit and counted.
-// global_load_lds_dwordx4: lane i's 16 bytes at `src` land at LDS byte address lds_base + 16 i (lds_base uniform)
 __device__ __forceinline__ void pf_copy16_to_lds(const void *src, uint32_t lds_base) {
-  lds_base = __builtin_amdgcn_readfirstlane(lds_base);
-  uint32_t m0_saved;  // the instruction takes the LDS address from m0; m0 is put back, the compiler owns it
-  asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, off\n\ts_mov_b32 m0, %0"
-               : "=&s"(m0_saved)
-               : "s"(lds_base), "v"(src)
-               : "memory");
+  kx_copy16_to_lds(src, __builtin_amdgcn_readfirstlane(lds_base));
 }
-// waits until at most N of this wave's copies are in flight (they complete in order)
 template <int N>
-__device__ __forceinline__ void pf_wait_copies() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
-// workgroup barrier without a fence: the wave's LDS operations are complete, nothing else is waited for
-__device__ __forceinline__ void pf_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+__device__ __forceinline__ void pf_wait_copies() { kx_wait_copies<N>(); }
+__device__ __forceinline__ void pf_barrier() { kx_lds_barrier(); }
 
 // dequantize one packed word (8 weights) to 8 bf16, columns ascending
 __device__ __forceinline__ kx_bf16x8 dequant_word(uint32_t w, float sc, float sc16, float c0, float c1, uint32_t magic) {

@@ -28,6 +28,7 @@
 // other matrix-core paths, and serves batches the token-identity checks do not run on.
 #include <atomic>
 #include "kx_common.h"
+#include "kx_lds_copy.h"
 #include "kx_dense.h"
 #include "kx_math.h"
 
@@ -43,18 +44,12 @@ struct SkinnyArgs {
   int rows, cols, tokens, x_stride, out_stride, mode;
 };
 
-// global_load_lds_dwordx4: lane i's 16 bytes at `src` land at LDS byte address lds_base + 16 i (lds_base uniform)
 __device__ __forceinline__ void sk_copy16_to_lds(const void *src, uint32_t lds_base) {
-  lds_base = __builtin_amdgcn_readfirstlane(lds_base);
-  uint32_t m0_saved;  // the instruction takes the LDS address from m0; m0 is put back, the compiler owns it
-  asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, off\n\ts_mov_b32 m0, %0"
-               : "=&s"(m0_saved)
-               : "s"(lds_base), "v"(src)
-               : "memory");
+  kx_copy16_to_lds(src, __builtin_amdgcn_readfirstlane(lds_base));
 }
 template <int N>
-__device__ __forceinline__ void sk_wait_copies() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
-__device__ __forceinline__ void sk_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+__device__ __forceinline__ void sk_wait_copies() { kx_wait_copies<N>(); }
+__device__ __forceinline__ void sk_barrier() { kx_lds_barrier(); }
 
 template <bool DUAL>
 __global__ void __launch_bounds__(512) skinny_staged_k(SkinnyArgs a) {

@@ -209,7 +209,11 @@ int copy_out(const std::vector<uint32_t> &ids, uint32_t *h_ids, size_t cap, size
 
 }  // namespace
 
-extern "C" int kx_tokenizer_open(const char *path, kx_tokenizer **out) {
+// ids index a table, so a hostile file must not be able to ask for gigabytes: no tokenizer.blok the reference
+// writes goes beyond 163,840 ids (scripts/model_fetch.py:92)
+constexpr unsigned long KX_TOK_MAX_ID = 1ul << 24;
+
+static int kx_tokenizer_open_body(const char *path, kx_tokenizer **out) {
   KX_REQUIRE(path && out, "kx_tokenizer_open: null argument");
   *out = nullptr;
   FILE *f = fopen(path, "rb");
@@ -231,7 +235,7 @@ extern "C" int kx_tokenizer_open(const char *path, kx_tokenizer **out) {
     char kind[16];
     unsigned long id = 0;
     int used = 0;
-    if (sscanf(buf, "%15s %lu %n", kind, &id, &used) < 2 || (strcmp(kind, "tok") && strcmp(kind, "special")) || id > 0x7fffffffu) { ok = false; break; }
+    if (sscanf(buf, "%15s %lu %n", kind, &id, &used) < 2 || (strcmp(kind, "tok") && strcmp(kind, "special")) || id >= KX_TOK_MAX_ID) { ok = false; break; }
     const char *hex = buf + used;
     const size_t hl = strlen(hex);
     if (hl == 0 || hl % 2) { ok = false; break; }
@@ -279,7 +283,7 @@ extern "C" int kx_tokenizer_info(const kx_tokenizer *tk, int32_t *n_tokens, int3
   return KX_OK;
 }
 
-extern "C" int kx_pretokenize(const char *text, size_t len, uint32_t *h_ends, size_t cap, size_t *n) {
+static int kx_pretokenize_body(const char *text, size_t len, uint32_t *h_ends, size_t cap, size_t *n) {
   KX_REQUIRE(text || len == 0, "kx_pretokenize: null text");
   std::vector<Cp> cps;
   decode_utf8((const unsigned char *)text, len, cps);
@@ -294,7 +298,7 @@ extern "C" int kx_pretokenize(const char *text, size_t len, uint32_t *h_ends, si
   return copy_out(ends, h_ends, cap, n, "kx_pretokenize");
 }
 
-extern "C" int kx_tokenizer_encode(const kx_tokenizer *tk, const char *text, size_t len, int allow_special, uint32_t *h_ids,
+static int kx_tokenizer_encode_body(const kx_tokenizer *tk, const char *text, size_t len, int allow_special, uint32_t *h_ids,
                                    size_t cap, size_t *n) {
   KX_REQUIRE(tk && (text || len == 0), "kx_tokenizer_encode: null argument");
   std::vector<uint32_t> ids;
@@ -318,7 +322,7 @@ extern "C" int kx_tokenizer_encode(const kx_tokenizer *tk, const char *text, siz
   return copy_out(ids, h_ids, cap, n, "kx_tokenizer_encode");
 }
 
-extern "C" int kx_tokenizer_decode(const kx_tokenizer *tk, const uint32_t *h_ids, size_t n_ids, char *h_bytes, size_t cap, size_t *len) {
+static int kx_tokenizer_decode_body(const kx_tokenizer *tk, const uint32_t *h_ids, size_t n_ids, char *h_bytes, size_t cap, size_t *len) {
   KX_REQUIRE(tk && (h_ids || n_ids == 0), "kx_tokenizer_decode: null argument");
   std::string out;
   for (size_t k = 0; k < n_ids; ++k) {
@@ -331,10 +335,27 @@ extern "C" int kx_tokenizer_decode(const kx_tokenizer *tk, const uint32_t *h_ids
   return KX_OK;
 }
 
-extern "C" int kx_encode_prompt(const kx_tokenizer *tk, const char *prompt, size_t len, uint32_t *h_ids, size_t cap, size_t *n) {
+static int kx_encode_prompt_body(const kx_tokenizer *tk, const char *prompt, size_t len, uint32_t *h_ids, size_t cap, size_t *n) {
   KX_REQUIRE(tk && (prompt || len == 0), "kx_encode_prompt: null argument");
   std::string text = "<|im_user|>user<|im_middle|>";  // runtime.py:139
   text.append(prompt, len);
   text += "<|im_end|><|im_assistant|>assistant<|im_middle|><think></think>";
   return kx_tokenizer_encode(tk, text.data(), text.size(), 1, h_ids, cap, n);
+}
+
+// ---- the C ABI: every body above runs under kx_guard, so that no exception leaves the library ----
+extern "C" int kx_tokenizer_open(const char *path, kx_tokenizer **out) {
+  return kx_guard("kx_tokenizer_open", [&] { return kx_tokenizer_open_body(path, out); });
+}
+extern "C" int kx_pretokenize(const char *text, size_t len, uint32_t *h_ends, size_t cap, size_t *n) {
+  return kx_guard("kx_pretokenize", [&] { return kx_pretokenize_body(text, len, h_ends, cap, n); });
+}
+extern "C" int kx_tokenizer_encode(const kx_tokenizer *tk, const char *text, size_t len, int allow_special, uint32_t *h_ids, size_t cap, size_t *n) {
+  return kx_guard("kx_tokenizer_encode", [&] { return kx_tokenizer_encode_body(tk, text, len, allow_special, h_ids, cap, n); });
+}
+extern "C" int kx_tokenizer_decode(const kx_tokenizer *tk, const uint32_t *h_ids, size_t n_ids, char *h_bytes, size_t cap, size_t *len) {
+  return kx_guard("kx_tokenizer_decode", [&] { return kx_tokenizer_decode_body(tk, h_ids, n_ids, h_bytes, cap, len); });
+}
+extern "C" int kx_encode_prompt(const kx_tokenizer *tk, const char *prompt, size_t len, uint32_t *h_ids, size_t cap, size_t *n) {
+  return kx_guard("kx_encode_prompt", [&] { return kx_encode_prompt_body(tk, prompt, len, h_ids, cap, n); });
 }
