@@ -36,9 +36,21 @@ def build_if_missing():
         __graft_entry__.build()
 
 
-# HBM bytes of one i4_gemv_k<dual> launch at T=1 (8 experts) from rocprofv3 counters: FETCH_SIZE 64,645 KiB x 2.0
-# (a 1 GiB kx_dev_copy reads 524,300 on that counter) + WRITE_SIZE 32 KiB x 1.0; see profiles/
-GATE_UP_TRAFFIC_T1 = 132423000
+# HBM bytes of one i4_gemv_k<dual> launch at T=1 (8 experts) as rocprofv3's FETCH_SIZE / WRITE_SIZE counters saw them,
+# scaled by what the same counters read for a 1 GiB kx_dev_copy.  Counters cannot be read inside this run; the figure is
+# taken from the committed summary of the counter runs of this same workload, which carries it on a line of the form
+# `traffic_bytes_per_launch: N`, and the JSON line names that file.
+TRAFFIC_PROFILE = "profiles/moe_layer_t1_pmc.md"
+
+
+def profiled_traffic():
+    try:
+        for line in open(os.path.join(ROOT, TRAFFIC_PROFILE)):
+            if line.startswith("traffic_bytes_per_launch:"):
+                return int(line.split(":")[1].split()[0].replace(",", ""))
+    except OSError:
+        pass
+    return None
 
 
 def moe_layer_bytes(cfg, tokens, distinct):
@@ -220,7 +232,8 @@ def run_moe_layer(args, emit=True):
                    "compute_units": cus.value},
         "roofline": {"bound": "hbm", "achieved": round(gate_up_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gate_up_gbs / HBM_PEAK_GBS, 4),
-                     "traffic": GATE_UP_TRAFFIC_T1 if (T == 1 and U_last == cfg.topk) else None,
+                     "traffic": profiled_traffic() if (T == 1 and U_last == cfg.topk) else None,
+                     "traffic_from": TRAFFIC_PROFILE if (T == 1 and U_last == cfg.topk) else None,
                      "kernel": "i4_gemv_k<dual> (routed gate+up + SwiGLU)",
                      "algorithmic_bytes_per_launch": int(U_last * by["gate_up"]),
                      "avg_launch_ms": round(alone[0], 5),
@@ -242,7 +255,8 @@ def run_moe_layer(args, emit=True):
 
 
 def stack_bytes_per_token(cfg, distinct_per_layer):
-    """Algorithmic HBM bytes of one batch-1 decode step of the truncated stack (weights read once)."""
+    """Algorithmic HBM bytes of the weights one decode step of the truncated stack reads (each once), with
+    distinct_per_layer routed experts selected per MoE layer (8 at batch 1; measured for a batch)."""
     H, V = cfg.hidden, cfg.vocab
     KD, VD = cfg.heads * (cfg.qk_nope + cfg.qk_rope), cfg.heads * cfg.v_head
     KVA, KVB = cfg.kv_rank + cfg.qk_rope, cfg.heads * (cfg.qk_nope + cfg.v_head)
@@ -298,10 +312,24 @@ def run_stack(args):
     check(lib.kx_event_elapsed_ms(e[1], e[2], C.byref(ms_dec)))
     last = np.zeros(B, dtype=np.uint32)
     check(lib.kx_greedy_sample(model, last.ctypes.data))
+    # distinct routed experts per MoE layer, which is what a batch's weight traffic depends on: counted over a few more
+    # (untimed) decode steps with the model's routing record switched on
+    distinct = float(cfg.topk)
+    if B > 1 and cfg.n_layers > cfg.first_dense:
+        check(lib.kx_model_set_routing_record(model, 1))
+        seen, d = [], C.c_int32()
+        for _ in range(6):
+            check(lib.kx_decode_step(model, None))
+            for layer in range(cfg.first_dense, cfg.n_layers):
+                check(lib.kx_model_routing(model, layer, None, C.byref(d)))
+                seen.append(d.value)
+        distinct = float(np.mean(seen))
     check(lib.kx_model_destroy(model))
     ms_per_step = ms_dec.value / K
     toks = B * 1e3 / ms_per_step
-    algo = stack_bytes_per_token(cfg, cfg.topk) if B == 1 else None
+    weights = stack_bytes_per_token(cfg, distinct)
+    kv = B * (P + W + K // 2) * (cfg.kv_rank + cfg.qk_rope) * 2 * cfg.n_layers   # latent cache rows read by a mid-run step
+    algo = weights if B == 1 else weights + kv
     return {
         "value": round(toks, 2), "ms_per_step": round(ms_per_step, 5), "wall_ms_per_step": round(wall_ms / K, 5),
         "prefill_ms_per_token": round(ms_pre.value / P, 5),
@@ -312,10 +340,12 @@ def run_stack(args):
         "resident_gb": {"weights": round(wb.value / 1e9, 2), "kv_cache": round(cb.value / 1e9, 3), "scratch": round(sb.value / 1e9, 3)},
         "model_create_s": round(t_create, 2), "device": name.value.decode(), "compute_units": cus.value,
         "last_ids": last.tolist(),
-        "stack_hbm": None if algo is None else {"algorithmic_bytes_per_token": int(algo),
-                                                "achieved_gbs": round(algo / (ms_per_step * 1e-3) / 1e9, 1),
-                                                "frac_of_peak": round(algo / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                                                "roof_tok_s": round(HBM_PEAK_GBS * 1e9 / algo, 1)},
+        "stack_hbm": {"algorithmic_bytes_per_step": int(algo), "weight_bytes": int(weights), "kv_cache_bytes": int(kv),
+                      "counted": "weights once per step" + ("" if B == 1 else " + latent cache rows of every sequence"),
+                      "distinct_experts_per_moe_layer": round(distinct, 1),
+                      "achieved_gbs": round(algo / (ms_per_step * 1e-3) / 1e9, 1),
+                      "frac_of_peak": round(algo / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                      "roof_tok_s": round(B * HBM_PEAK_GBS * 1e9 / algo, 1)},
     }
 
 
@@ -351,6 +381,11 @@ def run_default(args):
     margs = argparse.Namespace(**vars(args))
     margs.tokens, margs.steps, margs.warmup, margs.no_cpu = args.batch, 40, 8, True
     moe = run_moe_layer(margs, emit=False)
+    moe8 = None
+    if args.batch == 1:   # the same two kernels at T = 8 (BASELINE config 2 names T in {1, 8, 64}), where a launch is 7.5 waves of workgroups
+        margs8 = argparse.Namespace(**vars(margs))
+        margs8.tokens = 8
+        moe8 = run_moe_layer(margs8, emit=False)
     cpu = None if args.no_cpu else run_cpu_stack(args)
     out = {
         "metric": "decode tok/s + INT4 expert GEMV HBM GB/s (% of peak), Kimi-K2 shapes, 1 GPU",
@@ -364,6 +399,9 @@ def run_default(args):
         "stack": {k: stack[k] for k in ("wall_ms_per_step", "prefill_ms_per_token", "model_create_s", "stack_hbm", "last_ids")},
         "cpu_baseline": cpu,
     }
+    if moe8 is not None:
+        out["int4_expert_gemv_t8"] = dict(moe8["int4_expert_gemv"], workload=moe8["config"]["workload"],
+                                          gate_up_frac_of_peak=moe8["roofline"]["frac"])
     print(json.dumps(out), flush=True)
     return out
 

@@ -116,6 +116,7 @@ __global__ void __launch_bounds__(TT > 1 ? 512 : 1024) gemv_pair_k(KxGemvArgs a0
   __shared__ uint4 s_ids4[4];
   // The logits were stored with device-scope stores; after the barrier one thread counts the workgroup in
   // (release).  The workgroup that counts in last (acquire) reads all logits with device-scope loads.
+  kx_arrive_writes_done();
   __syncthreads();
   if (threadIdx.x == 0) s_last = kx_arrive_is_last(r.counter, n1);
   __syncthreads();
@@ -145,6 +146,7 @@ __global__ void __launch_bounds__(TT > 1 ? 512 : 1024) gemv_absorb_k(KxGemvArgs 
   }
   const int chunk = blockIdx.x - 1;
   gemv_body<1, RI, TT>(a, chunk, gridDim.x - 1, part);
+  kx_arrive_writes_done();
   __syncthreads();  // every lane's stores of q lie before the counting lane's release (kx_arrive.h)
   const int h = chunk / q.head_chunks;
   if (threadIdx.x == 0) s_last = kx_arrive_is_last(q.head_count + h, q.head_chunks);

@@ -168,6 +168,7 @@ __host__ __device__ constexpr int i4_chunk_rows(bool dual, int rt) { return dual
 __device__ __forceinline__ void moe_tail_arrive(const KxMoeTail &t, int blk_a, int blk_b, int block_rows, int rows,
                                                 const uint16_t *eout) {
   __shared__ int s_last[2];
+  kx_arrive_writes_done();
   __syncthreads();  // every lane's outputs lie before the counting lanes' release (kx_arrive.h)
   if (threadIdx.x < 2) {
     const int blk = threadIdx.x ? blk_b : blk_a;

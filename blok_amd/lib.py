@@ -114,22 +114,26 @@ _SIGS = {
 _lib = None
 
 
+def load_library(path):
+    """A library file with the signatures of include/kx.h bound.  Raises KxError when it is missing: there is no fallback."""
+    if not os.path.exists(path):
+        raise KxError(f"{path} is not built; run `make -C blok_amd/csrc` "
+                      "(or __graft_entry__.build())")
+    lib = C.CDLL(path)
+    lib.kx_last_error.restype = C.c_char_p
+    lib.kx_last_error.argtypes = []
+    for name, args in _SIGS.items():
+        fn = getattr(lib, name)
+        fn.argtypes = args
+        fn.restype = C.c_int
+    return lib
+
+
 def kx():
-    """The loaded library.  Raises KxError when libkx.so is missing: there is no fallback."""
+    """The loaded library (blok_amd/libkx.so)."""
     global _lib
     if _lib is None:
-        path = lib_path()
-        if not os.path.exists(path):
-            raise KxError(f"{path} is not built; run `make -C blok_amd/csrc` "
-                          "(or __graft_entry__.build())")
-        lib = C.CDLL(path)
-        lib.kx_last_error.restype = C.c_char_p
-        lib.kx_last_error.argtypes = []
-        for name, args in _SIGS.items():
-            fn = getattr(lib, name)
-            fn.argtypes = args
-            fn.restype = C.c_int
-        _lib = lib
+        _lib = load_library(lib_path())
     return _lib
 
 

@@ -595,6 +595,39 @@ def test_kimi_shape_batched_stack_against_single_sequences(kxlib, ox, batch):
     assert len(excused) <= batch // 4
 
 
+def test_model_form_of_the_handover_gives_the_same_bits(kxlib, ox):
+    # blok_amd/libkx_strict.so is the library with the hand-over between workgroups of one launch (the q_b GEMV that
+    # finishes a head's query, the router GEMV whose last workgroup routes, the routed down launch that combines)
+    # compiled in its memory-model form: release increment, acquire by the finisher.  The library that ships orders
+    # the same accesses by what the gfx950 instructions do, which is faster.  Both run here, on the paths that
+    # use the protocol (up to 4 sequences), and must agree to the bit on ids, hidden state, logits and cache rows.
+    import os
+    from blok_amd.lib import load_library
+    say("hand-over protocol: shipped form against the memory-model form")
+    strict = load_library(os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "blok_amd", "libkx_strict.so"))
+    cases = [("small", O.small_config(batch=3, context=64), 3, 11, 9)]
+    kimi = default_config()
+    kimi.n_layers, kimi.first_dense, kimi.max_batch, kimi.max_context, kimi.seed = 3, 1, 1, 48, 11
+    cases.append(("kimi", kimi, 1, 24, 8))
+    for name, cfg, batch, prompt_len, n_tokens in cases:
+        prompt = O.tokens_u32(batch * prompt_len, cfg.seed, 4, cfg.vocab).reshape(batch, prompt_len)
+        got = []
+        for lib in (kxlib, strict):
+            km = KxModel(lib, cfg)
+            rc, out, _ = km.generate(prompt, n_tokens)
+            assert rc == 0, lib.kx_last_error()
+            total = prompt_len + n_tokens - 1
+            h = np.empty((batch, cfg.hidden), dtype=np.uint16)
+            lg = np.empty((batch, cfg.vocab), dtype=np.float32)
+            assert lib.kx_model_hidden(km.h, ptr(h)) == 0 and lib.kx_model_logits(km.h, ptr(lg)) == 0
+            rows = np.empty((total, cfg.kv_rank + cfg.qk_rope), dtype=np.uint16)
+            assert lib.kx_model_latent(km.h, cfg.n_layers - 1, 0, 0, total, ptr(rows)) == 0
+            got.append((out.copy(), h, lg.view(np.uint32), rows))
+            km.close()
+        for a, b in zip(*got):
+            assert (a == b).all(), f"{name}: the two forms differ"
+
+
 def test_executor_json_line(kxlib):
     import json
     import os
