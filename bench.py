@@ -275,7 +275,7 @@ def run_stack(args):
     lib = kx()
     cfg = default_config()
     B, P, K, W = args.batch, args.prompt, args.steps, args.warmup
-    cfg.n_layers, cfg.max_batch, cfg.max_context, cfg.seed = args.stack_layers, B, P + K + W + 1, args.seed
+    cfg.n_layers, cfg.max_batch, cfg.max_context, cfg.seed = args.stack_layers, B, P + K + W + 9, args.seed
     name = C.create_string_buffer(256)
     cus, hbm = C.c_int32(), C.c_uint64()
     check(lib.kx_device_info(name, 256, C.byref(cus), C.byref(hbm)))
@@ -416,8 +416,8 @@ def run_prefill(args):
     layers = MoeLayerSet(lib, cfg, 2, args.seed)
     # Zipf-like load: bias += c*ln(1/rank)
     for li, w in enumerate(layers.layers):
-        bias = O.normal_f32(cfg.experts, args.seed + 1000 * li, 11, 0.01) + 0.1 * np.log(1.0 / np.arange(1, cfg.experts + 1))
-        check(lib.kx_h2d(w.d_router_bias, bias.astype(np.float32).ctypes.data, cfg.experts * 4))
+        bias = (O.normal_f32(cfg.experts, args.seed + 1000 * li, 11, 0.01) + 0.1 * np.log(1.0 / np.arange(1, cfg.experts + 1))).astype(np.float32)
+        check(lib.kx_h2d(w.d_router_bias, bias.ctypes.data, cfg.experts * 4))   # `bias` stays alive across the call
     ws = C.c_void_p()
     check(lib.kx_moe_workspace_create(C.byref(cfg), T, C.byref(ws)))
     n_host = O.normal_bf16(T * cfg.hidden, args.seed, 30, 1.0)
