@@ -41,6 +41,10 @@ struct kx_moe_workspace {
   uint16_t *smid;     // [T, shared_inter]
   uint16_t *sy;       // [T, hidden] shared expert output (prefill path)
   hipEvent_t ev[6];
+  // a second stream for the batched forms: the experts with one pair (GEMV kernels) and the shared expert run beside the
+  // grouped GEMMs of the experts with several pairs instead of in front of them.  Default priority, like every stream here.
+  hipStream_t side = nullptr;
+  hipEvent_t fork = nullptr, join = nullptr;
 };
 
 static int check_cfg(const kx_config *c) {
@@ -86,6 +90,9 @@ extern "C" int kx_moe_workspace_create(const kx_config *cfg, int32_t max_tokens,
   if (e == hipSuccess) e = hipMemset(ws->tail_count, 0, KX_TAIL_BLOCKS * 4);
   for (auto &ev : ws->ev)
     if (e == hipSuccess) e = hipEventCreate(&ev);
+  if (e == hipSuccess) e = hipStreamCreateWithFlags(&ws->side, hipStreamNonBlocking);
+  if (e == hipSuccess) e = hipEventCreateWithFlags(&ws->fork, hipEventDisableTiming);
+  if (e == hipSuccess) e = hipEventCreateWithFlags(&ws->join, hipEventDisableTiming);
   if (e != hipSuccess) {
     kx_set_error("kx_moe_workspace_create: %s", hipGetErrorString(e));
     kx_moe_workspace_destroy(ws);
@@ -103,6 +110,9 @@ extern "C" int kx_moe_workspace_destroy(kx_moe_workspace *ws) {
     if (p) (void)hipFree(p);
   for (auto &e : ws->ev)
     if (e) (void)hipEventDestroy(e);
+  if (ws->side) { (void)hipStreamSynchronize(ws->side); (void)hipStreamDestroy(ws->side); }
+  if (ws->fork) (void)hipEventDestroy(ws->fork);
+  if (ws->join) (void)hipEventDestroy(ws->join);
   delete ws;
   return KX_OK;
 }
@@ -221,14 +231,23 @@ int kx_moe_layer_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_work
   // routed gate/up + SwiGLU
   const bool rmm = (flags & KX_MOE_ROUTED_MATRIX_CORES) && tokens >= 5;
   const int n_slots = (long)tokens * K < E ? tokens * K : E;
-  if (rmm) {  // experts with one pair: the GEMV kernel (it streams them at its rate); the others: the grouped GEMM
+  if (rmm) {
+    // Experts with one pair: the GEMV kernels (they stream such an expert at their rate); the others: the grouped
+    // GEMMs.  The two classes touch different experts and different rows of mid and of the expert outputs, so they
+    // run side by side: the GEMV class (gate/up, then down) and after it the shared expert on the side stream, the
+    // GEMM class (gate/up, then down) on this one, joined before the combine.  A GEMM workgroup holds a whole CU
+    // for its 112 K steps and a batch of 32 brings about 280 of them for 256 CUs; side by side, the other class
+    // fills the CUs that the second round of those would leave idle (batch 32: two launches in sequence took
+    // 148 + 251 us for gate/up and 77 + 117 us for down).
     const int I = c->moe_inter;
-    if ((rc = kx_i4_launch(true, (const uint32_t *)w->d_gate_packed, (const uint16_t *)w->d_gate_scale,
-                           (const uint32_t *)w->d_up_packed, (const uint16_t *)w->d_up_scale, n, ws->mid, ws->work, ws->pairs, 0, I,
-                           H, K, (size_t)I * (H / 8), (size_t)I * (H / 32), 1, n_slots, 1, 1, st))) return rc;
+    KX_HIP(hipEventRecord(ws->fork, st));
+    KX_HIP(hipStreamWaitEvent(ws->side, ws->fork, 0));
     if ((rc = kx_grouped_gemm_launch(true, true, w->d_gate_packed, (const uint16_t *)w->d_gate_scale, w->d_up_packed,
                                      (const uint16_t *)w->d_up_scale, n, ws->mid, KX_GG_BF16, ws->work, ws->pairs, 0, n_slots, I, H,
                                      K, (size_t)I * (H / 8), (size_t)I * (H / 32), tokens, st, 2))) return rc;
+    if ((rc = kx_i4_launch(true, (const uint32_t *)w->d_gate_packed, (const uint16_t *)w->d_gate_scale,
+                           (const uint32_t *)w->d_up_packed, (const uint16_t *)w->d_up_scale, n, ws->mid, ws->work, ws->pairs, 0, I,
+                           H, K, (size_t)I * (H / 8), (size_t)I * (H / 32), 1, n_slots, 1, 1, ws->side))) return rc;
   } else if ((rc = routed_launch(c, w, ws, n, tokens, 0, st))) return rc;
   if (timed) KX_HIP(hipEventRecord(ws->ev[2], st));
   // shared down + combine + residual: as the epilogue of a GEMV of its own, or, for one token, inside the routed
@@ -250,33 +269,37 @@ int kx_moe_layer_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_work
   // routed down
   if (rmm) {
     const int I = c->moe_inter;
-    if ((rc = kx_i4_launch(false, (const uint32_t *)w->d_down_packed, (const uint16_t *)w->d_down_scale, nullptr, nullptr,
-                           ws->mid, ws->eout, ws->work, ws->pairs, 0, H, I, 1, (size_t)H * (I / 8), (size_t)H * (I / 32),
-                           1, n_slots, 1, 1, st, 2))) return rc;
     if ((rc = kx_grouped_gemm_launch(false, true, w->d_down_packed, (const uint16_t *)w->d_down_scale, nullptr, nullptr,
                                      ws->mid, ws->eout, KX_GG_BF16, ws->work, ws->pairs, 0, n_slots, H, I, 1, (size_t)H * (I / 8),
                                      (size_t)H * (I / 32), tokens, st, 2))) return rc;
+    if ((rc = kx_i4_launch(false, (const uint32_t *)w->d_down_packed, (const uint16_t *)w->d_down_scale, nullptr, nullptr,
+                           ws->mid, ws->eout, ws->work, ws->pairs, 0, H, I, 1, (size_t)H * (I / 8), (size_t)H * (I / 32),
+                           1, n_slots, 1, 1, ws->side, 2))) return rc;
   } else if (!tailed && (rc = routed_launch(c, w, ws, n, tokens, 1, st))) return rc;
   if (timed) KX_HIP(hipEventRecord(ws->ev[3], st));
   // shared gate/up + SwiGLU when it did not ride with the router
   // From 5 tokens on a caller may ask for the shared expert on the matrix cores (another summation order, held to
   // the 1e-2 bar; the router and the routed experts stay as they are, so the routing does not change)
   const bool mm = (flags & KX_MOE_SHARED_MATRIX_CORES) && tokens >= 5 && tokens <= 32;
+  hipStream_t sst = (rmm && mm) ? ws->side : st;  // the shared expert's matrix-core products follow the GEMV class on the side stream
   if (!paired) {
     if (norm_w) { s.x = n; s.norm_w = nullptr; }  // d_n holds the normed rows by now
     bool done = false;
     if (mm && !s.norm_w &&
-        (rc = kx_skinny_gemm_launch(true, s.w0, s.w1, s.x, s.x_stride, s.out, s.out_stride, KX_GG_BF16, tokens, s.rows, s.cols, &done, st)))
+        (rc = kx_skinny_gemm_launch(true, s.w0, s.w1, s.x, s.x_stride, s.out, s.out_stride, KX_GG_BF16, tokens, s.rows, s.cols, &done, sst)))
       return rc;
-    if (!done && (rc = kx_gemv_launch(KX_EPI_SWIGLU, s, st))) return rc;
+    if (!done && (rc = kx_gemv_launch(KX_EPI_SWIGLU, s, sst))) return rc;
   }
   if (timed) KX_HIP(hipEventRecord(ws->ev[4], st));
   if (!tailed) {
     bool done = false;
-    if (mm) {  // shared down into sy, then the combine as a kernel of its own
-      if ((rc = kx_skinny_gemm_launch(false, d.w0, nullptr, d.x, d.x_stride, ws->sy, H, KX_GG_BF16, tokens, d.rows, d.cols, &done, st))) return rc;
-      if (done && (rc = kx_moe_combine_launch(ws->eout, ws->weights, ws->sy, (uint16_t *)d_x, tokens, H, K, flags & 1u, st))) return rc;
+    if (mm &&  // shared down into sy, then the combine as a kernel of its own
+        (rc = kx_skinny_gemm_launch(false, d.w0, nullptr, d.x, d.x_stride, ws->sy, H, KX_GG_BF16, tokens, d.rows, d.cols, &done, sst))) return rc;
+    if (rmm) {  // both classes of routed experts and the shared expert are in before anything reads their outputs
+      KX_HIP(hipEventRecord(ws->join, ws->side));
+      KX_HIP(hipStreamWaitEvent(st, ws->join, 0));
     }
+    if (done && (rc = kx_moe_combine_launch(ws->eout, ws->weights, ws->sy, (uint16_t *)d_x, tokens, H, K, flags & 1u, st))) return rc;
     if (!done && (rc = kx_gemv_launch(KX_EPI_MOE_COMBINE, d, st))) return rc;
   }
   if (timed) KX_HIP(hipEventRecord(ws->ev[5], st));
@@ -324,6 +347,15 @@ extern "C" int kx_moe_prefill_layer(const kx_config *c, const kx_moe_weights *w,
   hipStream_t st = kx_stream(stream);
   const int H = c->hidden, I = c->moe_inter, SI = c->shared_inter, E = c->experts, K = c->topk;
   const uint16_t *n = (const uint16_t *)d_n;
+  // The shared expert needs nothing from the router or the routed experts: its two GEMMs run on the side stream
+  // while this one routes and runs the grouped GEMMs, and are joined before the combine.
+  KX_HIP(hipEventRecord(ws->fork, st));
+  KX_HIP(hipStreamWaitEvent(ws->side, ws->fork, 0));
+  if ((rc = kx_grouped_gemm_launch(true, false, w->d_shared_gate, nullptr, w->d_shared_up, nullptr, n, ws->smid, KX_GG_BF16,
+                                   nullptr, nullptr, tokens, 1, SI, H, 1, 0, 0, tokens, ws->side))) return rc;
+  if ((rc = kx_grouped_gemm_launch(false, false, w->d_shared_down, nullptr, nullptr, nullptr, ws->smid, ws->sy, KX_GG_BF16,
+                                   nullptr, nullptr, tokens, 1, H, SI, 1, 0, 0, tokens, ws->side))) return rc;
+  KX_HIP(hipEventRecord(ws->join, ws->side));
   // router: fp32 logits (unrounded) as one GEMM of all tokens against the gate, top-k, bucketing.  Up to 32 tokens
   // the decode GEMV is used instead (its summation order is the decode path's).
   if (tokens <= 32) {
@@ -347,10 +379,6 @@ extern "C" int kx_moe_prefill_layer(const kx_config *c, const kx_moe_weights *w,
   if ((rc = kx_grouped_gemm_launch(false, true, w->d_down_packed, (const uint16_t *)w->d_down_scale, nullptr, nullptr,
                                    ws->mid, ws->eout, KX_GG_BF16, ws->work, ws->pairs, 0, n_slots, H, I, 1, (size_t)H * (I / 8),
                                    (size_t)H * (I / 32), tokens, st))) return rc;
-  // shared expert: one group of all tokens, bf16 weights
-  if ((rc = kx_grouped_gemm_launch(true, false, w->d_shared_gate, nullptr, w->d_shared_up, nullptr, n, ws->smid, KX_GG_BF16,
-                                   nullptr, nullptr, tokens, 1, SI, H, 1, 0, 0, tokens, st))) return rc;
-  if ((rc = kx_grouped_gemm_launch(false, false, w->d_shared_down, nullptr, nullptr, nullptr, ws->smid, ws->sy, KX_GG_BF16,
-                                   nullptr, nullptr, tokens, 1, H, SI, 1, 0, 0, tokens, st))) return rc;
+  KX_HIP(hipStreamWaitEvent(st, ws->join, 0));  // the shared expert's output
   return kx_moe_combine_launch(ws->eout, ws->weights, ws->sy, (uint16_t *)d_x, tokens, H, K, flags, st);
 }
