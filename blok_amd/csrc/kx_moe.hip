@@ -217,6 +217,23 @@ int kx_moe_layer_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_work
     g.x = (const uint16_t *)d_x; g.norm_w = norm_w; g.norm_eps = c->rms_eps; g.norm_out = (uint16_t *)d_n;
     s.x = (const uint16_t *)d_x; s.norm_w = norm_w; s.norm_eps = c->rms_eps;
   }
+  // From 5 tokens on a caller may ask for the shared expert on the matrix cores (another summation order, held to
+  // the 1e-2 bar; the router and the routed experts stay as they are, so the routing does not change).  Its two
+  // products need nothing from the router or the routed experts: they run on the side stream while this one routes
+  // and runs the routed experts, and are joined before the combine.
+  const bool mm = (flags & KX_MOE_SHARED_MATRIX_CORES) && tokens >= 5 && tokens <= 32;
+  const bool rmm = (flags & KX_MOE_ROUTED_MATRIX_CORES) && tokens >= 5;
+  bool shared_up_done = false, shared_down_done = false, forked = false;
+  if (mm && !norm_w) {
+    KX_HIP(hipEventRecord(ws->fork, st));
+    KX_HIP(hipStreamWaitEvent(ws->side, ws->fork, 0));
+    forked = true;
+    if ((rc = kx_skinny_gemm_launch(true, s.w0, s.w1, s.x, s.x_stride, s.out, s.out_stride, KX_GG_BF16, tokens, s.rows, s.cols,
+                                    &shared_up_done, ws->side))) return rc;
+    if (shared_up_done &&
+        (rc = kx_skinny_gemm_launch(false, (const uint16_t *)w->d_shared_down, nullptr, ws->smid, c->shared_inter, ws->sy, H, KX_GG_BF16,
+                                    tokens, H, c->shared_inter, &shared_down_done, ws->side))) return rc;
+  }
   bool paired = false;
   if ((rc = kx_gemv_pair_route_launch(s, g, (const float *)w->d_router_bias, ws->ids, ws->weights, E, K, c->routed_scale,
                                       ws->counts, ws->offsets, ws->pairs, ws->work, ws->n_active, ws->route_counter, &paired,
@@ -229,7 +246,6 @@ int kx_moe_layer_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_work
   }
   if (timed) KX_HIP(hipEventRecord(ws->ev[1], st));
   // routed gate/up + SwiGLU
-  const bool rmm = (flags & KX_MOE_ROUTED_MATRIX_CORES) && tokens >= 5;
   const int n_slots = (long)tokens * K < E ? tokens * K : E;
   if (rmm) {
     // Experts with one pair: the GEMV kernels (they stream such an expert at their rate); the others: the grouped
@@ -240,8 +256,9 @@ int kx_moe_layer_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_work
     // fills the CUs that the second round of those would leave idle (batch 32: two launches in sequence took
     // 148 + 251 us for gate/up and 77 + 117 us for down).
     const int I = c->moe_inter;
-    KX_HIP(hipEventRecord(ws->fork, st));
+    KX_HIP(hipEventRecord(ws->fork, st));  // the routing is in
     KX_HIP(hipStreamWaitEvent(ws->side, ws->fork, 0));
+    forked = true;
     if ((rc = kx_grouped_gemm_launch(true, true, w->d_gate_packed, (const uint16_t *)w->d_gate_scale, w->d_up_packed,
                                      (const uint16_t *)w->d_up_scale, n, ws->mid, KX_GG_BF16, ws->work, ws->pairs, 0, n_slots, I, H,
                                      K, (size_t)I * (H / 8), (size_t)I * (H / 32), tokens, st, 2))) return rc;
@@ -277,30 +294,20 @@ int kx_moe_layer_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_work
                            1, n_slots, 1, 1, ws->side, 2))) return rc;
   } else if (!tailed && (rc = routed_launch(c, w, ws, n, tokens, 1, st))) return rc;
   if (timed) KX_HIP(hipEventRecord(ws->ev[3], st));
-  // shared gate/up + SwiGLU when it did not ride with the router
-  // From 5 tokens on a caller may ask for the shared expert on the matrix cores (another summation order, held to
-  // the 1e-2 bar; the router and the routed experts stay as they are, so the routing does not change)
-  const bool mm = (flags & KX_MOE_SHARED_MATRIX_CORES) && tokens >= 5 && tokens <= 32;
-  hipStream_t sst = (rmm && mm) ? ws->side : st;  // the shared expert's matrix-core products follow the GEMV class on the side stream
-  if (!paired) {
+  // shared gate/up + SwiGLU when it neither rode with the router nor ran on the side stream
+  if (!paired && !shared_up_done) {
     if (norm_w) { s.x = n; s.norm_w = nullptr; }  // d_n holds the normed rows by now
-    bool done = false;
-    if (mm && !s.norm_w &&
-        (rc = kx_skinny_gemm_launch(true, s.w0, s.w1, s.x, s.x_stride, s.out, s.out_stride, KX_GG_BF16, tokens, s.rows, s.cols, &done, sst)))
-      return rc;
-    if (!done && (rc = kx_gemv_launch(KX_EPI_SWIGLU, s, sst))) return rc;
+    if ((rc = kx_gemv_launch(KX_EPI_SWIGLU, s, st))) return rc;
   }
   if (timed) KX_HIP(hipEventRecord(ws->ev[4], st));
   if (!tailed) {
-    bool done = false;
-    if (mm &&  // shared down into sy, then the combine as a kernel of its own
-        (rc = kx_skinny_gemm_launch(false, d.w0, nullptr, d.x, d.x_stride, ws->sy, H, KX_GG_BF16, tokens, d.rows, d.cols, &done, sst))) return rc;
-    if (rmm) {  // both classes of routed experts and the shared expert are in before anything reads their outputs
+    if (forked) {  // the GEMV class of the routed experts and the shared expert are in before anything reads their outputs
       KX_HIP(hipEventRecord(ws->join, ws->side));
       KX_HIP(hipStreamWaitEvent(st, ws->join, 0));
     }
-    if (done && (rc = kx_moe_combine_launch(ws->eout, ws->weights, ws->sy, (uint16_t *)d_x, tokens, H, K, flags & 1u, st))) return rc;
-    if (!done && (rc = kx_gemv_launch(KX_EPI_MOE_COMBINE, d, st))) return rc;
+    if (shared_down_done) {  // the shared output is in sy: the combine is a kernel of its own
+      if ((rc = kx_moe_combine_launch(ws->eout, ws->weights, ws->sy, (uint16_t *)d_x, tokens, H, K, flags & 1u, st))) return rc;
+    } else if ((rc = kx_gemv_launch(KX_EPI_MOE_COMBINE, d, st))) return rc;
   }
   if (timed) KX_HIP(hipEventRecord(ws->ev[5], st));
   return KX_OK;
