@@ -244,15 +244,22 @@ __device__ __forceinline__ void gemv_body(const KxGemvArgs &a, const int bid, co
       const int rc = idx % CR, tok = idx / CR;
       const int row = c0 + rc;
       if (row < chunk * CR) continue;  // rows of a moved-back last chunk that the previous chunk owns
-      const float *p0 = part + ((0 * CR + rc) * T + tok) * S;
-      float y0 = p0[0];
-      for (int q = 1; q < S; ++q) y0 += p0[q];
+      // the slice sums are read eight at a time (one wait per eight instead of one per addition) and added in order
+      auto slice_sum = [&](const float *p) {
+        float y = p[0];
+        for (int q0 = 1; q0 < S; q0 += 8) {
+          float t[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) t[u] = p[min(q0 + u, S - 1)];
+#pragma unroll
+          for (int u = 0; u < 8; ++u)
+            if (q0 + u < S) y += t[u];
+        }
+        return y;
+      };
+      const float y0 = slice_sum(part + ((0 * CR + rc) * T + tok) * S);
       float y1 = 0.0f;
-      if (MATS == 2) {
-        const float *p1 = part + ((1 * CR + rc) * T + tok) * S;
-        y1 = p1[0];
-        for (int q = 1; q < S; ++q) y1 += p1[q];
-      }
+      if (MATS == 2) y1 = slice_sum(part + ((1 * CR + rc) * T + tok) * S);
       switch (a.epi) {
         case KX_EPI_BF16:
           if (a.flags & KX_GEMV_COHERENT_OUT)

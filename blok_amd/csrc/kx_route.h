@@ -18,13 +18,19 @@ __device__ __forceinline__ void topk_token(const float *lg, const float *__restr
                                            float routed_scale, int lane, uint16_t *s_ids = nullptr) {
   float sc[EPL], sel[EPL];
   const float NEG_INF = -__builtin_inff();
+  // all logits and biases of the lane are requested before the first is used (lanes past E read expert E - 1 and
+  // drop it): with the load inside the loop below, each of the EPL sigmoids waited for its own round trip
+  float x[EPL], bs[EPL];
 #pragma unroll
   for (int j = 0; j < EPL; ++j) {
-    int e = lane + 64 * j;
-    float x = 0.0f, b = e < E ? bias[e] : 0.0f;
-    if (e < E) x = COHERENT ? __hip_atomic_load(lg + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : lg[e];
-    sc[j] = kx_sigmoidf(x);
-    sel[j] = e < E ? sc[j] + b : NEG_INF;
+    const int ec = min(lane + 64 * j, E - 1);
+    x[j] = COHERENT ? __hip_atomic_load(lg + ec, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : lg[ec];
+    bs[j] = bias[ec];
+  }
+#pragma unroll
+  for (int j = 0; j < EPL; ++j) {
+    sc[j] = kx_sigmoidf(x[j]);
+    sel[j] = lane + 64 * j < E ? sc[j] + bs[j] : NEG_INF;
   }
   float sum = 0.0f;
   float my_w = 0.0f;  // lane k keeps the k-th winner's score
@@ -72,25 +78,51 @@ __device__ __forceinline__ void bucket_block(const uint16_t *__restrict__ ids, i
     __syncthreads();
   }
   const uint32_t me = (uint32_t)e, me2 = me | (me << 16);
-  int cnt = 0;
-  if (e < E)
-    for (int q = 0; q < n8; ++q) {
-      const uint4 u = s_ids4[q];
-      const uint32_t w[4] = {u.x ^ me2, u.y ^ me2, u.z ^ me2, u.w ^ me2};
-#pragma unroll
-      for (int j = 0; j < 4; ++j) cnt += ((w[j] & 0xffffu) == 0) + ((w[j] >> 16) == 0);
+  int cnt = 0, off, slot, total_active, total;
+  if (n_pairs <= 64) {
+    // Few pairs (decode steps of up to 8 tokens): every thread goes over the pairs itself.  Expert e's offset is the
+    // number of pairs with a smaller id and its slot the number of distinct smaller ids, so no scan over the
+    // workgroup is needed (18 barriers at 448 threads); s_act[q] marks the first pair of each id.
+    if (e < n8 * 8) {
+      const uint16_t id = s_ids[e];
+      int first = e < n_pairs;
+      for (int q = 0; q < e; ++q) first &= s_ids[q] != id;
+      s_act[e] = first;
     }
-  s_cnt[e] = cnt;
-  s_act[e] = cnt > 0 ? 1 : 0;
-  __syncthreads();
-  for (int d = 1; d < n; d <<= 1) {  // inclusive Hillis-Steele scans of both arrays
-    int a = e >= d ? s_cnt[e - d] : 0, b = e >= d ? s_act[e - d] : 0;
     __syncthreads();
-    s_cnt[e] += a;
-    s_act[e] += b;
+    off = slot = total_active = 0;
+    for (int q = 0; q < n_pairs; ++q) {
+      const uint32_t id = s_ids[q];
+      const int f = s_act[q];
+      cnt += id == me;
+      off += id < me;
+      slot += f && id < me;
+      total_active += f;
+    }
+    total = n_pairs;
+  } else {
+    if (e < E)
+      for (int q = 0; q < n8; ++q) {
+        const uint4 u = s_ids4[q];
+        const uint32_t w[4] = {u.x ^ me2, u.y ^ me2, u.z ^ me2, u.w ^ me2};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) cnt += ((w[j] & 0xffffu) == 0) + ((w[j] >> 16) == 0);
+      }
+    s_cnt[e] = cnt;
+    s_act[e] = cnt > 0 ? 1 : 0;
     __syncthreads();
+    for (int d = 1; d < n; d <<= 1) {  // inclusive Hillis-Steele scans of both arrays
+      int a = e >= d ? s_cnt[e - d] : 0, b = e >= d ? s_act[e - d] : 0;
+      __syncthreads();
+      s_cnt[e] += a;
+      s_act[e] += b;
+      __syncthreads();
+    }
+    off = s_cnt[e] - cnt;
+    slot = s_act[e] - (cnt > 0 ? 1 : 0);
+    total_active = s_act[n - 1];
+    total = s_cnt[n - 1];
   }
-  const int off = s_cnt[e] - cnt, slot = s_act[e] - (cnt > 0 ? 1 : 0), total_active = s_act[n - 1];
   if (e < E) {
     counts[e] = cnt;
     offsets[e] = off;
@@ -113,7 +145,7 @@ __device__ __forceinline__ void bucket_block(const uint16_t *__restrict__ ids, i
     if (e >= total_active) work[e] = make_int4(-1, 0, 0, 0);
   }
   if (e == 0) {
-    offsets[E] = s_cnt[n - 1];
+    offsets[E] = total;
     *n_active = total_active;
   }
 }
