@@ -100,7 +100,7 @@ struct KxRouteArgs {
   int *n_active;
   int4 *pair_work;  // optional second work list, one record per pair
 };
-template <int RI0, int TT>
+template <int RI0, int RI1, int TT>
 __global__ void __launch_bounds__(TT > 1 ? 512 : 1024) gemv_pair_k(KxGemvArgs a0, KxGemvArgs a1, int n0, KxRouteArgs r) {
   extern __shared__ float part[];
   const int n1 = gridDim.x - n0;  // the router's workgroups come first: its routing tail overlaps the rest
@@ -108,7 +108,7 @@ __global__ void __launch_bounds__(TT > 1 ? 512 : 1024) gemv_pair_k(KxGemvArgs a0
     gemv_body<2, RI0, TT>(a0, blockIdx.x - n1, n0, part);
     return;
   }
-  gemv_body<1, 1, TT>(a1, blockIdx.x, n1, part);
+  gemv_body<1, RI1, TT>(a1, blockIdx.x, n1, part);
   if (!r.counter) return;
   __shared__ int s_last;
   __shared__ int s_cnt[1024];
@@ -330,8 +330,17 @@ int kx_gemv_pair_route_launch(KxGemvArgs a0, KxGemvArgs a1, const float *bias, u
   *fused = false;
   if (a0.tokens != a1.tokens || a0.tokens > 4 || a0.tokens * topk > 32 || a0.cols != a1.cols || topk > 64 || topk > experts) return KX_OK;
   int ri0, ri1;
-  const int CR0 = gemv_plan(KX_EPI_SWIGLU, a0, ri0, 2), CR1 = gemv_plan(KX_EPI_F32, a1, ri1, 1, 128);
+  const int CR0 = gemv_plan(KX_EPI_SWIGLU, a0, ri0, 2);
+  int CR1 = gemv_plan(KX_EPI_F32, a1, ri1, 1, 128);
   if (CR0 < 0 || CR1 < 0) return KX_ERR_ARG;
+  // The routing waits for the last router workgroup, and a wave with one row per step spends a load's latency on every
+  // step (three tiles of two slices at Kimi shapes: 6.4 us for 43 KB).  Four rows per step and one tile per chunk
+  // where the rows allow: two steps.
+  if (a1.rows % (a1.rs * 4) == 0 && !a1.row_block) {
+    ri1 = 4;
+    a1.nt = 1;
+    CR1 = a1.rs * 4;
+  }
   const int threads = a0.nw * a0.rs * 64;
   if (threads != a1.nw * a1.rs * 64 || experts > threads || experts > 1024) return KX_OK;
   const int S = a0.cols / 512, T = a0.tokens;
@@ -346,9 +355,11 @@ int kx_gemv_pair_route_launch(KxGemvArgs a0, KxGemvArgs a1, const float *bias, u
   r.routed_scale = routed_scale; r.counts = counts; r.offsets = offsets; r.pairs = pairs; r.work = work; r.n_active = n_active; r.pair_work = pair_work;
   const int tt = T >= 4 ? 4 : T >= 2 ? 2 : 1;
   dim3 g(n0 + n1), blk(threads);
-#define KX_PAIR(R, TT_) hipLaunchKernelGGL((gemv_pair_k<R, TT_>), g, blk, lds, st, a0, a1, n0, r)
-  if (ri0 == 2) { if (tt == 4) KX_PAIR(2, 4); else if (tt == 2) KX_PAIR(2, 2); else KX_PAIR(2, 1); }
-  else          { if (tt == 4) KX_PAIR(1, 4); else if (tt == 2) KX_PAIR(1, 2); else KX_PAIR(1, 1); }
+#define KX_PAIR(R, R1, TT_) hipLaunchKernelGGL((gemv_pair_k<R, R1, TT_>), g, blk, lds, st, a0, a1, n0, r)
+#define KX_PAIR_TT(R, R1) do { if (tt == 4) KX_PAIR(R, R1, 4); else if (tt == 2) KX_PAIR(R, R1, 2); else KX_PAIR(R, R1, 1); } while (0)
+  if (ri0 == 2) { if (ri1 == 4) KX_PAIR_TT(2, 4); else KX_PAIR_TT(2, 1); }
+  else          { if (ri1 == 4) KX_PAIR_TT(1, 4); else KX_PAIR_TT(1, 1); }
+#undef KX_PAIR_TT
 #undef KX_PAIR
   KX_LAUNCH_CHECK();
   *fused = true;
