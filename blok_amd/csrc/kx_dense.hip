@@ -239,6 +239,10 @@ int gemv_plan(int epi, KxGemvArgs &a, int &ri, int ri_max, int target_chunks = 2
   for (int d = 2; d <= 8; ++d)
     if (S % d == 0) a.nw = d;
   a.rs = 8 / a.nw;
+  // 3, 5 or 6 slice waves leave the workgroup short of 8 waves (6, 5, 6; 7 slice waves are 7), and a wave that goes through its tiles one
+  // load latency at a time then has too little in flight for the CU: twice the row sets (12, 10, 12 waves).  The q_b
+  // GEMV (1536 columns) goes through six tiles per wave.
+  if ((a.nw == 3 || a.nw == 5 || a.nw == 6) && a.tokens == 1) a.rs *= 2;  // one token: the kernels that take 1024 threads
   while (a.rs > 1 && a.rs > a.rows) a.rs >>= 1;
   // rows per wave and tile, tiles per chunk: a few hundred chunks when the matrix allows
   ri = a.rows >= 2048 * a.rs ? 4 : a.rows >= 768 * a.rs ? 2 : 1;
