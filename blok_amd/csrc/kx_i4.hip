@@ -388,7 +388,8 @@ __device__ __forceinline__ void i4_body(const I4Args &a, const int bid, const in
       for (int idx = threadIdx.x; idx < CR * TT; idx += blockDim.x) {
         const int rc = idx % CR, t = idx / CR;
         if (pc + t < cur.p_end && cur.c0 + rc >= cur.c_first) {  // a moved-back chunk skips the rows it shares
-          const int pair = !a.work ? pc + t : a.pairs[pc + t];
+          // the first pair of the group is in the work record: no load in the tail of a one-pair group
+          const int pair = !a.work ? pc + t : (pc + t == cur.p_begin ? cur.first_pair : a.pairs[pc + t]);
           const float *p0 = part + ((0 * CR + rc) * TT + t) * ks;
           float y0 = p0[0];
           for (int q = 1; q < ks; ++q) y0 += p0[q];
