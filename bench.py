@@ -138,9 +138,9 @@ def run_moe_layer(args, emit=True):
     def step(i, timed=None):
         w = layers.layers[i % n_layers]
         if timed is None:
-            check(lib.kx_moe_decode_layer(C.byref(cfg), C.byref(w), ws, dn.ptr, dx.ptr, T, 0, None))
+            check(lib.kx_moe_decode_layer(C.byref(cfg), C.byref(w), ws, dn.ptr, dx.ptr, T, args.moe_flags, None))
         else:
-            check(lib.kx_moe_decode_layer_timed(C.byref(cfg), C.byref(w), ws, dn.ptr, dx.ptr, T, 0, None, timed))
+            check(lib.kx_moe_decode_layer_timed(C.byref(cfg), C.byref(w), ws, dn.ptr, dx.ptr, T, args.moe_flags, None, timed))
 
     for i in range(args.warmup):
         step(i)
@@ -228,7 +228,8 @@ def run_moe_layer(args, emit=True):
         "data": "synthetic",
         "config": {"workload": f"moe_decode_layer (BASELINE config 2), T={T}, hidden 7168, 384 experts top-8, "
                                f"moe_inter 2048, shared 2048; {n_layers} independent layers cycled (cold weights)",
-                   "tokens": T, "distinct_experts_per_step": round(U, 2), "device": name.value.decode(),
+                   "tokens": T, "distinct_experts_per_step": round(U, 2), "layer_flags": hex(args.moe_flags),
+                   "layer_gbs": round(layer_gbs, 1), "device": name.value.decode(),
                    "compute_units": cus.value},
         "roofline": {"bound": "hbm", "achieved": round(gate_up_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gate_up_gbs / HBM_PEAK_GBS, 4),
@@ -622,6 +623,9 @@ def main():
     ap.add_argument("--stack-layers", type=int, default=24)
     ap.add_argument("--cpu-layers", type=int, default=2)
     ap.add_argument("--tokens", type=int, default=1)
+    ap.add_argument("--moe-flags", type=lambda v: int(v, 0), default=0,
+                    help="moe_layer: flags of kx_moe_decode_layer (0: the bit-reproducible kernels; 0x400: routed experts with "
+                         "several pairs on the matrix cores, 0x200: the shared expert too, both within 1e-2 of the default)")
     ap.add_argument("--layers", type=int, default=4, help="independent layers cycled to keep weights cold")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true")
