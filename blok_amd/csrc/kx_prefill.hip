@@ -19,8 +19,9 @@
 //    of the step's j-th MFMA when that MFMA contracts over columns {8 j .. +7} and
 //    {32 + 8 j .. +7} (the contraction order within a step is free, the activation operand
 //    uses the same columns).  The 16-byte pieces of a row are stored xor-swizzled by the row
-//    so that the lanes' reads are free of bank conflicts.  Group scales are staged in LDS
-//    for eight K steps at a time (32 bytes per row and matrix, one load per thread);
+//    so that the lanes' reads are free of bank conflicts.  Group scales are copied to LDS
+//    the same way, sixteen K steps at a time: 64 bytes per row and matrix, a whole sector of the row (blocks of
+//    eight steps fetched half of every sector twice);
 //  * bf16 weights (shared expert, router gate) are loaded by the lanes themselves, 64
 //    contiguous bytes per lane and step, one step ahead;
 //  * the gathered activation rows go through a double-buffered LDS tile, one barrier per step; with INT4
@@ -54,7 +55,8 @@ typedef _Float16 kx_h2 __attribute__((ext_vector_type(2)));
 constexpr int BN = 256, BK = 64;  // a token tile has up to 4 blocks of 32 tokens (PfArgs::nb_max)
 constexpr int LDS_STRIDE = BK + 8;  // bf16 elements per LDS row: 144 B keeps 16-byte reads of a column of rows spread over banks
 constexpr int W_STAGE = BN * 64;               // bytes of one matrix's packed words for two K steps
-constexpr int SC_STRIDE = 40;                  // bytes per (row, matrix) of staged scales: 16 bf16 + pad against bank conflicts
+constexpr int SC_BLOCK = 16;                   // K steps per staged block of group scales
+constexpr int SC_STRIDE = SC_BLOCK * 4;        // bytes per (row, matrix) of a block: 32 bf16, one 64-byte sector of the row
 
 struct PfArgs {
   const void *w0, *w1;          // INT4: packed i32 [E][N][K/8]; BF16: bf16 [E][N][K]
@@ -113,11 +115,12 @@ __global__ void __launch_bounds__(WAVES * 64, (I4 || WAVES < 8) ? 1 : 2) grouped
   static_assert(!I4 || WAVES == 8, "the INT4 path is laid out for 8 waves");
   constexpr int MATS = DUAL ? 2 : 1;
   extern __shared__ __attribute__((aligned(16))) uint8_t pf_lds[];
-  const int BM = a.nb_max * 32, XT = BM * LDS_STRIDE;   // tokens and elements of one activation tile
+  const int BM = a.nb_max * 32, XT = BM * (I4 ? BK : LDS_STRIDE);  // tokens and elements of one activation tile
   uint16_t *xs_lds = (uint16_t *)pf_lds;                 // two activation tiles
   uint8_t *w_ring = pf_lds + 2 * XT * 2;                 // INT4: [2 stages][MATS][256 rows][4 pieces of 16 B]
-  uint8_t *sc_lds = w_ring + 2 * MATS * W_STAGE;         // INT4: [2][256 rows * MATS][SC_STRIDE]
+  uint8_t *sc_lds = w_ring + 2 * MATS * W_STAGE;         // INT4: [2 blocks][MATS][256 rows][SC_STRIDE]
   const uint32_t ring0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)w_ring;  // LDS address of the ring
+  const uint32_t sc0 = ring0 + 2 * MATS * W_STAGE;                                                  // of the scale blocks
   const uint32_t xs0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)pf_lds;    // and of the activation tiles
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lr = lane & 31, lh = lane >> 5;
@@ -155,23 +158,23 @@ __global__ void __launch_bounds__(WAVES * 64, (I4 || WAVES < 8) ? 1 : 2) grouped
         pf_copy16_to_lds(dma_src[u] + ss * 16, ring0 + (ss & 1) * MATS * W_STAGE + dma_dst[u]);
     }
   };
-  // scale staging: thread -> (row, matrix), 16 scales = 8 K steps per load
-  const int sc_row = MATS == 2 ? tid >> 1 : tid, sc_m = MATS == 2 ? (tid & 1) : 0;
-  const bool sc_active = I4 && sc_row < BN;
-  const uint16_t *sc_src = (sc_m ? a.s1 : a.s0) + (I4 ? (size_t)e * a.expert_s + (size_t)min(n0 + sc_row, a.N - 1) * (a.K >> 5) : 0);
-  uint2 sc_regs[4];
-  auto load_scales = [&](int blk) {
-    if (sc_active) {
-      const uint2 *p = (const uint2 *)(sc_src + blk * 16);
+  // group scales: blocks of SC_BLOCK K steps, 64 bytes per row and matrix -- whole sectors -- copied global -> LDS.
+  // Instruction c = wave * 2 MATS + i covers pieces 64 c .. +63 of [MATS][256 rows][4 pieces]; a last block of half
+  // the steps (K / 64 an odd multiple of 8) repeats its two pieces, the copies land in slots that are never read.
+  const uint16_t *sc_src[MATS * 2];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) sc_regs[i] = p[i];
-    }
-  };
-  auto store_scales = [&](int blk) {
-    if (sc_active) {
-      uint2 *d = (uint2 *)(sc_lds + (blk & 1) * (BN * MATS * SC_STRIDE) + (sc_row * MATS + sc_m) * SC_STRIDE);
+  for (int i = 0; i < MATS * 2; ++i) {
+    const int c = wave * MATS * 2 + i, m = c >> 4, row = (c & 15) * 16 + (lane >> 2);
+    sc_src[i] = (m ? a.s1 : a.s0) + (I4 ? (size_t)e * a.expert_s + (size_t)min(n0 + row, a.N - 1) * (a.K >> 5) : 0);
+  }
+  auto copy_scales = [&](int blk) {
+    if (I4) {
+      const int left = (nk - blk * SC_BLOCK) >> 2;  // 16-byte pieces of the row from this block on: 2 or at least 4
+      const int piece = min(lane & 3, left - 1);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) d[i] = sc_regs[i];
+      for (int i = 0; i < MATS * 2; ++i)
+        pf_copy16_to_lds(sc_src[i] + blk * (SC_BLOCK * 2) + piece * 8,
+                         sc0 + (blk & 1) * (BN * MATS * SC_STRIDE) + (wave * MATS * 2 + i) * 1024);
     }
   };
   // activation staging: thread -> rows tid/4 + q * (16 WAVES), 16 columns from (tid%4)*16
@@ -258,8 +261,8 @@ __global__ void __launch_bounds__(WAVES * 64, (I4 || WAVES < 8) ? 1 : 2) grouped
             const int q = (ks & 1) * 2 + lh;
             const uint8_t *st = w_ring + ((ks >> 1) & 1) * MATS * W_STAGE + m * W_STAGE;
             r.q[m] = *(const uint4 *)(st + (trow * 4 + (q ^ ((trow >> 2) & 3))) * 16);
-            const uint8_t *sb = sc_lds + ((ks >> 3) & 1) * (BN * MATS * SC_STRIDE) + (trow * MATS + m) * SC_STRIDE;
-            r.sc[m] = kx_bf16_f32(*(const uint16_t *)(sb + ((ks & 7) * 2 + lh) * 2));
+            const uint8_t *sb = sc_lds + ((ks / SC_BLOCK) & 1) * (BN * MATS * SC_STRIDE) + (m * BN + trow) * SC_STRIDE;
+            r.sc[m] = kx_bf16_f32(*(const uint16_t *)(sb + ((ks % SC_BLOCK) * 2 + lh) * 2));
           } else {
 #pragma unroll
             for (int j = 0; j < 4; ++j) r.b[m][j] = *(const uint4 *)(wb_ptr[m] + ks * BK + j * 8);
@@ -327,26 +330,27 @@ __global__ void __launch_bounds__(WAVES * 64, (I4 || WAVES < 8) ? 1 : 2) grouped
         else __syncthreads();
       };
       WRaw w0, w1;
-      load_scales(0);
       if (I4) {
+        copy_scales(0);
         copy_x(0);
         dma_stage(0);
       } else {
         load_x(0);
         fetch_w(w0, 0);
       }
-      store_scales(0);
       if (!I4) store_x(xs_lds);
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       barrier();
       for (int ks = 0; ks < nk; ks += 2) {
         // even step: the other ring stage and the other activation tile were last read behind a barrier.  Order of
-        // issue: scales, activations of the next step, then the ring copies; the activations have to land by the
-        // end of this step, the ring copies stay in flight until the end of the odd step
-        if ((ks & 7) == 0 && ks + 8 < nk) load_scales((ks >> 3) + 1);
+        // issue: activations of the next step, the ring copies, then (every SC_BLOCK steps) the next scale block; the
+        // activations have to land by the end of this step, the copies behind them stay in flight until the end of
+        // the odd step (a wave's copies complete in the order of issue)
+        const bool scales_now = I4 && ks % SC_BLOCK == 0 && ks + SC_BLOCK < nk;
         if (I4) {
           if (ks + 1 < nk) copy_x(ks + 1);
           if (ks + 2 < nk) dma_stage((ks >> 1) + 1);
+          if (scales_now) copy_scales(ks / SC_BLOCK + 1);
           fetch_w(w0, ks);
         } else {
           if (ks + 1 < nk) load_x(ks + 1);
@@ -354,7 +358,8 @@ __global__ void __launch_bounds__(WAVES * 64, (I4 || WAVES < 8) ? 1 : 2) grouped
         }
         step(w0, ks);
         if (I4) {
-          if (ks + 2 < nk) pf_wait_copies<MATS * 2>();
+          if (scales_now) pf_wait_copies<MATS * 4>();
+          else if (ks + 2 < nk) pf_wait_copies<MATS * 2>();
           else pf_wait_copies<0>();
         } else if (ks + 1 < nk) {
           store_x(xs_lds + XT);
@@ -370,7 +375,6 @@ __global__ void __launch_bounds__(WAVES * 64, (I4 || WAVES < 8) ? 1 : 2) grouped
           }
           step(w1, ks + 1);
           if (!I4 && ks + 2 < nk) store_x(xs_lds);
-          if ((ks & 7) == 6 && ks + 2 < nk) store_scales((ks >> 3) + 1);
           asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's copies (ring stage, activations) have landed
           barrier();
         }
@@ -450,7 +454,7 @@ int kx_grouped_gemm_launch(bool dual, bool i4, const void *w0, const uint16_t *s
   const int waves = i4 ? 8 : (N / 256 * tiles >= 192 ? 8 : N / 64 * tiles >= 192 ? 2 : 1);
   dim3 g(kx_cdiv(N, waves * 32), work ? n_slots : 1, mz), b(waves * 64);
   const int mats = dual ? 2 : 1;
-  const size_t lds = (size_t)2 * BM * LDS_STRIDE * 2 + (i4 ? (size_t)2 * mats * W_STAGE + (size_t)2 * BN * mats * SC_STRIDE : 0);
+  const size_t lds = (size_t)2 * BM * (i4 ? BK : LDS_STRIDE) * 2 + (i4 ? (size_t)2 * mats * W_STAGE + (size_t)2 * BN * mats * SC_STRIDE : 0);
   static std::atomic<bool> attr_set{false};  // setting it twice from two threads is harmless
   if (!attr_set) {  // more than 64 KB of dynamic LDS has to be allowed per kernel
     KX_HIP(hipFuncSetAttribute((const void *)grouped_gemm_k<true, true, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
