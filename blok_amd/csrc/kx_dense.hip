@@ -137,6 +137,8 @@ __global__ void __launch_bounds__(TT > 1 ? 512 : 1024) gemv_absorb_k(KxGemvArgs 
   __shared__ float ab_q[256];
   __shared__ float ab_ws[4];
   __shared__ int s_last;
+  // The cache row is the first workgroup's job: its dependent loads are answered fast while the launch is young (the
+  // same job given to the last workgroup, which starts once the memory pipeline is full, made the launch 2 us longer).
   if (blockIdx.x == 0) {
     const int kva = q.kv_rank + q.rope;
     for (int t = 0; t < a.tokens; ++t)
@@ -251,6 +253,11 @@ int gemv_plan(int epi, KxGemvArgs &a, int &ri, int ri_max, int target_chunks = 2
   if (ri > ri_max) ri = ri_max;
   const int rt = a.rs * ri;
   int nt = a.rows / (rt * target_chunks);
+  // From two tokens on a CU holds one workgroup of these kernels, not two (150-210 registers against 128): more chunks
+  // than CUs would be a second round of a few workgroups, so the chunks are made long enough for one round where
+  // eight tiles allow it.  (Twice the rows per tile on top of that, to put a one-token launch's bytes in flight per CU,
+  // changed nothing.)
+  if (a.tokens >= 2) nt = kx_cdiv(a.rows, rt * (target_chunks < 256 ? target_chunks : 256));
   nt = nt < 1 ? 1 : nt > 8 ? 8 : nt;
   if (a.row_block) {  // a chunk must not straddle blocks
     if (!(a.rows % a.row_block == 0 && a.row_block % rt == 0)) { kx_set_error("kx_gemv: row_block=%d does not fit tiles of %d rows", a.row_block, rt); return -1; }
@@ -313,7 +320,7 @@ int kx_gemv_launch(int epi, KxGemvArgs a, hipStream_t st) {
       b.expert_out = a.expert_out + (size_t)t0 * a.topk * a.rows;
       b.route_w = a.route_w + (size_t)t0 * a.topk;
     }
-    const int tt = b.tokens >= 4 ? 4 : b.tokens >= 2 ? 2 : 1;
+    const int tt = b.tokens >= 3 ? 4 : b.tokens >= 2 ? 2 : 1;
     const int chunks = kx_cdiv(a.rows, CR);
     const size_t lds = (size_t)mats * CR * b.tokens * S * sizeof(float);
     KX_REQUIRE(lds <= 160 * 1024, "kx_gemv: %zu bytes of LDS needed", lds);
@@ -334,9 +341,8 @@ int kx_gemv_pair_route_launch(KxGemvArgs a0, KxGemvArgs a1, const float *bias, u
   *fused = false;
   if (a0.tokens != a1.tokens || a0.tokens > 4 || a0.tokens * topk > 32 || a0.cols != a1.cols || topk > 64 || topk > experts) return KX_OK;
   int ri0, ri1;
-  const int CR0 = gemv_plan(KX_EPI_SWIGLU, a0, ri0, 2);
   int CR1 = gemv_plan(KX_EPI_F32, a1, ri1, 1, 128);
-  if (CR0 < 0 || CR1 < 0) return KX_ERR_ARG;
+  if (CR1 < 0) return KX_ERR_ARG;
   // The routing waits for the last router workgroup, and a wave with one row per step spends a load's latency on every
   // step (three tiles of two slices at Kimi shapes: 6.4 us for 43 KB).  Four rows per step and one tile per chunk
   // where the rows allow: two steps.
@@ -345,6 +351,10 @@ int kx_gemv_pair_route_launch(KxGemvArgs a0, KxGemvArgs a1, const float *bias, u
     a1.nt = 1;
     CR1 = a1.rs * 4;
   }
+  // from two tokens on the two parts share one round of workgroups (see gemv_plan)
+  const int left = 256 - kx_cdiv(a1.rows, CR1);
+  const int CR0 = gemv_plan(KX_EPI_SWIGLU, a0, ri0, 2, a0.tokens >= 2 && left >= 64 ? left : 256);
+  if (CR0 < 0) return KX_ERR_ARG;
   const int threads = a0.nw * a0.rs * 64;
   if (threads != a1.nw * a1.rs * 64 || experts > threads || experts > 1024) return KX_OK;
   const int S = a0.cols / 512, T = a0.tokens;
@@ -357,7 +367,7 @@ int kx_gemv_pair_route_launch(KxGemvArgs a0, KxGemvArgs a1, const float *bias, u
   r.counter = counter; r.bias = bias; r.ids = ids; r.weights = weights; r.experts = experts; r.topk = topk;
   a1.flags |= KX_GEMV_COHERENT_OUT;
   r.routed_scale = routed_scale; r.counts = counts; r.offsets = offsets; r.pairs = pairs; r.work = work; r.n_active = n_active; r.pair_work = pair_work;
-  const int tt = T >= 4 ? 4 : T >= 2 ? 2 : 1;
+  const int tt = T >= 3 ? 4 : T >= 2 ? 2 : 1;
   dim3 g(n0 + n1), blk(threads);
 #define KX_PAIR(R, R1, TT_) hipLaunchKernelGGL((gemv_pair_k<R, R1, TT_>), g, blk, lds, st, a0, a1, n0, r)
 #define KX_PAIR_TT(R, R1) do { if (tt == 4) KX_PAIR(R, R1, 4); else if (tt == 2) KX_PAIR(R, R1, 2); else KX_PAIR(R, R1, 1); } while (0)
@@ -378,8 +388,9 @@ int kx_gemv_absorb_launch(KxGemvArgs g, const QAbsArgs &q0, bool *fused, hipStre
       !q.head_count || !q.cache)
     return KX_OK;
   int ri;
-  const int CR = gemv_plan(KX_EPI_BF16, g, ri, 4);
+  int CR = gemv_plan(KX_EPI_BF16, g, ri, 4, g.tokens >= 2 ? 255 : 256);  // one workgroup more writes the cache row
   if (CR < 0) return KX_ERR_ARG;
+  while (qk % CR && g.nt < 16) CR = CR / g.nt * (g.nt + 1), ++g.nt;  // whole chunks per head
   const int threads = g.nw * g.rs * 64;
   if (qk % CR || g.rows / CR + 1 > 4096 || (threads < 256 && q.kv_rank / 8 > threads) || q.rope / 2 > threads) return KX_OK;
   q.head_chunks = qk / CR;
@@ -387,7 +398,7 @@ int kx_gemv_absorb_launch(KxGemvArgs g, const QAbsArgs &q0, bool *fused, hipStre
   const int S = g.cols / 512;
   const size_t lds = (size_t)CR * g.tokens * S * sizeof(float);
   KX_REQUIRE(lds <= 128 * 1024, "kx_gemv: %zu bytes of LDS needed", lds);
-  const int tt = g.tokens >= 4 ? 4 : g.tokens >= 2 ? 2 : 1;
+  const int tt = g.tokens >= 3 ? 4 : g.tokens >= 2 ? 2 : 1;
   dim3 grid(g.rows / CR + 1), blk(threads);
 #define KX_ABS(R, TT_) hipLaunchKernelGGL((gemv_absorb_k<R, TT_>), grid, blk, lds, st, g, q)
 #define KX_ABS_TT(R) do { if (tt == 4) KX_ABS(R, 4); else if (tt == 2) KX_ABS(R, 2); else KX_ABS(R, 1); } while (0)
