@@ -87,6 +87,16 @@ int kx_mla_span_tiles(int seq) {
 // sequences get more, shorter spans so that sequences x spans fills the chip -- up to 256 spans, merged 64 at a time.
 // Beyond 32 entries (the launches of a prefill step) the entries alone fill the chip and every span costs a row of
 // partials that is written and read back: down to 4 spans.
+static int mla_compute_units() {  // of the current device, asked once
+  static std::atomic<int> cus{0};
+  int v = cus.load();
+  if (!v) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
+    cus = v;
+  }
+  return v;
+}
 static int mfma_span_cap(int batch) {
   if (batch > 32) return 2048 / batch < 4 ? 4 : 2048 / batch;
   const int want = 1024 / (batch > 0 ? batch : 1);
@@ -202,15 +212,20 @@ struct MlaArgs {
 // of the score pass and the column-per-lane reads of the PV pass are free of bank conflicts).
 constexpr int MLA_R = 512, MLA_KVA = 576, MLA_PITCH = 584;  // bf16 elements; 1168 B per staged row
 
-template <int HG>
-__global__ void __launch_bounds__(256) mla_partial_k(MlaArgs a) {
+// W waves per workgroup, HG heads per wave.  The waves of a workgroup share the staged tile; with W = 6 .. 8 (HG = 1)
+// the last workgroup of a span may hold waves past the last head: they stage and keep the barriers, and compute the
+// last head again without storing it.
+template <int HG, int W = 4>
+__global__ void __launch_bounds__(W * 64) mla_partial_k(MlaArgs a) {
   constexpr int R = MLA_R, KVA = MLA_KVA, PITCH = MLA_PITCH;
-  extern __shared__ __attribute__((aligned(16))) uint16_t tile_lds[];  // [64][PITCH] then p [4][HG][64] floats
+  extern __shared__ __attribute__((aligned(16))) uint16_t tile_lds[];  // [64][PITCH] then p [W][HG][64] floats
   float(*p_lds)[HG][64] = (float(*)[HG][64])(tile_lds + 64 * PITCH);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: q is then read through the scalar path
   const int span = blockIdx.x, b = blockIdx.z;
-  const int h0 = (blockIdx.y * 4 + wave) * HG;
+  const int h_own = (blockIdx.y * W + wave) * HG;
+  const bool h_valid = h_own < a.heads;
+  const int h0 = h_valid ? h_own : a.heads - HG;
   const int seq = a.seqs ? a.seq - (int)(gridDim.z / a.seqs) + 1 + b / a.seqs : a.seq;
   const uint16_t *cache = a.cache + (size_t)(a.seqs ? b % a.seqs : b) * a.seq_stride;
   const float *q = a.qabs + ((size_t)b * a.heads + h0) * KVA;
@@ -229,16 +244,17 @@ __global__ void __launch_bounds__(256) mla_partial_k(MlaArgs a) {
     // stage rows t0 .. t0+n-1: 72 pieces of 16 bytes per row, 18 per thread
     {
       const uint4 *src = (const uint4 *)(cache + (size_t)t0 * KVA);
-      uint4 v[18];
+      constexpr int NP = (64 * 72 + W * 64 - 1) / (W * 64);  // pieces per thread: 18 with four waves
+      uint4 v[NP];
 #pragma unroll
-      for (int i = 0; i < 18; ++i) {
-        const int idx = threadIdx.x + i * 256;  // piece (row, j) = (idx / 72, idx % 72)
+      for (int i = 0; i < NP; ++i) {
+        const int idx = threadIdx.x + i * (W * 64);  // piece (row, j) = (idx / 72, idx % 72)
         v[i] = idx < n * 72 ? src[idx] : make_uint4(0, 0, 0, 0);
       }
 #pragma unroll
-      for (int i = 0; i < 18; ++i) {
-        const int idx = threadIdx.x + i * 256, row = idx / 72, j = idx - row * 72;
-        *(uint4 *)(tile_lds + row * PITCH + j * 8) = v[i];
+      for (int i = 0; i < NP; ++i) {
+        const int idx = threadIdx.x + i * (W * 64), row = idx / 72, j = idx - row * 72;
+        if ((64 * 72) % (W * 64) == 0 || idx < 64 * 72) *(uint4 *)(tile_lds + row * PITCH + j * 8) = v[i];
       }
     }
     __syncthreads();
@@ -296,6 +312,7 @@ __global__ void __launch_bounds__(256) mla_partial_k(MlaArgs a) {
   }
 #pragma unroll
   for (int h = 0; h < HG; ++h) {
+    if (!h_valid) break;
     const size_t idx = ((size_t)b * a.spans + span) * a.heads + h0 + h;
     if (lane == 0) { a.pm[idx] = M[h]; a.pz[idx] = Z[h]; }
     float4 *o = (float4 *)(a.po + idx * R + lane * 8);
@@ -742,11 +759,24 @@ int kx_mla_partials_launch(const kx_config *c, const uint16_t *cache, size_t seq
   const long waves1 = (long)batch * a.spans * c->heads;  // waves at one head per wave
   int hg = 1;
   while (hg < 8 && c->heads % (4 * hg * 2) == 0 && waves1 / (hg * 2) >= 4096) hg *= 2;
-  dim3 g(a.spans, c->heads / (4 * hg), batch), b(256);
-  const size_t lds = (size_t)64 * MLA_PITCH * 2 + (size_t)4 * hg * 64 * sizeof(float);
+  // One head per wave and more workgroups of four waves than CUs, but not many more (a context of 1100 positions and
+  // one sequence: 18 spans x 16 = 288): the CUs that get two take half as long again as the rest, and that is the
+  // launch.  Six to eight waves per workgroup -- fewer, wider workgroups that share a tile among more heads -- where
+  // that brings the launch to one workgroup per CU.  (Measured on the decode steps of the 24-layer stack at 1030-1290
+  // positions, tok/s: four waves 247.7, five 248.7 where they fit, six 251.2, seven 248.8, eight 248.9.)
+  int wv = 4;
+  if (hg == 1 && !use_mfma && (long)batch * a.spans * (c->heads / 4) > mla_compute_units()) {
+    for (int w = 6; w <= 8 && wv == 4; ++w)
+      if ((long)batch * a.spans * kx_cdiv(c->heads, w) <= mla_compute_units()) wv = w;
+  }
+  dim3 g(a.spans, kx_cdiv(c->heads, wv * hg), batch), b(wv * 64);
+  const size_t lds = (size_t)64 * MLA_PITCH * 2 + (size_t)wv * hg * 64 * sizeof(float);
   static std::atomic<bool> attr_set{false};  // setting it twice from two threads is harmless
   if (!attr_set) {  // more than 64 KB of dynamic LDS has to be allowed per kernel
     KX_HIP(hipFuncSetAttribute((const void *)mla_partial_k<1>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
+    KX_HIP(hipFuncSetAttribute((const void *)mla_partial_k<1, 6>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
+    KX_HIP(hipFuncSetAttribute((const void *)mla_partial_k<1, 7>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
+    KX_HIP(hipFuncSetAttribute((const void *)mla_partial_k<1, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
     KX_HIP(hipFuncSetAttribute((const void *)mla_partial_k<2>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
     KX_HIP(hipFuncSetAttribute((const void *)mla_partial_k<4>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
     KX_HIP(hipFuncSetAttribute((const void *)mla_partial_k<8>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
@@ -764,7 +794,10 @@ int kx_mla_partials_launch(const kx_config *c, const uint16_t *cache, size_t seq
     out->pm = a.pm; out->pz = a.pz; out->po = a.po; out->spans = a.spans;
     return KX_OK;
   }
-  if (hg == 1) hipLaunchKernelGGL(mla_partial_k<1>, g, b, lds, st, a);
+  if (hg == 1 && wv == 6) hipLaunchKernelGGL((mla_partial_k<1, 6>), g, b, lds, st, a);
+  else if (hg == 1 && wv == 7) hipLaunchKernelGGL((mla_partial_k<1, 7>), g, b, lds, st, a);
+  else if (hg == 1 && wv == 8) hipLaunchKernelGGL((mla_partial_k<1, 8>), g, b, lds, st, a);
+  else if (hg == 1) hipLaunchKernelGGL(mla_partial_k<1>, g, b, lds, st, a);
   else if (hg == 2) hipLaunchKernelGGL(mla_partial_k<2>, g, b, lds, st, a);
   else if (hg == 4) hipLaunchKernelGGL(mla_partial_k<4>, g, b, lds, st, a);
   else hipLaunchKernelGGL(mla_partial_k<8>, g, b, lds, st, a);

@@ -302,9 +302,10 @@ def test_q_absorb_operator(kxlib, ox, tokens):
     assert (exp.view(np.uint32) == got[:, :, :R].view(np.uint32)).all()
 
 
-@pytest.mark.parametrize("batch,seq", [(1, 1), (1, 100), (2, 700), (1, 5000)])
+@pytest.mark.parametrize("batch,seq", [(1, 1), (1, 100), (2, 700), (1, 1100), (1, 1500), (1, 2000), (1, 5000)])
 def test_mla_decode_operator(kxlib, ox, batch, seq):
-    # BASELINE config 3 shapes (64 heads, latent 512+64) at lengths the scalar oracle finishes quickly
+    # BASELINE config 3 shapes (64 heads, latent 512+64) at lengths the scalar oracle finishes quickly; 1100, 2 x 700,
+    # 1500 and 2000 positions take workgroups of six, six, seven and eight waves (one head each) instead of four
     say(f"mla decode batch={batch} seq={seq}")
     cfg = default_config()
     H, KVA, R = cfg.heads, 576, 512
