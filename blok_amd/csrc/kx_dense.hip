@@ -259,6 +259,12 @@ int gemv_plan(int epi, KxGemvArgs &a, int &ri, int ri_max, int target_chunks = 2
   // changed nothing.)
   if (a.tokens >= 2) nt = kx_cdiv(a.rows, rt * (target_chunks < 256 ? target_chunks : 256));
   nt = nt < 1 ? 1 : nt > 8 ? 8 : nt;
+  // One token: a CU holds two workgroups, and a plan that gives a few more chunks than CUs (q_a|kv_a at Kimi shapes:
+  // 264) leaves a few CUs with twice the bytes of the rest: one more tile per chunk (176 chunks; 250.3 -> 250.9 tok/s).
+  if (a.tokens == 1 && nt < 8) {
+    const int chunks = kx_cdiv(a.rows, rt * nt);
+    if (chunks > 256 && chunks <= 320) ++nt;
+  }
   if (a.row_block) {  // a chunk must not straddle blocks
     if (!(a.rows % a.row_block == 0 && a.row_block % rt == 0)) { kx_set_error("kx_gemv: row_block=%d does not fit tiles of %d rows", a.row_block, rt); return -1; }
     while (a.row_block % (rt * nt)) --nt;
