@@ -159,8 +159,10 @@ __global__ void __launch_bounds__(WAVES * 64, (I4 || WAVES < 8) ? 1 : 2) grouped
     }
   };
   // group scales: blocks of SC_BLOCK K steps, 64 bytes per row and matrix -- whole sectors -- copied global -> LDS.
-  // Instruction c = wave * 2 MATS + i covers pieces 64 c .. +63 of [MATS][256 rows][4 pieces]; a last block of half
-  // the steps (K / 64 an odd multiple of 8) repeats its two pieces, the copies land in slots that are never read.
+  // Instruction c = wave * 2 MATS + i covers pieces 64 c .. +63 of [MATS][256 rows][4 slots]; slot s of row r holds
+  // piece s ^ ((r / 2) % 4): a wave reads one 2-byte scale per row at the same offset of 32 consecutive rows, and with
+  // the pieces in place (64-byte rows) those fall into two banks; xor-ed by the row they fall into eight.  A last block of
+  // half the steps (K / 64 an odd multiple of 8) repeats its two pieces, the copies land in slots that are never read.
   const uint16_t *sc_src[MATS * 2];
 #pragma unroll
   for (int i = 0; i < MATS * 2; ++i) {
@@ -170,7 +172,7 @@ __global__ void __launch_bounds__(WAVES * 64, (I4 || WAVES < 8) ? 1 : 2) grouped
   auto copy_scales = [&](int blk) {
     if (I4) {
       const int left = (nk - blk * SC_BLOCK) >> 2;  // 16-byte pieces of the row from this block on: 2 or at least 4
-      const int piece = min(lane & 3, left - 1);
+      const int piece = min((lane & 3) ^ ((lane >> 3) & 3), left - 1);  // row = 16 (c % 16) + lane / 4
 #pragma unroll
       for (int i = 0; i < MATS * 2; ++i)
         pf_copy16_to_lds(sc_src[i] + blk * (SC_BLOCK * 2) + piece * 8,
@@ -262,7 +264,8 @@ __global__ void __launch_bounds__(WAVES * 64, (I4 || WAVES < 8) ? 1 : 2) grouped
             const uint8_t *st = w_ring + ((ks >> 1) & 1) * MATS * W_STAGE + m * W_STAGE;
             r.q[m] = *(const uint4 *)(st + (trow * 4 + (q ^ ((trow >> 2) & 3))) * 16);
             const uint8_t *sb = sc_lds + ((ks / SC_BLOCK) & 1) * (BN * MATS * SC_STRIDE) + (m * BN + trow) * SC_STRIDE;
-            r.sc[m] = kx_bf16_f32(*(const uint16_t *)(sb + ((ks % SC_BLOCK) * 2 + lh) * 2));
+            const int el = (ks % SC_BLOCK) * 2 + lh;  // the lane's group among the block's 32
+            r.sc[m] = kx_bf16_f32(*(const uint16_t *)(sb + (((el >> 3) ^ ((trow >> 1) & 3)) * 8 + (el & 7)) * 2));
           } else {
 #pragma unroll
             for (int j = 0; j < 4; ++j) r.b[m][j] = *(const uint4 *)(wb_ptr[m] + ks * BK + j * 8);
