@@ -31,6 +31,9 @@ def test_rmsnorm_parity(kxlib, ox, n, tokens):
     (384, 7168, 1, 1),      # router gate, fp32 logits
     (384, 7168, 8, 1),
     (2112, 7168, 1, 0),     # q_a + kv_a
+    (2112, 7168, 2, 0),     # the same for two and four tokens: one workgroup per CU, chunks planned for one round
+    (2112, 7168, 4, 0),
+    (7168, 8192, 3, 0),     # o_proj, three tokens on the four-token kernel
     (1000, 1536, 3, 0),     # q_b-like, ragged rows
     (128, 512, 2, 0),       # W_UV-like, one slice
     (64, 8192, 1, 0),       # o_proj width

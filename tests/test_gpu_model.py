@@ -206,16 +206,17 @@ def test_kimi_shape_truncated_stack_tokens_identical(kxlib, ox):
 
 def test_kimi_shape_stack_batch_invariance(kxlib, ox):
     # Properties that need no oracle, at Kimi-K2 shapes (4 layers: 1 dense + 3 MoE, full vocabulary): the summation
-    # order of every kernel on the path is independent of the batch, so identical prompts in a batch of 3 (the
-    # 2- and 4-token kernel variants, fused prologues) give the ids, hidden state and logits of the batch-1 run
-    # (1-token variants) to the bit, run after run, and a longer generation extends a shorter one.
+    # order of every kernel on the path is independent of the batch, so identical prompts in a batch of 2, 3 or 4 (the
+    # 2- and 4-token kernel variants with their own launch plans, fused prologues) give the ids, hidden state and
+    # logits of the batch-1 run (1-token variants) to the bit, run after run, and a longer generation extends a
+    # shorter one.
     say("kimi shape 4-layer stack, batch invariance")
     cfg = default_config()
     cfg.n_layers, cfg.first_dense, cfg.max_context, cfg.seed = 4, 1, 48, 5
     prompt_len, n_tokens = 9, 12
     one = O.tokens_u32(prompt_len, cfg.seed, 4, cfg.vocab).reshape(1, prompt_len)
     runs = {}
-    for batch in (1, 3, 1):
+    for batch in (1, 2, 3, 4, 1):
         cfg.max_batch = batch
         km = KxModel(kxlib, cfg)
         rc, out, counts = km.generate(np.repeat(one, batch, axis=0), n_tokens)
@@ -229,10 +230,11 @@ def test_kimi_shape_stack_batch_invariance(kxlib, ox):
             assert rc == 0 and (short[0] == out[0, :5]).all()
         km.close()
     o1, h1, l1 = runs[1]
-    o3, h3, l3 = runs[3]
-    for b in range(3):
-        assert (o3[b] == o1[0]).all(), f"row {b}: {o3[b]} vs {o1[0]}"
-        assert (h3[b] == h1[0]).all() and (l3[b] == l1[0]).all()
+    for batch in (2, 3, 4):
+        ob, hb, lb = runs[batch]
+        for b in range(batch):
+            assert (ob[b] == o1[0]).all(), f"batch {batch}, row {b}: {ob[b]} vs {o1[0]}"
+            assert (hb[b] == h1[0]).all() and (lb[b] == l1[0]).all(), f"batch {batch}, row {b}"
 
 
 @pytest.mark.parametrize("shape", ["small-1", "small-3", "kimi"])
