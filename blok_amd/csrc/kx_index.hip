@@ -240,6 +240,10 @@ static int kx_index_infer_config_body(const char *index_path, kx_config *cfg) {
     if ((t = ix.find(first_dense, "shared_expert_resident", "gate_proj")) && dims(t, r, c2)) cfg->shared_inter = (int32_t)r;
     if ((t = ix.find(first_dense, "routed_expert", "gate_proj.weight_scale", 0)) && dims(t, r, c2)) cfg->moe_inter = (int32_t)r;
   }
+  // A checkpoint is computed with the reference's constant, YARN_FACTOR 64 (src/kimi_exec.cu:184); the library
+  // default of 32 belongs to the seeded random-init configurations.  It enters the RoPE frequencies (:338) and,
+  // through mscale, the softmax scale at every context length (:428-429).
+  cfg->yarn_factor = 64.0f;
   return KX_OK;
 }
 

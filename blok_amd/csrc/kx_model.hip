@@ -92,6 +92,7 @@ struct kx_model {
   int x_row0 = 0;         // first row of x that belongs to the last position of the last step
   bool sampled = false;
   float ms_prefill = 0, ms_decode = 0;
+  int steps_decoded = 0;  // ids sampled per sequence by the last kx_generate (less than asked for when every sequence ended)
   uint64_t load_bytes = 0;  // checkpoint bytes copied in by kx_model_load, and the time that took
   double load_seconds = 0;
 };
@@ -638,20 +639,43 @@ extern "C" int kx_generate(kx_model *m, const uint32_t *h_prompt, int32_t batch,
   if ((rc = kx_prefill(m, h_prompt, batch, prompt_len))) return rc;
   KX_HIP(hipEventRecord(m->ev[1], m->st));
   const int cp = kx_cdiv(batch, 64);
+  // Steps are enqueued without waiting for the host.  When the end-of-sequence id counts, the ids sampled so far are
+  // read back every eighth step, and the loop ends once every sequence has sampled it (:887-888 stop there too):
+  // at most eight steps are decoded for nothing.
+  std::vector<uint32_t> hist((size_t)n_tokens * batch);
+  std::vector<char> ended(batch, 0);
+  int made = 0, seen = 0;  // history rows written on the device, and of those, rows the host has read
+  auto read_back = [&]() -> int {
+    if (seen == made) return KX_OK;
+    KX_HIP(hipMemcpyAsync(hist.data() + (size_t)seen * batch, m->history + (size_t)seen * batch, (size_t)(made - seen) * batch * 4,
+                          hipMemcpyDeviceToHost, m->st));
+    KX_HIP(hipStreamSynchronize(m->st));
+    for (; seen < made; ++seen)
+      for (int b = 0; b < batch; ++b)
+        if (hist[(size_t)seen * batch + b] == m->c.eos_id) ended[b] = 1;
+    return KX_OK;
+  };
   for (int i = 0; i < n_tokens; ++i) {  // :887-890
     hipLaunchKernelGGL(copy_ids_k, dim3(cp), dim3(64), 0, m->st, m->next, m->history + (size_t)i * batch, batch);
     KX_LAUNCH_CHECK();
+    made = i + 1;
+    if (!ignore_eos && (i & 7) == 7) {
+      if ((rc = read_back())) return rc;
+      bool all = true;
+      for (int b = 0; b < batch; ++b) all = all && ended[b];
+      if (all) break;
+    }
     if (i + 1 < n_tokens && (rc = step(m, m->history + (size_t)i * batch, true))) return rc;
   }
   KX_HIP(hipEventRecord(m->ev[2], m->st));
-  std::vector<uint32_t> hist((size_t)n_tokens * batch);
-  KX_HIP(hipMemcpyAsync(hist.data(), m->history, hist.size() * 4, hipMemcpyDeviceToHost, m->st));
+  if ((rc = read_back())) return rc;
   KX_HIP(hipStreamSynchronize(m->st));
   KX_HIP(hipEventElapsedTime(&m->ms_prefill, m->ev[0], m->ev[1]));
   KX_HIP(hipEventElapsedTime(&m->ms_decode, m->ev[1], m->ev[2]));
+  m->steps_decoded = made;
   for (int b = 0; b < batch; ++b) {  // generation stops before the end-of-sequence id is emitted (:887-888)
     int n = 0;
-    for (int i = 0; i < n_tokens; ++i) {
+    for (int i = 0; i < made; ++i) {
       const uint32_t id = hist[(size_t)i * batch + b];
       if (!ignore_eos && id == m->c.eos_id) break;
       h_out[(size_t)b * n_tokens + n++] = id;
@@ -715,6 +739,12 @@ extern "C" int kx_model_set_fusion(kx_model *m, uint32_t mask) {
   KX_REQUIRE(m, "kx_model_set_fusion: null model");
   KX_REQUIRE(!(mask & ~(uint32_t)KX_FUSE_ALL), "kx_model_set_fusion: unknown bits in mask 0x%x", mask);
   m->fusion = mask;
+  return KX_OK;
+}
+
+extern "C" int kx_model_steps_decoded(kx_model *m, int32_t *steps) {
+  KX_REQUIRE(m && steps, "kx_model_steps_decoded: null argument");
+  *steps = m->steps_decoded;
   return KX_OK;
 }
 

@@ -88,6 +88,7 @@ _SIGS = {
     "kx_model_logits": [_P, _P],
     "kx_model_latent": [_P, _I, _I, _I, _I, _P],
     "kx_model_timing": [_P, C.POINTER(C.c_float)],
+    "kx_model_steps_decoded": [_P, C.POINTER(C.c_int32)],
     "kx_model_set_fusion": [_P, C.c_uint32],
     "kx_model_set_attention_kernel": [_P, _I],
     "kx_model_set_routing_record": [_P, C.c_int],

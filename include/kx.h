@@ -270,8 +270,11 @@ int kx_generate(kx_model *model, const uint32_t *h_prompt, int32_t batch, int32_
  *                        reads and their data bytes.  Needs no GPU.
  * kx_index_infer_config: overwrites the shape fields of *cfg (vocab, hidden, n_layers, first_dense,
  *                        q_rank, kv_rank, heads, dense_inter, experts, shared_inter, moe_inter) with what
- *                        the index's tensor shapes say; head dimensions, topk and the numeric constants
- *                        are not in a checkpoint's shapes and stay as they are.  Needs no GPU.
+ *                        the index's tensor shapes say, and sets yarn_factor to 64, the constant the
+ *                        reference computes a checkpoint with (src/kimi_exec.cu:184; kx_config_default's 32
+ *                        is for the seeded random-init configurations; set the field afterwards to
+ *                        override).  Head dimensions, topk and the other numeric constants are not in a
+ *                        checkpoint's shapes and stay as they are.  Needs no GPU.
  * kx_model_load        : a kx_model whose weights are read from the index's files instead of being
  *                        random-init (load_tensor / load_rows, :608-649, which the reference runs per
  *                        tile per token; here once).  kv_b_proj stays whole: its rows h*256+d are
@@ -315,6 +318,10 @@ int kx_model_latent(kx_model *model, int32_t layer, int32_t seq_index, int32_t p
 int kx_model_stream(kx_model *model, void **stream);
 /* ms of GPU time of the last kx_generate: [0] prefill, [1] decode steps                         */
 int kx_model_timing(kx_model *model, float *ms2);
+/* ids sampled per sequence by the last kx_generate.  With ignore_eos = 0 the loop ends once every sequence has
+ * sampled the end-of-sequence id, as the reference's does (src/kimi_exec.cu:887-888); the ids are read back every
+ * eighth step for that, so up to seven steps past the last sequence's end are decoded.             */
+int kx_model_steps_decoded(kx_model *model, int32_t *steps);
 /* Which steps of a decode layer ride inside the launch of the GEMV before them (up to 4 tokens).
  * Results do not depend on the mask (same sums, same rounding points); it exists so that a test
  * can run both forms.  No counterpart in the reference, which launches every step on its own

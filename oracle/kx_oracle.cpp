@@ -45,6 +45,9 @@
 #include <stdlib.h>
 #include <string.h>
 #include <algorithm>
+#include <functional>
+#include <map>
+#include <memory>
 #include <vector>
 #ifdef _OPENMP
 #include <omp.h>
@@ -137,13 +140,18 @@ static inline float rng_normal_f32(uint64_t key, uint64_t i, float sigma) {
   return (float)rng_normal_int(key, i) * (sigma * 1.52587890625e-05f);
 }
 
-void ox_fill_normal_bf16(uint16_t *out, uint64_t n, uint64_t seed, uint64_t tid, float sigma, int absval) {
+// elements first .. first+n-1 of the tensor (a value depends on its index in the whole tensor only)
+static void fill_normal_bf16_at(uint16_t *out, uint64_t first, uint64_t n, uint64_t seed, uint64_t tid, float sigma,
+                                int absval) {
   uint64_t key = rng_key(seed, tid);
 #pragma omp parallel for schedule(static)
   for (int64_t i = 0; i < (int64_t)n; ++i) {
-    uint16_t h = bf16_bits(rng_normal_f32(key, (uint64_t)i, sigma));
+    uint16_t h = bf16_bits(rng_normal_f32(key, first + (uint64_t)i, sigma));
     out[i] = absval ? (uint16_t)(h & 0x7fff) : h;
   }
+}
+void ox_fill_normal_bf16(uint16_t *out, uint64_t n, uint64_t seed, uint64_t tid, float sigma, int absval) {
+  fill_normal_bf16_at(out, 0, n, seed, tid, sigma, absval);
 }
 // bf(mean + sigma*z): the norm weights of the random-init stack
 void ox_fill_affine_bf16(uint16_t *out, uint64_t n, uint64_t seed, uint64_t tid, float mean, float sigma) {
@@ -161,12 +169,23 @@ void ox_fill_normal_f32(float *out, uint64_t n, uint64_t seed, uint64_t tid, flo
 #pragma omp parallel for schedule(static)
   for (int64_t i = 0; i < (int64_t)n; ++i) out[i] = rng_normal_f32(key, (uint64_t)i, sigma);
 }
-void ox_fill_words_u32(uint32_t *out, uint64_t n, uint64_t seed, uint64_t tid) {
+static void fill_words_u32_at(uint32_t *out, uint64_t first, uint64_t n, uint64_t seed, uint64_t tid) {
   uint64_t key = rng_key(seed, tid);
+  auto word = [key](uint64_t k) { return (uint32_t)(rng_u64(key, k >> 1) >> (32u * (uint32_t)(k & 1))); };
+  if ((first & 1) || (n & 1)) {
 #pragma omp parallel for schedule(static)
-  for (int64_t i = 0; i < (int64_t)n; ++i)
-    out[i] = (uint32_t)(rng_u64(key, (uint64_t)i >> 1) >> (32u * (uint32_t)(i & 1)));
+    for (int64_t i = 0; i < (int64_t)n; ++i) out[i] = word(first + (uint64_t)i);
+    return;
+  }
+  // words 2j and 2j+1 are the two halves of one 64-bit draw
+#pragma omp parallel for schedule(static)
+  for (int64_t j = 0; j < (int64_t)(n >> 1); ++j) {
+    uint64_t h = rng_u64(key, (first >> 1) + (uint64_t)j);
+    out[2 * j] = (uint32_t)h;
+    out[2 * j + 1] = (uint32_t)(h >> 32);
+  }
 }
+void ox_fill_words_u32(uint32_t *out, uint64_t n, uint64_t seed, uint64_t tid) { fill_words_u32_at(out, 0, n, seed, tid); }
 
 // ---------------------------------------------------------------------------------
 // INT4: unpack (:309-311), dequant (:306,:312), GEMV (:300-323)
@@ -422,10 +441,20 @@ struct ox_moe_weights {
 void ox_moe_layer(const ox_moe_weights *w, const uint16_t *n, uint16_t *x, int tokens, int hidden, int moe_inter,
                   int shared_inter, int experts, int topk, float routed_scale, uint32_t flags, int mode,
                   float *o_logits, uint16_t *o_ids, float *o_weights, uint16_t *o_mid, uint16_t *o_eout);
+// the six tensors of one routed expert: packed i32 [N, K/8] and scales bf16 [N, K/32] per projection
+struct ExpertView {
+  const uint32_t *gate_p; const uint16_t *gate_s;
+  const uint32_t *up_p;   const uint16_t *up_s;
+  const uint32_t *down_p; const uint16_t *down_s;
+};
+// Where a layer's routed experts come from.  A null source reads them at expert * stride of the tensors in
+// ox_moe_weights; the decoder stack can pass one that produces an expert when it is first selected (a view is
+// only used until the next one is asked for).
+typedef std::function<ExpertView(int)> ExpertSource;
 static void moe_layer_impl(const ox_moe_weights *w, const uint16_t *n, uint16_t *x, int tokens, int hidden, int moe_inter,
                            int shared_inter, int experts, int topk, float routed_scale, uint32_t flags, int mode,
                            float *o_logits, uint16_t *o_ids, float *o_weights, uint16_t *o_mid, uint16_t *o_eout,
-                           const uint16_t *in_ids, const float *in_weights) {
+                           const uint16_t *in_ids, const float *in_weights, const ExpertSource *source = nullptr) {
   const int H = hidden, I = moe_inter, SI = shared_inter, E = experts, K = topk;
   std::vector<float> logits((size_t)tokens * E), weights((size_t)tokens * K);
   std::vector<uint16_t> ids((size_t)tokens * K);
@@ -445,12 +474,18 @@ static void moe_layer_impl(const ox_moe_weights *w, const uint16_t *n, uint16_t 
     std::vector<float> down(H, 0.0f);
     for (int slot = 0; slot < K; ++slot) {  // :845-870
       int e = ids[(size_t)t * K + slot];
-      size_t wo = (size_t)e * I * (H / 8), so = (size_t)e * I * (H / 32);
-      ox_i4_gemv(w->gate_packed + wo, w->gate_scale + so, nt, g.data(), I, H, 1, mode);
-      ox_i4_gemv(w->up_packed + wo, w->up_scale + so, nt, u.data(), I, H, 1, mode);
+      ExpertView v;
+      if (source) {
+        v = (*source)(e);
+      } else {
+        size_t wo = (size_t)e * I * (H / 8), so = (size_t)e * I * (H / 32);
+        v = {w->gate_packed + wo, w->gate_scale + so, w->up_packed + wo, w->up_scale + so, w->down_packed + wo,
+             w->down_scale + so};
+      }
+      ox_i4_gemv(v.gate_p, v.gate_s, nt, g.data(), I, H, 1, mode);
+      ox_i4_gemv(v.up_p, v.up_s, nt, u.data(), I, H, 1, mode);
       for (int r = 0; r < I; ++r) mid[r] = bf16_bits(swiglu_m(bf16_val(g[r]), bf16_val(u[r]), mode));
-      size_t dwo = (size_t)e * H * (I / 8), dso = (size_t)e * H * (I / 32);
-      ox_i4_gemv(w->down_packed + dwo, w->down_scale + dso, mid.data(), y.data(), H, I, 1, mode);
+      ox_i4_gemv(v.down_p, v.down_s, mid.data(), y.data(), H, I, 1, mode);
       float wk = weights[(size_t)t * K + slot];
       for (int r = 0; r < H; ++r) down[r] = fmaf(bf16_val(y[r]), wk, down[r]);  // :401
       if (o_mid) memcpy(o_mid + ((size_t)t * K + slot) * I, mid.data(), (size_t)I * 2);
@@ -547,6 +582,13 @@ struct OxLayer {
   std::vector<uint16_t> router, gate_s, up_s, down_s, sh_gate, sh_up, sh_down;
   std::vector<float> router_bias;
   std::vector<uint32_t> gate_p, up_p, down_p;
+  // a model whose experts are produced on demand keeps the ones in use here instead of in the six tensors above
+  struct Expert {
+    std::vector<uint32_t> gate_p, up_p, down_p;
+    std::vector<uint16_t> gate_s, up_s, down_s;
+    bool given = false;  // holds a tensor handed over with ox_model_set_tensor: never dropped
+  };
+  std::map<int, std::unique_ptr<Expert>> on_demand;
   // latent cache [B][max_context][kv_rank + qk_rope] bf16; mode 0 also keeps the expanded
   // fp32 K [B][ctx][heads*(nope+rope)] and V [B][ctx][heads*v_head] of the reference (:192-238)
   std::vector<uint16_t> latent;
@@ -556,6 +598,13 @@ struct OxLayer {
 struct ox_model {
   ox_config c;
   int mode;
+  // experts on demand: a decode step touches topk experts per layer, so the stack of BASELINE config 5 (24 layers
+  // x 384 experts = 228 GB of routed tensors) needs a few GB of host memory this way.  The generator's values
+  // depend on (seed, tensor, index) only, so an expert produced alone equals its part of the whole tensor.
+  bool on_demand = false;
+  size_t kept = 0, keep_at_most = 192;  // experts held over all layers before the ones not handed over are dropped
+  uint64_t produced = 0;                // experts generated so far (for the tests)
+  std::vector<std::unique_ptr<OxLayer::Expert>> spare;
   float expert_scale_sigma;
   std::vector<uint16_t> embed, final_norm, lm_head, rope_tab;
   std::vector<OxLayer> layers;
@@ -576,11 +625,13 @@ static void fill_words(std::vector<uint32_t> &v, size_t n, uint64_t seed, uint64
   ox_fill_words_u32(v.data(), n, seed, tid);
 }
 
-ox_model *ox_model_create(const ox_config *cfg, int mode) {
+// flags bit 0: routed experts are produced when first selected instead of all at creation
+ox_model *ox_model_create_ex(const ox_config *cfg, int mode, uint32_t flags) {
   const float expert_scale_sigma = cfg->expert_scale_sigma;
   ox_model *m = new ox_model();
   m->c = *cfg;
   m->mode = mode;
+  m->on_demand = (flags & 1u) != 0;
   m->expert_scale_sigma = expert_scale_sigma;
   const ox_config &c = m->c;
   const size_t H = c.hidden, V = c.vocab, E = c.experts, I = c.moe_inter, SI = c.shared_inter, D = c.dense_inter;
@@ -613,12 +664,14 @@ ox_model *ox_model_create(const ox_config *cfg, int mode) {
       fill_bf16(L.router, E * H, c.seed, b + TL_ROUTER, 1.0f / sqrtf((float)H));
       L.router_bias.resize(E);
       ox_fill_normal_f32(L.router_bias.data(), E, c.seed, b + TL_ROUTER_BIAS, 0.01f);
-      fill_words(L.gate_p, E * I * H / 8, c.seed, b + TL_GATE_P);
-      fill_bf16(L.gate_s, E * I * H / 32, c.seed, b + TL_GATE_S, expert_scale_sigma, 1);
-      fill_words(L.up_p, E * I * H / 8, c.seed, b + TL_UP_P);
-      fill_bf16(L.up_s, E * I * H / 32, c.seed, b + TL_UP_S, expert_scale_sigma, 1);
-      fill_words(L.down_p, E * H * I / 8, c.seed, b + TL_DOWN_P);
-      fill_bf16(L.down_s, E * H * I / 32, c.seed, b + TL_DOWN_S, expert_scale_sigma, 1);
+      if (!m->on_demand) {
+        fill_words(L.gate_p, E * I * H / 8, c.seed, b + TL_GATE_P);
+        fill_bf16(L.gate_s, E * I * H / 32, c.seed, b + TL_GATE_S, expert_scale_sigma, 1);
+        fill_words(L.up_p, E * I * H / 8, c.seed, b + TL_UP_P);
+        fill_bf16(L.up_s, E * I * H / 32, c.seed, b + TL_UP_S, expert_scale_sigma, 1);
+        fill_words(L.down_p, E * H * I / 8, c.seed, b + TL_DOWN_P);
+        fill_bf16(L.down_s, E * H * I / 32, c.seed, b + TL_DOWN_S, expert_scale_sigma, 1);
+      }
       fill_bf16(L.sh_gate, SI * H, c.seed, b + TL_SH_GATE, sg);
       fill_bf16(L.sh_up, SI * H, c.seed, b + TL_SH_UP, sg);
       fill_bf16(L.sh_down, H * SI, c.seed, b + TL_SH_DOWN, sg);
@@ -633,7 +686,52 @@ ox_model *ox_model_create(const ox_config *cfg, int mode) {
   m->last_logits.assign((size_t)c.max_batch * V, 0.0f);
   return m;
 }
+ox_model *ox_model_create(const ox_config *cfg, int mode) { return ox_model_create_ex(cfg, mode, 0); }
 void ox_model_destroy(ox_model *m) { delete m; }
+uint64_t ox_model_experts_produced(const ox_model *m) { return m->produced; }
+// how many on-demand experts are held before the ones that can be produced again are dropped (at least 1)
+void ox_model_keep_experts(ox_model *m, int n) { m->keep_at_most = n < 1 ? 1 : (size_t)n; }
+
+// expert e of layer l of a model that produces its experts on demand.  Dropped experts go to a list of spares and
+// their buffers are filled again for the next expert: fresh pages cost more than the values that go into them.
+static OxLayer::Expert &expert_on_demand(ox_model *m, int l, int e) {
+  OxLayer &L = m->layers[l];
+  auto it = L.on_demand.find(e);
+  if (it != L.on_demand.end()) return *it->second;
+  if (m->kept >= m->keep_at_most) {  // drop every expert that can be produced again
+    m->kept = 0;
+    for (OxLayer &o : m->layers)
+      for (auto j = o.on_demand.begin(); j != o.on_demand.end();) {
+        if (j->second->given) {
+          ++j, ++m->kept;
+        } else {
+          m->spare.push_back(std::move(j->second));
+          j = o.on_demand.erase(j);
+        }
+      }
+  }
+  std::unique_ptr<OxLayer::Expert> &slot = L.on_demand[e];
+  if (m->spare.empty()) {
+    slot.reset(new OxLayer::Expert());
+  } else {
+    slot = std::move(m->spare.back());
+    m->spare.pop_back();
+  }
+  OxLayer::Expert &x = *slot;
+  const ox_config &c = m->c;
+  const uint64_t b = (uint64_t)(l + 1) * 64, words = (uint64_t)c.moe_inter * c.hidden / 8, scales = words / 4;
+  x.gate_p.resize(words); x.up_p.resize(words); x.down_p.resize(words);
+  x.gate_s.resize(scales); x.up_s.resize(scales); x.down_s.resize(scales);
+  fill_words_u32_at(x.gate_p.data(), e * words, words, c.seed, b + TL_GATE_P);
+  fill_normal_bf16_at(x.gate_s.data(), e * scales, scales, c.seed, b + TL_GATE_S, m->expert_scale_sigma, 1);
+  fill_words_u32_at(x.up_p.data(), e * words, words, c.seed, b + TL_UP_P);
+  fill_normal_bf16_at(x.up_s.data(), e * scales, scales, c.seed, b + TL_UP_S, m->expert_scale_sigma, 1);
+  fill_words_u32_at(x.down_p.data(), e * words, words, c.seed, b + TL_DOWN_P);
+  fill_normal_bf16_at(x.down_s.data(), e * scales, scales, c.seed, b + TL_DOWN_S, m->expert_scale_sigma, 1);
+  ++m->kept;
+  ++m->produced;
+  return x;
+}
 
 // Overwrites one weight tensor of the model with `bytes` bytes from `src` (the element type the model keeps:
 // bf16, u32 words, f32 for the router bias).  layer < 0: id is TID_EMBED / TID_FINAL_NORM / TID_LM_HEAD; else a
@@ -650,6 +748,22 @@ int ox_model_set_tensor(ox_model *m, int layer, int id, int expert, const void *
     dst = v.data() + per * (size_t)expert;
     have = per * esz;
   };
+  if (m->on_demand && layer >= m->c.first_dense && layer < m->c.n_layers && id >= TL_GATE_P && id <= TL_DOWN_S) {
+    if (expert < 0 || expert >= m->c.experts) return -1;
+    OxLayer::Expert &x = expert_on_demand(m, layer, expert);
+    x.given = true;
+    switch (id) {
+      case TL_GATE_P: dst = x.gate_p.data(); have = x.gate_p.size() * 4; break;
+      case TL_GATE_S: dst = x.gate_s.data(); have = x.gate_s.size() * 2; break;
+      case TL_UP_P: dst = x.up_p.data(); have = x.up_p.size() * 4; break;
+      case TL_UP_S: dst = x.up_s.data(); have = x.up_s.size() * 2; break;
+      case TL_DOWN_P: dst = x.down_p.data(); have = x.down_p.size() * 4; break;
+      default: dst = x.down_s.data(); have = x.down_s.size() * 2; break;
+    }
+    if (have != bytes) return -1;
+    memcpy(dst, src, bytes);
+    return 0;
+  }
   if (layer < 0) {
     if (id == TID_EMBED) whole16(m->embed);
     else if (id == TID_FINAL_NORM) whole16(m->final_norm);
@@ -932,8 +1046,13 @@ static void model_step(ox_model *m, const uint32_t *ids, int B, int pos, int sam
         ox_moe_weights w = {L.router.data(), L.router_bias.data(), L.gate_p.data(), L.gate_s.data(), L.up_p.data(),
                             L.up_s.data(), L.down_p.data(), L.down_s.data(), L.sh_gate.data(), L.sh_up.data(),
                             L.sh_down.data()};
-        ox_moe_layer(&w, n.data(), x, 1, H, c.moe_inter, c.shared_inter, c.experts, c.topk, c.routed_scale, 0, mode,
-                     nullptr, nullptr, nullptr, nullptr, nullptr);
+        ExpertSource source = [m, l](int e) {
+          const OxLayer::Expert &x = expert_on_demand(m, l, e);
+          return ExpertView{x.gate_p.data(), x.gate_s.data(), x.up_p.data(), x.up_s.data(), x.down_p.data(),
+                            x.down_s.data()};
+        };
+        moe_layer_impl(&w, n.data(), x, 1, H, c.moe_inter, c.shared_inter, c.experts, c.topk, c.routed_scale, 0, mode,
+                       nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, m->on_demand ? &source : nullptr);
       }
     }
     if (sample) {  // final norm, lm_head, lowest-index argmax over bf16-rounded logits (:880-881, :718-734)
@@ -978,6 +1097,17 @@ int ox_generate(ox_model *m, const uint32_t *prompt, int B, int P, int n_tokens,
       model_step(m, cur.data(), B, P + i, 1, next.data());
     }
   }
+  return 0;
+}
+// One step of run() (:801-884) for every sequence of the batch at position pos, so that a caller can walk a long
+// generation itself (and watch it).  ids u32 [B]; out_ids u32 [B] is written when sample is set.  Returns 0, or 1 on
+// a bad argument.
+int ox_model_step(ox_model *m, const uint32_t *ids, int B, int pos, int sample, uint32_t *out_ids) {
+  const ox_config &c = m->c;
+  if (B < 1 || B > c.max_batch || pos < 0 || pos >= c.max_context || (sample && !out_ids)) return 1;
+  for (int b = 0; b < B; ++b)
+    if (ids[b] >= (uint32_t)c.vocab) return 1;
+  model_step(m, ids, B, pos, sample, out_ids);
   return 0;
 }
 const float *ox_model_logits(ox_model *m) { return m->last_logits.data(); }

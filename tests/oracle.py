@@ -46,8 +46,12 @@ _SIGS = {
     "ox_mla_span_tiles": ([_I], _I),
     "ox_mla_decode": ([_P, _P, C.c_size_t, _P, _P, _I, _I, _I], None),
     "ox_model_create": ([_P, _I], _P),
+    "ox_model_create_ex": ([_P, _I, C.c_uint32], _P),
+    "ox_model_experts_produced": ([_P], _U64),
+    "ox_model_keep_experts": ([_P, _I], None),
     "ox_model_destroy": ([_P], None),
     "ox_model_set_tensor": ([_P, _I, _I, _I, _P, _U64], _I),
+    "ox_model_step": ([_P, _P, _I, _I, _I, _P], _I),
     "ox_generate": ([_P, _P, _I, _I, _I, _I, _P, _P], _I),
     "ox_model_logits": ([_P], C.POINTER(C.c_float)),
     "ox_model_hidden": ([_P], C.POINTER(C.c_uint16)),
@@ -148,9 +152,11 @@ def small_config(n_layers=3, first_dense=1, batch=1, context=96):
 
 
 class OxModel:
-    def __init__(self, cfg, mode):
+    def __init__(self, cfg, mode, experts_on_demand=False):
+        """experts_on_demand: the routed experts are generated when a token first selects them (same values: the
+        generator is a function of seed, tensor and index), so a stack with hundreds of GB of experts fits."""
         self.cfg, self.lib = cfg, load()
-        self.h = self.lib.ox_model_create(C.byref(cfg), mode)
+        self.h = self.lib.ox_model_create_ex(C.byref(cfg), mode, 1 if experts_on_demand else 0)
 
     def generate(self, prompt, n_tokens, ignore_eos=True):
         B, P = prompt.shape
@@ -158,6 +164,14 @@ class OxModel:
         counts = np.zeros(B, dtype=np.int32)
         rc = self.lib.ox_generate(self.h, ptr(np.ascontiguousarray(prompt)), B, P, n_tokens, int(ignore_eos), ptr(out), ptr(counts))
         return rc, out, counts
+
+    def step(self, ids, pos, sample):
+        """one decode step of every sequence at position pos; returns the sampled ids (or None)"""
+        ids = np.ascontiguousarray(ids, dtype=np.uint32)
+        out = np.zeros(len(ids), dtype=np.uint32)
+        if self.lib.ox_model_step(self.h, ptr(ids), len(ids), pos, int(sample), ptr(out)) != 0:
+            raise ValueError("ox_model_step: bad argument")
+        return out if sample else None
 
     def set_tensor(self, layer, tid, expert, arr):
         arr = np.ascontiguousarray(arr)

@@ -9,6 +9,8 @@ from the Hugging Face tensor names; and the error messages of runtime_index() (:
 """
 import ctypes as C
 
+import numpy as np
+
 import pytest
 
 import ckpt
@@ -93,6 +95,15 @@ def test_infer_config_recovers_the_shapes(tmp_path):
         assert getattr(got, f) == getattr(cfg, f), f
     rc, _, _, err = _check(got, report["index"])
     assert rc == 0, err
+    # the numeric constants after the call are the reference's for a checkpoint (src/kimi_exec.cu:181-186): a caller
+    # of the C ABI that loads one computes RoPE and the softmax scale with YARN_FACTOR 64, not the 32 of the
+    # library's random-init default
+    assert got.yarn_factor == 64.0 and (got.yarn_beta_fast, got.yarn_beta_slow, got.yarn_orig_ctx) == (32.0, 1.0, 4096.0)
+    assert got.rope_theta == 50000.0 and abs(got.rms_eps - 1e-5) < 1e-12 and abs(got.routed_scale - 2.827) < 1e-6
+    assert got.eos_id == 163586 and got.yarn_mscale_all_dim == 1.0
+    rs, ms = C.c_float(), C.c_float()
+    assert kx().kx_softmax_scale(C.byref(got), C.byref(rs), C.byref(ms)) == 0
+    assert abs(ms.value - (0.1 * np.log(64.0) + 1.0)) < 1e-6                   # :428
 
 
 def _rewrite(index, fn):

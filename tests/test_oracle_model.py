@@ -91,6 +91,63 @@ def test_generate_is_deterministic_and_batch_independent(ox):
         assert (out1[0] == out2[b]).all()       # a sequence does not depend on its batch neighbours
 
 
+@pytest.mark.parametrize("mode", [0, 1])
+def test_experts_on_demand_equal_the_whole_tensors(ox, mode):
+    # A model that produces a routed expert when a token first selects it (what lets the 24-layer stack fit in host
+    # memory) must be the model that holds every expert: ids, logits, hidden state, cache rows to the bit -- also when
+    # it keeps at most three experts at a time (each step then produces its experts again), and with an expert's
+    # tensors handed over from outside, which must survive the dropping.
+    cfg = O.small_config(batch=2, context=40)
+    prompt = O.tokens_u32(2 * 9, cfg.seed, 4, cfg.vocab).reshape(2, 9)
+    whole = O.OxModel(cfg, mode)
+    given = O.words_u32(cfg.moe_inter * cfg.hidden // 8, 99, 1)
+    runs = []
+    for m, keep in ((whole, None), (O.OxModel(cfg, mode, experts_on_demand=True), None),
+                    (O.OxModel(cfg, mode, experts_on_demand=True), 3)):
+        if keep:
+            ox.ox_model_keep_experts(m.h, keep)
+        for e in range(cfg.experts):      # every expert of layer 1 gets the same foreign gate_proj words
+            m.set_tensor(1, 14, e, given)
+        rc, out, counts = m.generate(prompt, 7)
+        assert rc == 0
+        runs.append((out, counts, m.logits(2).view(np.uint32), m.hidden(2), m.latent(1), m.latent(2)))
+        if m is not whole:
+            made = ox.ox_model_experts_produced(m.h)
+            # 2 MoE layers x 16 experts exist; with room for all of them none is produced twice
+            assert (made <= 32) if keep is None else (made > 32), made
+        m.close()
+    for other in runs[1:]:
+        assert all((a == b).all() for a, b in zip(runs[0], other))
+    # and the foreign words did change the result (the hand-over is not a no-op)
+    plain = O.OxModel(cfg, mode, experts_on_demand=True)
+    rc, out_p, _ = plain.generate(prompt, 7)
+    assert not (plain.logits(2).view(np.uint32) == runs[0][2]).all()
+    plain.close()
+
+
+def test_step_by_step_equals_generate(ox):
+    cfg = O.small_config(batch=2, context=24)
+    prompt = O.tokens_u32(2 * 6, cfg.seed, 4, cfg.vocab).reshape(2, 6)
+    m = O.OxModel(cfg, 1)
+    rc, out, _ = m.generate(prompt, 5)
+    logits, hidden = m.logits(2), m.hidden(2)
+    m.close()
+    m = O.OxModel(cfg, 1, experts_on_demand=True)
+    got, nxt = [], None
+    for pos in range(6 + 4):
+        ids = prompt[:, pos] if pos < 6 else nxt
+        nxt = m.step(ids, pos, pos >= 5)
+        if nxt is not None:
+            got.append(nxt)
+    assert (np.stack(got, axis=1) == out).all()
+    assert (m.logits(2).view(np.uint32) == logits.view(np.uint32)).all() and (m.hidden(2) == hidden).all()
+    with pytest.raises(ValueError):
+        m.step(np.array([cfg.vocab, 0]), 3, False)
+    with pytest.raises(ValueError):
+        m.step(prompt[:, 0], cfg.max_context, False)
+    m.close()
+
+
 def test_generate_eos_and_argument_rules(ox):
     cfg = O.small_config()
     prompt = O.tokens_u32(10, cfg.seed, 4, cfg.vocab).reshape(1, 10)
