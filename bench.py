@@ -44,13 +44,33 @@ TRAFFIC_PROFILE = "profiles/moe_layer_t1_pmc.md"
 
 
 def profiled_traffic():
+    return _profile_figure(TRAFFIC_PROFILE, "traffic_bytes_per_launch:", int)
+
+
+# Average duration of the same kernel in the committed `rocprofv3 --kernel-trace --stats` summary of the same
+# command (a line `kernel_avg_us: N` there).  The profiler widens the launches and the event figure includes the
+# gap between launches, so the line carries both, and the fraction each gives.
+KERNEL_PROFILE = "profiles/moe_layer_t1.md"
+
+
+def _profile_figure(path, key, kind):
     try:
-        for line in open(os.path.join(ROOT, TRAFFIC_PROFILE)):
-            if line.startswith("traffic_bytes_per_launch:"):
-                return int(line.split(":")[1].split()[0].replace(",", ""))
+        for line in open(os.path.join(ROOT, path)):
+            if line.startswith(key):
+                return kind(line.split(":")[1].split()[0].replace(",", ""))
     except OSError:
         pass
     return None
+
+
+def device_tokens(lib, n, seed, vocab):
+    """n uniform-random token ids generated on the device (tensor id 4 of the seed) and copied back: what kx_prefill
+    takes is a host array, as the reference's executor takes its prompt from argv."""
+    from blok_amd.lib import DevBuf, check
+    buf = DevBuf(n * 4)
+    check(lib.kx_fill_tokens_u32(buf.ptr, n, seed, 4, vocab, None))
+    check(lib.kx_sync(None))
+    return buf.to_numpy(np.uint32, (n,))
 
 
 def moe_layer_bytes(cfg, tokens, distinct):
@@ -117,7 +137,6 @@ class MoeLayerSet:
 
 
 def run_moe_layer(args, emit=True):
-    import oracle as O
     from blok_amd.lib import DevBuf, check, default_config, kx
     lib = kx()
     cfg = default_config()
@@ -129,9 +148,9 @@ def run_moe_layer(args, emit=True):
     layers = MoeLayerSet(lib, cfg, n_layers, args.seed)
     ws = C.c_void_p()
     check(lib.kx_moe_workspace_create(C.byref(cfg), T, C.byref(ws)))
-    n_host = O.normal_bf16(T * cfg.hidden, args.seed, 30, 1.0).reshape(T, cfg.hidden)
-    x_host = O.normal_bf16(T * cfg.hidden, args.seed, 31, 1.0).reshape(T, cfg.hidden)
-    dn, dx = DevBuf.from_numpy(n_host), DevBuf.from_numpy(x_host)
+    dn, dx = DevBuf(T * cfg.hidden * 2), DevBuf(T * cfg.hidden * 2)     # activations generated on the device
+    check(lib.kx_fill_normal_bf16(dn.ptr, T * cfg.hidden, args.seed, 30, 1.0, 0, None))
+    check(lib.kx_fill_normal_bf16(dx.ptr, T * cfg.hidden, args.seed, 31, 1.0, 0, None))
     views = [C.c_void_p() for _ in range(8)]
     check(lib.kx_moe_workspace_views(ws, *[C.byref(v) for v in views]))
 
@@ -199,8 +218,11 @@ def run_moe_layer(args, emit=True):
     # CPU baseline: the oracle's reference schedule on the same layer-0 weights, bounded sample
     cpu = None
     if not args.no_cpu:
+        import oracle as O
         from kxt import moe_oracle_weights
         ox = O.load()
+        n_host = dn.to_numpy(np.uint16, (T, cfg.hidden))
+        x_host = dx.to_numpy(np.uint16, (T, cfg.hidden))
         host = layers.host_layer(0)
         wo = moe_oracle_weights(host)
         tc = min(T, 4)
@@ -269,31 +291,15 @@ def stack_bytes_per_token(cfg, distinct_per_layer):
     return cfg.n_layers * attn + cfg.first_dense * dense + n_moe * moe + 2 * V * H
 
 
-def run_stack(args):
-    """BASELINE config 5: the truncated Kimi-K2-shaped stack, greedy decode after a uniform-random prompt."""
-    import oracle as O
-    from blok_amd.lib import check, default_config, kx
-    lib = kx()
-    cfg = default_config()
-    B, P, K, W = args.batch, args.prompt, args.steps, args.warmup
-    cfg.n_layers, cfg.max_batch, cfg.max_context, cfg.seed = args.stack_layers, B, P + K + W + 9, args.seed
-    name = C.create_string_buffer(256)
-    cus, hbm = C.c_int32(), C.c_uint64()
-    check(lib.kx_device_info(name, 256, C.byref(cus), C.byref(hbm)))
-    wb, cb, sb = C.c_uint64(), C.c_uint64(), C.c_uint64()
-    check(lib.kx_model_bytes(C.byref(cfg), C.byref(wb), C.byref(cb), C.byref(sb)))
-    t0 = time.perf_counter()
-    model = C.c_void_p()
-    check(lib.kx_model_create(C.byref(cfg), C.byref(model)))
-    t_create = time.perf_counter() - t0
-    st = C.c_void_p()
-    check(lib.kx_model_stream(model, C.byref(st)))
-    prompt = O.tokens_u32(B * P, args.seed, 4, cfg.vocab).reshape(B, P)
+def stack_leg(lib, cfg, model, st, B, P, K, W, seed, prefill_chunk):
+    """One timed run of the stack on an existing model: prefill B prompts of P tokens, W warm-up and K timed greedy
+    decode steps; ids never leave the device inside the timed region."""
+    from blok_amd.lib import check
+    prompt = device_tokens(lib, B * P, seed, cfg.vocab).reshape(B, P)
     e = [C.c_void_p() for _ in range(4)]
     for ev in e:
         check(lib.kx_event_create(C.byref(ev)))
-    if args.prefill_chunk > 1:              # several prompt positions per prefill step (tolerance path; default: 1)
-        check(lib.kx_model_set_prefill_chunk(model, args.prefill_chunk))
+    check(lib.kx_model_set_prefill_chunk(model, max(1, prefill_chunk)))  # 1: token by token, the reference's loop
     check(lib.kx_event_record(e[0], st))
     check(lib.kx_prefill(model, prompt.ctypes.data, B, P))
     check(lib.kx_event_record(e[3], st))
@@ -302,7 +308,6 @@ def run_stack(args):
     check(lib.kx_event_record(e[1], st))
     check(lib.kx_sync(st))
     t0 = time.perf_counter()
-    ids = np.zeros((K, B), dtype=np.uint32)
     for i in range(K):                      # K timed decode steps; ids stay on the device
         check(lib.kx_decode_step(model, None))
     check(lib.kx_event_record(e[2], st))
@@ -311,6 +316,8 @@ def run_stack(args):
     ms_pre, ms_dec = C.c_float(), C.c_float()
     check(lib.kx_event_elapsed_ms(e[0], e[3], C.byref(ms_pre)))
     check(lib.kx_event_elapsed_ms(e[1], e[2], C.byref(ms_dec)))
+    for ev in e:
+        check(lib.kx_event_destroy(ev))
     last = np.zeros(B, dtype=np.uint32)
     check(lib.kx_greedy_sample(model, last.ctypes.data))
     # distinct routed experts per MoE layer, which is what a batch's weight traffic depends on: counted over a few more
@@ -325,22 +332,15 @@ def run_stack(args):
                 check(lib.kx_model_routing(model, layer, None, C.byref(d)))
                 seen.append(d.value)
         distinct = float(np.mean(seen))
-    check(lib.kx_model_destroy(model))
+        check(lib.kx_model_set_routing_record(model, 0))
     ms_per_step = ms_dec.value / K
-    toks = B * 1e3 / ms_per_step
     weights = stack_bytes_per_token(cfg, distinct)
     kv = B * (P + W + K // 2) * (cfg.kv_rank + cfg.qk_rope) * 2 * cfg.n_layers   # latent cache rows read by a mid-run step
     algo = weights if B == 1 else weights + kv
     return {
-        "value": round(toks, 2), "ms_per_step": round(ms_per_step, 5), "wall_ms_per_step": round(wall_ms / K, 5),
-        "prefill_ms_per_token": round(ms_pre.value / P, 5),
-        "workload": f"truncated Kimi-K2 stack (BASELINE config 5): {cfg.n_layers} layers (1 dense + {cfg.n_layers - 1} MoE), "
-                    f"vocab {cfg.vocab}, batch {B}, {P}-token uniform-random prompt prefilled "
-                    + ("token by token" if args.prefill_chunk <= 1 else f"{min(args.prefill_chunk, max(1, 2048 // B))} positions per step") + ", then "
-                    f"{W} warm-up and {K} timed greedy decode steps; seeded random-init weights resident in HBM",
-        "resident_gb": {"weights": round(wb.value / 1e9, 2), "kv_cache": round(cb.value / 1e9, 3), "scratch": round(sb.value / 1e9, 3)},
-        "model_create_s": round(t_create, 2), "device": name.value.decode(), "compute_units": cus.value,
-        "last_ids": last.tolist(),
+        "value": round(B * 1e3 / ms_per_step, 2), "ms_per_step": round(ms_per_step, 5), "wall_ms_per_step": round(wall_ms / K, 5),
+        "prefill_ms_per_token": round(ms_pre.value / P, 5), "last_ids": last.tolist(),
+        "prefill": "token by token" if prefill_chunk <= 1 else f"{min(prefill_chunk, max(1, 2048 // B))} positions per step",
         "stack_hbm": {"algorithmic_bytes_per_step": int(algo), "weight_bytes": int(weights), "kv_cache_bytes": int(kv),
                       "counted": "weights once per step" + ("" if B == 1 else " + latent cache rows of every sequence"),
                       "distinct_experts_per_moe_layer": round(distinct, 1),
@@ -350,35 +350,74 @@ def run_stack(args):
     }
 
 
+def run_stack(args, extra_batches=()):
+    """BASELINE config 5: the truncated Kimi-K2-shaped stack, greedy decode after a uniform-random prompt.  The model
+    is created once, for the largest batch asked for; the headline leg (--batch) runs first, then one leg per extra
+    batch on the same resident weights."""
+    from blok_amd.lib import check, default_config, kx
+    lib = kx()
+    cfg = default_config()
+    B, P, K, W = args.batch, args.prompt, args.steps, args.warmup
+    cfg.n_layers, cfg.max_batch, cfg.max_context, cfg.seed = args.stack_layers, max((B,) + tuple(extra_batches)), P + K + W + 9, args.seed
+    name = C.create_string_buffer(256)
+    cus, hbm = C.c_int32(), C.c_uint64()
+    check(lib.kx_device_info(name, 256, C.byref(cus), C.byref(hbm)))
+    wb, cb, sb = C.c_uint64(), C.c_uint64(), C.c_uint64()
+    check(lib.kx_model_bytes(C.byref(cfg), C.byref(wb), C.byref(cb), C.byref(sb)))
+    t0 = time.perf_counter()
+    model = C.c_void_p()
+    check(lib.kx_model_create(C.byref(cfg), C.byref(model)))
+    check(lib.kx_sync(None))
+    t_create = time.perf_counter() - t0
+    st = C.c_void_p()
+    check(lib.kx_model_stream(model, C.byref(st)))
+    out = stack_leg(lib, cfg, model, st, B, P, K, W, args.seed, args.prefill_chunk)
+    out["extra"] = {b: stack_leg(lib, cfg, model, st, b, P, K, W, args.seed, args.prefill_chunk) for b in extra_batches}
+    check(lib.kx_model_destroy(model))
+    out.update({
+        "workload": f"truncated Kimi-K2 stack (BASELINE config 5): {cfg.n_layers} layers (1 dense + {cfg.n_layers - 1} MoE), "
+                    f"vocab {cfg.vocab}, batch {B}, {P}-token uniform-random prompt prefilled {out['prefill']}, then "
+                    f"{W} warm-up and {K} timed greedy decode steps; seeded random-init weights resident in HBM",
+        "resident_gb": {"weights": round(wb.value / 1e9, 2), "kv_cache": round(cb.value / 1e9, 3), "scratch": round(sb.value / 1e9, 3)},
+        "model_create_s": round(t_create, 2), "device": name.value.decode(), "compute_units": cus.value})
+    return out
+
+
 def run_cpu_stack(args):
-    """CPU baseline: the oracle's reference schedule on a bounded sample of config 5 (fewer layers, few tokens)."""
+    """CPU baseline: the oracle's reference schedule (mode 0) on config 5's stack itself -- all --cpu-layers layers
+    (default 24), full vocabulary, batch 1 -- for a bounded number of token steps.  The oracle holds the dense tensors
+    and produces a routed expert when a token first selects it, so the stack fits in host memory; producing the
+    experts is part of what is timed (the reference reads its tiles from NVMe inside the layer loop, too)."""
     import oracle as O
     from blok_amd.lib import default_config
     cfg = default_config()
     cfg.n_layers, cfg.max_batch, cfg.max_context, cfg.seed = args.cpu_layers, 1, 64, args.seed
-    P, K = 2, args.cpu_tokens
     t0 = time.perf_counter()
-    m = O.OxModel(cfg, 0)
+    m = O.OxModel(cfg, 0, experts_on_demand=True)
     t_init = time.perf_counter() - t0
-    prompt = O.tokens_u32(P, args.seed, 4, cfg.vocab).reshape(1, P)
+    ids = O.tokens_u32(1, args.seed, 4, cfg.vocab)
     t0 = time.perf_counter()
-    rc, out, _ = m.generate(prompt, K + 1)      # P prefill steps (one sampled) + K sampled decode steps
+    steps = 0
+    while steps < args.cpu_tokens and (steps < 2 or time.perf_counter() - t0 < args.cpu_seconds * 2):
+        ids = m.step(ids, steps, True)          # every step samples, as a decode step does
+        steps += 1
     dt = time.perf_counter() - t0
     m.close()
-    steps = P + K
     per_step = dt / steps
     full = default_config()
-    scaled = per_step * ((full.n_layers - 1) / max(1, cfg.n_layers - 1))
+    scaled = per_step * ((full.n_layers - 1) / max(1, cfg.n_layers - 1)) if cfg.n_layers != full.n_layers else per_step
     return {"value": round(1.0 / per_step, 4), "unit": "tok/s", "cores": O.load().ox_num_threads(), "kind": "port",
-            "sample": f"oracle reference schedule (mode 0), {cfg.n_layers}-layer truncation of config 5 (1 dense + "
-                      f"{cfg.n_layers - 1} MoE, full vocabulary), {steps} token steps in {dt:.1f} s after {t_init:.1f} s of "
-                      f"weight generation; OpenMP over output rows; scaled by MoE-layer count to 24 layers this is about "
-                      f"{1.0 / scaled:.3f} tok/s"}
+            "layers": cfg.n_layers, "steps": steps, "seconds": round(dt, 2),
+            "scaled_to_24_layers_tok_s": round(1.0 / scaled, 4),
+            "sample": f"oracle reference schedule (mode 0) on config 5's stack, {cfg.n_layers} layers (1 dense + "
+                      f"{cfg.n_layers - 1} MoE, 384 experts produced on demand, full vocabulary), batch 1: {steps} sampled token "
+                      f"steps in {dt:.1f} s after {t_init:.1f} s of dense-weight generation; OpenMP over output rows"}
 
 
 def run_default(args):
     """Config 5 for `value`, plus the routed INT4 gate/up kernel of config 2 (T = batch) for `roofline`."""
-    stack = run_stack(args)
+    extra = (32,) if (args.batch == 1 and not args.no_b32) else ()
+    stack = run_stack(args, extra)
     margs = argparse.Namespace(**vars(args))
     margs.tokens, margs.steps, margs.warmup, margs.no_cpu = args.batch, 40, 8, True
     moe = run_moe_layer(margs, emit=False)
@@ -388,6 +427,12 @@ def run_default(args):
         margs8.tokens = 8
         moe8 = run_moe_layer(margs8, emit=False)
     cpu = None if args.no_cpu else run_cpu_stack(args)
+    roof = {k: v for k, v in moe["roofline"].items()}
+    prof_us = _profile_figure(KERNEL_PROFILE, "kernel_avg_us:", float) if args.batch == 1 else None
+    if prof_us:
+        roof["profile_kernel_avg_us"] = prof_us
+        roof["profile_frac"] = round(roof["algorithmic_bytes_per_launch"] / (prof_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)
+        roof["profile_from"] = KERNEL_PROFILE
     out = {
         "metric": "decode tok/s + INT4 expert GEMV HBM GB/s (% of peak), Kimi-K2 shapes, 1 GPU",
         "value": stack["value"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -395,11 +440,15 @@ def run_default(args):
         "dtype": "int4 weights x bf16 activations, f32 accumulate", "data": "synthetic",
         "config": {"workload": stack["workload"], "batch": args.batch, "prompt": args.prompt, "device": stack["device"],
                    "compute_units": stack["compute_units"], "resident_gb": stack["resident_gb"]},
-        "roofline": moe["roofline"],
+        "roofline": roof,
         "int4_expert_gemv": dict(moe["int4_expert_gemv"], workload=moe["config"]["workload"], phase_ms=moe["phase_ms"]),
         "stack": {k: stack[k] for k in ("wall_ms_per_step", "prefill_ms_per_token", "model_create_s", "stack_hbm", "last_ids")},
         "cpu_baseline": cpu,
     }
+    for b, leg in stack["extra"].items():     # config 5 names batch 32 too: the same resident model, same prompt length
+        out[f"stack_b{b}"] = {"tok_s": leg["value"], "ms_per_step": leg["ms_per_step"], "steps": args.steps, "warmup": args.warmup,
+                              "prompt": args.prompt, "prefill": leg["prefill"], "prefill_ms_per_token": leg["prefill_ms_per_token"],
+                              "distinct_experts": leg["stack_hbm"]["distinct_experts_per_moe_layer"], "stack_hbm": leg["stack_hbm"]}
     if moe8 is not None:
         out["int4_expert_gemv_t8"] = dict(moe8["int4_expert_gemv"], workload=moe8["config"]["workload"],
                                           gate_up_frac_of_peak=moe8["roofline"]["frac"])
@@ -621,7 +670,8 @@ def main():
     ap.add_argument("--prompt", type=int, default=1024)
     ap.add_argument("--prefill-chunk", type=int, default=1, help="prompt positions per prefill step (1: the reference's token-by-token prefill)")
     ap.add_argument("--stack-layers", type=int, default=24)
-    ap.add_argument("--cpu-layers", type=int, default=2)
+    ap.add_argument("--cpu-layers", type=int, default=24)
+    ap.add_argument("--no-b32", action="store_true", help="default run: skip the batch-32 leg of config 5")
     ap.add_argument("--tokens", type=int, default=1)
     ap.add_argument("--moe-flags", type=lambda v: int(v, 0), default=0,
                     help="moe_layer: flags of kx_moe_decode_layer (0: the bit-reproducible kernels; 0x400: routed experts with "
@@ -629,7 +679,7 @@ def main():
     ap.add_argument("--layers", type=int, default=4, help="independent layers cycled to keep weights cold")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--cpu-tokens", type=int, default=40)
+    ap.add_argument("--cpu-tokens", type=int, default=12)
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     args = ap.parse_args()
     if args.gpus != 1:

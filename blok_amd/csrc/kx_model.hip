@@ -89,6 +89,7 @@ struct kx_model {
   hipEvent_t ev[3] = {nullptr, nullptr, nullptr};
   int batch = 0, pos = 0;
   int prefill_chunk = 1;  // prompt positions per prefill step (kx_model_set_prefill_chunk)
+  uint32_t exact = 0;     // kx_model_set_exact: KX_EXACT_* parts that keep the bit-reproducible kernels at every batch size
   int x_row0 = 0;         // first row of x that belongs to the last position of the last step
   bool sampled = false;
   float ms_prefill = 0, ms_decode = 0;
@@ -289,7 +290,8 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample, int C = 1) {
   const bool fuse = B <= 4 && C == 1;  // RMSNorms ride in the prologue of the GEMV that consumes them
   // From 5 sequences on (the fused prologues cover up to 4), the dense projections run as GEMMs on the matrix cores: the
   // GEMV is bound by its fma count there.  Same values, another summation order (the bf16 rounding points stay).
-  const bool mm = B >= 5;
+  const bool mm = B >= 5 && !(m->exact & KX_EXACT_PROJECTIONS);
+  const int mla_kernel = (m->exact & KX_EXACT_ATTENTION) ? KX_MLA_VALU : m->mla_kernel;
   auto dense = [&](int epi, const KxGemvArgs &g) -> int {
     if (!mm) return kx_gemv_launch(epi, g, st);
     const bool dual = epi == KX_EPI_SWIGLU;
@@ -337,7 +339,7 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample, int C = 1) {
     g.w_block_off = c.qk_nope; g.x_block_stride = c.kv_rank;
     if (fuse) {                                                                                 // :825
       KxMlaPartials mp;
-      KX_TRY(kx_mla_partials_launch(&c, L.cache, seq_stride, m->qabs, m->partial, B, pos + 1, &mp, st, 0, m->mla_kernel));
+      KX_TRY(kx_mla_partials_launch(&c, L.cache, seq_stride, m->qabs, m->partial, B, pos + 1, &mp, st, 0, mla_kernel));
       if (mp.spans <= 64) {  // the GEMV's activations are the attention partials, merged as they are loaded
         g.mla_pm = mp.pm; g.mla_pz = mp.pz; g.mla_po = mp.po; g.mla_spans = mp.spans; g.mla_heads = c.heads;
       } else {               // long context, few sequences: more spans than the GEMV's merge takes
@@ -349,7 +351,7 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample, int C = 1) {
       for (int i0 = 0; i0 < C; i0 += cs) {
         const int np = C - i0 < cs ? C - i0 : cs;
         KX_TRY(kx_mla_attend_launch(&c, L.cache, seq_stride, m->qabs + (size_t)i0 * NB * c.heads * KVA, m->partial,
-                                    m->o_lat + (size_t)i0 * NB * c.heads * c.kv_rank, np * NB, pos + i0 + np, st, C > 1 ? NB : 0, m->mla_kernel));
+                                    m->o_lat + (size_t)i0 * NB * c.heads * c.kv_rank, np * NB, pos + i0 + np, st, C > 1 ? NB : 0, mla_kernel));
       }
     }
     if (C > 1 && B > 32 && c.kv_rank % 128 == 0) {  // a long prefill step: one grouped GEMM over the heads
@@ -388,8 +390,8 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample, int C = 1) {
         // streams them faster than the GEMM kernel does at one token.  With 32 sequences that decode alike (70-100
         // distinct experts for 256 pairs, up to 23 pairs on one expert) the step goes from 24.5 to 18.1 ms; at 12
         // sequences the two forms are level (12.1 against 12.4 ms), at 8 the GEMV kernels win (9.8 against 10.9 ms).
-        const uint32_t flags = ((m->fusion & KX_FUSE_MOE_TAIL) ? 0u : KX_MOE_SEPARATE_TAIL) | (mm ? KX_MOE_SHARED_MATRIX_CORES : 0u) |
-                               (B >= 12 ? KX_MOE_ROUTED_MATRIX_CORES : 0u);
+        const uint32_t flags = ((m->fusion & KX_FUSE_MOE_TAIL) ? 0u : KX_MOE_SEPARATE_TAIL) | (B >= 5 && !(m->exact & KX_EXACT_SHARED) ? KX_MOE_SHARED_MATRIX_CORES : 0u) |
+                               (B >= 12 && !(m->exact & KX_EXACT_ROUTED) ? KX_MOE_ROUTED_MATRIX_CORES : 0u);
         KX_TRY(kx_moe_layer_launch(&c, &L.moe, m->moe_ws, m->n, m->x, B, flags, fuse ? L.post_ln : nullptr, st, false));  // :835-877
       }
       if (m->route_logits) {  // the routing record: logits of the first rows and the number of distinct experts
@@ -590,7 +592,7 @@ extern "C" int kx_prefill(kx_model *m, const uint32_t *h_ids, int32_t batch, int
   m->pos = 0;
   // :886: one run() per prompt token, sampling on the last; with a prefill chunk set, up to that many positions per step
   int chunk = m->prefill_chunk < STEP_TOKENS / batch ? m->prefill_chunk : STEP_TOKENS / batch;
-  if (chunk < 1) chunk = 1;
+  if (chunk < 1 || m->exact == KX_EXACT_ALL) chunk = 1;  // a step of several positions is a tolerance path
   for (int i = 0; i < prompt_len; i += chunk) {
     const int n = prompt_len - i < chunk ? prompt_len - i : chunk;
     if ((rc = step(m, m->ids + (size_t)i * batch, i + n == prompt_len, n))) return rc;
@@ -689,6 +691,22 @@ extern "C" int kx_model_set_prefill_chunk(kx_model *m, int32_t positions) {
   KX_REQUIRE(m, "kx_model_set_prefill_chunk: null model");
   KX_REQUIRE(positions >= 1 && positions <= STEP_TOKENS, "kx_model_set_prefill_chunk: positions=%d outside [1, %d]", positions, STEP_TOKENS);
   m->prefill_chunk = positions;
+  return KX_OK;
+}
+
+extern "C" int kx_model_set_exact(kx_model *m, uint32_t mask) {
+  KX_REQUIRE(m, "kx_model_set_exact: null model");
+  KX_REQUIRE(!(mask & ~(uint32_t)KX_EXACT_ALL), "kx_model_set_exact: unknown bits in mask 0x%x", mask);
+  m->exact = mask;
+  return KX_OK;
+}
+
+extern "C" int kx_model_rewind(kx_model *m, int32_t positions) {
+  KX_REQUIRE(m, "kx_model_rewind: null model");
+  KX_REQUIRE(m->batch > 0, "kx_model_rewind: no prefill has run");
+  KX_REQUIRE(positions >= 0 && positions <= m->pos, "kx_model_rewind: positions=%d outside [0, %d]", positions, m->pos);
+  m->pos -= positions;
+  if (positions) m->sampled = false;  // the sampled ids belonged to the last position
   return KX_OK;
 }
 

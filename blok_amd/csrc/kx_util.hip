@@ -120,6 +120,11 @@ __global__ void fill_words_k(uint32_t *out, uint64_t n, uint64_t key) {
   uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
   for (; i < n; i += stride) out[i] = kx_rng_u32(key, i);
 }
+__global__ void fill_tokens_k(uint32_t *out, uint64_t n, uint64_t key, uint32_t vocab) {
+  uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (; i < n; i += stride) out[i] = (uint32_t)(kx_rng_u64(key, i) % vocab);
+}
 unsigned fill_grid(uint64_t n) {
   uint64_t b = (n + 255) / 256;
   return (unsigned)(b < 1 ? 1 : (b > 65536 ? 65536 : b));
@@ -162,6 +167,15 @@ extern "C" int kx_fill_words_u32(void *d_out, uint64_t n, uint64_t seed, uint64_
   if (!n) return KX_OK;
   hipLaunchKernelGGL(fill_words_k, dim3(fill_grid(n)), dim3(256), 0, kx_stream(stream), (uint32_t *)d_out, n,
                      kx_rng_key(seed, tensor_id));
+  KX_LAUNCH_CHECK();
+  return KX_OK;
+}
+extern "C" int kx_fill_tokens_u32(void *d_out, uint64_t n, uint64_t seed, uint64_t tensor_id, uint32_t vocab, void *stream) {
+  KX_REQUIRE(d_out || !n, "kx_fill_tokens_u32: null pointer");
+  KX_REQUIRE(vocab > 0, "kx_fill_tokens_u32: vocab must be positive");
+  if (!n) return KX_OK;
+  hipLaunchKernelGGL(fill_tokens_k, dim3(fill_grid(n)), dim3(256), 0, kx_stream(stream), (uint32_t *)d_out, n,
+                     kx_rng_key(seed, tensor_id), vocab);
   KX_LAUNCH_CHECK();
   return KX_OK;
 }

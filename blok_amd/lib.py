@@ -56,6 +56,7 @@ _SIGS = {
     "kx_fill_normal_bf16": [_P, _U64, _U64, _U64, _F, C.c_int, _P],
     "kx_fill_normal_f32": [_P, _U64, _U64, _U64, _F, _P],
     "kx_fill_words_u32": [_P, _U64, _U64, _U64, _P],
+    "kx_fill_tokens_u32": [_P, _U64, _U64, _U64, C.c_uint32, _P],
     "kx_dev_copy": [_P, _P, _U64, _P],
     "kx_i4_unpack": [_P, _P, _I, _I, _P],
     "kx_i4_dequant": [_P, _P, _P, _I, _I, _P],
@@ -92,6 +93,8 @@ _SIGS = {
     "kx_model_set_fusion": [_P, C.c_uint32],
     "kx_model_set_attention_kernel": [_P, _I],
     "kx_model_set_routing_record": [_P, C.c_int],
+    "kx_model_set_exact": [_P, C.c_uint32],
+    "kx_model_rewind": [_P, _I],
     "kx_model_routing": [_P, _I, _P, _P],
     "kx_model_set_prefill_chunk": [_P, _I],
     "kx_model_stream": [_P, _PP],

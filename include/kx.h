@@ -89,6 +89,8 @@ int kx_fill_normal_bf16(void *d_out, uint64_t n, uint64_t seed, uint64_t tensor_
 int kx_fill_normal_f32(void *d_out, uint64_t n, uint64_t seed, uint64_t tensor_id, float sigma,
                        void *stream);
 int kx_fill_words_u32(void *d_out, uint64_t n, uint64_t seed, uint64_t tensor_id, void *stream);
+/* token ids uniform in [0, vocab): the uniform-random prompts of the benchmark configurations */
+int kx_fill_tokens_u32(void *d_out, uint64_t n, uint64_t seed, uint64_t tensor_id, uint32_t vocab, void *stream);
 
 /* ---- INT4 operators ------------------------------------------------------
  * kx_i4_unpack : nibble extraction of matvec_i4_bf16_scale_k (:309-311);
@@ -333,6 +335,23 @@ int kx_model_set_fusion(kx_model *model, uint32_t mask);
 /* The attention kernel this model's steps use: KX_MLA_AUTO (default), KX_MLA_VALU or KX_MLA_MATRIX_CORES, as for
  * kx_mla_decode.  A property of the model: other models of the process keep theirs.                          */
 int kx_model_set_attention_kernel(kx_model *model, int32_t kernel);
+/* kx_model_set_exact(model, KX_EXACT_ALL): every step takes the kernels of the bit-reproducible path -- the GEMV
+ * kernels, the VALU attention kernel, one prompt position per prefill step -- whatever the batch size, instead of
+ * moving to the matrix cores from 5 sequences on.  A sequence then comes out to the bit as it does alone (every sum
+ * of that path is a fixed tree that does not depend on the batch), at a few times the cost per step for large
+ * batches.  The mask selects the parts (so that a deviation can be traced to one of them); 0, the default, none.
+ * No counterpart in the reference, whose batch is always 1 (src/kimi_exec.cu:792-799).
+ * kx_model_rewind(model, n): the next step runs at a position n lower than it would have: the last n cache rows of
+ * every sequence are written again by the steps that follow (rows above the current position are never read).  After
+ * a rewind kx_decode_step needs host ids.  What a caller that rejects drafted tokens needs, and what lets a test run
+ * the same step twice, once on each path, from the same cache.                                                 */
+#define KX_EXACT_PROJECTIONS 1u /* q_a|kv_a, q_b, o_proj, dense MLP, lm_head as GEMVs */
+#define KX_EXACT_ATTENTION 2u   /* the VALU attention kernel */
+#define KX_EXACT_SHARED 4u      /* the shared expert as GEMVs */
+#define KX_EXACT_ROUTED 8u      /* every routed expert through the INT4 GEMV kernels */
+#define KX_EXACT_ALL 15u
+int kx_model_set_exact(kx_model *model, uint32_t mask);
+int kx_model_rewind(kx_model *model, int32_t positions);
 /* A record of the routing for tests and measurement.  The reference's host knows the expert ids of every layer
  * (it copies them back, src/kimi_exec.cu:844); here they stay on the device, and this is the way to look at them.
  * kx_model_set_routing_record(model, 1): from now on every step also keeps, per MoE layer, the router logits of its

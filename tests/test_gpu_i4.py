@@ -29,6 +29,10 @@ def test_fill_kernels_match_oracle(kxlib, ox):
     check(kxlib.kx_fill_words_u32(b.ptr, n, 42, 6, None))
     check(kxlib.kx_sync(None))
     assert (b.to_numpy(np.uint32, (n,)) == O.words_u32(n, 42, 6)).all()
+    check(kxlib.kx_fill_tokens_u32(b.ptr, n, 42, 4, 163840, None))
+    check(kxlib.kx_sync(None))
+    assert (b.to_numpy(np.uint32, (n,)) == O.tokens_u32(n, 42, 4, 163840)).all()
+    assert kxlib.kx_fill_tokens_u32(b.ptr, n, 42, 4, 0, None) != 0
 
 
 def test_unpack_and_dequant_bit_exact(kxlib, ox):

@@ -175,6 +175,16 @@ def test_eos_and_errors(kxlib, ox):
     km = KxModel(kxlib, cfg)
     rc, out_e, counts_e = km.generate(prompt, 8, ignore_eos=False)
     assert rc == 0 and counts_e[0] == first and (out_e[0, :first] == out[0, :first]).all()
+    # the loop ends once every sequence has sampled the end-of-sequence id (:887-888); the ids are looked at every
+    # eighth step, so of 28 steps asked for 8 are decoded; with ignore_eos all of them
+    steps = C.c_int32()
+    rc, out_l, counts_l = km.generate(prompt, 28, ignore_eos=False)
+    assert rc == 0 and counts_l[0] == first and (out_l[0, :first] == out[0, :first]).all()
+    check(kxlib.kx_model_steps_decoded(km.h, C.byref(steps)))
+    assert steps.value == 8
+    rc, out_l, counts_l = km.generate(prompt, 28, ignore_eos=True)
+    check(kxlib.kx_model_steps_decoded(km.h, C.byref(steps)))
+    assert rc == 0 and counts_l[0] == 28 and steps.value == 28 and (out_l[0, :8] == out[0]).all()
     assert km.generate(prompt, 31)[0] != 0 and b"context" in kxlib.kx_last_error()
     bad = prompt.copy(); bad[0, 1] = cfg.vocab
     assert km.generate(bad, 2)[0] != 0 and b"vocabulary" in kxlib.kx_last_error()
@@ -661,6 +671,134 @@ def test_kimi_shape_batched_stack_against_single_sequences(kxlib, ox, batch):
                               np.stack(ref_logits))
     print(f"batch {batch}: logits max-rel per sequence: median {np.median(errs):.2e}, worst {max(errs):.2e}; excused: {excused or 'none'}", flush=True)
     assert len(excused) <= batch // 4
+
+
+def test_config5_batch32_full_size_step_by_step_against_the_exact_path(kxlib, ox, capsys):
+    # BASELINE config 5 at batch 32 and full size: 24 layers, 32 uniform-random prompts of 1024 tokens, 256 greedy
+    # tokens.  At this batch the projections, the shared expert, the attention and the routed experts with several
+    # tokens run on the matrix cores: another summation order, a tolerance path.  The reference is the same model with
+    # kx_model_set_exact: the GEMV kernels and the VALU attention kernel at batch 32, whose sums do not depend on the
+    # batch.  The exact path prefills the prompts and decodes greedily; every one of the 256 decode steps is run
+    # three times from the same cache and the same input ids -- twice on the default path, then, after
+    # kx_model_rewind(1), on the exact path, which also leaves the exact cache row behind -- so what is compared is
+    # one step's own deviation.  Checked:
+    #  1. the exact path's sequences 0..3 equal, to the bit, the same sequences decoded four at a time (the path the
+    #     tests above hold to the oracle, at 24 layers too): ids, logits, router logits of the first three tokens;
+    #  2. the two default runs of every step agree to the bit (ids, logits, the router logits of all 23 MoE layers of
+    #     all 32 sequences): two streams per MoE layer and arrival counters leave no room for a run-to-run difference
+    #     unless something races;
+    #  3. for every (sequence, step): the router logits of the first MoE layer -- what the dense layer and two
+    #     attention blocks on the matrix cores hand to the first router -- within max-rel 1e-2 of the exact path's;
+    #  4. for every (sequence, step), one of three verdicts, each checked:
+    #     "agrees": the same expert set in all 23 MoE layers, logits within the stack-level 3e-2, the same sampled id;
+    #     "argmax near-tie": as before, but another id, and the exact path's two largest logits closer than the bar;
+    #     "router flip": the expert sets differ first in layer j, and the exact path's selection gap there is below
+    #        2.5e-2, i.e. what a router-logit change of a few percent can cross.  A token that took another expert is
+    #        off by tens of percent in the next layer, so such a pair is not judged further in this step.
+    # Why the bars of a 24-layer stack are wider than the operator bars (1e-2 given identical inputs, held in the
+    # operator tests): with INT4 values in [-8, 7] times group scales |N(0, 0.02)| a routed expert has a gain of
+    # several hundred, every MoE layer's output swamps the residual stream it is added to, and a deviation of 4e-3 in
+    # layer 1 is 1e-2 to 6e-2 a few layers later for some sequences before it decays again -- with any one of the
+    # matrix-core parts switched on alone, the others exact.  The counts of the three verdicts and the worst figures are
+    # printed.
+    import time
+    batch, plen, n_tokens = 32, 1024, 256
+    say(f"config 5 at full size: 24 layers, batch {batch}, prompt {plen}, {n_tokens} tokens, default path against exact path step by step")
+    cfg = default_config()
+    cfg.max_batch, cfg.max_context, cfg.seed = batch, plen + n_tokens, 0
+    assert cfg.n_layers == 24 and cfg.first_dense == 1 and cfg.vocab == 163840
+    prompt = O.tokens_u32(batch * plen, cfg.seed, 4, cfg.vocab).reshape(batch, plen)
+    moe_layers = list(range(cfg.first_dense, cfg.n_layers))
+    bias = np.stack([O.normal_f32(cfg.experts, cfg.seed, (l + 1) * 64 + 13, 0.01).astype(np.float64) for l in moe_layers])
+    t0 = time.time()
+
+    def note(msg):
+        with capsys.disabled():
+            print(f"  [{time.time() - t0:4.0f} s] {msg}", flush=True)
+
+    km = KxModel(kxlib, cfg)
+    check(kxlib.kx_model_set_routing_record(km.h, 1))
+
+    def observe(nb):
+        """sampled ids, logits (as bits), router logits [nb, layers, experts] of the last step"""
+        ids = np.zeros(nb, dtype=np.uint32)
+        check(kxlib.kx_greedy_sample(km.h, ptr(ids)))
+        rl = np.empty((nb, len(moe_layers), cfg.experts), dtype=np.float32)
+        lg = np.empty((nb, cfg.experts), dtype=np.float32)
+        for j, l in enumerate(moe_layers):
+            check(kxlib.kx_model_routing(km.h, l, ptr(lg), None))
+            rl[:, j] = lg
+        return ids, km.logits(nb), rl
+
+    def same_bits(a, b):
+        return all((x.view(np.uint32) == y.view(np.uint32)).all() for x, y in zip(a, b))
+
+    # four sequences at a time, default path (GEMV kernels at this batch): prompt + 3 tokens
+    four = []
+    check(kxlib.kx_prefill(km.h, ptr(np.ascontiguousarray(prompt[:4])), 4, plen))
+    for i in range(3):
+        if i:
+            check(kxlib.kx_decode_step(km.h, None))
+        four.append(observe(4))
+    note("sequences 0..3 decoded four at a time")
+    # exact path at batch 32: prefill, then step back onto the last prompt position
+    check(kxlib.kx_model_set_exact(km.h, 15))
+    check(kxlib.kx_prefill(km.h, ptr(prompt), batch, plen))
+    check(kxlib.kx_sync(None))
+    note("exact path: 32 prompts prefilled")
+    check(kxlib.kx_model_rewind(km.h, 1))
+    feed = np.ascontiguousarray(prompt[:, plen - 1])
+    verdicts = {"agrees": 0, "argmax near-tie": 0, "router flip": 0}
+    worst = {"first router": 0.0, "logits": 0.0, "flipped gap": 0.0}
+    for i in range(n_tokens):
+        runs = []
+        for mask in (0, 0, 15):
+            if runs:
+                check(kxlib.kx_model_rewind(km.h, 1))
+            check(kxlib.kx_model_set_exact(km.h, mask))
+            check(kxlib.kx_decode_step(km.h, ptr(feed)))
+            runs.append(observe(batch))
+        assert same_bits(runs[0], runs[1]), f"token {i}: two runs of the default path differ"
+        (ids_f, log_f, rl_f), (ids_e, log_e, rl_e) = runs[0], runs[2]
+        if i < 3:
+            assert same_bits([x[:4] for x in runs[2]], four[i]), f"token {i}: the exact path at batch 32 differs from four at a time"
+        first_router = np.abs(rl_f[:, 0] - rl_e[:, 0]).max(axis=1) / np.abs(rl_e[:, 0]).max(axis=1)
+        worst["first router"] = max(worst["first router"], float(first_router.max()))
+        assert first_router.max() < 1e-2, f"token {i}, sequence {int(first_router.argmax())}: router logits of the first MoE layer differ by max-rel {first_router.max():.3e}"
+        sel_f = 1.0 / (1.0 + np.exp(-rl_f.astype(np.float64))) + bias[None]
+        sel_e = 1.0 / (1.0 + np.exp(-rl_e.astype(np.float64))) + bias[None]
+        order_e = np.argsort(-sel_e, axis=2, kind="stable")
+        set_e = np.sort(order_e[:, :, :cfg.topk], axis=2)
+        set_f = np.sort(np.argsort(-sel_f, axis=2, kind="stable")[:, :, :cfg.topk], axis=2)
+        srt_e = np.take_along_axis(sel_e, order_e[:, :, :cfg.topk + 1], axis=2)
+        gap_e = srt_e[:, :, cfg.topk - 1] - srt_e[:, :, cfg.topk]
+        errs = np.abs(log_f - log_e).max(axis=1) / np.abs(log_e).max(axis=1)
+        for b in range(batch):
+            differs = np.nonzero((set_f[b] != set_e[b]).any(axis=1))[0]
+            if len(differs):
+                j = int(differs[0])
+                assert gap_e[b, j] < 2.5e-2, (f"sequence {b}, token {i}: experts differ in layer {moe_layers[j]} although the exact path's "
+                                              f"selection gap there is {gap_e[b, j]:.2e}")
+                worst["flipped gap"] = max(worst["flipped gap"], float(gap_e[b, j]))
+                verdicts["router flip"] += 1
+                continue
+            worst["logits"] = max(worst["logits"], float(errs[b]))
+            assert errs[b] < 3e-2, f"sequence {b}, token {i}: the same experts in every layer, logits err {errs[b]:.3e}"
+            if ids_f[b] != ids_e[b]:
+                top = np.sort(log_e[b])[-2:]
+                gap = float(top[1] - top[0]) / float(np.abs(log_e[b]).max())
+                assert gap < 3e-2, f"sequence {b}, token {i}: id {ids_f[b]} vs {ids_e[b]} although the top-2 logit gap is {gap:.2e}"
+                verdicts["argmax near-tie"] += 1
+                continue
+            verdicts["agrees"] += 1
+        feed = ids_e.copy()
+        if i % 32 == 31:
+            note(f"{i + 1} steps: verdicts {verdicts}; worst {({k: float(f'{v:.2e}') for k, v in worst.items()})}")
+    km.close()
+    note(f"{batch * n_tokens} (sequence, step) pairs: {verdicts}; worst first-router max-rel {worst['first router']:.2e}, worst logits max-rel among "
+         f"pairs with the same experts everywhere {worst['logits']:.2e}, largest selection gap "
+         f"flipped {worst['flipped gap']:.2e}; default path deterministic over {n_tokens} steps")
+    assert sum(verdicts.values()) == batch * n_tokens
 
 
 def test_model_form_of_the_handover_gives_the_same_bits(kxlib, ox):
