@@ -84,6 +84,7 @@ struct kx_model {
   int mla_kernel = KX_MLA_AUTO;    // kx_model_set_attention_kernel
   float *route_logits = nullptr;   // routing record (kx_model_set_routing_record): [n_layers][max_batch][experts]
   int *route_distinct = nullptr;   // [n_layers] distinct experts of the last step
+  float *route_history = nullptr;  // record level 2: router logits of every position, [n_layers][max_context][max_batch][experts]
   kx_moe_workspace *moe_ws = nullptr;
   hipStream_t st = nullptr;
   hipEvent_t ev[3] = {nullptr, nullptr, nullptr};
@@ -401,6 +402,11 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample, int C = 1) {
         KX_HIP(hipMemcpyAsync(m->route_logits + (size_t)l * c.max_batch * c.experts, d_logits, (size_t)rows * c.experts * 4,
                               hipMemcpyDeviceToDevice, st));
         KX_HIP(hipMemcpyAsync(m->route_distinct + l, kx_moe_workspace_n_active(m->moe_ws), 4, hipMemcpyDeviceToDevice, st));
+        if (m->route_history) {  // every token of the step: token i * NB + b is position pos + i of sequence b
+          const size_t row = (size_t)c.experts * 4;
+          KX_HIP(hipMemcpy2DAsync(m->route_history + (((size_t)l * c.max_context + pos) * c.max_batch) * c.experts, (size_t)c.max_batch * row,
+                                  d_logits, (size_t)NB * row, (size_t)NB * row, (size_t)C, hipMemcpyDeviceToDevice, st));
+        }
       }
     }
   }
@@ -567,6 +573,7 @@ extern "C" int kx_model_destroy(kx_model *m) {
   if (m->arena) (void)hipFree(m->arena);
   if (m->route_logits) (void)hipFree(m->route_logits);
   if (m->route_distinct) (void)hipFree(m->route_distinct);
+  if (m->route_history) (void)hipFree(m->route_history);
   delete m;
   return KX_OK;
 }
@@ -721,11 +728,21 @@ extern "C" int kx_model_set_routing_record(kx_model *m, int on) {
   KX_REQUIRE(m, "kx_model_set_routing_record: null model");
   KX_REQUIRE(m->c.first_dense < m->c.n_layers, "kx_model_set_routing_record: the model has no MoE layer");
   KX_HIP(hipStreamSynchronize(m->st));
+  KX_REQUIRE(on >= 0 && on <= 2, "kx_model_set_routing_record: level %d outside [0, 2]", on);
+  if (on < 2 && m->route_history) {
+    (void)hipFree(m->route_history);
+    m->route_history = nullptr;
+  }
   if (!on) {
     if (m->route_logits) (void)hipFree(m->route_logits);
     if (m->route_distinct) (void)hipFree(m->route_distinct);
     m->route_logits = nullptr; m->route_distinct = nullptr;
     return KX_OK;
+  }
+  if (on == 2 && !m->route_history) {
+    const size_t bytes = (size_t)m->c.n_layers * m->c.max_context * m->c.max_batch * m->c.experts * 4;
+    KX_HIP(hipMalloc((void **)&m->route_history, bytes));
+    KX_HIP(hipMemset(m->route_history, 0, bytes));
   }
   if (m->route_logits) return KX_OK;
   const size_t nl = (size_t)m->c.n_layers;
@@ -750,6 +767,15 @@ extern "C" int kx_model_routing(kx_model *m, int32_t layer, float *h_logits, int
     KX_HIP(hipMemcpyAsync(h_logits, m->route_logits + (size_t)layer * m->c.max_batch * m->c.experts, (size_t)m->batch * m->c.experts * 4,
                           hipMemcpyDeviceToHost, m->st));
   if (h_distinct) KX_HIP(hipMemcpyAsync(h_distinct, m->route_distinct + layer, 4, hipMemcpyDeviceToHost, m->st));
+  KX_HIP(hipStreamSynchronize(m->st));
+  return KX_OK;
+}
+extern "C" int kx_model_routing_history(kx_model *m, int32_t layer, int32_t pos0, int32_t n, float *h_logits) {
+  KX_REQUIRE(m && h_logits && m->route_history, "kx_model_routing_history: null argument, or kx_model_set_routing_record is not at level 2");
+  KX_REQUIRE(layer >= m->c.first_dense && layer < m->c.n_layers, "kx_model_routing_history: layer %d is not a MoE layer of this model", layer);
+  KX_REQUIRE(pos0 >= 0 && n >= 0 && pos0 + n <= m->c.max_context, "kx_model_routing_history: positions [%d, %d) outside the context of %d", pos0, pos0 + n, m->c.max_context);
+  KX_HIP(hipMemcpyAsync(h_logits, m->route_history + (((size_t)layer * m->c.max_context + pos0) * m->c.max_batch) * m->c.experts,
+                        (size_t)n * m->c.max_batch * m->c.experts * 4, hipMemcpyDeviceToHost, m->st));
   KX_HIP(hipStreamSynchronize(m->st));
   return KX_OK;
 }

@@ -96,6 +96,7 @@ _SIGS = {
     "kx_model_set_exact": [_P, C.c_uint32],
     "kx_model_rewind": [_P, _I],
     "kx_model_routing": [_P, _I, _P, _P],
+    "kx_model_routing_history": [_P, _I, _I, _I, _P],
     "kx_model_set_prefill_chunk": [_P, _I],
     "kx_model_stream": [_P, _PP],
     "kx_moe_prefill_layer": [C.POINTER(KxConfig), C.POINTER(KxMoeWeights), _P, _P, _P, _I, C.c_uint32, _P],

@@ -358,9 +358,14 @@ int kx_model_rewind(kx_model *model, int32_t positions);
  * first min(tokens, max_batch) tokens and the number of distinct experts its tokens selected (two small device
  * copies per layer; off by default).
  * kx_model_routing: the record of the last step for `layer`: h_logits f32 [batch][experts] (or NULL), h_distinct
- * i32 [1] (or NULL).  Synchronises.  A dense layer is an error.                                              */
+ * i32 [1] (or NULL).  Synchronises.  A dense layer is an error.
+ * kx_model_set_routing_record(model, 2) also keeps the router logits of every position of every sequence, whichever
+ * step computed them (n_layers x max_context x max_batch x experts floats of device memory), so that a prefill in
+ * steps of several positions can be compared with one token by token, position by position.
+ * kx_model_routing_history: h_logits f32 [n][max_batch][experts] for positions pos0 .. pos0 + n - 1 of `layer`.   */
 int kx_model_set_routing_record(kx_model *model, int on);
 int kx_model_routing(kx_model *model, int32_t layer, float *h_logits, int32_t *h_distinct);
+int kx_model_routing_history(kx_model *model, int32_t layer, int32_t pos0, int32_t n, float *h_logits);
 /* Prompt positions per prefill step.  1 (default) is the reference's prefill, one run() per prompt token (:886),
  * and the bit-reproducible path.  With n > 1, kx_prefill and kx_generate take up to n consecutive positions of
  * every sequence in one step (at most 2048 tokens a step, so min(n, 2048 / batch) positions): the projections, the
