@@ -1,0 +1,436 @@
+// kx_front.hip -- the front of the attention block for one token as one launch:
+//   q_a GEMV with the input RMSNorm      (src/kimi_exec.cu:812-813)
+//   q_b GEMV with the q_a RMSNorm        (:814-815)
+//   kv_a GEMV, its RMSNorm, RoPE of the shared key, the cache row   (:816-817, :820-824)
+//   q_abs = (bf(W_UK^T q_nope) | rope(q_rope)) per head             (:818 as W_UK, rope_k :346-357)
+// The reference runs these as seven launches with a tile read from NVMe in front of each; the separate-launch
+// form of this library runs them as two (gemv_bf16_k for q_a|kv_a, gemv_absorb_k).  q_b needs all of q_a and the
+// absorb needs a whole head of q, so the steps are a chain, and as launches each of them pays its start and its
+// drain while the memory system idles.  Here one workgroup per CU stays resident, and its 48 rows of q_b (144 KB)
+// are copied global -> LDS while q_a is computed, so that the q_b step reads them at LDS speed.
+//
+//   every workgroup: 6 rows of q_a and 2 or 3 of kv_a, all loads out at once (waves 0..6) -> hand the 8 or 9 values
+//                    over; waves 4..7 start the copy of the workgroup's 48 rows of q_b into LDS -> take all of q_a ->
+//                    q rows [48 b, 48 b + 48) from LDS -> hand them over -> (workgroup 0: take kv_a, norm, RoPE,
+//                    cache row) -> take its head's q -> a quarter of the head's q_abs
+//
+// Sums are the ones of the separate-launch kernels (kx_gemv_body.h, kx_attn_parts.h): results are equal to the
+// bit, which the fused / separate test of the stack checks.
+//
+// Hand-over between workgroups: no barrier and no counter.  A value travels as one 32-bit word that carries the
+// launch's tag above its bf16 bits; the reader polls the words it needs until they carry the tag.  A word is one
+// relaxed atomic object, so nothing has to be ordered, acknowledged or reset.  All workgroups must be resident at
+// once (a reader waits for writers): the launcher refuses a device with fewer CUs than workgroups, and the LDS a
+// workgroup takes keeps a second one off its CU.  The wait is bounded: after FR_SPIN_LIMIT polls a reader sets the
+// error flag and goes on (with wrong results), so the grid always drains; the model reports the flag at its next
+// synchronisation.
+#include "kx_attn_parts.h"
+#include "kx_common.h"
+#include "kx_dense.h"
+#include "kx_front.h"
+#include "kx_gemv_body.h"
+#include "kx_lds_copy.h"
+#include "kx_math.h"
+#include "kx_wave.h"
+
+namespace {
+
+using namespace kxg;
+
+constexpr int FR_THREADS = 512;      // 8 waves; in the first step wave w < 7 owns the 512-column slices w and w + 7 of a 7168-wide row
+constexpr int FR_ROWS = 9;           // rows of q_a | kv_a a workgroup computes: 6 + 2 (+ 1 for the first 64 workgroups)
+constexpr int FR_PART_BYTES = 6144;  // head of the dynamic LDS: 2 KB of slice partials, then the q_a row / the head's q
+constexpr int FR_SPIN_LIMIT = 1 << 16;  // polls of a microsecond or so each
+
+struct FrontArgs {
+  const uint16_t *x, *input_ln;  // residual row, input RMSNorm weights [hidden]
+  const uint16_t *w_qkv;         // bf16 [q_rank + kv_rank + rope, hidden]
+  const uint16_t *qa_ln, *w_qb;  // q_a RMSNorm weights [q_rank], bf16 [heads * (nope + rope), q_rank]
+  QAbsArgs qa;                   // kvb, rope_row, qabs, w_kv_ln, cache, dims, pos
+  uint32_t *hand;                // tagged words: [q_rank] q_a, [kv_rank + rope] kv_a, [heads * (nope + rope)] q
+  int hidden, q_rank, rows_b;
+  float eps;
+  uint32_t tag;                  // this launch's tag, in the upper half of every word handed over
+  int *err;
+};
+
+// A value handed to other workgroups of the launch travels as one 32-bit word, the launch's tag above the bf16
+// bits: whoever reads the word with the right tag has the value, so there is no counter to arrive at, no store to
+// wait for and nothing to order -- each word is one relaxed atomic object.
+__device__ __forceinline__ void hand_store(uint32_t *p, uint32_t tag, uint16_t v) {
+  __hip_atomic_store(p, (tag << 16) | v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// reads n (at most 8) consecutive words until all carry the tag; gives up after FR_SPIN_LIMIT polls (flag set,
+// values as they are), so that the grid always drains
+template <int N>
+__device__ __forceinline__ void hand_load(const uint32_t *p, uint32_t tag, int *err, uint32_t (&w)[N]) {
+  int polls = 0;
+  while (true) {
+    bool ok = true;
+#pragma unroll
+    for (int i = 0; i < N; ++i) w[i] = __hip_atomic_load(p + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+    for (int i = 0; i < N; ++i) ok = ok && (w[i] >> 16) == tag;
+    if (ok) return;
+    if (++polls > FR_SPIN_LIMIT || (polls == 1 && __hip_atomic_load(err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) {
+      __hip_atomic_store(err, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      return;
+    }
+    __builtin_amdgcn_s_sleep(2);
+  }
+}
+
+__global__ void __launch_bounds__(FR_THREADS) attn_front_k(FrontArgs a) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t fr_lds[];
+  __shared__ float s_ws[4];
+  __shared__ float s_scale;
+  float *part = (float *)fr_lds;                 // [FR_ROWS][S] of phase A, [rows_b][4] of the q_b step, [8][cq] of the absorb
+  uint16_t *s_row = (uint16_t *)(fr_lds + 2048); // the q_a row (q_rank bf16); later the head's q as floats
+  uint8_t *big = fr_lds + FR_PART_BYTES;         // the q_b rows of this workgroup
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int bid = blockIdx.x;
+  const int H = a.hidden, S = H >> 9, kva = a.qa.kv_rank + a.qa.rope;
+  const int rows_a = a.q_rank / (int)gridDim.x;  // 6
+  uint32_t *hand_qa = a.hand, *hand_kv = a.hand + a.q_rank, *hand_q = hand_kv + kva;
+
+  // rows of [q_a ; kv_a] this workgroup computes: rows_a of q_a, two of kv_a, and one more of kv_a while they last
+  auto row_of = [&](int i) {
+    if (i < rows_a) return bid * rows_a + i;
+    const int k = i < rows_a + 2 ? 2 * bid + (i - rows_a) : 2 * (int)gridDim.x + bid;
+    return k < kva ? a.q_rank + k : -1;
+  };
+
+  const int row_bytes = a.q_rank * 2;
+  // ---- every load that does not depend on another workgroup goes out now, in the order of need: the row for the
+  // RMSNorm, this wave's activations and weights, and behind them the operands of the later steps (the q_a RMSNorm
+  // weights of the q_b step, the W_UK block of the absorb), which then lie in registers when their step comes
+  uint4 wbuf[FR_ROWS][2], xr[2], gr[2], nx[4], gb[4], wuk_r[16];
+  const int s0 = wave, s1 = wave + 7;  // this wave's slices (wave 7 computes nothing in phase A)
+  const int SB = a.q_rank >> 9;        // slices of the q_b GEMV: 3 at Kimi-K2 shapes; the launcher allows up to 4
+  const int cq = a.qa.kv_rank >> 2, ncg = cq >> 3;  // absorb: columns per workgroup, groups of 8 of them
+  const int ab_chain = tid / ncg, ab_cg = tid - ab_chain * ncg;  // absorb item of this thread (tid < 8 * ncg)
+  if (tid < 256) {
+    const int chunks = H >> 3;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) nx[j] = ((const uint4 *)a.x)[min(tid + 256 * j, chunks - 1)];
+  }
+  if (wave < 7) {
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const uint32_t col = (uint32_t)(k ? s1 : s0) * 512u + (uint32_t)lane * 8u;
+      xr[k] = *(const uint4 *)(a.x + col);
+      gr[k] = *(const uint4 *)(a.input_ln + col);
+    }
+#pragma unroll
+    for (int i = 0; i < FR_ROWS; ++i) {
+      const int row = max(row_of(i), 0);
+#pragma unroll
+      for (int k = 0; k < 2; ++k)
+        wbuf[i][k] = ld_stream16(a.w_qkv + (size_t)row * H + (uint32_t)(k ? s1 : s0) * 512u + (uint32_t)lane * 8u);
+    }
+  }
+#pragma unroll
+  for (int s = 0; s < 4; ++s)
+    if (s < SB) gb[s] = *(const uint4 *)(a.qa_ln + s * 512 + lane * 8);
+  if (tid < 8 * ncg) {  // 16 rows of W_UK[h] for this thread's chain and column group (nope = 128: the launcher checks)
+    const uint16_t *wuk = a.qa.kvb + (size_t)(bid >> 2) * (a.qa.nope + a.qa.v_head) * a.qa.kv_rank + (bid & 3) * cq + ab_cg * 8;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) wuk_r[i] = ld_stream16(wuk + (size_t)(ab_chain + 8 * i) * a.qa.kv_rank);
+  }
+  // input RMSNorm scale: gemv_body's prologue (the first 256 threads own the 8-element chunks t, t + 256, ...)
+  {
+    const int chunks = H >> 3;
+    float v = 0.0f;
+    if (tid < 256) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (tid + 256 * j < chunks) {
+          float f[8];
+          unpack8(f, nx[j]);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v = __builtin_fmaf(f[e], f[e], v);
+        }
+    }
+    float vv[1] = {v};
+    kxw::reduce<1, 64>(vv, lane);
+    if (lane == 0 && wave < 4) s_ws[wave] = vv[0];
+    kx_lds_barrier();
+    if (tid == 0) s_scale = kx_rsqrtf((((s_ws[0] + s_ws[1]) + s_ws[2]) + s_ws[3]) / (float)H + a.eps);
+    kx_lds_barrier();
+  }
+  if (wave < 7) {
+    float xs[2][8];
+    const float sc = s_scale;
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      float g[8];
+      unpack8(xs[k], xr[k]);
+      unpack8(g, gr[k]);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) xs[k][e] = kx_bfround(kx_bfround(xs[k][e] * sc) * g[e]);
+    }
+    auto dot = [&](const uint4 &w, const float (&x8)[8]) {
+      float wf[8];
+      unpack8(wf, w);
+      float acc = 0.0f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc = __builtin_fmaf(wf[e], x8[e], acc);
+      return acc;
+    };
+    float v[16];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      v[2 * i] = dot(wbuf[i][0], xs[0]);
+      v[2 * i + 1] = dot(wbuf[i][1], xs[1]);
+    }
+    kxw::reduce<16, 64>(v, lane);
+    if (kxw::reduce_writer<16, 64>(lane)) {
+#pragma unroll
+      for (int j = 0; j < kxw::reduce_out<16, 64>(); ++j) {
+        const int idx = kxw::reduce_index<16, 64>(lane, j);
+        part[(idx >> 1) * S + ((idx & 1) ? s1 : s0)] = v[j];
+      }
+    }
+    float v2[2] = {dot(wbuf[8][0], xs[0]), dot(wbuf[8][1], xs[1])};
+    kxw::reduce<2, 64>(v2, lane);
+    if (kxw::reduce_writer<2, 64>(lane)) {
+#pragma unroll
+      for (int j = 0; j < kxw::reduce_out<2, 64>(); ++j) {
+        const int idx = kxw::reduce_index<2, 64>(lane, j);
+        part[8 * S + (idx ? s1 : s0)] = v2[j];
+      }
+    }
+  }
+  kx_lds_barrier();
+  if (tid < FR_ROWS) {  // slices left to right, one rounding, handed over
+    const int row = row_of(tid);
+    if (row >= 0) {
+      const float *p = part + tid * S;
+      float y = p[0];
+      for (int s = 1; s < S; ++s) y += p[s];
+      hand_store(a.hand + row, a.tag, kx_bf16_rne(y));
+    }
+  }
+
+  // ---- waves 4..7: the q_b rows of this workgroup, global -> LDS, 1 KB per copy instruction.  Not earlier: the copies
+  // are needed last, and a wave that is held up issuing them (the memory pipeline is full by now) would hold the
+  // workgroup's barriers up with it.
+  if (wave >= 4) {
+    const int units = a.rows_b * row_bytes >> 10;
+    const uint8_t *src = (const uint8_t *)a.w_qb + (size_t)bid * a.rows_b * row_bytes + lane * 16;
+    const uint32_t dst = (uint32_t)(uintptr_t)big;
+    for (int u = wave - 4; u < units; u += 4) kx_copy16_to_lds(src + (size_t)u * 1024, __builtin_amdgcn_readfirstlane(dst + u * 1024));
+  }
+
+  // ---- q_a from every workgroup: its RMSNorm scale (the same prologue schedule) and the row itself into LDS
+  {
+    const int chunks = a.q_rank >> 3;  // at most 256: one chunk per thread
+    float v = 0.0f;
+    if (tid < chunks) {
+      uint32_t w[8];
+      hand_load<8>(hand_qa + tid * 8, a.tag, a.err, w);
+      uint32_t o[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = (w[2 * e] & 0xffffu) | (w[2 * e + 1] << 16);
+      ((uint4 *)s_row)[tid] = make_uint4(o[0], o[1], o[2], o[3]);
+      float f[8];
+      unpack8(f, make_uint4(o[0], o[1], o[2], o[3]));
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v = __builtin_fmaf(f[e], f[e], v);
+    }
+    float vv[1] = {v};
+    kxw::reduce<1, 64>(vv, lane);
+    if (lane == 0 && wave < 4) s_ws[wave] = vv[0];
+    kx_wait_copies<0>();  // waves 4..7: their copies have landed
+    __syncthreads();
+    if (tid == 0) s_scale = kx_rsqrtf((((s_ws[0] + s_ws[1]) + s_ws[2]) + s_ws[3]) / (float)a.q_rank + a.eps);
+    __syncthreads();
+  }
+  // ---- q rows [rows_b * bid, +rows_b) from LDS
+  {
+    float xs[4][8];
+    const float sc = s_scale;
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+      if (s < SB) {
+        float g[8];
+        unpack8(xs[s], *(const uint4 *)(s_row + s * 512 + lane * 8));
+        unpack8(g, gb[s]);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) xs[s][e] = kx_bfround(kx_bfround(xs[s][e] * sc) * g[e]);
+      }
+    // wave w takes rows w, w + 8, ..., w + 40 (the launcher makes rows_b 48): all their LDS reads first, then the
+    // products, then one butterfly for four rows and one for two
+    auto dot = [&](int r, int s) {
+      float wf[8];
+      unpack8(wf, *(const uint4 *)(big + (size_t)r * row_bytes + s * 1024 + lane * 16));
+      float acc = 0.0f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc = __builtin_fmaf(wf[e], xs[s][e], acc);
+      return acc;
+    };
+    float v[16], v2[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int s = 0; s < 4; ++s) v[i * 4 + s] = s < SB ? dot(wave + 8 * i, s) : 0.0f;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int s = 0; s < 4; ++s) v2[i * 4 + s] = s < SB ? dot(wave + 8 * (4 + i), s) : 0.0f;
+    kxw::reduce<16, 64>(v, lane);
+    if (kxw::reduce_writer<16, 64>(lane)) {
+#pragma unroll
+      for (int j = 0; j < kxw::reduce_out<16, 64>(); ++j) {
+        const int idx = kxw::reduce_index<16, 64>(lane, j);
+        part[(wave + 8 * (idx >> 2)) * 4 + (idx & 3)] = v[j];
+      }
+    }
+    kxw::reduce<8, 64>(v2, lane);
+    if (kxw::reduce_writer<8, 64>(lane)) {
+#pragma unroll
+      for (int j = 0; j < kxw::reduce_out<8, 64>(); ++j) {
+        const int idx = kxw::reduce_index<8, 64>(lane, j);
+        part[(wave + 8 * (4 + (idx >> 2))) * 4 + (idx & 3)] = v2[j];
+      }
+    }
+    __syncthreads();
+    if (tid < a.rows_b) {
+      const float *p = part + tid * 4;
+      float y = p[0];
+      for (int s = 1; s < SB; ++s) y += p[s];
+      hand_store(hand_q + (size_t)bid * a.rows_b + tid, a.tag, kx_bf16_rne(y));
+    }
+  }
+  // ---- workgroup 0: kv_a from everybody -> RMSNorm of the latent part, RoPE of the shared key, the cache row.
+  // kxa::kv_finish_block's schedule, with the row taken from the tagged words.
+  if (bid == 0) {
+    const int kv_rank = a.qa.kv_rank, rope = a.qa.rope, half = rope >> 1, chunks = kv_rank >> 3;
+    uint16_t *crow = a.qa.cache + (size_t)a.qa.pos * kva;
+    uint4 mine = make_uint4(0, 0, 0, 0);
+    float v = 0.0f;
+    if (tid < chunks) {  // chunks <= 256 (the launcher checks)
+      uint32_t w[8];
+      hand_load<8>(hand_kv + tid * 8, a.tag, a.err, w);
+      mine = make_uint4((w[0] & 0xffffu) | (w[1] << 16), (w[2] & 0xffffu) | (w[3] << 16), (w[4] & 0xffffu) | (w[5] << 16),
+                        (w[6] & 0xffffu) | (w[7] << 16));
+      float f[8];
+      unpack8(f, mine);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v = __builtin_fmaf(f[e], f[e], v);
+    }
+    float vv[1] = {v};
+    kxw::reduce<1, 64>(vv, lane);
+    __syncthreads();
+    if (tid < 4) s_ws[tid] = 0.0f;
+    __syncthreads();
+    if (tid < 256 && lane == 0) s_ws[wave] = vv[0];
+    __syncthreads();
+    const float scale = kx_rsqrtf((((s_ws[0] + s_ws[1]) + s_ws[2]) + s_ws[3]) / (float)kv_rank + a.qa.eps);
+    if (tid < chunks) {
+      float f[8], g[8];
+      unpack8(f, mine);
+      unpack8(g, ((const uint4 *)a.qa.w_kv_ln)[tid]);
+      uint32_t o[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        o[e] = (uint32_t)kx_bf16_rne(kx_bfround(f[2 * e] * scale) * g[2 * e]) | ((uint32_t)kx_bf16_rne(kx_bfround(f[2 * e + 1] * scale) * g[2 * e + 1]) << 16);
+      ((uint4 *)crow)[tid] = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+    if (tid >= 256 && tid < 256 + half) {
+      const int p = tid - 256;
+      uint32_t w[2];
+      hand_load<2>(hand_kv + kv_rank + 2 * p, a.tag, a.err, w);
+      float lo, hi;
+      kxa::rope_pair(kx_bf16_f32((uint16_t)w[0]), kx_bf16_f32((uint16_t)w[1]), kx_bf16_f32(a.qa.rope_row[p]), kx_bf16_f32(a.qa.rope_row[half + p]), lo, hi);
+      crow[kv_rank + p] = kx_bf16_rne(lo);
+      crow[kv_rank + half + p] = kx_bf16_rne(hi);
+    }
+  }
+  // ---- a quarter of the head's q_abs: the sums of kxa::absorb_head_block for columns [cq * j, cq * (j + 1))
+  {
+    const int nope = a.qa.nope, rope = a.qa.rope, kv_rank = a.qa.kv_rank, qk = nope + rope, half = rope >> 1;
+    const int h = bid >> 2, j = bid & 3;
+    float *ab_part = (float *)big;     // [8][cq]: the q_b rows are spent
+    float *qs = (float *)s_row;        // [qk]
+    float *out = a.qa.qabs + (size_t)h * (kv_rank + rope);
+    __syncthreads();  // s_row (the q_a row) and the q_b rows are no longer read
+    if (tid < (qk >> 2)) {
+      uint32_t w[4];
+      hand_load<4>(hand_q + (size_t)h * qk + tid * 4, a.tag, a.err, w);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) qs[tid * 4 + e] = kx_bf16_f32((uint16_t)w[e]);
+    }
+    __syncthreads();
+    if (tid < 8 * ncg) {  // chain ab_chain over d = ab_chain, ab_chain + 8, ..., W_UK rows from the registers
+      float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        float wf[8];
+        unpack8(wf, wuk_r[i]);
+        const float qd = qs[ab_chain + 8 * i];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] = __builtin_fmaf(wf[e], qd, acc[e]);
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ab_part[ab_chain * cq + ab_cg * 8 + e] = acc[e];
+    }
+    __syncthreads();
+    for (int c = tid; c < cq; c += FR_THREADS) {
+      const float *p = ab_part + c;
+      const float s = ((p[0] + p[cq]) + (p[2 * cq] + p[3 * cq])) + ((p[4 * cq] + p[5 * cq]) + (p[6 * cq] + p[7 * cq]));
+      out[j * cq + c] = kx_bfround(s);
+    }
+    if (j == 3 && tid < half) {
+      float lo, hi;
+      kxa::rope_pair(qs[nope + 2 * tid], qs[nope + 2 * tid + 1], kx_bf16_f32(a.qa.rope_row[tid]), kx_bf16_f32(a.qa.rope_row[half + tid]),
+                     lo, hi);
+      out[kv_rank + tid] = lo;
+      out[kv_rank + half + tid] = hi;
+    }
+  }
+}
+
+}  // namespace
+
+// g_qkv: the q_a | kv_a GEMV as the separate launch would get it (w0 = [q_rank + kv_rank + rope, hidden], x = the
+// residual row, norm_w = the input RMSNorm weights); g_qb: the q_b GEMV (w0 = [heads * (nope + rope), q_rank],
+// norm_w = the q_a RMSNorm weights).  hand: (q_rank + kv_rank + rope + heads * (nope + rope)) words of device memory;
+// tag: a value in [1, 65535] that differs from the previous launch's on the same `hand`; err: one int, zero until a
+// wait of some launch gave up.  *done = false, nothing launched, when the shapes or the device do not allow the
+// fused form.  The q_a | kv_a and q rows are not written to g_qkv.out / g_qb.out: nothing after this launch reads them.
+int kx_attn_front_launch(const KxGemvArgs &g_qkv, const KxGemvArgs &g_qb, const QAbsArgs &q, uint32_t *hand, uint32_t tag, int *err,
+                         bool *done, hipStream_t st) {
+  *done = false;
+  static int cus = 0;
+  if (!cus) {
+    int dev = 0;
+    KX_HIP(hipGetDevice(&dev));
+    KX_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+  }
+  const int hidden = g_qkv.cols, q_rank = g_qb.cols, qk = q.nope + q.rope, G = 4 * q.heads, kva = q.kv_rank + q.rope;
+  if (g_qkv.tokens != 1 || g_qb.tokens != 1 || !hand || !err || !q.cache || !g_qkv.norm_w || !g_qb.norm_w || tag < 1 || tag > 65535) return KX_OK;
+  if (G > cus || hidden != 14 * 512 || q_rank % 512 || q_rank / 512 > 4 || q_rank / 8 > 256) return KX_OK;
+  if (g_qkv.rows != q_rank + kva || g_qb.rows != q.heads * qk || qk % 16 || q.rope % 2 || q.rope / 2 > 256 || qk / 4 > FR_THREADS) return KX_OK;
+  const int rows_a = q_rank / G, rows_b = qk / 4;
+  if (rows_b != 48 || q.nope != 128 || q.kv_rank / 4 > FR_THREADS || q_rank % G || rows_a != FR_ROWS - 3 || kva < 2 * G || kva > 3 * G || q.kv_rank % 32 || q.kv_rank / 8 > 256) return KX_OK;
+  const size_t qb_bytes = (size_t)rows_b * q_rank * 2;
+  if (qb_bytes % 1024 || (size_t)rows_b * 16 > 2048 || (size_t)FR_ROWS * 14 * 4 > 2048 || (size_t)q_rank * 2 > FR_PART_BYTES - 2048 ||
+      (size_t)qk * 4 > FR_PART_BYTES - 2048 || qb_bytes < (size_t)8 * (q.kv_rank / 4) * 4)
+    return KX_OK;
+  const size_t lds = FR_PART_BYTES + qb_bytes;
+  if (lds > 156 * 1024) return KX_OK;
+  static bool attr_set = false;
+  if (!attr_set) {
+    KX_HIP(hipFuncSetAttribute((const void *)attn_front_k, hipFuncAttributeMaxDynamicSharedMemorySize, 156 * 1024));
+    attr_set = true;
+  }
+  FrontArgs a = {};
+  a.x = g_qkv.x; a.input_ln = g_qkv.norm_w; a.w_qkv = g_qkv.w0; a.qa_ln = g_qb.norm_w; a.w_qb = g_qb.w0;
+  a.qa = q;
+  a.hand = hand; a.hidden = hidden; a.q_rank = q_rank; a.rows_b = rows_b; a.eps = g_qkv.norm_eps; a.tag = tag; a.err = err;
+  hipLaunchKernelGGL(attn_front_k, dim3(G), dim3(FR_THREADS), lds, st, a);
+  KX_LAUNCH_CHECK();
+  *done = true;
+  return KX_OK;
+}

@@ -24,6 +24,7 @@
 #include "kx_attn_parts.h"
 #include "kx_common.h"
 #include "kx_dense.h"
+#include "kx_front.h"
 #include "kx_index.h"
 #include "kx_load.h"
 #include "kx_mla.h"
@@ -78,6 +79,9 @@ struct kx_model {
   float *qabs, *partial, *logits, *argmax_scratch;
   uint32_t *ids, *next, *history;  // [max_context][B], [B], [max_context][B]
   int *head_count;                 // [heads] arrival counters of the q_b GEMV that finishes the query; zero between launches
+  int *front_err;                  // error flag of the fused attention front (kx_front.hip): a wait gave up
+  uint32_t *front_hand;            // its tagged words
+  uint32_t front_tag = 0;          // tag of its last launch
   int4 *head_work;                 // [heads], [step tokens * heads]: the groups of head_groups_k
   int *head_pairs;
   uint32_t fusion = KX_FUSE_ALL;
@@ -201,6 +205,8 @@ int layout(const kx_config *c, Plan &p, kx_model *m) {
   auto *next = KX_AT(uint32_t *, B * 4);
   auto *history = KX_AT(uint32_t *, (size_t)c->max_context * B * 4);
   auto *head_count = KX_AT(int *, (size_t)c->heads * 4);
+  auto *front_err = KX_AT(int *, 4);
+  auto *front_hand = KX_AT(uint32_t *, kx_front_hand_words(c->q_rank, (int)KVA, (int)KD) * 4);
   auto *head_work = KX_AT(int4 *, (size_t)c->heads * 16);
   auto *head_pairs = KX_AT(int *, BT * c->heads * 4);
 #undef KX_AT
@@ -208,7 +214,7 @@ int layout(const kx_config *c, Plan &p, kx_model *m) {
   if (m) {
     m->x = x; m->n = n; m->qkv = qkv; m->qa = qa; m->q = q; m->o_lat = o_lat; m->att = att; m->dmid = dmid;
     m->qabs = qabs; m->partial = partial; m->logits = logits; m->argmax_scratch = argmax_scratch; m->ids = ids; m->next = next; m->history = history;
-    m->head_count = head_count; m->head_work = head_work; m->head_pairs = head_pairs;
+    m->head_count = head_count; m->front_err = front_err; m->front_hand = front_hand; m->head_work = head_work; m->head_pairs = head_pairs;
   }
   return KX_OK;
 }
@@ -312,27 +318,35 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample, int C = 1) {
     KxGemvArgs g = {};
     g.w0 = L.qkv_a; g.x = m->n; g.x_stride = H; g.out = m->qkv; g.out_stride = QKV; g.rows = QKV; g.cols = H; g.tokens = B;
     if (fuse) { g.x = m->x; g.norm_w = L.input_ln; g.norm_eps = c.rms_eps; }
-    else KX_TRY(kx_rmsnorm_launch(m->x, L.input_ln, m->n, B, H, H, H, c.rms_eps, st));                 // :812
-    KX_TRY(dense(KX_EPI_BF16, g));                                                                      // :813, :816
-    g = {};
-    g.w0 = L.qb; g.x = m->qa; g.x_stride = c.q_rank; g.out = m->q; g.out_stride = KD; g.rows = KD; g.cols = c.q_rank; g.tokens = B;
-    if (fuse) { g.x = m->qkv; g.x_stride = QKV; g.norm_w = L.qa_ln; g.norm_eps = c.rms_eps; }
-    else KX_TRY(kx_rmsnorm_launch(m->qkv, L.qa_ln, m->qa, B, c.q_rank, QKV, c.q_rank, c.rms_eps, st)); // :814
-    // W_UK absorb + rope(q); kv_a norm, rope of the shared key, cache row (:817-824): inside the q_b launch when
-    // the shapes allow, else as a kernel of their own
-    bool absorbed = false;
-    if (fuse && (m->fusion & KX_FUSE_ABSORB)) {
-      QAbsArgs qa = {};
-      qa.q = m->q; qa.kvb = L.kvb; qa.rope_row = rope_row; qa.qabs = m->qabs; qa.kva = m->qkv + c.q_rank; qa.kva_stride = QKV;
-      qa.w_kv_ln = L.kv_ln; qa.cache = L.cache; qa.seq_stride = seq_stride; qa.heads = c.heads; qa.nope = c.qk_nope;
-      qa.rope = c.qk_rope; qa.v_head = c.v_head; qa.kv_rank = c.kv_rank; qa.pos = pos; qa.eps = c.rms_eps;
-      qa.head_count = m->head_count;
-      KX_TRY(kx_gemv_absorb_launch(g, qa, &absorbed, st));                                             // :815
+    KxGemvArgs gb = {};
+    gb.w0 = L.qb; gb.x = m->qa; gb.x_stride = c.q_rank; gb.out = m->q; gb.out_stride = KD; gb.rows = KD; gb.cols = c.q_rank; gb.tokens = B;
+    if (fuse) { gb.x = m->qkv; gb.x_stride = QKV; gb.norm_w = L.qa_ln; gb.norm_eps = c.rms_eps; }
+    QAbsArgs qa = {};
+    qa.q = m->q; qa.kvb = L.kvb; qa.rope_row = rope_row; qa.qabs = m->qabs; qa.kva = m->qkv + c.q_rank; qa.kva_stride = QKV;
+    qa.w_kv_ln = L.kv_ln; qa.cache = L.cache; qa.seq_stride = seq_stride; qa.heads = c.heads; qa.nope = c.qk_nope;
+    qa.rope = c.qk_rope; qa.v_head = c.v_head; qa.kv_rank = c.kv_rank; qa.pos = pos; qa.eps = c.rms_eps;
+    qa.head_count = m->head_count;
+    // One token: the whole front of the attention block -- q_a | kv_a, q_b, the W_UK absorb, RoPE, the cache row -- as
+    // one resident launch where the shapes and the device allow it (kx_front.hip; same sums, same bits)
+    bool front = false;
+    if (fuse && B == 1 && (m->fusion & KX_FUSE_FRONT)) {
+      const uint32_t tag = m->front_tag % 65535u + 1u;
+      KX_TRY(kx_attn_front_launch(g, gb, qa, m->front_hand, tag, m->front_err, &front, st));
+      if (front) m->front_tag = tag;
     }
-    if (!absorbed) {
-      KX_TRY(dense(KX_EPI_BF16, g));                                                                    // :815
-      KX_TRY(kx_q_absorb_launch(m->q, L.kvb, rope_row, m->qabs, B, c.heads, c.qk_nope, c.qk_rope, c.v_head, c.kv_rank,
-                                m->qkv + c.q_rank, QKV, L.kv_ln, L.cache, seq_stride, pos, c.rms_eps, st, C > 1 ? NB : 0));
+    if (!front) {
+      if (!fuse) KX_TRY(kx_rmsnorm_launch(m->x, L.input_ln, m->n, B, H, H, H, c.rms_eps, st));                 // :812
+      KX_TRY(dense(KX_EPI_BF16, g));                                                                      // :813, :816
+      if (!fuse) KX_TRY(kx_rmsnorm_launch(m->qkv, L.qa_ln, m->qa, B, c.q_rank, QKV, c.q_rank, c.rms_eps, st)); // :814
+      // W_UK absorb + rope(q); kv_a norm, rope of the shared key, cache row (:817-824): inside the q_b launch when
+      // the shapes allow, else as a kernel of their own
+      bool absorbed = false;
+      if (fuse && (m->fusion & KX_FUSE_ABSORB)) KX_TRY(kx_gemv_absorb_launch(gb, qa, &absorbed, st));     // :815
+      if (!absorbed) {
+        KX_TRY(dense(KX_EPI_BF16, gb));                                                                   // :815
+        KX_TRY(kx_q_absorb_launch(m->q, L.kvb, rope_row, m->qabs, B, c.heads, c.qk_nope, c.qk_rope, c.v_head, c.kv_rank,
+                                  m->qkv + c.q_rank, QKV, L.kv_ln, L.cache, seq_stride, pos, c.rms_eps, st, C > 1 ? NB : 0));
+      }
     }
     g = {};  // W_UV of :818 per head
     g.w0 = L.kvb; g.x = m->o_lat; g.x_stride = c.heads * c.kv_rank; g.out = m->att; g.out_stride = VD; g.rows = VD;
@@ -468,7 +482,9 @@ static int model_new(const kx_config *cfg, const char *who, kx_model **out) {
   for (auto &ev : m->ev)
     if (!rc && hipEventCreate(&ev) != hipSuccess) rc = KX_ERR_HIP;
   if (!rc && cfg->first_dense < cfg->n_layers) rc = kx_moe_workspace_create(cfg, step_tokens(cfg), &m->moe_ws);
-  if (!rc && (hipMemsetAsync(m->head_count, 0, (size_t)cfg->heads * 4, m->st) != hipSuccess || hipStreamSynchronize(m->st) != hipSuccess))
+  if (!rc && (hipMemsetAsync(m->head_count, 0, (size_t)cfg->heads * 4, m->st) != hipSuccess ||
+              hipMemsetAsync(m->front_err, 0, 4, m->st) != hipSuccess ||
+              hipMemsetAsync(m->front_hand, 0, kx_front_hand_words(cfg->q_rank, cfg->kv_rank + cfg->qk_rope, cfg->heads * (cfg->qk_nope + cfg->qk_rope)) * 4, m->st) != hipSuccess || hipStreamSynchronize(m->st) != hipSuccess))
     rc = KX_ERR_HIP;
   if (rc) {
     if (rc == KX_ERR_HIP && !kx_last_error()[0]) kx_set_error("%s: HIP resource creation failed", who);
@@ -584,6 +600,20 @@ static int check_ids(const kx_model *m, const uint32_t *ids, size_t n) {
   return KX_OK;
 }
 
+// Synchronises the model's stream and reports a grid barrier of the fused attention front that gave up waiting
+// (kx_front.hip): the steps since then computed with values that were not there yet.
+static int check_front(kx_model *m) {
+  int flag = 0;
+  KX_HIP(hipMemcpyAsync(&flag, m->front_err, 4, hipMemcpyDeviceToHost, m->st));
+  KX_HIP(hipStreamSynchronize(m->st));
+  if (flag) {
+    kx_set_error("kx_model: a grid barrier of the fused attention front timed out (not all of its workgroups were resident); "
+                 "results since then are invalid -- switch it off with kx_model_set_fusion(model, KX_FUSE_ALL & ~KX_FUSE_FRONT)");
+    return KX_ERR_STATE;
+  }
+  return KX_OK;
+}
+
 extern "C" int kx_prefill(kx_model *m, const uint32_t *h_ids, int32_t batch, int32_t prompt_len) {
   KX_REQUIRE(m && h_ids, "kx_prefill: null argument");
   KX_REQUIRE(batch > 0 && batch <= m->c.max_batch, "kx_prefill: batch=%d outside [1, %d]", batch, m->c.max_batch);
@@ -634,8 +664,7 @@ extern "C" int kx_greedy_sample(kx_model *m, uint32_t *h_out) {
   KX_REQUIRE(m && h_out, "kx_greedy_sample: null argument");
   KX_REQUIRE(m->sampled, "kx_greedy_sample: the last step did not sample");
   KX_HIP(hipMemcpyAsync(h_out, m->next, (size_t)m->batch * 4, hipMemcpyDeviceToHost, m->st));
-  KX_HIP(hipStreamSynchronize(m->st));
-  return KX_OK;
+  return check_front(m);
 }
 
 extern "C" int kx_generate(kx_model *m, const uint32_t *h_prompt, int32_t batch, int32_t prompt_len, int32_t n_tokens,
@@ -678,7 +707,7 @@ extern "C" int kx_generate(kx_model *m, const uint32_t *h_prompt, int32_t batch,
   }
   KX_HIP(hipEventRecord(m->ev[2], m->st));
   if ((rc = read_back())) return rc;
-  KX_HIP(hipStreamSynchronize(m->st));
+  if ((rc = check_front(m))) return rc;
   KX_HIP(hipEventElapsedTime(&m->ms_prefill, m->ev[0], m->ev[1]));
   KX_HIP(hipEventElapsedTime(&m->ms_decode, m->ev[1], m->ev[2]));
   m->steps_decoded = made;

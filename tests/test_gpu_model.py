@@ -314,9 +314,10 @@ def test_kimi_shape_stack_batch_invariance(kxlib, ox):
 
 @pytest.mark.parametrize("shape", ["small-1", "small-3", "kimi"])
 def test_fused_and_separate_launches_agree(kxlib, ox, shape):
-    # the q_b GEMV that finishes the query in its own launch, and (batch 1) the routed down launch that finishes the
-    # MoE layer, against the same steps as kernels of their own: cache rows, hidden state, logits and ids to the bit
-    # (the oracle comparisons above run the fused forms)
+    # the q_b GEMV that finishes the query in its own launch, (batch 1) the routed down launch that finishes the MoE
+    # layer, and (batch 1, Kimi shapes) the resident launch that runs the whole front of the attention block, against
+    # the same steps as kernels of their own: cache rows, hidden state, logits and ids to the bit (the oracle
+    # comparisons above run the fused forms)
     say(f"fusion on/off {shape}")
     if shape == "kimi":
         cfg = default_config()
@@ -328,7 +329,7 @@ def test_fused_and_separate_launches_agree(kxlib, ox, shape):
         prompt_len, n_tokens = 11, 9
     prompt = O.tokens_u32(batch * prompt_len, cfg.seed, 4, cfg.vocab).reshape(batch, prompt_len)
     got = []
-    for mask in (3, 0, 1, 2):
+    for mask in (7, 0, 1, 2, 3, 4):
         km = KxModel(kxlib, cfg)
         check(kxlib.kx_model_set_fusion(km.h, mask))
         rc, out, _ = km.generate(prompt, n_tokens)
@@ -339,10 +340,10 @@ def test_fused_and_separate_launches_agree(kxlib, ox, shape):
         km.close()
     assert kxlib.kx_model_set_fusion(None, 1) != 0
     km = KxModel(kxlib, cfg)
-    assert kxlib.kx_model_set_fusion(km.h, 4) != 0 and b"mask" in kxlib.kx_last_error()
+    assert kxlib.kx_model_set_fusion(km.h, 8) != 0 and b"mask" in kxlib.kx_last_error()
     km.close()
     o0, h0, l0, c0 = got[1]   # every launch on its own
-    for (o1, h1, l1, c1) in (got[0], got[2], got[3]):
+    for (o1, h1, l1, c1) in got[:1] + got[2:]:
         assert all((a == b).all() for a, b in zip(c1, c0)), "latent cache differs"
         assert (h1 == h0).all() and (l1 == l0).all() and (o1 == o0).all()
 
