@@ -371,6 +371,8 @@ def run_stack(args, extra_batches=()):
     t_create = time.perf_counter() - t0
     st = C.c_void_p()
     check(lib.kx_model_stream(model, C.byref(st)))
+    if args.fusion is not None:             # which steps ride inside the launch before them (KX_FUSE_* of include/kx.h); same results
+        check(lib.kx_model_set_fusion(model, args.fusion))
     out = stack_leg(lib, cfg, model, st, B, P, K, W, args.seed, args.prefill_chunk)
     out["extra"] = {b: stack_leg(lib, cfg, model, st, b, P, K, W, args.seed, args.prefill_chunk) for b in extra_batches}
     check(lib.kx_model_destroy(model))
@@ -670,6 +672,7 @@ def main():
     ap.add_argument("--prompt", type=int, default=1024)
     ap.add_argument("--prefill-chunk", type=int, default=1, help="prompt positions per prefill step (1: the reference's token-by-token prefill)")
     ap.add_argument("--stack-layers", type=int, default=24)
+    ap.add_argument("--fusion", type=lambda v: int(v, 0), default=None, help="stack: mask for kx_model_set_fusion (default: the library's, all on)")
     ap.add_argument("--cpu-layers", type=int, default=24)
     ap.add_argument("--no-b32", action="store_true", help="default run: skip the batch-32 leg of config 5")
     ap.add_argument("--tokens", type=int, default=1)

@@ -8,3 +8,4 @@
 inline size_t kx_front_hand_words(int q_rank, int kva, int q_rows) { return (size_t)q_rank + kva + q_rows; }
 int kx_attn_front_launch(const KxGemvArgs &g_qkv, const KxGemvArgs &g_qb, const QAbsArgs &q, uint32_t *hand, uint32_t tag, int *err,
                          bool *done, hipStream_t st);
+int kx_attn_back_launch(const KxGemvArgs &g_uv, const KxGemvArgs &g_o, uint32_t *hand, uint32_t tag, int *err, bool *done, hipStream_t st);

@@ -1,4 +1,5 @@
-// kx_front.hip -- the front of the attention block for one token as one launch:
+// kx_front.hip -- the two halves of the attention block around the attention itself, for one token, as one resident
+// launch each (the back: attn_back_k below).  The front:
 //   q_a GEMV with the input RMSNorm      (src/kimi_exec.cu:812-813)
 //   q_b GEMV with the q_a RMSNorm        (:814-815)
 //   kv_a GEMV, its RMSNorm, RoPE of the shared key, the cache row   (:816-817, :820-824)
@@ -7,7 +8,7 @@
 // form of this library runs them as two (gemv_bf16_k for q_a|kv_a, gemv_absorb_k).  q_b needs all of q_a and the
 // absorb needs a whole head of q, so the steps are a chain, and as launches each of them pays its start and its
 // drain while the memory system idles.  Here one workgroup per CU stays resident, and its 48 rows of q_b (144 KB)
-// are copied global -> LDS while q_a is computed, so that the q_b step reads them at LDS speed.
+// are copied global -> LDS while q_a travels between the workgroups, so that the q_b step reads them at LDS speed.
 //
 //   every workgroup: 6 rows of q_a and 2 or 3 of kv_a, all loads out at once (waves 0..6) -> hand the 8 or 9 values
 //                    over; waves 4..7 start the copy of the workgroup's 48 rows of q_b into LDS -> take all of q_a ->
@@ -60,23 +61,50 @@ struct FrontArgs {
 __device__ __forceinline__ void hand_store(uint32_t *p, uint32_t tag, uint16_t v) {
   __hip_atomic_store(p, (tag << 16) | v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-// reads n (at most 8) consecutive words until all carry the tag; gives up after FR_SPIN_LIMIT polls (flag set,
-// values as they are), so that the grid always drains
+// Four consecutive words at agent scope (served by the point of coherence, not by a line an L2 may still hold) as one
+// 16-byte request; hand_wait completes the requests of a wave and ties the registers to the wait, so that no use of
+// them is scheduled before it.
+// the compiler may not move a memory access across this point: loads are requested in the order they are written
+__device__ __forceinline__ void issue_order() { asm volatile("" ::: "memory"); }
+typedef unsigned int hand4 __attribute__((ext_vector_type(4)));  // a register quad, as inline asm takes it
+__device__ __forceinline__ void hand_request4(const uint32_t *p, hand4 &v) {
+  asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v) : "v"(p) : "memory");
+}
+__device__ __forceinline__ void hand_wait(hand4 &a) { asm volatile("s_waitcnt vmcnt(0)" : "+v"(a)::"memory"); }
+__device__ __forceinline__ void hand_wait(hand4 &a, hand4 &b) { asm volatile("s_waitcnt vmcnt(0)" : "+v"(a), "+v"(b)::"memory"); }
+__device__ __forceinline__ bool hand_tagged(const hand4 &v, uint32_t tag) {
+  return (v.x >> 16) == tag && (v.y >> 16) == tag && (v.z >> 16) == tag && (v.w >> 16) == tag;
+}
+// the bf16 halves of four tagged words as two packed words
+__device__ __forceinline__ uint2 hand_pack(const hand4 &v) { return make_uint2((v.x & 0xffffu) | (v.y << 16), (v.z & 0xffffu) | (v.w << 16)); }
+// one more poll has failed: true when the reader should give up (the flag is set: too many polls, or an earlier
+// launch gave up already), so that the grid always drains
+__device__ __forceinline__ bool hand_give_up(int &polls, int *err) {
+  if (++polls > FR_SPIN_LIMIT || (polls == 1 && __hip_atomic_load(err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) {
+    __hip_atomic_store(err, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return true;
+  }
+  __builtin_amdgcn_s_sleep(2);
+  return false;
+}
+// reads N (4 or 8) consecutive words, 16-byte aligned, until all carry the tag; returns their bf16 halves packed
 template <int N>
-__device__ __forceinline__ void hand_load(const uint32_t *p, uint32_t tag, int *err, uint32_t (&w)[N]) {
+__device__ __forceinline__ void hand_load(const uint32_t *p, uint32_t tag, int *err, uint32_t (&packed)[N / 2]) {
+  static_assert(N == 4 || N == 8, "words per call");
   int polls = 0;
+  hand4 v0, v1 = {0, 0, 0, 0};
   while (true) {
-    bool ok = true;
-#pragma unroll
-    for (int i = 0; i < N; ++i) w[i] = __hip_atomic_load(p + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-#pragma unroll
-    for (int i = 0; i < N; ++i) ok = ok && (w[i] >> 16) == tag;
-    if (ok) return;
-    if (++polls > FR_SPIN_LIMIT || (polls == 1 && __hip_atomic_load(err, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) {
-      __hip_atomic_store(err, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      return;
-    }
-    __builtin_amdgcn_s_sleep(2);
+    hand_request4(p, v0);
+    if (N == 8) hand_request4(p + 4, v1);
+    if (N == 8) hand_wait(v0, v1);
+    else hand_wait(v0);
+    if ((hand_tagged(v0, tag) && (N == 4 || hand_tagged(v1, tag))) || hand_give_up(polls, err)) break;
+  }
+  const uint2 a = hand_pack(v0);
+  packed[0] = a.x; packed[1] = a.y;
+  if (N == 8) {
+    const uint2 b = hand_pack(v1);
+    packed[2] = b.x; packed[3] = b.y;
   }
 }
 
@@ -114,6 +142,7 @@ __global__ void __launch_bounds__(FR_THREADS) attn_front_k(FrontArgs a) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) nx[j] = ((const uint4 *)a.x)[min(tid + 256 * j, chunks - 1)];
   }
+  issue_order();
   if (wave < 7) {
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
@@ -129,6 +158,7 @@ __global__ void __launch_bounds__(FR_THREADS) attn_front_k(FrontArgs a) {
         wbuf[i][k] = ld_stream16(a.w_qkv + (size_t)row * H + (uint32_t)(k ? s1 : s0) * 512u + (uint32_t)lane * 8u);
     }
   }
+  issue_order();
 #pragma unroll
   for (int s = 0; s < 4; ++s)
     if (s < SB) gb[s] = *(const uint4 *)(a.qa_ln + s * 512 + lane * 8);
@@ -227,11 +257,8 @@ __global__ void __launch_bounds__(FR_THREADS) attn_front_k(FrontArgs a) {
     const int chunks = a.q_rank >> 3;  // at most 256: one chunk per thread
     float v = 0.0f;
     if (tid < chunks) {
-      uint32_t w[8];
-      hand_load<8>(hand_qa + tid * 8, a.tag, a.err, w);
       uint32_t o[4];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) o[e] = (w[2 * e] & 0xffffu) | (w[2 * e + 1] << 16);
+      hand_load<8>(hand_qa + tid * 8, a.tag, a.err, o);
       ((uint4 *)s_row)[tid] = make_uint4(o[0], o[1], o[2], o[3]);
       float f[8];
       unpack8(f, make_uint4(o[0], o[1], o[2], o[3]));
@@ -310,10 +337,9 @@ __global__ void __launch_bounds__(FR_THREADS) attn_front_k(FrontArgs a) {
     uint4 mine = make_uint4(0, 0, 0, 0);
     float v = 0.0f;
     if (tid < chunks) {  // chunks <= 256 (the launcher checks)
-      uint32_t w[8];
-      hand_load<8>(hand_kv + tid * 8, a.tag, a.err, w);
-      mine = make_uint4((w[0] & 0xffffu) | (w[1] << 16), (w[2] & 0xffffu) | (w[3] << 16), (w[4] & 0xffffu) | (w[5] << 16),
-                        (w[6] & 0xffffu) | (w[7] << 16));
+      uint32_t o[4];
+      hand_load<8>(hand_kv + tid * 8, a.tag, a.err, o);
+      mine = make_uint4(o[0], o[1], o[2], o[3]);
       float f[8];
       unpack8(f, mine);
 #pragma unroll
@@ -337,14 +363,17 @@ __global__ void __launch_bounds__(FR_THREADS) attn_front_k(FrontArgs a) {
         o[e] = (uint32_t)kx_bf16_rne(kx_bfround(f[2 * e] * scale) * g[2 * e]) | ((uint32_t)kx_bf16_rne(kx_bfround(f[2 * e + 1] * scale) * g[2 * e + 1]) << 16);
       ((uint4 *)crow)[tid] = make_uint4(o[0], o[1], o[2], o[3]);
     }
-    if (tid >= 256 && tid < 256 + half) {
-      const int p = tid - 256;
-      uint32_t w[2];
-      hand_load<2>(hand_kv + kv_rank + 2 * p, a.tag, a.err, w);
-      float lo, hi;
-      kxa::rope_pair(kx_bf16_f32((uint16_t)w[0]), kx_bf16_f32((uint16_t)w[1]), kx_bf16_f32(a.qa.rope_row[p]), kx_bf16_f32(a.qa.rope_row[half + p]), lo, hi);
-      crow[kv_rank + p] = kx_bf16_rne(lo);
-      crow[kv_rank + half + p] = kx_bf16_rne(hi);
+    if (tid >= 256 && tid < 256 + (half >> 1)) {  // two interleaved pairs per thread (rope is a multiple of 4)
+      uint32_t o[2];
+      hand_load<4>(hand_kv + kv_rank + 4 * (tid - 256), a.tag, a.err, o);
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int p = 2 * (tid - 256) + u;
+        float lo, hi;
+        kxa::rope_pair(bf_lo(o[u]), bf_hi(o[u]), kx_bf16_f32(a.qa.rope_row[p]), kx_bf16_f32(a.qa.rope_row[half + p]), lo, hi);
+        crow[kv_rank + p] = kx_bf16_rne(lo);
+        crow[kv_rank + half + p] = kx_bf16_rne(hi);
+      }
     }
   }
   // ---- a quarter of the head's q_abs: the sums of kxa::absorb_head_block for columns [cq * j, cq * (j + 1))
@@ -356,10 +385,10 @@ __global__ void __launch_bounds__(FR_THREADS) attn_front_k(FrontArgs a) {
     float *out = a.qa.qabs + (size_t)h * (kv_rank + rope);
     __syncthreads();  // s_row (the q_a row) and the q_b rows are no longer read
     if (tid < (qk >> 2)) {
-      uint32_t w[4];
-      hand_load<4>(hand_q + (size_t)h * qk + tid * 4, a.tag, a.err, w);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) qs[tid * 4 + e] = kx_bf16_f32((uint16_t)w[e]);
+      uint32_t o[2];
+      hand_load<4>(hand_q + (size_t)h * qk + tid * 4, a.tag, a.err, o);
+      qs[tid * 4 + 0] = bf_lo(o[0]); qs[tid * 4 + 1] = bf_hi(o[0]);
+      qs[tid * 4 + 2] = bf_lo(o[1]); qs[tid * 4 + 3] = bf_hi(o[1]);
     }
     __syncthreads();
     if (tid < 8 * ncg) {  // chain ab_chain over d = ab_chain, ab_chain + 8, ..., W_UK rows from the registers
@@ -391,6 +420,173 @@ __global__ void __launch_bounds__(FR_THREADS) attn_front_k(FrontArgs a) {
   }
 }
 
+
+// ---------------------------------------------------------------------------------------------------------------
+// The back of the attention block for one token as one launch: the merge of the attention's span partials, the
+// per-head W_UV product (src/kimi_exec.cu:818 as W_UV) and o_proj with the residual add (:826-827).  As launches
+// of their own (the W_UV GEMV that merges while it loads, the o_proj GEMV) the second one streams 117 MB and
+// cannot ask for a byte of it before the first has drained.  Here every workgroup merges and multiplies its quarter
+// of a head, hands the 32 values over as tagged words, requests the first five tiles of its o_proj rows and then
+// takes all 8192 values from the other workgroups.  A wave's loads return in order, so its polls come back behind
+// the weights it has asked for -- which is when the others have handed over, about: five of a workgroup's seven
+// tiles are in registers by then.  The tiles are not requested before the hand-over: a CU's memory pipeline takes
+// requests in order, and the 32 stores would sit behind 160 KB of them (measured: 2.5 us later, no gain from the
+// earlier start).  Sums as in kx_gemv_body.h (lane partial over 8 columns, butterfly over the wave, slices left to
+// right) and in its merge of the partials: equal to the separate launches to the bit.
+constexpr int BK_THREADS = 512;  // 8 waves: wave w owns rows 4 w .. of its quarter head, then the slices w and w + 8 of o_proj
+constexpr int BK_PRE = 5;        // o_proj tiles (4 rows x 2 slices per wave) in flight per wave
+constexpr int BK_SPANS = 32;     // span partials a thread holds in registers
+
+struct BackArgs {
+  const float *pm, *pz, *po;  // attention partials of the token: [spans][heads], same, [spans][heads][kv_rank]
+  int spans, heads;
+  const uint16_t *kvb;        // kv_b: W_UV[h] = rows h * (nope + v_head) + nope .. of it
+  int nope, v_head, kv_rank;
+  const uint16_t *w_o;        // bf16 [hidden, heads * v_head]
+  uint16_t *x;                // the residual row, updated in place
+  int hidden, vd;
+  uint32_t *hand;             // [heads * v_head] tagged words
+  uint32_t tag;
+  int *err;
+};
+
+__global__ void __launch_bounds__(BK_THREADS) attn_back_k(BackArgs a) {
+  __shared__ float s_x[512];                                   // the head's merged attention output, bf16 values
+  __shared__ __attribute__((aligned(16))) uint16_t s_att[8192];  // the token's attention output, all heads
+  __shared__ float s_part[8 * 4 * 16];                         // [row of the workgroup][slice]
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int bid = blockIdx.x, h = bid >> 2, jq = bid & 3;
+  const int rows_o = a.hidden / (int)gridDim.x, tiles = rows_o >> 2;  // 28 rows, 7 tiles of 4 at Kimi-K2 shapes
+  const int s0 = wave, s1 = wave + 8;
+  // ---- requests, in the order of need: the head's partials, this wave's W_UV rows
+  const size_t my = (size_t)min(lane, a.spans - 1) * a.heads + h;
+  const float mj = a.pm[my], zj = a.pz[my];
+  float o[BK_SPANS];
+#pragma unroll
+  for (int j = 0; j < BK_SPANS; ++j) o[j] = j < a.spans ? a.po[((size_t)j * a.heads + h) * a.kv_rank + tid] : 0.0f;
+  issue_order();
+  uint4 wuv[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    wuv[i] = ld_stream16(a.kvb + ((size_t)h * (a.nope + a.v_head) + a.nope + jq * 32 + wave * 4 + i) * a.kv_rank + lane * 8);
+  issue_order();
+  uint4 wo[BK_PRE][4][2];
+  const uint16_t *wo_base = a.w_o + (size_t)bid * rows_o * a.vd + lane * 8;
+  auto load_tile = [&](uint4 (&buf)[4][2], int t) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      buf[i][0] = ld_stream16(wo_base + (size_t)(t * 4 + i) * a.vd + s0 * 512);
+      buf[i][1] = ld_stream16(wo_base + (size_t)(t * 4 + i) * a.vd + s1 * 512);
+    }
+  };
+  // ---- the merge of the span partials (kx_gemv_body.h load_x): M = max M_j; w_j = exp(M_j - M);
+  // Z = fma(Z_j, w_j, Z), O = fma(O_j, w_j, O) over the spans in order; x = bf(O / Z).  Thread c owns column c.
+  {
+    const float M = kxw::wave_max_f32(lane < a.spans ? mj : -__builtin_inff());
+    const float wj = kx_expf(mj - M);
+    float Z = 0.0f, O = 0.0f;
+    for (int j = 0; j < a.spans; ++j)
+      Z = __builtin_fmaf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, zj), j)),
+                         __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wj), j)), Z);
+#pragma unroll
+    for (int j = 0; j < BK_SPANS; ++j)
+      if (j < a.spans) O = __builtin_fmaf(o[j], __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wj), j)), O);
+    s_x[tid] = kx_bfround(O / Z);
+  }
+  kx_lds_barrier();
+  // ---- W_UV: rows 32 jq + 4 wave + i of the head; one 512-column slice, so the butterfly's value is the row's
+  {
+    float xs[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) xs[e] = s_x[lane * 8 + e];
+    float v[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float wf[8];
+      unpack8(wf, wuv[i]);
+      float acc = 0.0f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc = __builtin_fmaf(wf[e], xs[e], acc);
+      v[i] = acc;
+    }
+    kxw::reduce<4, 64>(v, lane);
+    if (kxw::reduce_writer<4, 64>(lane)) {
+#pragma unroll
+      for (int j = 0; j < kxw::reduce_out<4, 64>(); ++j) {
+        const int i = kxw::reduce_index<4, 64>(lane, j);
+        hand_store(a.hand + (size_t)h * a.v_head + jq * 32 + wave * 4 + i, a.tag, kx_bf16_rne(v[j]));
+      }
+    }
+  }
+  // ---- the first o_proj tiles, behind the hand-over and in front of the polls
+#pragma unroll
+  for (int t = 0; t < BK_PRE; ++t) load_tile(wo[t], min(t, tiles - 1));
+  issue_order();
+  // ---- all of the token's attention output: 8192 words = 2048 requests of 16 bytes, four per thread; request i of
+  // thread t is number 512 i + t, so that a wave's request covers 1 KB in a row.  Asked for again until every word
+  // carries the tag.
+  {
+    const uint32_t *src = a.hand + (size_t)tid * 4;
+    hand4 v[4];
+    int polls = 0;
+    while (true) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) hand_request4(src + (size_t)i * 2048, v[i]);
+      asm volatile("s_waitcnt vmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3])::"memory");
+      if ((hand_tagged(v[0], a.tag) && hand_tagged(v[1], a.tag) && hand_tagged(v[2], a.tag) && hand_tagged(v[3], a.tag)) || hand_give_up(polls, a.err)) break;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) ((uint2 *)s_att)[i * 512 + tid] = hand_pack(v[i]);
+  }
+  kx_lds_barrier();
+  // ---- o_proj rows [rows_o * bid, +rows_o): BK_PRE tiles in flight, a tile's registers take the tile BK_PRE further on
+  float xo[2][8];
+  unpack8(xo[0], *(const uint4 *)(s_att + s0 * 512 + lane * 8));
+  unpack8(xo[1], *(const uint4 *)(s_att + s1 * 512 + lane * 8));
+  auto compute_tile = [&](const uint4 (&buf)[4][2], int t) {
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        float wf[8];
+        unpack8(wf, buf[i][k]);
+        float acc = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc = __builtin_fmaf(wf[e], xo[k][e], acc);
+        v[i * 2 + k] = acc;
+      }
+    kxw::reduce<8, 64>(v, lane);
+    if (kxw::reduce_writer<8, 64>(lane)) {
+#pragma unroll
+      for (int j = 0; j < kxw::reduce_out<8, 64>(); ++j) {
+        const int idx = kxw::reduce_index<8, 64>(lane, j);
+        s_part[(t * 4 + (idx >> 1)) * 16 + ((idx & 1) ? s1 : s0)] = v[j];
+      }
+    }
+  };
+  for (int t0 = 0; t0 < tiles; t0 += BK_PRE) {
+#pragma unroll
+    for (int u = 0; u < BK_PRE; ++u) {
+      const int t = t0 + u;
+      if (t < tiles) {
+        compute_tile(wo[u], t);
+        if (t + BK_PRE < tiles) load_tile(wo[u], t + BK_PRE);
+      }
+    }
+  }
+  kx_lds_barrier();
+  // ---- slices left to right, then x = bf(x + bf(y))  (add_k, :248-251)
+  if (tid < rows_o) {
+    const float *p = s_part + tid * 16;
+    float y = p[0];
+#pragma unroll
+    for (int s = 1; s < 16; ++s) y += p[s];
+    uint16_t *xr = a.x + (size_t)bid * rows_o + tid;
+    *xr = kx_bf16_rne(kx_bf16_f32(*xr) + kx_bfround(y));
+  }
+}
+
 }  // namespace
 
 // g_qkv: the q_a | kv_a GEMV as the separate launch would get it (w0 = [q_rank + kv_rank + rope, hidden], x = the
@@ -411,7 +607,7 @@ int kx_attn_front_launch(const KxGemvArgs &g_qkv, const KxGemvArgs &g_qb, const 
   const int hidden = g_qkv.cols, q_rank = g_qb.cols, qk = q.nope + q.rope, G = 4 * q.heads, kva = q.kv_rank + q.rope;
   if (g_qkv.tokens != 1 || g_qb.tokens != 1 || !hand || !err || !q.cache || !g_qkv.norm_w || !g_qb.norm_w || tag < 1 || tag > 65535) return KX_OK;
   if (G > cus || hidden != 14 * 512 || q_rank % 512 || q_rank / 512 > 4 || q_rank / 8 > 256) return KX_OK;
-  if (g_qkv.rows != q_rank + kva || g_qb.rows != q.heads * qk || qk % 16 || q.rope % 2 || q.rope / 2 > 256 || qk / 4 > FR_THREADS) return KX_OK;
+  if (g_qkv.rows != q_rank + kva || g_qb.rows != q.heads * qk || qk % 16 || q.rope % 4 || q.kv_rank % 4 || q.rope / 2 > 256 || qk / 4 > FR_THREADS) return KX_OK;
   const int rows_a = q_rank / G, rows_b = qk / 4;
   if (rows_b != 48 || q.nope != 128 || q.kv_rank / 4 > FR_THREADS || q_rank % G || rows_a != FR_ROWS - 3 || kva < 2 * G || kva > 3 * G || q.kv_rank % 32 || q.kv_rank / 8 > 256) return KX_OK;
   const size_t qb_bytes = (size_t)rows_b * q_rank * 2;
@@ -430,6 +626,33 @@ int kx_attn_front_launch(const KxGemvArgs &g_qkv, const KxGemvArgs &g_qb, const 
   a.qa = q;
   a.hand = hand; a.hidden = hidden; a.q_rank = q_rank; a.rows_b = rows_b; a.eps = g_qkv.norm_eps; a.tag = tag; a.err = err;
   hipLaunchKernelGGL(attn_front_k, dim3(G), dim3(FR_THREADS), lds, st, a);
+  KX_LAUNCH_CHECK();
+  *done = true;
+  return KX_OK;
+}
+
+// The W_UV GEMV that merges the attention partials (g_uv: mla_* set, row_block = v_head) and the o_proj GEMV with the
+// residual add (g_o: w0 = [hidden, heads * v_head], out = the residual row) of one token as one launch.  hand:
+// heads * v_head words; tag and err as for kx_attn_front_launch.  The W_UV output row (g_uv.out) is not written.
+int kx_attn_back_launch(const KxGemvArgs &g_uv, const KxGemvArgs &g_o, uint32_t *hand, uint32_t tag, int *err, bool *done, hipStream_t st) {
+  *done = false;
+  static int cus = 0;
+  if (!cus) {
+    int dev = 0;
+    KX_HIP(hipGetDevice(&dev));
+    KX_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+  }
+  const int heads = g_uv.mla_heads, G = 4 * heads;
+  if (g_uv.tokens != 1 || g_o.tokens != 1 || !g_uv.mla_po || !hand || !err || tag < 1 || tag > 65535) return KX_OK;
+  if (g_uv.mla_spans < 1 || g_uv.mla_spans > BK_SPANS || G > cus || g_uv.cols != 512 || g_uv.row_block != 128 || g_uv.rows != heads * 128) return KX_OK;
+  if (g_o.cols != g_uv.rows || g_o.cols != 16 * 512 || g_o.rows % G || (g_o.rows / G) % 4 || g_o.rows / G > 32 || g_o.rows / G < 4 * BK_PRE || g_o.norm_w) return KX_OK;
+  BackArgs a = {};
+  a.pm = g_uv.mla_pm; a.pz = g_uv.mla_pz; a.po = g_uv.mla_po; a.spans = g_uv.mla_spans; a.heads = heads;
+  a.kvb = g_uv.w0; a.nope = g_uv.w_block_off; a.v_head = g_uv.row_block; a.kv_rank = g_uv.cols;
+  if (g_uv.w_block_stride != a.nope + a.v_head) return KX_OK;
+  a.w_o = g_o.w0; a.x = (uint16_t *)g_o.out; a.hidden = g_o.rows; a.vd = g_o.cols;
+  a.hand = hand; a.tag = tag; a.err = err;
+  hipLaunchKernelGGL(attn_back_k, dim3(G), dim3(BK_THREADS), 0, st, a);
   KX_LAUNCH_CHECK();
   *done = true;
   return KX_OK;

@@ -82,6 +82,8 @@ struct kx_model {
   int *front_err;                  // error flag of the fused attention front (kx_front.hip): a wait gave up
   uint32_t *front_hand;            // its tagged words
   uint32_t front_tag = 0;          // tag of its last launch
+  uint32_t *back_hand;             // tagged words of the fused back of the attention block (W_UV output)
+  uint32_t back_tag = 0;
   int4 *head_work;                 // [heads], [step tokens * heads]: the groups of head_groups_k
   int *head_pairs;
   uint32_t fusion = KX_FUSE_ALL;
@@ -207,6 +209,7 @@ int layout(const kx_config *c, Plan &p, kx_model *m) {
   auto *head_count = KX_AT(int *, (size_t)c->heads * 4);
   auto *front_err = KX_AT(int *, 4);
   auto *front_hand = KX_AT(uint32_t *, kx_front_hand_words(c->q_rank, (int)KVA, (int)KD) * 4);
+  auto *back_hand = KX_AT(uint32_t *, VD * 4);
   auto *head_work = KX_AT(int4 *, (size_t)c->heads * 16);
   auto *head_pairs = KX_AT(int *, BT * c->heads * 4);
 #undef KX_AT
@@ -214,7 +217,7 @@ int layout(const kx_config *c, Plan &p, kx_model *m) {
   if (m) {
     m->x = x; m->n = n; m->qkv = qkv; m->qa = qa; m->q = q; m->o_lat = o_lat; m->att = att; m->dmid = dmid;
     m->qabs = qabs; m->partial = partial; m->logits = logits; m->argmax_scratch = argmax_scratch; m->ids = ids; m->next = next; m->history = history;
-    m->head_count = head_count; m->front_err = front_err; m->front_hand = front_hand; m->head_work = head_work; m->head_pairs = head_pairs;
+    m->head_count = head_count; m->front_err = front_err; m->front_hand = front_hand; m->back_hand = back_hand; m->head_work = head_work; m->head_pairs = head_pairs;
   }
   return KX_OK;
 }
@@ -377,12 +380,25 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample, int C = 1) {
       KX_TRY(kx_grouped_gemm_launch(false, false, L.kvb + (size_t)c.qk_nope * c.kv_rank, nullptr, nullptr, nullptr, m->o_lat, m->att,
                                     KX_GG_BF16, m->head_work, m->head_pairs, 0, c.heads, c.v_head, c.kv_rank, 1,
                                     (size_t)(c.qk_nope + c.v_head) * c.kv_rank, 0, B, st));
+      KxGemvArgs go = {};
+      go.w0 = L.o; go.x = m->att; go.x_stride = VD; go.out = m->x; go.out_stride = H; go.rows = H; go.cols = VD; go.tokens = B;
+      KX_TRY(dense(KX_EPI_RESID, go));                                                                  // :826-827
     } else {
-      KX_TRY(kx_gemv_launch(KX_EPI_BF16, g, st));
+      KxGemvArgs go = {};
+      go.w0 = L.o; go.x = m->att; go.x_stride = VD; go.out = m->x; go.out_stride = H; go.rows = H; go.cols = VD; go.tokens = B;
+      // One token: the merge of the attention partials, W_UV and o_proj with the residual add as one resident launch
+      // where the shapes and the device allow it (kx_front.hip; same sums, same bits)
+      bool back = false;
+      if (fuse && B == 1 && g.mla_po && (m->fusion & KX_FUSE_BACK)) {
+        const uint32_t tag = m->back_tag % 65535u + 1u;
+        KX_TRY(kx_attn_back_launch(g, go, m->back_hand, tag, m->front_err, &back, st));
+        if (back) m->back_tag = tag;
+      }
+      if (!back) {
+        KX_TRY(kx_gemv_launch(KX_EPI_BF16, g, st));
+        KX_TRY(dense(KX_EPI_RESID, go));                                                                // :826-827
+      }
     }
-    g = {};
-    g.w0 = L.o; g.x = m->att; g.x_stride = VD; g.out = m->x; g.out_stride = H; g.rows = H; g.cols = VD; g.tokens = B;
-    KX_TRY(dense(KX_EPI_RESID, g));                                                                     // :826-827
     if (l < c.first_dense) {                                                                            // bf16_mlp (:674-686)
       g = {};
       g.w0 = L.dgate; g.w1 = L.dup; g.x = m->n; g.x_stride = H; g.out = m->dmid; g.out_stride = c.dense_inter;
@@ -484,6 +500,7 @@ static int model_new(const kx_config *cfg, const char *who, kx_model **out) {
   if (!rc && cfg->first_dense < cfg->n_layers) rc = kx_moe_workspace_create(cfg, step_tokens(cfg), &m->moe_ws);
   if (!rc && (hipMemsetAsync(m->head_count, 0, (size_t)cfg->heads * 4, m->st) != hipSuccess ||
               hipMemsetAsync(m->front_err, 0, 4, m->st) != hipSuccess ||
+              hipMemsetAsync(m->back_hand, 0, (size_t)cfg->heads * cfg->v_head * 4, m->st) != hipSuccess ||
               hipMemsetAsync(m->front_hand, 0, kx_front_hand_words(cfg->q_rank, cfg->kv_rank + cfg->qk_rope, cfg->heads * (cfg->qk_nope + cfg->qk_rope)) * 4, m->st) != hipSuccess || hipStreamSynchronize(m->st) != hipSuccess))
     rc = KX_ERR_HIP;
   if (rc) {

@@ -332,7 +332,9 @@ int kx_model_steps_decoded(kx_model *model, int32_t *steps);
 #define KX_FUSE_MOE_TAIL 2u /* one token: shared down GEMV + combine + residual inside the routed down launch */
 #define KX_FUSE_FRONT 4u    /* one token, Kimi-K2 shapes, a device with at least 4 * heads CUs: q_a | kv_a, q_b, the absorb, RoPE and
                                the cache row as one resident launch with two grid barriers (takes precedence over KX_FUSE_ABSORB) */
-#define KX_FUSE_ALL 7u
+#define KX_FUSE_BACK 8u     /* one token, same conditions, up to 32 attention spans: the merge of the attention partials, W_UV and
+                               o_proj with the residual add as one resident launch */
+#define KX_FUSE_ALL 15u
 int kx_model_set_fusion(kx_model *model, uint32_t mask);
 /* The attention kernel this model's steps use: KX_MLA_AUTO (default), KX_MLA_VALU or KX_MLA_MATRIX_CORES, as for
  * kx_mla_decode.  A property of the model: other models of the process keep theirs.                          */

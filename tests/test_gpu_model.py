@@ -329,7 +329,7 @@ def test_fused_and_separate_launches_agree(kxlib, ox, shape):
         prompt_len, n_tokens = 11, 9
     prompt = O.tokens_u32(batch * prompt_len, cfg.seed, 4, cfg.vocab).reshape(batch, prompt_len)
     got = []
-    for mask in (7, 0, 1, 2, 3, 4):
+    for mask in (15, 0, 1, 2, 3, 4, 8):
         km = KxModel(kxlib, cfg)
         check(kxlib.kx_model_set_fusion(km.h, mask))
         rc, out, _ = km.generate(prompt, n_tokens)
@@ -340,7 +340,7 @@ def test_fused_and_separate_launches_agree(kxlib, ox, shape):
         km.close()
     assert kxlib.kx_model_set_fusion(None, 1) != 0
     km = KxModel(kxlib, cfg)
-    assert kxlib.kx_model_set_fusion(km.h, 8) != 0 and b"mask" in kxlib.kx_last_error()
+    assert kxlib.kx_model_set_fusion(km.h, 16) != 0 and b"mask" in kxlib.kx_last_error()
     km.close()
     o0, h0, l0, c0 = got[1]   # every launch on its own
     for (o1, h1, l1, c1) in got[:1] + got[2:]:
