@@ -121,6 +121,9 @@ struct kx_moe_workspace;
 // (kx_prefill.hip) instead of the GEMV kernels: such an expert's weights are streamed and dequantised once for all its
 // tokens (tolerance instead of bit parity); the experts with one pair keep the GEMV kernel
 #define KX_MOE_ROUTED_MATRIX_CORES 0x400u
+// internal (not among the public flags): the layer's first launch -- normed row in d_n, router logits, routing, shared
+// gate/up -- has been done by the caller's own launch (kx_front.hip's back launch with kx_moe_head_args): one token
+#define KX_MOE_HEAD_DONE 0x800u
 int *kx_moe_workspace_n_active(kx_moe_workspace *ws);  // device address of the count of distinct experts of the last call
 // the flags a caller of kx_moe_decode_layer may pass (include/kx.h documents them)
 #define KX_MOE_PUBLIC_FLAGS (1u | KX_MOE_SEPARATE_TAIL | KX_MOE_SHARED_MATRIX_CORES | KX_MOE_ROUTED_MATRIX_CORES)

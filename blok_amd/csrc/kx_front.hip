@@ -32,6 +32,7 @@
 #include "kx_gemv_body.h"
 #include "kx_lds_copy.h"
 #include "kx_math.h"
+#include "kx_route.h"
 #include "kx_wave.h"
 
 namespace {
@@ -102,7 +103,7 @@ __device__ __forceinline__ void hand_load(const uint32_t *p, uint32_t tag, int *
   }
   const uint2 a = hand_pack(v0);
   packed[0] = a.x; packed[1] = a.y;
-  if (N == 8) {
+  if constexpr (N == 8) {
     const uint2 b = hand_pack(v1);
     packed[2] = b.x; packed[3] = b.y;
   }
@@ -445,19 +446,44 @@ struct BackArgs {
   const uint16_t *w_o;        // bf16 [hidden, heads * v_head]
   uint16_t *x;                // the residual row, updated in place
   int hidden, vd;
-  uint32_t *hand;             // [heads * v_head] tagged words
+  uint32_t *hand;             // tagged words: [heads * v_head] attention output; HEAD: [hidden] residual row, [2 * experts] router logits
   uint32_t tag;
   int *err;
+  KxMoeHeadArgs hd;           // HEAD only
 };
 
+constexpr int HD_TILES = 5;   // the head's rows as tiles of 4: 8 gate, 8 up, 2 router rows, 2 unused
+constexpr int HD_O_TILES = 7; // o_proj tiles of a workgroup when the head rides along (hidden = 28 * 256)
+
+// HEAD: the launch goes on with the head of the MoE layer (the router and shared gate/up launch of kx_moe.hip):
+// post-attention RMSNorm, the shared expert's gate and up rows with SwiGLU, the router's logits, top-k and bucketing.
+// The residual row travels between the workgroups as the attention output does; a workgroup's 18 rows of the three
+// matrices are requested into the o_proj tiles' registers as those are used up, so the weight stream does not stop
+// for the hand-over.  The last workgroup takes the logits from the others and routes (kx_route.h, the same code the
+// router launch runs).  Sums as in kx_gemv_body.h.
+template <bool HEAD>
 __global__ void __launch_bounds__(BK_THREADS) attn_back_k(BackArgs a) {
   __shared__ float s_x[512];                                   // the head's merged attention output, bf16 values
   __shared__ __attribute__((aligned(16))) uint16_t s_att[8192];  // the token's attention output, all heads
   __shared__ float s_part[8 * 4 * 16];                         // [row of the workgroup][slice]
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int bid = blockIdx.x, h = bid >> 2, jq = bid & 3;
-  const int rows_o = a.hidden / (int)gridDim.x, tiles = rows_o >> 2;  // 28 rows, 7 tiles of 4 at Kimi-K2 shapes
+  const int rows_o = a.hidden / (int)gridDim.x, tiles = HEAD ? HD_O_TILES : rows_o >> 2;  // 28 rows, 7 tiles of 4 at Kimi-K2 shapes
   const int s0 = wave, s1 = wave + 8;
+  // the residual value this thread will add to (a load at that point would come back behind every weight request)
+  uint16_t x_old = 0;
+  uint4 hd_g[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};  // HEAD: post-attention RMSNorm weights of this lane's columns
+  if (tid < rows_o) x_old = a.x[(size_t)bid * rows_o + tid];
+  __shared__ float s_logits[HEAD ? 512 : 1], s_bias[HEAD ? 512 : 1];  // the routing workgroup's: one thread per expert
+  __shared__ int s_cnt[HEAD ? BK_THREADS : 1], s_act[HEAD ? BK_THREADS : 1];
+  __shared__ uint4 s_ids4[4];
+  if (HEAD) {
+    hd_g[0] = *(const uint4 *)(a.hd.post_ln + s0 * 512 + lane * 8);
+    if (s1 * 512 < a.hidden) hd_g[1] = *(const uint4 *)(a.hd.post_ln + s1 * 512 + lane * 8);
+    float b = 0.0f;  // the router bias, for the workgroup that routes: in LDS long before it is needed
+    if (bid == (int)gridDim.x - 1 && tid < a.hd.experts) b = a.hd.bias[tid];
+    s_bias[tid] = b;
+  }
   // ---- requests, in the order of need: the head's partials, this wave's W_UV rows
   const size_t my = (size_t)min(lane, a.spans - 1) * a.heads + h;
   const float mj = a.pm[my], zj = a.pz[my];
@@ -565,26 +591,188 @@ __global__ void __launch_bounds__(BK_THREADS) attn_back_k(BackArgs a) {
       }
     }
   };
-  for (int t0 = 0; t0 < tiles; t0 += BK_PRE) {
+  // HEAD: row r of the workgroup's head tiles -> the weight row it stands for (nullptr: none).  Tile 0 comes first in
+  // every sense: two router rows (the first experts / 2 workgroups), or a gate and an up row of the eight shared rows
+  // that the last workgroup, which routes instead, leaves to the eight workgroups behind the router's; then the
+  // workgroup's eight gate rows and eight up rows.
+  const int E = a.hd.experts, last = (int)gridDim.x - 1;
+  const int extra = HEAD && bid >= (E >> 1) && bid < (E >> 1) + 8 ? 8 * last + bid - (E >> 1) : -1;  // shared row taken over
+  auto head_row = [&](int r) -> const uint16_t * {
+    if (bid == last) return nullptr;
+    if (r < 2) return 2 * bid < E ? a.hd.w_router + (size_t)(2 * bid + r) * a.hidden : nullptr;
+    if (r < 4) return extra >= 0 ? (r == 2 ? a.hd.w_gate : a.hd.w_up) + (size_t)extra * a.hidden : nullptr;
+    if (r < 12) return a.hd.w_gate + (size_t)(8 * bid + r - 4) * a.hidden;
+    return a.hd.w_up + (size_t)(8 * bid + r - 12) * a.hidden;
+  };
+  auto load_head_tile = [&](uint4 (&buf)[4][2], int j) {
 #pragma unroll
-    for (int u = 0; u < BK_PRE; ++u) {
-      const int t = t0 + u;
-      if (t < tiles) {
-        compute_tile(wo[u], t);
-        if (t + BK_PRE < tiles) load_tile(wo[u], t + BK_PRE);
+    for (int i = 0; i < 4; ++i) {
+      const uint16_t *row = head_row(4 * j + i);
+      buf[i][0] = buf[i][1] = make_uint4(0, 0, 0, 0);
+      if (row) {
+        buf[i][0] = ld_stream16(row + s0 * 512 + lane * 8);
+        if (s1 * 512 < a.hidden) buf[i][1] = ld_stream16(row + s1 * 512 + lane * 8);
+      }
+    }
+  };
+  if constexpr (HEAD) {
+#pragma unroll
+    for (int t = 0; t < HD_O_TILES; ++t) {
+      compute_tile(wo[t % BK_PRE], t);
+      if (t + BK_PRE < HD_O_TILES) load_tile(wo[t % BK_PRE], t + BK_PRE);
+      else load_head_tile(wo[t % BK_PRE], t + BK_PRE - HD_O_TILES);  // head tile j lies in wo[(HD_O_TILES + j) % BK_PRE]
+    }
+  } else {
+    for (int t0 = 0; t0 < tiles; t0 += BK_PRE) {
+#pragma unroll
+      for (int u = 0; u < BK_PRE; ++u) {
+        const int t = t0 + u;
+        if (t < tiles) {
+          compute_tile(wo[u], t);
+          if (t + BK_PRE < tiles) load_tile(wo[u], t + BK_PRE);
+        }
       }
     }
   }
   kx_lds_barrier();
   // ---- slices left to right, then x = bf(x + bf(y))  (add_k, :248-251)
+  uint32_t *hand_x = a.hand + (size_t)a.heads * a.v_head;
   if (tid < rows_o) {
     const float *p = s_part + tid * 16;
     float y = p[0];
 #pragma unroll
     for (int s = 1; s < 16; ++s) y += p[s];
-    uint16_t *xr = a.x + (size_t)bid * rows_o + tid;
-    *xr = kx_bf16_rne(kx_bf16_f32(*xr) + kx_bfround(y));
+    const uint16_t x_new = kx_bf16_rne(kx_bf16_f32(x_old) + kx_bfround(y));
+    a.x[(size_t)bid * rows_o + tid] = x_new;
+    if (HEAD) hand_store(hand_x + (size_t)bid * rows_o + tid, a.tag, x_new);
   }
+  if constexpr (!HEAD) return;
+  // ================================================================ the head of the MoE layer
+  const int H = a.hidden, S = H >> 9;
+  uint16_t *s_xrow = s_att;  // the residual row; the attention output is spent
+  __shared__ float s_ws[4];
+  __shared__ float s_scale;
+  uint32_t *hand_lg = hand_x + H;
+  if (bid == last) {
+    // ---- the last workgroup routes: logits from the tagged words into LDS (the bias lies there since the start),
+    // then kx_route.h
+    if (tid < (E >> 1)) {  // two logits = four words
+      uint32_t o[2];
+      hand_load<4>(hand_lg + tid * 4, a.tag, a.err, o);
+      s_logits[2 * tid] = __builtin_bit_cast(float, o[0]);
+      s_logits[2 * tid + 1] = __builtin_bit_cast(float, o[1]);
+    }
+    __syncthreads();
+    kxr::route_block_any<false>(s_logits, s_bias, a.hd.ids, a.hd.weights, 1, E, a.hd.topk, a.hd.routed_scale, a.hd.counts, a.hd.offsets,
+                                a.hd.pairs, a.hd.work, a.hd.n_active, s_ids4, s_cnt, s_act, nullptr);
+    return;
+  }
+  {  // the residual row from every workgroup: H / 4 requests of 16 bytes, request i of thread t is number 512 i + t
+    const uint32_t *src = hand_x + (size_t)tid * 4;
+    const int nreq = H >> 2;
+    hand4 v[4] = {{0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}, {0, 0, 0, 0}};
+    int polls = 0;
+    while (true) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (i * 512 + tid < nreq) hand_request4(src + (size_t)i * 2048, v[i]);
+      asm volatile("s_waitcnt vmcnt(0)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3])::"memory");
+      bool ok = true;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) ok = ok && (i * 512 + tid >= nreq || hand_tagged(v[i], a.tag));
+      if (ok || hand_give_up(polls, a.err)) break;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (i * 512 + tid < nreq) ((uint2 *)s_xrow)[i * 512 + tid] = hand_pack(v[i]);
+  }
+  __syncthreads();  // every request of this kernel has landed by now
+  {  // the row's RMSNorm scale: gemv_body's prologue (the first 256 threads own the 8-element chunks t, t + 256, ...)
+    const int chunks = H >> 3;
+    float v = 0.0f;
+    if (tid < 256)
+      for (int c = tid; c < chunks; c += 256) {
+        float f[8];
+        unpack8(f, ((const uint4 *)s_xrow)[c]);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v = __builtin_fmaf(f[e], f[e], v);
+      }
+    float vv[1] = {v};
+    kxw::reduce<1, 64>(vv, lane);
+    if (lane == 0 && wave < 4) s_ws[wave] = vv[0];
+    __syncthreads();
+    if (tid == 0) s_scale = kx_rsqrtf((((s_ws[0] + s_ws[1]) + s_ws[2]) + s_ws[3]) / (float)H + a.hd.eps);
+    __syncthreads();
+  }
+  const float sc = s_scale;
+  auto normed8 = [&](float (&o)[8], uint4 raw, uint4 g8) {
+    float g[8];
+    unpack8(o, raw);
+    unpack8(g, g8);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = kx_bfround(kx_bfround(o[e] * sc) * g[e]);
+  };
+  float xh[2][8];
+  normed8(xh[0], *(const uint4 *)(s_xrow + s0 * 512 + lane * 8), hd_g[0]);
+  normed8(xh[1], *(const uint4 *)(s_xrow + min(s1, S - 1) * 512 + lane * 8), hd_g[1]);
+  auto head_tile = [&](const uint4 (&buf)[4][2], int j) {
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        float wf[8];
+        unpack8(wf, buf[i][k]);
+        float acc = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc = __builtin_fmaf(wf[e], xh[k][e], acc);
+        v[i * 2 + k] = acc;
+      }
+    kxw::reduce<8, 64>(v, lane);
+    if (kxw::reduce_writer<8, 64>(lane)) {
+#pragma unroll
+      for (int q = 0; q < kxw::reduce_out<8, 64>(); ++q) {
+        const int idx = kxw::reduce_index<8, 64>(lane, q);
+        if (!(idx & 1) || s1 < S) s_part[(j * 4 + (idx >> 1)) * 16 + ((idx & 1) ? s1 : s0)] = v[q];
+      }
+    }
+  };
+  auto slice_sum = [&](int r) {
+    const float *p = s_part + r * 16;
+    float y = p[0];
+    for (int q = 1; q < S; ++q) y += p[q];
+    return y;
+  };
+  // ---- tile 0 first and on its own: the router's logits are what the last workgroup waits for
+  const bool tile0 = 2 * bid < E || extra >= 0;
+  if (tile0) {
+    head_tile(wo[HD_O_TILES % BK_PRE], 0);
+    __syncthreads();
+    if (tid < 2 && 2 * bid < E) {  // a router logit: fp32 (KX_EPI_F32), handed over as two tagged halves
+      const int e = 2 * bid + tid;
+      const float y = slice_sum(tid);
+      const uint32_t u = __builtin_bit_cast(uint32_t, y);
+      hand_store(hand_lg + 2 * e, a.tag, (uint16_t)(u & 0xffffu));
+      hand_store(hand_lg + 2 * e + 1, a.tag, (uint16_t)(u >> 16));
+      a.hd.logits[e] = y;
+    }
+  }
+  // the normed row for the routed experts' launch: 8 chunks of 8 values by each of the first workgroups
+  if (tid >= 64 && tid < 72 && 8 * bid + tid - 64 < (H >> 3)) {
+    const int c = 8 * bid + tid - 64;
+    float f[8];
+    normed8(f, ((const uint4 *)s_xrow)[c], ((const uint4 *)a.hd.post_ln)[c]);
+    uint32_t o[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = (uint32_t)kx_bf16_rne(f[2 * e]) | ((uint32_t)kx_bf16_rne(f[2 * e + 1]) << 16);
+    ((uint4 *)a.hd.n_out)[c] = make_uint4(o[0], o[1], o[2], o[3]);
+  }
+#pragma unroll
+  for (int j = 1; j < HD_TILES; ++j) head_tile(wo[(HD_O_TILES + j) % BK_PRE], j);
+  __syncthreads();
+  // KX_EPI_SWIGLU: rows 4 + t (gate) and 12 + t (up) of the tiles; the row taken over from the last workgroup: 2 and 3
+  if (tid < 8) a.hd.smid[8 * bid + tid] = kx_bf16_rne(kx_swiglu(kx_bfround(slice_sum(4 + tid)), kx_bfround(slice_sum(12 + tid))));
+  if (tid == 8 && extra >= 0) a.hd.smid[extra] = kx_bf16_rne(kx_swiglu(kx_bfround(slice_sum(2)), kx_bfround(slice_sum(3))));
 }
 
 }  // namespace
@@ -633,9 +821,13 @@ int kx_attn_front_launch(const KxGemvArgs &g_qkv, const KxGemvArgs &g_qb, const 
 
 // The W_UV GEMV that merges the attention partials (g_uv: mla_* set, row_block = v_head) and the o_proj GEMV with the
 // residual add (g_o: w0 = [hidden, heads * v_head], out = the residual row) of one token as one launch.  hand:
-// heads * v_head words; tag and err as for kx_attn_front_launch.  The W_UV output row (g_uv.out) is not written.
-int kx_attn_back_launch(const KxGemvArgs &g_uv, const KxGemvArgs &g_o, uint32_t *hand, uint32_t tag, int *err, bool *done, hipStream_t st) {
+// kx_back_hand_words words; tag and err as for kx_attn_front_launch.  The W_UV output row (g_uv.out) is not written.
+// head: the head of the MoE layer that follows (post-attention norm, shared gate/up, router, routing), taken along
+// when its shapes fit the launch's workgroups; *head_done says so.
+int kx_attn_back_launch(const KxGemvArgs &g_uv, const KxGemvArgs &g_o, const KxMoeHeadArgs *head, uint32_t *hand, uint32_t tag, int *err,
+                        bool *done, bool *head_done, hipStream_t st) {
   *done = false;
+  *head_done = false;
   static int cus = 0;
   if (!cus) {
     int dev = 0;
@@ -652,8 +844,20 @@ int kx_attn_back_launch(const KxGemvArgs &g_uv, const KxGemvArgs &g_o, uint32_t 
   if (g_uv.w_block_stride != a.nope + a.v_head) return KX_OK;
   a.w_o = g_o.w0; a.x = (uint16_t *)g_o.out; a.hidden = g_o.rows; a.vd = g_o.cols;
   a.hand = hand; a.tag = tag; a.err = err;
-  hipLaunchKernelGGL(attn_back_k, dim3(G), dim3(BK_THREADS), 0, st, a);
+  // the head: 8 gate and 8 up rows and up to 2 router rows per workgroup, columns as 512-wide slices over 8 waves x 2,
+  // one thread per expert in the routing; the last workgroup routes, and the 8 workgroups behind the router's take
+  // a gate and an up row each for it
+  const bool with_head = head && g_o.rows / G == 4 * HD_O_TILES && head->shared_inter == 8 * G && g_o.rows % 512 == 0 && g_o.rows / 512 <= 16 &&
+                         g_o.rows <= 8192 && head->experts % 2 == 0 && head->experts / 2 + 8 < G && head->experts <= 512 &&
+                         head->topk >= 1 && head->topk <= 32 && head->topk <= head->experts && g_o.rows / 8 >= 1 && g_o.rows / 64 <= G;
+  if (with_head) {
+    a.hd = *head;
+    hipLaunchKernelGGL(attn_back_k<true>, dim3(G), dim3(BK_THREADS), 0, st, a);
+  } else {
+    hipLaunchKernelGGL(attn_back_k<false>, dim3(G), dim3(BK_THREADS), 0, st, a);
+  }
   KX_LAUNCH_CHECK();
   *done = true;
+  *head_done = with_head;
   return KX_OK;
 }

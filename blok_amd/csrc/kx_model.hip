@@ -209,7 +209,7 @@ int layout(const kx_config *c, Plan &p, kx_model *m) {
   auto *head_count = KX_AT(int *, (size_t)c->heads * 4);
   auto *front_err = KX_AT(int *, 4);
   auto *front_hand = KX_AT(uint32_t *, kx_front_hand_words(c->q_rank, (int)KVA, (int)KD) * 4);
-  auto *back_hand = KX_AT(uint32_t *, VD * 4);
+  auto *back_hand = KX_AT(uint32_t *, kx_back_hand_words((int)VD, c->hidden, c->experts) * 4);
   auto *head_work = KX_AT(int4 *, (size_t)c->heads * 16);
   auto *head_pairs = KX_AT(int *, BT * c->heads * 4);
 #undef KX_AT
@@ -317,6 +317,7 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample, int C = 1) {
                                   g.tokens, 1, g.rows, g.cols, 1, 0, 0, g.tokens, st);
   };
   for (int l = 0; l < c.n_layers; ++l) {
+    bool moe_head_done = false;  // the MoE layer's router + shared gate/up step rode in the attention block's last launch
     Layer &L = m->layers[l];
     KxGemvArgs g = {};
     g.w0 = L.qkv_a; g.x = m->n; g.x_stride = H; g.out = m->qkv; g.out_stride = QKV; g.rows = QKV; g.cols = H; g.tokens = B;
@@ -388,10 +389,14 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample, int C = 1) {
       go.w0 = L.o; go.x = m->att; go.x_stride = VD; go.out = m->x; go.out_stride = H; go.rows = H; go.cols = VD; go.tokens = B;
       // One token: the merge of the attention partials, W_UV and o_proj with the residual add as one resident launch
       // where the shapes and the device allow it (kx_front.hip; same sums, same bits)
+      // and, in front of a MoE layer, that layer's head too (post-attention norm, shared gate/up, router, routing)
       bool back = false;
       if (fuse && B == 1 && g.mla_po && (m->fusion & KX_FUSE_BACK)) {
         const uint32_t tag = m->back_tag % 65535u + 1u;
-        KX_TRY(kx_attn_back_launch(g, go, m->back_hand, tag, m->front_err, &back, st));
+        KxMoeHeadArgs hd;
+        const bool want_head = l >= c.first_dense && (m->fusion & KX_FUSE_MOE_HEAD);
+        if (want_head) kx_moe_head_args(&c, &L.moe, m->moe_ws, m->n, L.post_ln, &hd);
+        KX_TRY(kx_attn_back_launch(g, go, want_head ? &hd : nullptr, m->back_hand, tag, m->front_err, &back, &moe_head_done, st));
         if (back) m->back_tag = tag;
       }
       if (!back) {
@@ -421,7 +426,7 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample, int C = 1) {
         // streams them faster than the GEMM kernel does at one token.  With 32 sequences that decode alike (70-100
         // distinct experts for 256 pairs, up to 23 pairs on one expert) the step goes from 24.5 to 18.1 ms; at 12
         // sequences the two forms are level (12.1 against 12.4 ms), at 8 the GEMV kernels win (9.8 against 10.9 ms).
-        const uint32_t flags = ((m->fusion & KX_FUSE_MOE_TAIL) ? 0u : KX_MOE_SEPARATE_TAIL) | (B >= 5 && !(m->exact & KX_EXACT_SHARED) ? KX_MOE_SHARED_MATRIX_CORES : 0u) |
+        const uint32_t flags = ((m->fusion & KX_FUSE_MOE_TAIL) ? 0u : KX_MOE_SEPARATE_TAIL) | (moe_head_done ? KX_MOE_HEAD_DONE : 0u) | (B >= 5 && !(m->exact & KX_EXACT_SHARED) ? KX_MOE_SHARED_MATRIX_CORES : 0u) |
                                (B >= 12 && !(m->exact & KX_EXACT_ROUTED) ? KX_MOE_ROUTED_MATRIX_CORES : 0u);
         KX_TRY(kx_moe_layer_launch(&c, &L.moe, m->moe_ws, m->n, m->x, B, flags, fuse ? L.post_ln : nullptr, st, false));  // :835-877
       }
@@ -500,7 +505,7 @@ static int model_new(const kx_config *cfg, const char *who, kx_model **out) {
   if (!rc && cfg->first_dense < cfg->n_layers) rc = kx_moe_workspace_create(cfg, step_tokens(cfg), &m->moe_ws);
   if (!rc && (hipMemsetAsync(m->head_count, 0, (size_t)cfg->heads * 4, m->st) != hipSuccess ||
               hipMemsetAsync(m->front_err, 0, 4, m->st) != hipSuccess ||
-              hipMemsetAsync(m->back_hand, 0, (size_t)cfg->heads * cfg->v_head * 4, m->st) != hipSuccess ||
+              hipMemsetAsync(m->back_hand, 0, kx_back_hand_words(cfg->heads * cfg->v_head, cfg->hidden, cfg->experts) * 4, m->st) != hipSuccess ||
               hipMemsetAsync(m->front_hand, 0, kx_front_hand_words(cfg->q_rank, cfg->kv_rank + cfg->qk_rope, cfg->heads * (cfg->qk_nope + cfg->qk_rope)) * 4, m->st) != hipSuccess || hipStreamSynchronize(m->st) != hipSuccess))
     rc = KX_ERR_HIP;
   if (rc) {

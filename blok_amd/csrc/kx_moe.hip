@@ -19,6 +19,7 @@
 // with one pair, experts with more).
 #include "kx_common.h"
 #include "kx_dense.h"
+#include "kx_front.h"
 
 constexpr int KX_TAIL_BLOCKS = 1024;
 
@@ -118,6 +119,17 @@ extern "C" int kx_moe_workspace_destroy(kx_moe_workspace *ws) {
 }
 
 int *kx_moe_workspace_n_active(kx_moe_workspace *ws) { return ws->n_active; }
+
+void kx_moe_head_args(const kx_config *c, const kx_moe_weights *w, kx_moe_workspace *ws, void *d_n, const uint16_t *norm_w, KxMoeHeadArgs *out) {
+  KxMoeHeadArgs h = {};
+  h.post_ln = norm_w;
+  h.w_gate = (const uint16_t *)w->d_shared_gate; h.w_up = (const uint16_t *)w->d_shared_up; h.w_router = (const uint16_t *)w->d_router_gate;
+  h.bias = (const float *)w->d_router_bias;
+  h.n_out = (uint16_t *)d_n; h.smid = ws->smid; h.logits = ws->logits; h.ids = ws->ids; h.weights = ws->weights;
+  h.counts = ws->counts; h.offsets = ws->offsets; h.pairs = ws->pairs; h.work = ws->work; h.n_active = ws->n_active;
+  h.shared_inter = c->shared_inter; h.experts = c->experts; h.topk = c->topk; h.routed_scale = c->routed_scale; h.eps = c->rms_eps;
+  *out = h;
+}
 
 extern "C" int kx_moe_workspace_views(kx_moe_workspace *ws, void **d_logits, void **d_ids, void **d_weights,
                                       void **d_counts, void **d_offsets, void **d_pairs, void **d_mid,
@@ -234,8 +246,8 @@ int kx_moe_layer_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_work
         (rc = kx_skinny_gemm_launch(false, (const uint16_t *)w->d_shared_down, nullptr, ws->smid, c->shared_inter, ws->sy, H, KX_GG_BF16,
                                     tokens, H, c->shared_inter, &shared_down_done, ws->side))) return rc;
   }
-  bool paired = false;
-  if ((rc = kx_gemv_pair_route_launch(s, g, (const float *)w->d_router_bias, ws->ids, ws->weights, E, K, c->routed_scale,
+  bool paired = (flags & KX_MOE_HEAD_DONE) && tokens == 1 && norm_w && !mm;  // the caller's launch has done this step
+  if (!paired && (rc = kx_gemv_pair_route_launch(s, g, (const float *)w->d_router_bias, ws->ids, ws->weights, E, K, c->routed_scale,
                                       ws->counts, ws->offsets, ws->pairs, ws->work, ws->n_active, ws->route_counter, &paired,
                                       st, routed_per_pair(tokens, K, E) ? ws->pair_work : nullptr))) return rc;
   if (!paired) {

@@ -331,10 +331,13 @@ int kx_model_steps_decoded(kx_model *model, int32_t *steps);
 #define KX_FUSE_ABSORB 1u   /* W_UK absorb, RoPE of q, kv_a norm + cache row: inside the q_b GEMV */
 #define KX_FUSE_MOE_TAIL 2u /* one token: shared down GEMV + combine + residual inside the routed down launch */
 #define KX_FUSE_FRONT 4u    /* one token, Kimi-K2 shapes, a device with at least 4 * heads CUs: q_a | kv_a, q_b, the absorb, RoPE and
-                               the cache row as one resident launch with two grid barriers (takes precedence over KX_FUSE_ABSORB) */
+                               the cache row as one resident launch (takes precedence over KX_FUSE_ABSORB) */
 #define KX_FUSE_BACK 8u     /* one token, same conditions, up to 32 attention spans: the merge of the attention partials, W_UV and
                                o_proj with the residual add as one resident launch */
-#define KX_FUSE_ALL 15u
+#define KX_FUSE_MOE_HEAD 16u /* with KX_FUSE_BACK, in front of a MoE layer (shared_inter = 32 * heads, an even number of at most 510
+                               experts): the post-attention norm, the router, the routing and the shared expert's gate/up ride in
+                               that launch */
+#define KX_FUSE_ALL 31u
 int kx_model_set_fusion(kx_model *model, uint32_t mask);
 /* The attention kernel this model's steps use: KX_MLA_AUTO (default), KX_MLA_VALU or KX_MLA_MATRIX_CORES, as for
  * kx_mla_decode.  A property of the model: other models of the process keep theirs.                          */

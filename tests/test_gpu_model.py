@@ -315,7 +315,8 @@ def test_kimi_shape_stack_batch_invariance(kxlib, ox):
 @pytest.mark.parametrize("shape", ["small-1", "small-3", "kimi"])
 def test_fused_and_separate_launches_agree(kxlib, ox, shape):
     # the q_b GEMV that finishes the query in its own launch, (batch 1) the routed down launch that finishes the MoE
-    # layer, and (batch 1, Kimi shapes) the resident launch that runs the whole front of the attention block, against
+    # layer, and (batch 1, Kimi shapes) the resident launches that run the whole front of the attention block and its
+    # back (bit 3; with bit 4 the head of the MoE layer behind it: norm, router, routing, shared gate/up), against
     # the same steps as kernels of their own: cache rows, hidden state, logits and ids to the bit (the oracle
     # comparisons above run the fused forms)
     say(f"fusion on/off {shape}")
@@ -329,7 +330,7 @@ def test_fused_and_separate_launches_agree(kxlib, ox, shape):
         prompt_len, n_tokens = 11, 9
     prompt = O.tokens_u32(batch * prompt_len, cfg.seed, 4, cfg.vocab).reshape(batch, prompt_len)
     got = []
-    for mask in (15, 0, 1, 2, 3, 4, 8):
+    for mask in (31, 0, 1, 2, 3, 4, 8, 15, 24):
         km = KxModel(kxlib, cfg)
         check(kxlib.kx_model_set_fusion(km.h, mask))
         rc, out, _ = km.generate(prompt, n_tokens)
@@ -340,7 +341,7 @@ def test_fused_and_separate_launches_agree(kxlib, ox, shape):
         km.close()
     assert kxlib.kx_model_set_fusion(None, 1) != 0
     km = KxModel(kxlib, cfg)
-    assert kxlib.kx_model_set_fusion(km.h, 16) != 0 and b"mask" in kxlib.kx_last_error()
+    assert kxlib.kx_model_set_fusion(km.h, 32) != 0 and b"mask" in kxlib.kx_last_error()
     km.close()
     o0, h0, l0, c0 = got[1]   # every launch on its own
     for (o1, h1, l1, c1) in got[:1] + got[2:]:
