@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 
 import oracle as O
-from kxt import check, dev, judge_sequences, routing_of, say
+from kxt import assert_excused, check, dev, judge_sequences, routing_of, say
 from oracle import ptr
 
 pytestmark = pytest.mark.gpu
@@ -49,6 +49,18 @@ class KxModel:
         if self.h:
             self.lib.kx_model_destroy(self.h)
             self.h = None
+
+
+
+# The sequences a tolerance path may differ on, for the fixed seeds of the tests below: (sequence, "router" or
+# "argmax", first MoE layer whose expert set differs).  Every entry was checked when it was recorded -- the reference
+# run's selection gap in that layer is below kxt.NEAR_TIE, or its two largest logits lie closer than the bar -- and
+# judge_sequences checks it again on every run.  A set that changes means the arithmetic of a kernel changed.
+EXCUSED_SMALL_STACK = {(16, 1): [], (16, 0): [], (8, 1): [], (8, 0): [], (5, 1): [], (5, 0): [],
+                       (40, 1): [("sequence 16", "argmax", None)], (40, 0): [("sequence 16", "argmax", None)]}
+EXCUSED_ATTENTION_PATHS = []
+EXCUSED_AGAINST_SINGLE = {16: [("sequence 0", "router", 1)],
+                          32: [("sequence 0", "router", 1), ("sequence 20", "router", 1), ("sequence 29", "argmax", None)]}
 
 
 def test_rope_table_matches_oracle(kxlib, ox):
@@ -138,7 +150,7 @@ def test_small_stack_matrix_core_projections(kxlib, ox, batch):
         errs = [O.max_rel(got[b], ref[b]) for b in range(batch)]
         excused = judge_sequences(names, errs, 3e-2, routes, ref_routes, out[:, 0], out_o[:, 0], ref)
         print(f"batch-{batch} stack vs oracle mode {mode}: worst logits max-rel {max(errs):.3e}; excused: {excused or 'none'}", flush=True)
-        assert len(excused) <= batch // 4
+        assert_excused(excused, EXCUSED_SMALL_STACK[batch, mode], f"small stack, batch {batch}, oracle mode {mode}")
         om.close()
 
 
@@ -561,7 +573,7 @@ def test_kimi_shape_batched_stack_attention_paths(kxlib, ox):
     excused = judge_sequences([f"sequence {b}" for b in range(batch)], errs, 3e-2, got[0][2], got[1][2], got[0][0][:, 0],
                               got[1][0][:, 0], got[1][1])
     print(f"batch-8 stack, matrix-core vs VALU attention: worst logits max-rel {max(errs):.3e}; excused: {excused or 'none'}", flush=True)
-    assert len(excused) <= 2
+    assert_excused(excused, EXCUSED_ATTENTION_PATHS, "Kimi-shape stack, batch 8, attention paths")
 
 
 @pytest.mark.parametrize("shape,batch,prompt_len,chunk", [
@@ -694,7 +706,7 @@ def test_kimi_shape_batched_stack_against_single_sequences(kxlib, ox, batch):
     excused = judge_sequences([f"sequence {b}" for b in range(batch)], errs, 3e-2, routes, ref_routes, out[:, 0], ref_ids,
                               np.stack(ref_logits))
     print(f"batch {batch}: logits max-rel per sequence: median {np.median(errs):.2e}, worst {max(errs):.2e}; excused: {excused or 'none'}", flush=True)
-    assert len(excused) <= batch // 4
+    assert_excused(excused, EXCUSED_AGAINST_SINGLE[batch], f"Kimi-shape stack, batch {batch} against the sequences alone")
 
 
 def test_config5_batch32_full_size_step_by_step_against_the_exact_path(kxlib, ox, capsys):
