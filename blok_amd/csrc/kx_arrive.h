@@ -81,5 +81,15 @@ KX_ARRIVE_FN bool kx_arrive_is_last(int *counter, int target) {
   if (last && KX_ARRIVE_ORDER != __ATOMIC_RELAXED) (void)KX_ARRIVE_LOAD_ACQUIRE(counter);
   return last;
 }
+// The data accesses of the hand-over: every value one group writes for the finisher goes through kx_arrive_store,
+// every read of such a value by the finisher through kx_arrive_load (relaxed, agent scope: written through to / read
+// from the device's point of coherence).  A plain store or load on these paths would break the argument above
+// silently, so the accesses carry a name that can be searched for.
+#if defined(__HIPCC__)
+template <class T>
+__device__ __forceinline__ void kx_arrive_store(T *p, T v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+template <class T>
+__device__ __forceinline__ T kx_arrive_load(const T *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+#endif
 // By the finishing group, once it is done: the counter is zero again for the next launch.
 KX_ARRIVE_FN void kx_arrive_reset(int *counter) { __atomic_store_n(counter, 0, __ATOMIC_RELAXED); }

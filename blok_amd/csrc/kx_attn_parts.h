@@ -107,7 +107,7 @@ __device__ __forceinline__ void absorb_head_block(const QAbsArgs &a, int h, int 
     const uint32_t *qh = (const uint32_t *)(a.q + ((size_t)t * a.heads + h) * qk);
     float *out = a.qabs + ((size_t)t * a.heads + h) * kva;
     for (int i = threadIdx.x; i < (qk >> 1); i += blockDim.x) {
-      const uint32_t u = __hip_atomic_load(qh + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const uint32_t u = kx_arrive_load(qh + i);
       qs[2 * i] = kxg::bf_lo(u);
       qs[2 * i + 1] = kxg::bf_hi(u);
     }

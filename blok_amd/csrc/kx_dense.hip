@@ -496,6 +496,13 @@ extern "C" int kx_lm_head_argmax_static(const void *d_w, const void *d_n, void *
   KX_REQUIRE(tokens <= KX_STATIC_ARGMAX_TOKENS,
              "kx_lm_head_argmax_static: tokens=%d is more than the %d rows the built-in scratch holds; use kx_lm_head_argmax with a buffer of your own",
              tokens, KX_STATIC_ARGMAX_TOKENS);
+  // the array is the current device's: pointers that live on another device would be handed this device's array
+  int dev = -1;
+  hipPointerAttribute_t attr;
+  KX_HIP(hipGetDevice(&dev));
+  KX_HIP(hipPointerGetAttributes(&attr, d_logits));
+  KX_REQUIRE(attr.device == dev, "kx_lm_head_argmax_static: d_logits lives on device %d, the current device is %d: make the buffers' device current",
+             attr.device, dev);
   void *scratch = nullptr;
   int rc = argmax_scratch_for_current_device(&scratch);
   if (rc) return rc;

@@ -2,6 +2,7 @@
 // Used by the GEMV kernels of kx_dense.hip: the plain one, the pair that runs the shared expert's gate/up and the
 // router in one launch, and the q_b GEMV that finishes the query (W_UK absorb, RoPE) in the same launch.
 #pragma once
+#include "kx_arrive.h"
 #include "kx_common.h"
 #include "kx_dense.h"
 #include "kx_math.h"
@@ -263,13 +264,13 @@ __device__ __forceinline__ void gemv_body(const KxGemvArgs &a, const int bid, co
       switch (a.epi) {
         case KX_EPI_BF16:
           if (a.flags & KX_GEMV_COHERENT_OUT)
-            __hip_atomic_store((uint16_t *)a.out + (size_t)tok * a.out_stride + row, kx_bf16_rne(y0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            kx_arrive_store((uint16_t *)a.out + (size_t)tok * a.out_stride + row, kx_bf16_rne(y0));
           else
             ((uint16_t *)a.out)[(size_t)tok * a.out_stride + row] = kx_bf16_rne(y0);
           break;
         case KX_EPI_F32:
           if (a.flags & KX_GEMV_COHERENT_OUT)  // read back by another workgroup of this launch: store through to memory
-            __hip_atomic_store((float *)a.out + (size_t)tok * a.out_stride + row, y0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            kx_arrive_store((float *)a.out + (size_t)tok * a.out_stride + row, y0);
           else
             ((float *)a.out)[(size_t)tok * a.out_stride + row] = y0;
           break;

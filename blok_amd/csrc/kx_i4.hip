@@ -185,18 +185,18 @@ __device__ __forceinline__ void moe_tail_arrive(const KxMoeTail &t, int blk_a, i
       const int rc = idx % block_rows, tok = idx / block_rows, row = r0 + rc;
       const uint16_t *y = eout + (size_t)tok * t.topk * rows + row;
       const float *w = t.route_w + (size_t)tok * t.topk;
-      const uint16_t sh = __hip_atomic_load(t.sy + (size_t)tok * rows + row, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const uint16_t sh = kx_arrive_load(t.sy + (size_t)tok * rows + row);
       float acc = 0.0f;
       int k = 0;
       for (; k + 8 <= t.topk; k += 8) {  // the loads of eight slots go out together; the sum stays in slot order
         uint16_t v[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] = __hip_atomic_load(y + (size_t)(k + j) * rows, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int j = 0; j < 8; ++j) v[j] = kx_arrive_load(y + (size_t)(k + j) * rows);
 #pragma unroll
         for (int j = 0; j < 8; ++j) acc = __builtin_fmaf(kx_bf16_f32(v[j]), w[k + j], acc);
       }
       for (; k < t.topk; ++k)
-        acc = __builtin_fmaf(kx_bf16_f32(__hip_atomic_load(y + (size_t)k * rows, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)), w[k], acc);
+        acc = __builtin_fmaf(kx_bf16_f32(kx_arrive_load(y + (size_t)k * rows)), w[k], acc);
       const float down = kx_bfround(kx_bfround(acc) + kx_bf16_f32(sh));
       uint16_t *xr = t.x + (size_t)tok * t.x_stride + row;
       *xr = (t.flags & 1u) ? kx_bf16_rne(down) : kx_bf16_rne(kx_bf16_f32(*xr) + down);
@@ -401,7 +401,7 @@ __device__ __forceinline__ void i4_body(const I4Args &a, const int bid, const in
             res = kx_swiglu(kx_bfround(y0), kx_bfround(y1));
           }
           if (!DUAL && a.tail.counter)  // read back by another workgroup of this launch
-            __hip_atomic_store(a.out + (size_t)pair * a.rows + cur.c0 + rc, kx_bf16_rne(res), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            kx_arrive_store(a.out + (size_t)pair * a.rows + cur.c0 + rc, kx_bf16_rne(res));
           else
             a.out[(size_t)pair * a.rows + cur.c0 + rc] = kx_bf16_rne(res);
         }
@@ -493,7 +493,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))
     const float *p = lds + threadIdx.x * S;
     float y = p[0];
     for (int q = 1; q < S; ++q) y += p[q];
-    __hip_atomic_store((uint16_t *)g.out + bid * CR + threadIdx.x, kx_bf16_rne(y), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    kx_arrive_store((uint16_t *)g.out + bid * CR + threadIdx.x, kx_bf16_rne(y));
   }
   moe_tail_arrive(a.tail, routed_blk, bid * CR / BLOCK, BLOCK, a.rows, a.out);
 }

@@ -206,8 +206,21 @@ static int routed_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_wor
   return KX_OK;
 }
 
+static int moe_layer_body(const kx_config *c, const kx_moe_weights *w, kx_moe_workspace *ws, void *d_n, void *d_x,
+                          int tokens, uint32_t flags, const uint16_t *norm_w, hipStream_t st, bool timed, bool &forked);
+
+// An error after the layer has put work on its side stream must not leave that work unjoined: the caller's stream
+// waits for it here, so whatever the caller does next (free the buffers, run the layer again) comes after it.
 int kx_moe_layer_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_workspace *ws, void *d_n, void *d_x,
                         int tokens, uint32_t flags, const uint16_t *norm_w, hipStream_t st, bool timed) {
+  bool forked = false;
+  const int rc = moe_layer_body(c, w, ws, d_n, d_x, tokens, flags, norm_w, st, timed, forked);
+  if (rc && forked && hipEventRecord(ws->join, ws->side) == hipSuccess) (void)hipStreamWaitEvent(st, ws->join, 0);
+  return rc;
+}
+
+static int moe_layer_body(const kx_config *c, const kx_moe_weights *w, kx_moe_workspace *ws, void *d_n, void *d_x,
+                          int tokens, uint32_t flags, const uint16_t *norm_w, hipStream_t st, bool timed, bool &forked) {
   int rc = check_cfg(c);
   if (rc) return rc;
   KX_REQUIRE(w && ws && d_n && d_x, "kx_moe_decode_layer: null argument");
@@ -235,7 +248,7 @@ int kx_moe_layer_launch(const kx_config *c, const kx_moe_weights *w, kx_moe_work
   // and runs the routed experts, and are joined before the combine.
   const bool mm = (flags & KX_MOE_SHARED_MATRIX_CORES) && tokens >= 5 && tokens <= 32;
   const bool rmm = (flags & KX_MOE_ROUTED_MATRIX_CORES) && tokens >= 5;
-  bool shared_up_done = false, shared_down_done = false, forked = false;
+  bool shared_up_done = false, shared_down_done = false;
   if (mm && !norm_w) {
     KX_HIP(hipEventRecord(ws->fork, st));
     KX_HIP(hipStreamWaitEvent(ws->side, ws->fork, 0));

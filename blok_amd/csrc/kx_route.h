@@ -2,6 +2,7 @@
 // the token -> expert bucketing by one workgroup.  Shared by the stand-alone router
 // kernels and by the GEMV whose last workgroup routes the logits it has just produced.
 #pragma once
+#include "kx_arrive.h"
 #include "kx_common.h"
 #include "kx_math.h"
 #include "kx_wave.h"
@@ -24,7 +25,7 @@ __device__ __forceinline__ void topk_token(const float *lg, const float *__restr
 #pragma unroll
   for (int j = 0; j < EPL; ++j) {
     const int ec = min(lane + 64 * j, E - 1);
-    x[j] = COHERENT ? __hip_atomic_load(lg + ec, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : lg[ec];
+    x[j] = COHERENT ? kx_arrive_load(lg + ec) : lg[ec];
     bs[j] = bias[ec];
   }
 #pragma unroll

@@ -60,6 +60,11 @@ extern "C" int kx_dev_memset(void *d_ptr, int value, size_t bytes, void *stream)
   KX_HIP(hipMemsetAsync(d_ptr, value, bytes, kx_stream(stream)));
   return KX_OK;
 }
+extern "C" int kx_dev_mem_info(size_t *free_bytes, size_t *total_bytes) {
+  KX_REQUIRE(free_bytes && total_bytes, "kx_dev_mem_info: null pointer");
+  KX_HIP(hipMemGetInfo(free_bytes, total_bytes));
+  return KX_OK;
+}
 extern "C" int kx_h2d(void *d_dst, const void *h_src, size_t bytes) {
   KX_REQUIRE((d_dst && h_src) || !bytes, "kx_h2d: null pointer");
   KX_HIP(hipMemcpy(d_dst, h_src, bytes, hipMemcpyHostToDevice));

@@ -46,6 +46,7 @@ _SIGS = {
     "kx_dev_malloc": [_PP, _SZ],
     "kx_dev_free": [_P],
     "kx_dev_memset": [_P, C.c_int, _SZ, _P],
+    "kx_dev_mem_info": [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)],
     "kx_h2d": [_P, _P, _SZ],
     "kx_d2h": [_P, _P, _SZ],
     "kx_sync": [_P],

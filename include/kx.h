@@ -70,6 +70,8 @@ int kx_device_info(char *name, size_t name_len, int32_t *compute_units, uint64_t
 int kx_dev_malloc(void **d_ptr, size_t bytes);
 int kx_dev_free(void *d_ptr);
 int kx_dev_memset(void *d_ptr, int value, size_t bytes, void *stream);
+/* free and total device memory of the current device, in bytes (hipMemGetInfo) */
+int kx_dev_mem_info(size_t *free_bytes, size_t *total_bytes);
 int kx_h2d(void *d_dst, const void *h_src, size_t bytes);
 int kx_d2h(void *h_dst, const void *d_src, size_t bytes);
 int kx_sync(void *stream);
@@ -201,7 +203,9 @@ int kx_moe_prefill_layer(const kx_config *cfg, const kx_moe_weights *w, kx_moe_w
                          const void *d_n, void *d_x, int32_t tokens, uint32_t flags, void *stream);
 /* per-phase kernel time of the most recent kx_moe_decode_layer_timed call, ms:
  * [0] router+bucket [1] routed gate/up [2] routed down [3] shared gate/up
- * [4] shared down + combine.  Synchronises.                                 */
+ * [4] shared down + combine.  Synchronises.  The intervals are taken on `stream`: up to 4 tokens the
+ * shared gate/up rides in the router's launch ([0] holds it, [3] reads about 0); with bit9 or bit10
+ * the work the layer puts on its side stream lies outside [0]..[3] and is waited for inside [4].  */
 int kx_moe_decode_layer_timed(const kx_config *cfg, const kx_moe_weights *w, kx_moe_workspace *ws,
                               const void *d_n, void *d_x, int32_t tokens, uint32_t flags,
                               void *stream, float *ms5);

@@ -847,27 +847,38 @@ def test_model_form_of_the_handover_gives_the_same_bits(kxlib, ox):
     from blok_amd.lib import load_library
     say("hand-over protocol: shipped form against the memory-model form")
     strict = load_library(os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "blok_amd", "libkx_strict.so"))
-    cases = [("small", O.small_config(batch=3, context=64), 3, 11, 9)]
+    # (name, config, sequences, prompt, tokens, fusion masks): the small stack at 3 sequences; Kimi shapes at one
+    # sequence with the launches that use the protocol (mask 3: the q_b GEMV finishes the query, the routed down
+    # launch finishes the layer; mask 1: the layer's tail as launches of its own) and with the default (the resident
+    # launches, whose hand-over is another one, plus the routed down launch); Kimi shapes at 3 sequences (the router
+    # and shared gate/up pair launch whose last router workgroup routes, the q_b GEMV at several tokens)
+    cases = [("small", O.small_config(batch=3, context=64), 3, 11, 9, (31,))]
     kimi = default_config()
     kimi.n_layers, kimi.first_dense, kimi.max_batch, kimi.max_context, kimi.seed = 3, 1, 1, 48, 11
-    cases.append(("kimi", kimi, 1, 24, 8))
-    for name, cfg, batch, prompt_len, n_tokens in cases:
+    cases.append(("kimi", kimi, 1, 24, 8, (3, 1, 31)))
+    kimi3 = default_config()
+    kimi3.n_layers, kimi3.first_dense, kimi3.max_batch, kimi3.max_context, kimi3.seed = 2, 1, 3, 24, 12
+    cases.append(("kimi, 3 sequences", kimi3, 3, 9, 4, (31,)))
+    for name, cfg, batch, prompt_len, n_tokens, masks in cases:
         prompt = O.tokens_u32(batch * prompt_len, cfg.seed, 4, cfg.vocab).reshape(batch, prompt_len)
-        got = []
-        for lib in (kxlib, strict):
-            km = KxModel(lib, cfg)
-            rc, out, _ = km.generate(prompt, n_tokens)
-            assert rc == 0, lib.kx_last_error()
-            total = prompt_len + n_tokens - 1
-            h = np.empty((batch, cfg.hidden), dtype=np.uint16)
-            lg = np.empty((batch, cfg.vocab), dtype=np.float32)
-            assert lib.kx_model_hidden(km.h, ptr(h)) == 0 and lib.kx_model_logits(km.h, ptr(lg)) == 0
-            rows = np.empty((total, cfg.kv_rank + cfg.qk_rope), dtype=np.uint16)
-            assert lib.kx_model_latent(km.h, cfg.n_layers - 1, 0, 0, total, ptr(rows)) == 0
-            got.append((out.copy(), h, lg.view(np.uint32), rows))
-            km.close()
-        for a, b in zip(*got):
-            assert (a == b).all(), f"{name}: the two forms differ"
+        for mask in masks:
+            got = []
+            for lib in (kxlib, strict):
+                km = KxModel(lib, cfg)
+                assert lib.kx_model_set_fusion(km.h, mask) == 0
+                rc, out, _ = km.generate(prompt, n_tokens)
+                assert rc == 0, lib.kx_last_error()
+                total = prompt_len + n_tokens - 1
+                h = np.empty((batch, cfg.hidden), dtype=np.uint16)
+                lg = np.empty((batch, cfg.vocab), dtype=np.float32)
+                assert lib.kx_model_hidden(km.h, ptr(h)) == 0 and lib.kx_model_logits(km.h, ptr(lg)) == 0
+                rows = np.empty((batch, total, cfg.kv_rank + cfg.qk_rope), dtype=np.uint16)
+                for b in range(batch):
+                    assert lib.kx_model_latent(km.h, cfg.n_layers - 1, b, 0, total, ptr(rows[b])) == 0
+                got.append((out.copy(), h, lg.view(np.uint32), rows))
+                km.close()
+            for a, b in zip(*got):
+                assert (a == b).all(), f"{name}, fusion mask {mask}: the two forms differ"
 
 
 def test_executor_json_line(kxlib):

@@ -3,7 +3,10 @@
 The two share their kernels; what differs is where the argmax partials live (a device array inside the library
 instead of the caller's buffer).  Logits and ids must agree to the bit, on two calls in a row of which the
 second is smaller (fewer rows, a shorter vocabulary): the array then still holds the first call's partials.
+The second test checks the property the entry point is named for: device memory free before a call = free after it.
 """
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -40,6 +43,29 @@ def test_static_entry_point_matches_the_allocating_one(kxlib):
         assert (l0 == l1).all(), f"{np.count_nonzero(l0 != l1)} logits differ"
         assert (i0 == i1).all(), (i0, i1)
         assert (i0 < vocab).all()
+
+
+@pytest.mark.gpu
+def test_static_entry_point_takes_no_device_memory(kxlib):
+    check(kxlib.kx_static_scratch_init())
+    vocab, hidden, tokens = 3000, 512, 5
+    w = O.normal_bf16(vocab * hidden, 23, 1, 0.02).reshape(vocab, hidden)
+    x = O.normal_bf16(tokens * hidden, 23, 2, 1.0).reshape(tokens, hidden)
+    dw, dx, dl, di = dev(w), dev(x), DevBuf(tokens * vocab * 4), DevBuf(tokens * 4)
+
+    def free_now():
+        free, total = C.c_size_t(), C.c_size_t()
+        check(kxlib.kx_dev_mem_info(C.byref(free), C.byref(total)))
+        return free.value
+
+    check(kxlib.kx_lm_head_argmax_static(dw.ptr, dx.ptr, dl.ptr, di.ptr, vocab, hidden, tokens, None))   # code objects, streams: loaded
+    check(kxlib.kx_sync(None))
+    before = free_now()
+    for _ in range(3):
+        check(kxlib.kx_lm_head_argmax_static(dw.ptr, dx.ptr, dl.ptr, di.ptr, vocab, hidden, tokens, None))
+        assert free_now() == before, "a call of the entry point that allocates nothing changed the free device memory"
+    check(kxlib.kx_sync(None))
+    assert free_now() == before
 
 
 @pytest.mark.gpu
