@@ -75,6 +75,13 @@ struct KxMoeTail {
 int kx_i4_down_shared_launch(const uint32_t *packed, const uint16_t *scale, const uint16_t *x, uint16_t *out, const int4 *work,
                              const int *pairs, int rows, int cols, int x_div, size_t expert_words, size_t expert_scales,
                              int n_slots, KxGemvArgs shared, KxMoeTail tail, bool *fused, hipStream_t st);
+// The same with the routed gate/up + SwiGLU in front, as one resident launch whose workgroups hand the mid values to
+// each other as tagged words (kx_hand.h; hand: n_slots * inter words, tag in [1, 65535] and different from the last
+// launch's, err: the flag a wait that gives up sets).  *fused = false, nothing launched, when shapes or device do not fit.
+int kx_i4_routed_shared_launch(const uint32_t *gate_packed, const uint16_t *gate_scale, const uint32_t *up_packed, const uint16_t *up_scale,
+                               const uint32_t *down_packed, const uint16_t *down_scale, const uint16_t *x, uint16_t *mid, uint16_t *eout,
+                               const int4 *work, const int *pairs, int hidden, int inter, int topk, int n_slots, KxGemvArgs shared,
+                               KxMoeTail tail, uint32_t *hand, uint32_t tag, int *err, bool *fused, hipStream_t st);
 // the launch shape kx_gemv_launch would give a GEMV (fills a.nw, a.rs, a.nt, a.epi); returns rows per chunk or -1
 int kx_gemv_plan(int epi, KxGemvArgs &a, int *ri);
 // cnt_lo..cnt_hi: only the experts of the work list with that many pairs are processed (0, INT_MAX: all)
@@ -124,6 +131,10 @@ struct kx_moe_workspace;
 // internal (not among the public flags): the layer's first launch -- normed row in d_n, router logits, routing, shared
 // gate/up -- has been done by the caller's own launch (kx_front.hip's back launch with kx_moe_head_args): one token
 #define KX_MOE_HEAD_DONE 0x800u
+// internal: one token, the routed experts (gate/up, down, shared down, combine) as one resident launch where shapes
+// and device allow it; the workspace must have been given an error flag (kx_moe_workspace_set_err)
+#define KX_MOE_ROUTED_RESIDENT 0x1000u
+void kx_moe_workspace_set_err(kx_moe_workspace *ws, int *d_err);
 int *kx_moe_workspace_n_active(kx_moe_workspace *ws);  // device address of the count of distinct experts of the last call
 // the flags a caller of kx_moe_decode_layer may pass (include/kx.h documents them)
 #define KX_MOE_PUBLIC_FLAGS (1u | KX_MOE_SEPARATE_TAIL | KX_MOE_SHARED_MATRIX_CORES | KX_MOE_ROUTED_MATRIX_CORES)

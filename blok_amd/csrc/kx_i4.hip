@@ -27,6 +27,7 @@
 // All arithmetic is IEEE binary32 (fma, mul, add), so a scalar host program
 // that follows the same order reproduces the result bit for bit.
 #include "kx_arrive.h"
+#include "kx_hand.h"
 #include "kx_common.h"
 #include "kx_dense.h"
 #include "kx_gemv_body.h"
@@ -151,6 +152,9 @@ struct I4Args {
   size_t expert_words, expert_scales;
   int cnt_lo, cnt_hi;  // only experts with cnt_lo <= pairs <= cnt_hi are processed by this launch
   KxMoeTail tail;      // tail.counter != nullptr: single-matrix launches finish the MoE layer (see moe_tail_arrive)
+  uint32_t *hand;      // HAND: the gate/up outputs as tagged words [pair][rows] (kx_hand.h), written (1) or read as activations (2)
+  uint32_t tag;
+  int *err;
 };
 
 constexpr int I4_RI = 2;  // rows per half-wave per tile
@@ -219,7 +223,11 @@ __device__ __forceinline__ void moe_tail_arrive(const KxMoeTail &t, int blk_a, i
 // FILTER: the launch processes only the experts whose pair count lies in [cnt_lo, cnt_hi]
 // `idle` is called once, where the last chunk's loads have landed and nothing more will be requested: what it
 // requests arrives during the epilogue.
-template <bool DUAL, int TT, int KS_T, bool FILTER, int CM = 1, class Idle>
+// HAND (one token, one chunk per workgroup, inside a launch whose workgroups are all resident): 1 = every output is
+// also handed over as a tagged word, and the workgroup may have more waves than the chunk shape uses (they keep the
+// barriers); 2 = the activations are not read from a.x but collected from the tagged words of the pair's row, one
+// 16-byte request per thread (4 * blockDim.x = cols), through LDS.
+template <bool DUAL, int TT, int KS_T, bool FILTER, int CM = 1, int HAND = 0, class Idle>
 __device__ __forceinline__ void i4_body(const I4Args &a, const int bid, const int nblocks, float *lds, Idle &&idle) {
   constexpr int MATS = DUAL ? 2 : 1;
   constexpr int RI = I4_RI;
@@ -233,11 +241,13 @@ __device__ __forceinline__ void i4_body(const I4Args &a, const int bid, const in
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int l = lane & 31, h = lane >> 5;
   const int s = wave % ks, rset = wave / ks;
+  const bool active = HAND == 1 ? wave < ks * rs : true;
   const int groups = ks * 32, row_words = ks * 128;
   const int n16 = CR * groups / 8;                                // 16-byte pieces of one matrix's chunk scales
   const int sc_pieces = (MATS * n16 + 63) & ~63;                  // per buffer, whole 1 KB runs
   float *part = lds;                                              // [mats][CR][TT][ks]
   uint4 *sc_base = (uint4 *)(lds + ((MATS * CR * TT * ks + 3) & ~3));  // 2 x [mats][CR][groups] bf16
+  uint16_t *s_xh = (uint16_t *)(sc_base + 2 * sc_pieces);               // HAND == 2: the pair's activation row, cols bf16
   const int cpe = (a.rows + CR - 1) / CR;                         // chunks per expert
   const int n_chunks = (a.work ? a.n_slots : 1) * cpe;
   const int row_lane = rset * RI * 2 + h;                         // row of this lane in tile 0, i = 0
@@ -312,8 +322,21 @@ __device__ __forceinline__ void i4_body(const I4Args &a, const int bid, const in
   uint4 xraw[TT][4];
   int sb = 0;
   copy_scales(cur, sc_base);
-  load_tile(bufA, cur, 0);
-  load_xraw(xraw, cur, cur.p_begin);
+  if (active) load_tile(bufA, cur, 0);
+  if (HAND == 2) {
+    // behind the first tile's requests: a wave's loads return in order, so the answer comes when those have landed
+    const uint32_t *src = a.hand + (size_t)cur.first_pair * a.cols + threadIdx.x * 4;
+    kxh::hand4 v;
+    int polls = 0;
+    while (true) {
+      kxh::hand_request4(src, v);
+      kxh::hand_wait(v);
+      if (kxh::hand_tagged(v, a.tag) || kxh::hand_give_up(polls, a.err)) break;
+    }
+    ((uint2 *)s_xh)[threadIdx.x] = kxh::hand_pack(v);
+  } else if (active) {
+    load_xraw(xraw, cur, cur.p_begin);
+  }
   bool fresh = true;  // the scales of `cur` have not been made visible to the workgroup yet
 
   while (true) {
@@ -330,12 +353,19 @@ __device__ __forceinline__ void i4_body(const I4Args &a, const int bid, const in
 
     for (int pc = cur.p_begin; pc < cur.p_end; pc += TT) {
       XGroup xg[TT];
+      if (HAND != 2) {
 #pragma unroll
-      for (int t = 0; t < TT; ++t) prep_xgroup(xg[t], xraw[t]);
+        for (int t = 0; t < TT; ++t) prep_xgroup(xg[t], xraw[t]);
+      }
       if (fresh) {  // first chunk of the workgroup: wait for the scale copies of every wave
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
         fresh = false;
+      }
+      if (HAND == 2) {  // the row every thread has collected a piece of
+#pragma unroll
+        for (int q = 0; q < 4; ++q) xraw[0][q] = ((const uint4 *)s_xh)[(s * 32 + l) * 4 + q];
+        prep_xgroup(xg[0], xraw[0]);
       }
 
       auto compute_tile = [&](uint4 (&buf)[MATS][RI], int tile) {
@@ -362,17 +392,18 @@ __device__ __forceinline__ void i4_body(const I4Args &a, const int bid, const in
         }
       };
 
-      for (int tile = 0; tile < nt; tile += 2) {
-        if (tile + 1 < nt) load_tile(bufB, cur, tile + 1);
-        compute_tile(bufA, tile);
-        if (tile + 2 < nt) load_tile(bufA, cur, tile + 2);
-        if (tile + 1 < nt) compute_tile(bufB, tile + 1);
-      }
+      if (active)
+        for (int tile = 0; tile < nt; tile += 2) {
+          if (tile + 1 < nt) load_tile(bufB, cur, tile + 1);
+          compute_tile(bufA, tile);
+          if (tile + 2 < nt) load_tile(bufA, cur, tile + 2);
+          if (tile + 1 < nt) compute_tile(bufB, tile + 1);
+        }
       // every load of this wave has landed, the scale copies for the next chunk included; its first tile
       // and activations are requested now and arrive during the epilogue
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       const bool last_pass = pc + TT >= cur.p_end;
-      if (!last_pass || more) {  // a further pass over this chunk (an expert with more than TT pairs), or the next chunk
+      if (HAND == 0 && (!last_pass || more)) {  // a further pass over this chunk (an expert with more than TT pairs), or the next chunk
         const Work &t = last_pass ? nxt : cur;
         load_tile(bufA, t, 0);
         load_xraw(xraw, t, last_pass ? nxt.p_begin : pc + TT);
@@ -404,11 +435,12 @@ __device__ __forceinline__ void i4_body(const I4Args &a, const int bid, const in
             kx_arrive_store(a.out + (size_t)pair * a.rows + cur.c0 + rc, kx_bf16_rne(res));
           else
             a.out[(size_t)pair * a.rows + cur.c0 + rc] = kx_bf16_rne(res);
+          if (HAND == 1) kxh::hand_store(a.hand + (size_t)pair * a.rows + cur.c0 + rc, a.tag, kx_bf16_rne(res));
         }
       }
       __syncthreads();  // `part` is free again; the next chunk's scale copies are visible to every wave
     }
-    if (!more) break;
+    if (!more || HAND != 0) break;
     cur = nxt;
     chunk = nchunk;
     sb ^= 1;
@@ -428,9 +460,8 @@ __global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(WPE, 
 // Both chunks finish through moe_tail_arrive: the launch leaves the layer's output in x.
 // The shared chunk is computed as kx_gemv_launch computes it for this shape (4 slice waves x 2 row sets, 4 rows per
 // wave and tile, 2 tiles): lane partials over 8 columns, butterfly over the wave, slices summed left to right.
-__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) i4_down_shared_k(I4Args a, KxGemvArgs g, int n_i4,
-                                                                                                 int n_g) {
-  extern __shared__ float lds[];
+template <int HAND>
+__device__ __forceinline__ void down_shared_body(const I4Args &a, const KxGemvArgs &g, int n_i4, int n_g, float *lds) {
   constexpr int S = 4, RI = 4, RT = 8, CR = 16;  // two tiles of RT rows per chunk
   const int bid = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -454,7 +485,7 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))
   constexpr int BLOCK = i4_chunk_rows(false, 16);
   int routed_blk = -1;
   if (bid < n_i4) {
-    i4_body<false, 1, 2, false>(a, bid, n_i4, lds, load_shared);
+    i4_body<false, 1, 2, false, 1, HAND>(a, bid, n_i4, lds, load_shared);
     if (a.work[bid / (a.rows / BLOCK)].x >= 0) routed_blk = bid % (a.rows / BLOCK);
   }
   load_shared();  // a workgroup without routed work
@@ -496,6 +527,26 @@ __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))
     kx_arrive_store((uint16_t *)g.out + bid * CR + threadIdx.x, kx_bf16_rne(y));
   }
   moe_tail_arrive(a.tail, routed_blk, bid * CR / BLOCK, BLOCK, a.rows, a.out);
+}
+
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) i4_down_shared_k(I4Args a, KxGemvArgs g, int n_i4,
+                                                                                                 int n_g) {
+  extern __shared__ float lds[];
+  down_shared_body<0>(a, g, n_i4, n_g, lds);
+}
+
+// The routed experts of one token as one launch: workgroup b computes chunk b of gate/up (32 rows of both matrices
+// of one expert, SwiGLU) with seven of its eight waves, hands the 32 values over as tagged words, and goes on as
+// workgroup b of the launch above with the activations of its down chunk -- the expert's 2048 mid values, from the 64
+// workgroups of the same expert -- collected from those words.  As launches of their own the second one cannot ask
+// for a byte before the first has drained; here a workgroup requests its down chunk's scales and first tile, then
+// polls.  Every workgroup must be resident (two per CU): the launcher checks CUs, LDS and the grid.
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4))) i4_routed_shared_k(I4Args gu, I4Args a, KxGemvArgs g,
+                                                                                                   int n_i4, int n_g) {
+  extern __shared__ float lds[];
+  i4_body<true, 1, 7, false, 1, 1>(gu, blockIdx.x, gridDim.x, lds, [] {});
+  __syncthreads();  // a workgroup without a gate/up chunk returns from the body early; the LDS changes hands here
+  down_shared_body<2>(a, g, n_i4, n_g, lds);
 }
 
 struct I4Launch {
@@ -561,7 +612,7 @@ int kx_i4_launch(bool dual, const uint32_t *packed0, const uint16_t *scale0, con
   if (dual2) cm = 2;
   int rc = plan(cols, rows, dual ? 2 : 1, tt, pl, cm, dual2);
   if (rc) return rc;
-  I4Args a;
+  I4Args a = {};
   a.packed0 = packed0; a.scale0 = scale0; a.packed1 = packed1; a.scale1 = scale1;
   a.x = x; a.out = out; a.work = work; a.pairs = pairs; a.n_pairs = n_pairs; a.n_slots = n_slots;
   a.rows = rows; a.cols = cols; a.x_div = x_div; a.ks = pl.ks; a.rs = pl.rs; a.nt = pl.nt;
@@ -617,7 +668,7 @@ int kx_i4_down_shared_launch(const uint32_t *packed, const uint16_t *scale, cons
   if (n_i4 > 32768 || n_g > 32768) return KX_OK;
   const size_t lds_g = (size_t)g_cr * 4 * sizeof(float);
   const size_t lds = pl.lds > lds_g ? pl.lds : lds_g;
-  I4Args a;
+  I4Args a = {};
   a.packed0 = packed; a.scale0 = scale; a.packed1 = nullptr; a.scale1 = nullptr;
   a.x = x; a.out = out; a.work = work; a.pairs = pairs; a.n_pairs = 0; a.n_slots = n_slots;
   a.rows = rows; a.cols = cols; a.x_div = x_div; a.ks = pl.ks; a.rs = pl.rs; a.nt = pl.nt;
@@ -625,6 +676,72 @@ int kx_i4_down_shared_launch(const uint32_t *packed, const uint16_t *scale, cons
   a.cnt_lo = 0; a.cnt_hi = 0x7fffffff;
   a.tail = tail;
   hipLaunchKernelGGL(i4_down_shared_k, dim3((unsigned)(n_i4 > n_g ? n_i4 : n_g)), dim3(512), lds, st, a, shared, (int)n_i4, (int)n_g);
+  KX_LAUNCH_CHECK();
+  *fused = true;
+  return KX_OK;
+}
+
+// The routed experts of one token -- gate/up + SwiGLU, down, the shared expert's down GEMV, combine, residual -- as one
+// launch (i4_routed_shared_k).  x: the normed row [hidden]; mid: [n_slots, inter] (also written, as the separate
+// launches leave it); hand: n_slots * inter words; tag in [1, 65535], different from the previous launch's on `hand`;
+// err: the flag a workgroup sets when it gives a wait up.  *fused = false and nothing launched when the shapes or the
+// device do not allow the resident form.
+int kx_i4_routed_shared_launch(const uint32_t *gate_packed, const uint16_t *gate_scale, const uint32_t *up_packed, const uint16_t *up_scale,
+                               const uint32_t *down_packed, const uint16_t *down_scale, const uint16_t *x, uint16_t *mid, uint16_t *eout,
+                               const int4 *work, const int *pairs, int hidden, int inter, int topk, int n_slots, KxGemvArgs shared,
+                               KxMoeTail tail, uint32_t *hand, uint32_t tag, int *err, bool *fused, hipStream_t st) {
+  *fused = false;
+  if (tail.tokens != 1 || shared.tokens != 1 || !tail.counter || !work || shared.rows != hidden || !hand || !err || tag < 1 || tag > 65535)
+    return KX_OK;
+  static int cus = 0;
+  if (!cus) {
+    int dev = 0;
+    KX_HIP(hipGetDevice(&dev));
+    KX_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+  }
+  I4Launch pu, pd;
+  int rc = plan(hidden, inter, 2, 1, pu);
+  if (rc) return rc;
+  if ((rc = plan(inter, hidden, 1, 1, pd))) return rc;
+  // gate/up: 7 slice waves, chunks of 32 rows; down: 2 slices x 4 row sets, chunks of 112 rows, 4 * 512 columns
+  if (!(pu.ks == 7 && pu.rs == 1 && pu.cr == 32 && inter % pu.cr == 0)) return KX_OK;
+  if (!(pd.ks == 2 && pd.rs == 4 && pd.cr == i4_chunk_rows(false, 16) && hidden % pd.cr == 0 && inter == 4 * 512)) return KX_OK;
+  int ri;
+  shared.out = (void *)tail.sy;
+  shared.out_stride = hidden;
+  if (kx_gemv_plan(KX_EPI_BF16, shared, &ri) < 0) return KX_ERR_ARG;
+  if (!(shared.cols == 2048 && ri == 4 && shared.nw == 4 && shared.rs == 2) || shared.row_block || shared.norm_w) return KX_OK;
+  const int g_cr = 16;
+  if (pd.cr % g_cr || hidden % g_cr) return KX_OK;
+  tail.shared_chunks = pd.cr / g_cr;
+  const long n_gu = (long)n_slots * (inter / pu.cr), n_i4 = (long)n_slots * (hidden / pd.cr), n_g = hidden / g_cr;
+  // every workgroup waits for others of the launch: all of them resident, two per CU
+  const size_t lds_d = pd.lds + (size_t)inter * 2, lds_g = (size_t)g_cr * 4 * sizeof(float);
+  size_t lds = pu.lds > lds_d ? pu.lds : lds_d;
+  lds = lds > lds_g ? lds : lds_g;
+  if (n_gu != n_i4 || n_g > n_i4 || n_i4 > 2L * cus || lds > 78 * 1024) return KX_OK;
+  static bool attr_set = false;
+  if (!attr_set) {
+    KX_HIP(hipFuncSetAttribute((const void *)i4_routed_shared_k, hipFuncAttributeMaxDynamicSharedMemorySize, 78 * 1024));
+    attr_set = true;
+  }
+  I4Args u = {};
+  u.packed0 = gate_packed; u.scale0 = gate_scale; u.packed1 = up_packed; u.scale1 = up_scale;
+  u.x = x; u.out = mid; u.work = work; u.pairs = pairs; u.n_pairs = 0; u.n_slots = n_slots;
+  u.rows = inter; u.cols = hidden; u.x_div = topk; u.ks = pu.ks; u.rs = pu.rs; u.nt = pu.nt;
+  u.expert_words = (size_t)inter * (hidden / 8); u.expert_scales = (size_t)inter * (hidden / 32);
+  u.cnt_lo = 0; u.cnt_hi = 0x7fffffff;
+  u.tail = KxMoeTail{};
+  u.hand = hand; u.tag = tag; u.err = err;
+  I4Args d = {};
+  d.packed0 = down_packed; d.scale0 = down_scale;
+  d.x = mid; d.out = eout; d.work = work; d.pairs = pairs; d.n_pairs = 0; d.n_slots = n_slots;
+  d.rows = hidden; d.cols = inter; d.x_div = 1; d.ks = pd.ks; d.rs = pd.rs; d.nt = pd.nt;
+  d.expert_words = (size_t)hidden * (inter / 8); d.expert_scales = (size_t)hidden * (inter / 32);
+  d.cnt_lo = 0; d.cnt_hi = 0x7fffffff;
+  d.tail = tail;
+  d.hand = hand; d.tag = tag; d.err = err;
+  hipLaunchKernelGGL(i4_routed_shared_k, dim3((unsigned)n_i4), dim3(512), lds, st, u, d, shared, (int)n_i4, (int)n_g);
   KX_LAUNCH_CHECK();
   *fused = true;
   return KX_OK;

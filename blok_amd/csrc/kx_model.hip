@@ -426,7 +426,8 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample, int C = 1) {
         // streams them faster than the GEMM kernel does at one token.  With 32 sequences that decode alike (70-100
         // distinct experts for 256 pairs, up to 23 pairs on one expert) the step goes from 24.5 to 18.1 ms; at 12
         // sequences the two forms are level (12.1 against 12.4 ms), at 8 the GEMV kernels win (9.8 against 10.9 ms).
-        const uint32_t flags = ((m->fusion & KX_FUSE_MOE_TAIL) ? 0u : KX_MOE_SEPARATE_TAIL) | (moe_head_done ? KX_MOE_HEAD_DONE : 0u) | (B >= 5 && !(m->exact & KX_EXACT_SHARED) ? KX_MOE_SHARED_MATRIX_CORES : 0u) |
+        const uint32_t flags = ((m->fusion & KX_FUSE_MOE_TAIL) ? 0u : KX_MOE_SEPARATE_TAIL) | (moe_head_done ? KX_MOE_HEAD_DONE : 0u) |
+                               ((m->fusion & KX_FUSE_ROUTED) ? KX_MOE_ROUTED_RESIDENT : 0u) | (B >= 5 && !(m->exact & KX_EXACT_SHARED) ? KX_MOE_SHARED_MATRIX_CORES : 0u) |
                                (B >= 12 && !(m->exact & KX_EXACT_ROUTED) ? KX_MOE_ROUTED_MATRIX_CORES : 0u);
         KX_TRY(kx_moe_layer_launch(&c, &L.moe, m->moe_ws, m->n, m->x, B, flags, fuse ? L.post_ln : nullptr, st, false));  // :835-877
       }
@@ -503,6 +504,7 @@ static int model_new(const kx_config *cfg, const char *who, kx_model **out) {
   for (auto &ev : m->ev)
     if (!rc && hipEventCreate(&ev) != hipSuccess) rc = KX_ERR_HIP;
   if (!rc && cfg->first_dense < cfg->n_layers) rc = kx_moe_workspace_create(cfg, step_tokens(cfg), &m->moe_ws);
+  if (!rc && m->moe_ws) kx_moe_workspace_set_err(m->moe_ws, m->front_err);
   if (!rc && (hipMemsetAsync(m->head_count, 0, (size_t)cfg->heads * 4, m->st) != hipSuccess ||
               hipMemsetAsync(m->front_err, 0, 4, m->st) != hipSuccess ||
               hipMemsetAsync(m->back_hand, 0, kx_back_hand_words(cfg->heads * cfg->v_head, cfg->hidden, cfg->experts) * 4, m->st) != hipSuccess ||
@@ -622,15 +624,16 @@ static int check_ids(const kx_model *m, const uint32_t *ids, size_t n) {
   return KX_OK;
 }
 
-// Synchronises the model's stream and reports a grid barrier of the fused attention front that gave up waiting
-// (kx_front.hip): the steps since then computed with values that were not there yet.
+// Synchronises the model's stream and reports a wait inside a resident launch (kx_front.hip, the routed experts'
+// launch of kx_i4.hip) that was given up: the steps since then computed with values that were not there yet.
 static int check_front(kx_model *m) {
   int flag = 0;
   KX_HIP(hipMemcpyAsync(&flag, m->front_err, 4, hipMemcpyDeviceToHost, m->st));
   KX_HIP(hipStreamSynchronize(m->st));
   if (flag) {
-    kx_set_error("kx_model: a grid barrier of the fused attention front timed out (not all of its workgroups were resident); "
-                 "results since then are invalid -- switch it off with kx_model_set_fusion(model, KX_FUSE_ALL & ~KX_FUSE_FRONT)");
+    kx_set_error("kx_model: a workgroup of a resident launch gave up waiting for values from the others (not all workgroups of the launch "
+                 "were on the device at once); results since then are invalid -- switch the resident launches off with "
+                 "kx_model_set_fusion(model, KX_FUSE_ABSORB | KX_FUSE_MOE_TAIL)");
     return KX_ERR_STATE;
   }
   return KX_OK;

@@ -41,6 +41,9 @@ struct kx_moe_workspace {
   uint16_t *eout;     // [T*topk, hidden]
   uint16_t *smid;     // [T, shared_inter]
   uint16_t *sy;       // [T, hidden] shared expert output (prefill path)
+  uint32_t *mid_hand; // [topk, moe_inter] tagged words: one token's mid values inside the resident routed launch
+  uint32_t mid_tag = 0;
+  int *err = nullptr; // the caller's flag for waits given up inside resident launches (not owned)
   hipEvent_t ev[6];
   // a second stream for the batched forms: the experts with one pair (GEMV kernels) and the shared expert run beside the
   // grouped GEMMs of the experts with several pairs instead of in front of them.  Default priority, like every stream here.
@@ -73,7 +76,8 @@ extern "C" int kx_moe_workspace_create(const kx_config *cfg, int32_t max_tokens,
       {(void **)&ws->counts, E * 4}, {(void **)&ws->offsets, (E + 1) * 4}, {(void **)&ws->pairs, T * K * 4},
       {(void **)&ws->work, E * 16}, {(void **)&ws->pair_work, T * K * 16}, {(void **)&ws->n_active, 8}, {(void **)&ws->tail_count, KX_TAIL_BLOCKS * 4},
       {(void **)&ws->mid, T * K * (size_t)cfg->moe_inter * 2}, {(void **)&ws->eout, T * K * (size_t)cfg->hidden * 2},
-      {(void **)&ws->smid, T * (size_t)cfg->shared_inter * 2}, {(void **)&ws->sy, T * (size_t)cfg->hidden * 2}};
+      {(void **)&ws->smid, T * (size_t)cfg->shared_inter * 2}, {(void **)&ws->sy, T * (size_t)cfg->hidden * 2},
+      {(void **)&ws->mid_hand, K * (size_t)cfg->moe_inter * 4}};
   for (auto &al : allocs) {
     hipError_t e = hipMalloc(al.p, al.bytes);
     if (e != hipSuccess) {
@@ -89,6 +93,7 @@ extern "C" int kx_moe_workspace_create(const kx_config *cfg, int32_t max_tokens,
   if (e == hipSuccess) e = hipMemset(ws->pair_work, 0xff, T * K * 16);
   if (e == hipSuccess) e = hipMemset(ws->n_active, 0, 8);
   if (e == hipSuccess) e = hipMemset(ws->tail_count, 0, KX_TAIL_BLOCKS * 4);
+  if (e == hipSuccess) e = hipMemset(ws->mid_hand, 0, K * (size_t)cfg->moe_inter * 4);
   for (auto &ev : ws->ev)
     if (e == hipSuccess) e = hipEventCreate(&ev);
   if (e == hipSuccess) e = hipStreamCreateWithFlags(&ws->side, hipStreamNonBlocking);
@@ -106,7 +111,7 @@ extern "C" int kx_moe_workspace_create(const kx_config *cfg, int32_t max_tokens,
 extern "C" int kx_moe_workspace_destroy(kx_moe_workspace *ws) {
   if (!ws) return KX_OK;
   void *ptrs[] = {ws->logits, ws->ids, ws->weights, ws->counts, ws->offsets, ws->pairs,
-                  ws->work, ws->pair_work, ws->n_active, ws->tail_count, ws->mid, ws->eout, ws->smid, ws->sy};
+                  ws->work, ws->pair_work, ws->n_active, ws->tail_count, ws->mid, ws->eout, ws->smid, ws->sy, ws->mid_hand};
   for (void *p : ptrs)
     if (p) (void)hipFree(p);
   for (auto &e : ws->ev)
@@ -119,6 +124,7 @@ extern "C" int kx_moe_workspace_destroy(kx_moe_workspace *ws) {
 }
 
 int *kx_moe_workspace_n_active(kx_moe_workspace *ws) { return ws->n_active; }
+void kx_moe_workspace_set_err(kx_moe_workspace *ws, int *d_err) { ws->err = d_err; }
 
 void kx_moe_head_args(const kx_config *c, const kx_moe_weights *w, kx_moe_workspace *ws, void *d_n, const uint16_t *norm_w, KxMoeHeadArgs *out) {
   KxMoeHeadArgs h = {};
@@ -270,8 +276,30 @@ static int moe_layer_body(const kx_config *c, const kx_moe_weights *w, kx_moe_wo
                               routed_per_pair(tokens, K, E) ? ws->pair_work : nullptr))) return rc;
   }
   if (timed) KX_HIP(hipEventRecord(ws->ev[1], st));
-  // routed gate/up + SwiGLU
   const int n_slots = (long)tokens * K < E ? tokens * K : E;
+  // one token: the routed experts and the layer's tail as one resident launch
+  bool resident = false;
+  if ((flags & KX_MOE_ROUTED_RESIDENT) && ws->err && paired && tokens == 1 && !(flags & KX_MOE_SEPARATE_TAIL) && H / 16 <= KX_TAIL_BLOCKS) {
+    KxGemvArgs d = {};
+    d.w0 = (const uint16_t *)w->d_shared_down; d.x = ws->smid; d.x_stride = c->shared_inter; d.out = d_x;
+    d.out_stride = H; d.rows = H; d.cols = c->shared_inter; d.tokens = tokens; d.expert_out = ws->eout;
+    d.route_w = ws->weights; d.topk = K; d.flags = flags & 1u;
+    KxMoeTail t = {};
+    t.counter = ws->tail_count; t.n_active = ws->n_active; t.sy = ws->sy; t.route_w = ws->weights; t.x = (uint16_t *)d_x;
+    t.x_stride = H; t.tokens = tokens; t.topk = K; t.flags = flags & 1u;
+    const uint32_t tag = ws->mid_tag % 65535u + 1u;
+    if ((rc = kx_i4_routed_shared_launch((const uint32_t *)w->d_gate_packed, (const uint16_t *)w->d_gate_scale, (const uint32_t *)w->d_up_packed,
+                                         (const uint16_t *)w->d_up_scale, (const uint32_t *)w->d_down_packed, (const uint16_t *)w->d_down_scale,
+                                         n, ws->mid, ws->eout, ws->work, ws->pairs, H, c->moe_inter, K, n_slots, d, t, ws->mid_hand, tag, ws->err,
+                                         &resident, st))) return rc;
+    if (resident) {
+      ws->mid_tag = tag;
+      if (timed)
+        for (int i = 2; i <= 5; ++i) KX_HIP(hipEventRecord(ws->ev[i], st));
+      return KX_OK;
+    }
+  }
+  // routed gate/up + SwiGLU
   if (rmm) {
     // Experts with one pair: the GEMV kernels (they stream such an expert at their rate); the others: the grouped
     // GEMMs.  The two classes touch different experts and different rows of mid and of the expert outputs, so they

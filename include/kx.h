@@ -341,7 +341,9 @@ int kx_model_steps_decoded(kx_model *model, int32_t *steps);
 #define KX_FUSE_MOE_HEAD 16u /* with KX_FUSE_BACK, in front of a MoE layer (shared_inter = 32 * heads, an even number of at most 510
                                experts): the post-attention norm, the router, the routing and the shared expert's gate/up ride in
                                that launch */
-#define KX_FUSE_ALL 31u
+#define KX_FUSE_ROUTED 32u  /* one token, Kimi-K2 shapes, a device with at least 256 CUs, with KX_FUSE_MOE_TAIL: the routed experts' gate/up
+                               rides in the launch of their down projection (one resident launch for the routed experts and the tail) */
+#define KX_FUSE_ALL 63u
 int kx_model_set_fusion(kx_model *model, uint32_t mask);
 /* The attention kernel this model's steps use: KX_MLA_AUTO (default), KX_MLA_VALU or KX_MLA_MATRIX_CORES, as for
  * kx_mla_decode.  A property of the model: other models of the process keep theirs.                          */

@@ -328,8 +328,8 @@ def test_kimi_shape_stack_batch_invariance(kxlib, ox):
 def test_fused_and_separate_launches_agree(kxlib, ox, shape):
     # the q_b GEMV that finishes the query in its own launch, (batch 1) the routed down launch that finishes the MoE
     # layer, and (batch 1, Kimi shapes) the resident launches that run the whole front of the attention block and its
-    # back (bit 3; with bit 4 the head of the MoE layer behind it: norm, router, routing, shared gate/up), against
-    # the same steps as kernels of their own: cache rows, hidden state, logits and ids to the bit (the oracle
+    # back (bit 3; with bit 4 the head of the MoE layer behind it: norm, router, routing, shared gate/up) and the routed
+    # experts with the layer's tail (bit 5), against the same steps as kernels of their own: cache rows, hidden state, logits and ids to the bit (the oracle
     # comparisons above run the fused forms)
     say(f"fusion on/off {shape}")
     if shape == "kimi":
@@ -342,7 +342,7 @@ def test_fused_and_separate_launches_agree(kxlib, ox, shape):
         prompt_len, n_tokens = 11, 9
     prompt = O.tokens_u32(batch * prompt_len, cfg.seed, 4, cfg.vocab).reshape(batch, prompt_len)
     got = []
-    for mask in (31, 0, 1, 2, 3, 4, 8, 15, 24):
+    for mask in (63, 0, 1, 2, 3, 4, 8, 15, 24, 31, 34):
         km = KxModel(kxlib, cfg)
         check(kxlib.kx_model_set_fusion(km.h, mask))
         rc, out, _ = km.generate(prompt, n_tokens)
@@ -353,7 +353,7 @@ def test_fused_and_separate_launches_agree(kxlib, ox, shape):
         km.close()
     assert kxlib.kx_model_set_fusion(None, 1) != 0
     km = KxModel(kxlib, cfg)
-    assert kxlib.kx_model_set_fusion(km.h, 32) != 0 and b"mask" in kxlib.kx_last_error()
+    assert kxlib.kx_model_set_fusion(km.h, 64) != 0 and b"mask" in kxlib.kx_last_error()
     km.close()
     o0, h0, l0, c0 = got[1]   # every launch on its own
     for (o1, h1, l1, c1) in got[:1] + got[2:]:
@@ -849,16 +849,17 @@ def test_model_form_of_the_handover_gives_the_same_bits(kxlib, ox):
     strict = load_library(os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "blok_amd", "libkx_strict.so"))
     # (name, config, sequences, prompt, tokens, fusion masks): the small stack at 3 sequences; Kimi shapes at one
     # sequence with the launches that use the protocol (mask 3: the q_b GEMV finishes the query, the routed down
-    # launch finishes the layer; mask 1: the layer's tail as launches of its own) and with the default (the resident
-    # launches, whose hand-over is another one, plus the routed down launch); Kimi shapes at 3 sequences (the router
+    # launch finishes the layer; mask 1: the layer's tail as launches of its own), with the resident launches of the
+    # attention block (31: their hand-over is another one; the routed down launch finishes the layer) and with the
+    # default (63: the routed experts' resident launch finishes it); Kimi shapes at 3 sequences (the router
     # and shared gate/up pair launch whose last router workgroup routes, the q_b GEMV at several tokens)
-    cases = [("small", O.small_config(batch=3, context=64), 3, 11, 9, (31,))]
+    cases = [("small", O.small_config(batch=3, context=64), 3, 11, 9, (63,))]
     kimi = default_config()
     kimi.n_layers, kimi.first_dense, kimi.max_batch, kimi.max_context, kimi.seed = 3, 1, 1, 48, 11
-    cases.append(("kimi", kimi, 1, 24, 8, (3, 1, 31)))
+    cases.append(("kimi", kimi, 1, 24, 8, (3, 1, 31, 63)))
     kimi3 = default_config()
     kimi3.n_layers, kimi3.first_dense, kimi3.max_batch, kimi3.max_context, kimi3.seed = 2, 1, 3, 24, 12
-    cases.append(("kimi, 3 sequences", kimi3, 3, 9, 4, (31,)))
+    cases.append(("kimi, 3 sequences", kimi3, 3, 9, 4, (63,)))
     for name, cfg, batch, prompt_len, n_tokens, masks in cases:
         prompt = O.tokens_u32(batch * prompt_len, cfg.seed, 4, cfg.vocab).reshape(batch, prompt_len)
         for mask in masks:
