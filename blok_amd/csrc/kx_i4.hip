@@ -26,10 +26,8 @@
 //
 // All arithmetic is IEEE binary32 (fma, mul, add), so a scalar host program
 // that follows the same order reproduces the result bit for bit.
-#include <stdlib.h>
 #include "kx_arrive.h"
 #include "kx_hand.h"
-#include "kx_lds_copy.h"
 #include "kx_common.h"
 #include "kx_dense.h"
 #include "kx_gemv_body.h"
@@ -113,8 +111,7 @@ struct I4Dec {  // the eight f16 pairs of one 128-bit load... four words, four p
   kx_h2 a[16];
 };
 
-template <class V4>
-__device__ __forceinline__ void decode_words(I4Dec &d, const V4 &v, uint32_t magic) {
+__device__ __forceinline__ void decode_words(I4Dec &d, uint4 v, uint32_t magic) {
   const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
   for (int p = 0; p < 4; ++p) {
@@ -230,21 +227,16 @@ __device__ __forceinline__ void moe_tail_arrive(const KxMoeTail &t, int blk_a, i
 // also handed over as a tagged word, and the workgroup may have more waves than the chunk shape uses (they keep the
 // barriers); 2 = the activations are not read from a.x but collected from the tagged words of the pair's row, one
 // 16-byte request per thread (4 * blockDim.x = cols), through LDS.
-// RING3 (one token, the fused gate/up shape, one chunk per workgroup): three tiles under way per wave instead of
-// one -- two in registers and one in LDS, in the place of the second scale buffer, which a workgroup with one chunk
-// does not use -- requested from inline asm and waited for by count, because the compiler's own waits would complete
-// every request in flight in front of the oldest.  Same values, same sums: only the way the packed words travel.
-template <bool DUAL, int TT, int KS_T, bool FILTER, int CM = 1, int HAND = 0, bool RING3 = false, class Idle>
+template <bool DUAL, int TT, int KS_T, bool FILTER, int CM = 1, int HAND = 0, class Idle>
 __device__ __forceinline__ void i4_body(const I4Args &a, const int bid, const int nblocks, float *lds, Idle &&idle) {
   constexpr int MATS = DUAL ? 2 : 1;
   constexpr int RI = I4_RI;
   constexpr int NV = RI * MATS * TT;
   constexpr int NOUT = kxw::reduce_out<NV, 32>();
   const int ks = KS_T ? KS_T : a.ks;
-  constexpr int KS_D = KS_T ? KS_T : 1;  // divisor that is never zero in the branches not taken
-  const int rs = KS_T ? (KS_T >= 5 ? 1 : 8 / KS_D) : a.rs;
+  const int rs = KS_T ? (KS_T >= 5 ? 1 : 8 / KS_T) : a.rs;
   const int RT = rs * 2 * RI;
-  const int nt = KS_T ? CM * (i4_chunk_rows(DUAL, KS_T >= 5 ? 4 : 32 / KS_D) / (KS_T >= 5 ? 4 : 32 / KS_D)) : a.nt;  // CM: chunks of CM times the rows
+  const int nt = KS_T ? CM * (i4_chunk_rows(DUAL, KS_T >= 5 ? 4 : 32 / KS_T) / (KS_T >= 5 ? 4 : 32 / KS_T)) : a.nt;  // CM: chunks of CM times the rows
   const int CR = RT * nt;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int l = lane & 31, h = lane >> 5;
@@ -330,23 +322,7 @@ __device__ __forceinline__ void i4_body(const I4Args &a, const int bid, const in
   uint4 xraw[TT][4];
   int sb = 0;
   copy_scales(cur, sc_base);
-  kx_u32x4 rx[MATS][RI], ry[MATS][RI];  // RING3: the register slots of the tiles under way
-  // addresses as a scalar base (matrix, tile, row pair) plus this lane's byte offset: no address registers per request
-  const uint32_t ring_off = w_off * 4u;
-  auto ring_base = [&](int m, int i, int tile) { return (uint64_t)(uintptr_t)(tile_ptr(cur, m) + (size_t)((tile * RT + i * 2) * row_words)); };
-  auto ring_regs = [&](kx_u32x4 (&buf)[MATS][RI], int tile) {
-#pragma unroll
-    for (int i = 0; i < RI; ++i)
-#pragma unroll
-      for (int m = 0; m < MATS; ++m)
-        // s_nop 4: the scalar base may have been written by a VALU instruction (v_readlane of a spilled SGPR) just in
-        // front of this statement, and a memory instruction may read such an SGPR only five wait states later; the
-        // compiler keeps that distance for its own instructions and cannot see into this one
-        asm volatile("s_nop 4\n\tglobal_load_dwordx4 %0, %1, %2 nt" : "=v"(buf[m][i]) : "v"(ring_off), "s"(ring_base(m, i, tile)) : "memory");
-  };
-  if (RING3) {
-    if (active) ring_regs(rx, 0);
-  } else if (active) load_tile(bufA, cur, 0);
+  if (active) load_tile(bufA, cur, 0);
   if (HAND == 2) {
     // behind the first tile's requests: a wave's loads return in order, so the answer comes when those have landed
     const uint32_t *src = a.hand + (size_t)cur.first_pair * a.cols + threadIdx.x * 4;
@@ -392,14 +368,14 @@ __device__ __forceinline__ void i4_body(const I4Args &a, const int bid, const in
         prep_xgroup(xg[0], xraw[0]);
       }
 
-      auto compute_from = [&](auto &&get, int tile) {
+      auto compute_tile = [&](uint4 (&buf)[MATS][RI], int tile) {
         float v[NV];
 #pragma unroll
         for (int i = 0; i < RI; ++i)
 #pragma unroll
           for (int m = 0; m < MATS; ++m) {
             I4Dec dec;
-            decode_words(dec, get(m, i), magic);
+            decode_words(dec, buf[m][i], magic);
             const float sc = kx_bf16_f32(sc_lane[(m * CR + tile * RT + i * 2) * groups]);
 #pragma unroll
             for (int t = 0; t < TT; ++t) v[(i * MATS + m) * TT + t] = sc * group_dot(dec, xg[t]);
@@ -415,50 +391,8 @@ __device__ __forceinline__ void i4_body(const I4Args &a, const int bid, const in
           }
         }
       };
-      auto compute_tile = [&](uint4 (&buf)[MATS][RI], int tile) {
-        compute_from([&](int m, int i) { return buf[m][i]; }, tile);
-      };
 
-      if constexpr (RING3) {
-        static_assert(!RING3 || (DUAL && TT == 1 && KS_T == 7 && !FILTER && CM == 1), "RING3 is the one-token gate/up shape");
-        if (active) {
-          constexpr int NT = 8;  // = nt for this shape
-          uint8_t *ring = (uint8_t *)(sc_base + sc_pieces) + wave * (MATS * RI * 1024);  // this wave's 4 KB of the unused scale buffer
-          const uint32_t ring_lds = (uint32_t)(uintptr_t)ring;
-          auto issue_regs = ring_regs;
-          auto issue_lds = [&](int tile) {
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // this wave's reads of the tile that lay here are done
-#pragma unroll
-            for (int i = 0; i < RI; ++i)
-#pragma unroll
-              for (int m = 0; m < MATS; ++m) {
-                uint32_t m0_saved;
-                asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 4\n\tglobal_load_lds_dwordx4 %2, %3 nt\n\ts_mov_b32 m0, %0"
-                             : "=&s"(m0_saved)
-                             : "s"(__builtin_amdgcn_readfirstlane(ring_lds + (i * MATS + m) * 1024)), "v"(ring_off), "s"(ring_base(m, i, tile))
-                             : "memory");
-              }
-          };
-          auto from_regs = [&](kx_u32x4 (&buf)[MATS][RI]) {
-            return [&](int m, int i) -> const kx_u32x4 & { return buf[m][i]; };
-          };
-          auto from_lds = [&](int m, int i) { return *(const uint4 *)(ring + (i * MATS + m) * 1024 + lane * 16); };
-#define KX_I4_WAIT(N, B) asm volatile("s_waitcnt vmcnt(" #N ")" : "+v"(B[0][0]), "+v"(B[0][1]), "+v"(B[1][0]), "+v"(B[1][1])::"memory")
-          // tile 0 is in rx (requested before the scales were waited for); tiles 0, 3, 6 go through rx, 1, 4 and 7
-          // through ry, 2 and 5 through LDS; behind the tile being waited for, two more are in flight
-          issue_regs(ry, 1);
-          issue_lds(2);
-          KX_I4_WAIT(8, rx); compute_from(from_regs(rx), 0); issue_regs(rx, 3);
-          KX_I4_WAIT(8, ry); compute_from(from_regs(ry), 1); issue_regs(ry, 4);
-          asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); compute_from(from_lds, 2); issue_lds(5);
-          KX_I4_WAIT(8, rx); compute_from(from_regs(rx), 3); issue_regs(rx, 6);
-          KX_I4_WAIT(8, ry); compute_from(from_regs(ry), 4); issue_regs(ry, 7);
-          asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); compute_from(from_lds, 5);
-          KX_I4_WAIT(4, rx); compute_from(from_regs(rx), 6);
-          KX_I4_WAIT(0, ry); compute_from(from_regs(ry), NT - 1);
-#undef KX_I4_WAIT
-        }
-      } else if (active)
+      if (active)
         for (int tile = 0; tile < nt; tile += 2) {
           if (tile + 1 < nt) load_tile(bufB, cur, tile + 1);
           compute_tile(bufA, tile);
@@ -513,10 +447,10 @@ __device__ __forceinline__ void i4_body(const I4Args &a, const int bid, const in
   }
 }
 
-template <bool DUAL, int TT, int KS_T, int MAXT, int WPE, bool FILTER, int CM = 1, bool RING3 = false>
+template <bool DUAL, int TT, int KS_T, int MAXT, int WPE, bool FILTER, int CM = 1>
 __global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(WPE, WPE))) i4_gemv_k(I4Args a) {
   extern __shared__ float lds[];
-  i4_body<DUAL, TT, KS_T, FILTER, CM, 0, RING3>(a, blockIdx.x, gridDim.x, lds, [] {});
+  i4_body<DUAL, TT, KS_T, FILTER, CM>(a, blockIdx.x, gridDim.x, lds, [] {});
 }
 
 // The routed down GEMV of one token and the shared expert's down GEMV ([rows, 2048] bf16) in one launch.  Workgroup b
@@ -695,8 +629,6 @@ int kx_i4_launch(bool dual, const uint32_t *packed0, const uint16_t *scale0, con
     if (tt == 2) hipLaunchKernelGGL((i4_gemv_k<false, 2, 2, 512, 4, true, 2>), g, b, pl.lds, st, a);
     else if (filter) hipLaunchKernelGGL((i4_gemv_k<false, 1, 2, 512, 4, true, 2>), g, b, pl.lds, st, a);
     else hipLaunchKernelGGL((i4_gemv_k<false, 1, 2, 512, 4, false, 2>), g, b, pl.lds, st, a);
-  } else if (full && pl.ks == 7 && dual && tt == 1 && !filter && chunks == (long)g.x && getenv("KX_I4_RING3")) {
-    hipLaunchKernelGGL((i4_gemv_k<true, 1, 7, 448, 4, false, 1, true>), g, b, pl.lds, st, a);
   } else if (full && pl.ks == 7) {        // Kimi-K2 gate/up: K = 7168
     if (dual) launch_tt<true, 7, 448>(a, tt, g, b, pl.lds, st);
     else launch_tt<false, 7, 448>(a, tt, g, b, pl.lds, st);
