@@ -771,6 +771,14 @@ extern "C" int kx_model_rewind(kx_model *m, int32_t positions) {
   return KX_OK;
 }
 
+extern "C" int kx_model_debug_fail_waits(kx_model *m) {
+  KX_REQUIRE(m, "kx_model_debug_fail_waits: null model");
+  const int one = 1;
+  KX_HIP(hipMemcpyAsync(m->front_err, &one, 4, hipMemcpyHostToDevice, m->st));
+  KX_HIP(hipStreamSynchronize(m->st));
+  return KX_OK;
+}
+
 extern "C" int kx_model_set_attention_kernel(kx_model *m, int32_t kernel) {
   KX_REQUIRE(m, "kx_model_set_attention_kernel: null model");
   KX_REQUIRE(kernel >= KX_MLA_AUTO && kernel <= KX_MLA_MATRIX_CORES, "kx_model_set_attention_kernel: kernel=%d outside [0, 2]", kernel);

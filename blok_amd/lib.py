@@ -92,6 +92,7 @@ _SIGS = {
     "kx_model_timing": [_P, C.POINTER(C.c_float)],
     "kx_model_steps_decoded": [_P, C.POINTER(C.c_int32)],
     "kx_model_set_fusion": [_P, C.c_uint32],
+    "kx_model_debug_fail_waits": [_P],
     "kx_model_set_attention_kernel": [_P, _I],
     "kx_model_set_routing_record": [_P, C.c_int],
     "kx_model_set_exact": [_P, C.c_uint32],

@@ -345,6 +345,12 @@ int kx_model_steps_decoded(kx_model *model, int32_t *steps);
                                rides in the launch of their down projection (one resident launch for the routed experts and the tail) */
 #define KX_FUSE_ALL 63u
 int kx_model_set_fusion(kx_model *model, uint32_t mask);
+/* Test hook for the failure path of the resident launches (KX_FUSE_FRONT, _BACK, _MOE_HEAD, _ROUTED): sets the
+ * model's device-side flag as a workgroup does that has given a wait for another workgroup's values up.  From then
+ * on a workgroup whose first poll does not succeed gives up at once, every launch still ends normally, and the next
+ * call that synchronises (kx_greedy_sample, kx_generate) returns KX_ERR_STATE with a message naming
+ * kx_model_set_fusion.  The flag stays set: the model is only good for kx_model_destroy afterwards.              */
+int kx_model_debug_fail_waits(kx_model *model);
 /* The attention kernel this model's steps use: KX_MLA_AUTO (default), KX_MLA_VALU or KX_MLA_MATRIX_CORES, as for
  * kx_mla_decode.  A property of the model: other models of the process keep theirs.                          */
 int kx_model_set_attention_kernel(kx_model *model, int32_t kernel);

@@ -837,6 +837,35 @@ def test_config5_batch32_full_size_step_by_step_against_the_exact_path(kxlib, ox
     assert sum(verdicts.values()) == batch * n_tokens
 
 
+def test_a_wait_given_up_inside_a_resident_launch_is_reported(kxlib, ox):
+    # The workgroups of the resident launches wait for each other's values with a bounded number of polls; one that
+    # gives up sets a flag, the launch ends normally, and the model reports the flag at its next synchronisation.
+    # Forced from the host: with the flag set beforehand, every workgroup whose first poll fails gives up at once, so
+    # all launches drain (nothing hangs) and generate must come back with an error that names the way out.
+    say("resident launches: a wait given up is reported, the launches still end")
+    cfg = default_config()
+    cfg.n_layers, cfg.first_dense, cfg.max_batch, cfg.max_context, cfg.seed = 2, 1, 1, 32, 11
+    prompt = O.tokens_u32(5, cfg.seed, 4, cfg.vocab).reshape(1, 5)
+    km = KxModel(kxlib, cfg)
+    check(kxlib.kx_model_debug_fail_waits(km.h))
+    rc, _, _ = km.generate(prompt, 3)
+    assert rc != 0 and b"kx_model_set_fusion" in kxlib.kx_last_error(), kxlib.kx_last_error()
+    rc, _, _ = km.generate(prompt, 3)   # the flag stays: so does the error
+    assert rc != 0
+    km.close()
+    assert kxlib.kx_model_debug_fail_waits(None) != 0
+    # the process is fine: a new model, with and without the resident launches, decodes the same ids
+    outs = []
+    for mask in (63, 3):
+        km = KxModel(kxlib, cfg)
+        check(kxlib.kx_model_set_fusion(km.h, mask))
+        rc, out, _ = km.generate(prompt, 3)
+        assert rc == 0, kxlib.kx_last_error()
+        outs.append(out.copy())
+        km.close()
+    assert (outs[0] == outs[1]).all()
+
+
 def test_model_form_of_the_handover_gives_the_same_bits(kxlib, ox):
     # blok_amd/libkx_strict.so is the library with the hand-over between workgroups of one launch (the q_b GEMV that
     # finishes a head's query, the router GEMV whose last workgroup routes, the routed down launch that combines)
