@@ -124,9 +124,9 @@ struct kx_moe_workspace;
 #define KX_MOE_SEPARATE_TAIL 0x100u
 // 5 to 32 tokens: the shared expert's GEMVs on the matrix cores (kx_skinny.hip; tolerance instead of bit parity)
 #define KX_MOE_SHARED_MATRIX_CORES 0x200u
-// 5 tokens and more: the routed experts with more than one pair as W4A16 grouped GEMMs on the matrix cores
+// 5 tokens and more: the routed experts with three or more pairs as W4A16 grouped GEMMs on the matrix cores
 // (kx_prefill.hip) instead of the GEMV kernels: such an expert's weights are streamed and dequantised once for all its
-// tokens (tolerance instead of bit parity); the experts with one pair keep the GEMV kernel
+// tokens (tolerance instead of bit parity); the experts with one or two pairs keep the GEMV kernel
 #define KX_MOE_ROUTED_MATRIX_CORES 0x400u
 // internal (not among the public flags): the layer's first launch -- normed row in d_n, router logits, routing, shared
 // gate/up -- has been done by the caller's own launch (kx_front.hip's back launch with kx_moe_head_args): one token

@@ -254,6 +254,11 @@ static int moe_layer_body(const kx_config *c, const kx_moe_weights *w, kx_moe_wo
   // and runs the routed experts, and are joined before the combine.
   const bool mm = (flags & KX_MOE_SHARED_MATRIX_CORES) && tokens >= 5 && tokens <= 32;
   const bool rmm = (flags & KX_MOE_ROUTED_MATRIX_CORES) && tokens >= 5;
+  // The grouped GEMMs take the experts with at least three pairs, the GEMV kernels those with one or two: a GEMM
+  // workgroup holds a CU for the whole of its 112 K steps whatever its tokens, and at 32 sequences the experts with
+  // two pairs made the GEMMs a round of 256 workgroups and a twelfth (measured, batch 32: 1897 tok/s with the line
+  // at two pairs, 1983 at three, 1941 at four, 1812 at six; batch 16: 1313 -> 1325; batch 12: level)
+  constexpr int rmm_min = 3;
   bool shared_up_done = false, shared_down_done = false;
   if (mm && !norm_w) {
     KX_HIP(hipEventRecord(ws->fork, st));
@@ -314,10 +319,10 @@ static int moe_layer_body(const kx_config *c, const kx_moe_weights *w, kx_moe_wo
     forked = true;
     if ((rc = kx_grouped_gemm_launch(true, true, w->d_gate_packed, (const uint16_t *)w->d_gate_scale, w->d_up_packed,
                                      (const uint16_t *)w->d_up_scale, n, ws->mid, KX_GG_BF16, ws->work, ws->pairs, 0, n_slots, I, H,
-                                     K, (size_t)I * (H / 8), (size_t)I * (H / 32), tokens, st, 2))) return rc;
+                                     K, (size_t)I * (H / 8), (size_t)I * (H / 32), tokens, st, rmm_min))) return rc;
     if ((rc = kx_i4_launch(true, (const uint32_t *)w->d_gate_packed, (const uint16_t *)w->d_gate_scale,
                            (const uint32_t *)w->d_up_packed, (const uint16_t *)w->d_up_scale, n, ws->mid, ws->work, ws->pairs, 0, I,
-                           H, K, (size_t)I * (H / 8), (size_t)I * (H / 32), 1, n_slots, 1, 1, ws->side))) return rc;
+                           H, K, (size_t)I * (H / 8), (size_t)I * (H / 32), 1, n_slots, 1, rmm_min - 1, ws->side))) return rc;
   } else if ((rc = routed_launch(c, w, ws, n, tokens, 0, st))) return rc;
   if (timed) KX_HIP(hipEventRecord(ws->ev[2], st));
   // shared down + combine + residual: as the epilogue of a GEMV of its own, or, for one token, inside the routed
@@ -341,10 +346,10 @@ static int moe_layer_body(const kx_config *c, const kx_moe_weights *w, kx_moe_wo
     const int I = c->moe_inter;
     if ((rc = kx_grouped_gemm_launch(false, true, w->d_down_packed, (const uint16_t *)w->d_down_scale, nullptr, nullptr,
                                      ws->mid, ws->eout, KX_GG_BF16, ws->work, ws->pairs, 0, n_slots, H, I, 1, (size_t)H * (I / 8),
-                                     (size_t)H * (I / 32), tokens, st, 2))) return rc;
+                                     (size_t)H * (I / 32), tokens, st, rmm_min))) return rc;
     if ((rc = kx_i4_launch(false, (const uint32_t *)w->d_down_packed, (const uint16_t *)w->d_down_scale, nullptr, nullptr,
                            ws->mid, ws->eout, ws->work, ws->pairs, 0, H, I, 1, (size_t)H * (I / 8), (size_t)H * (I / 32),
-                           1, n_slots, 1, 1, ws->side, 2))) return rc;
+                           1, n_slots, 1, rmm_min - 1, ws->side, 2))) return rc;
   } else if (!tailed && (rc = routed_launch(c, w, ws, n, tokens, 1, st))) return rc;
   if (timed) KX_HIP(hipEventRecord(ws->ev[3], st));
   // shared gate/up + SwiGLU when it neither rode with the router nor ran on the side stream

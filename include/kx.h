@@ -188,8 +188,8 @@ int kx_moe_workspace_views(kx_moe_workspace *ws, void **d_logits, void **d_ids, 
  *             for one token (by default they ride in the routed down launch; same results).
  *       bit9: 5 to 32 tokens: the shared expert's two GEMVs as bf16 matrix-core products (another
  *             summation order: within max-rel 1e-2 of the default instead of equal to the bit).
- *       bit10: 5 tokens and more: the routed experts that have more than one (token, slot) pair as W4A16
- *             grouped GEMMs on the matrix cores, the experts with one pair through the GEMV kernel (same
+ *       bit10: 5 tokens and more: the routed experts that have three or more (token, slot) pairs as W4A16
+ *             grouped GEMMs on the matrix cores, the experts with one or two pairs through the GEMV kernel (same
  *             tolerance).  The router is not affected by either bit, so the routing stays the default's.
  *             The decoder stack sets bit9 from 5 sequences on and bit10 from 12. */
 int kx_moe_decode_layer(const kx_config *cfg, const kx_moe_weights *w, kx_moe_workspace *ws,
