@@ -209,68 +209,73 @@ def test_eos_and_errors(kxlib, ox):
     assert kxlib.kx_model_create(C.byref(bad_cfg), C.byref(h)) != 0
 
 
-def test_config5_24_layer_stack_tokens_identical_to_the_oracle(kxlib, ox, capsys):
+@pytest.mark.parametrize("batch,plen,n_tokens", [(1, 70, 32), (3, 6, 5)])
+def test_config5_24_layer_stack_tokens_identical_to_the_oracle(kxlib, ox, capsys, batch, plen, n_tokens):
     # BASELINE config 5's stack at its full depth and width -- 24 layers (one dense, 23 MoE of 384 experts), vocabulary
     # 163840, 231 GB resident on the GPU -- against the CPU oracle's kx schedule (generate(), :885-890; run(),
     # :801-884).  The oracle holds the dense tensors and produces a routed expert when a token first selects it (the
     # generator is a function of seed, tensor and index; the CPU suite checks that such a model equals the one holding
-    # every expert), which makes 24 layers fit in host memory.  A 70-token prompt crosses the 64-position tile of the
-    # attention kernel; 32 greedy tokens follow.  Required: every sampled id identical, the logits of every sampled step
-    # identical to the bit, and at the end the hidden state and the cache rows of all 24 layers identical to the bit.
-    # The top-1/top-2 margin of every sampled step is printed: identity is not owed to wide margins alone when some of
-    # them are a few bf16 steps.  The oracle takes about half a second a step on sixteen cores: progress is printed.
+    # every expert), which makes 24 layers fit in host memory.  One sequence: a 70-token prompt crosses the 64-position
+    # tile of the attention kernel; 32 greedy tokens follow (the path of the resident launches).  Three sequences, a
+    # short run: the kernels that take two to four tokens per pass, at the full depth.  Required: every sampled id
+    # identical, the logits of every sampled step identical to the bit, and at the end the hidden state and the cache
+    # rows of all 24 layers identical to the bit.  The top-1/top-2 margin of every sampled step is printed: identity
+    # is not owed to wide margins alone when some of them are a few bf16 steps.  The oracle takes about half a second
+    # a step and sequence on sixteen cores: progress is printed.
     import time
-    plen, n_tokens = 70, 32
-    say(f"config 5, 24 layers, batch 1, prompt {plen}, {n_tokens} tokens against the oracle")
+    say(f"config 5, 24 layers, batch {batch}, prompt {plen}, {n_tokens} tokens against the oracle")
     cfg = default_config()
-    cfg.max_batch, cfg.max_context, cfg.seed = 1, plen + n_tokens, 0
+    cfg.max_batch, cfg.max_context, cfg.seed = batch, plen + n_tokens, 0
     assert cfg.n_layers == 24 and cfg.first_dense == 1 and cfg.experts == 384 and cfg.vocab == 163840
-    prompt = O.tokens_u32(plen, cfg.seed, 4, cfg.vocab).reshape(1, plen)
+    prompt = O.tokens_u32(batch * plen, cfg.seed, 4, cfg.vocab).reshape(batch, plen)
 
     def note(msg):
         with capsys.disabled():
             print("  " + msg, flush=True)
 
     km = KxModel(kxlib, cfg)
-    check(kxlib.kx_prefill(km.h, ptr(prompt), 1, plen))
+    check(kxlib.kx_prefill(km.h, ptr(prompt), batch, plen))
     ids_gpu, logits_gpu = [], []
-    one = np.zeros(1, dtype=np.uint32)
+    got = np.zeros(batch, dtype=np.uint32)
     for i in range(n_tokens):
         if i:
-            check(kxlib.kx_decode_step(km.h, None))        # feeds the id sampled on the device
-        check(kxlib.kx_greedy_sample(km.h, ptr(one)))
-        ids_gpu.append(int(one[0]))
-        logits_gpu.append(km.logits(1)[0].view(np.uint32).copy())
-    hidden_gpu = km.hidden(1)
+            check(kxlib.kx_decode_step(km.h, None))        # feeds the ids sampled on the device
+        check(kxlib.kx_greedy_sample(km.h, ptr(got)))
+        ids_gpu.append(got.copy())
+        logits_gpu.append(km.logits(batch).view(np.uint32).copy())
+    hidden_gpu = km.hidden(batch)
     total = plen + n_tokens - 1
-    rows_gpu = [km.latent(layer, 0, total) for layer in range(cfg.n_layers)]
+    rows_gpu = [[km.latent(layer, b, total) for b in range(batch)] for layer in range(cfg.n_layers)]
     km.close()
-    note(f"GPU ids {ids_gpu}")
+    note(f"GPU ids {[g.tolist() for g in ids_gpu]}")
 
     om = O.OxModel(cfg, 1, experts_on_demand=True)
     t0 = time.time()
     for pos in range(plen - 1):
-        om.step(prompt[:, pos], pos, False)
+        om.step(np.ascontiguousarray(prompt[:, pos]), pos, False)
         if pos % 8 == 7:
             note(f"oracle: prompt position {pos + 1} of {plen}, {time.time() - t0:.0f} s")
-    cur = prompt[:, plen - 1]
+    cur = np.ascontiguousarray(prompt[:, plen - 1])
     for i in range(n_tokens):
         nxt = om.step(cur, plen - 1 + i, True)
-        lg = om.logits(1)[0]
-        top = np.sort(lg)[-2:]
-        steps = (top[1] - top[0]) / (abs(top[1]) * 2.0 ** -8)      # in bf16 steps of the winner
-        note(f"token {i}: oracle {int(nxt[0])} GPU {ids_gpu[i]}; top-1 {top[1]:.4f}, top-2 {top[0]:.4f} "
-             f"({steps:.1f} bf16 steps apart); {time.time() - t0:.0f} s")
-        assert int(nxt[0]) == ids_gpu[i], f"token {i}: the oracle samples {int(nxt[0])}, the GPU {ids_gpu[i]}"
+        lg = om.logits(batch)
+        margins = []
+        for b in range(batch):
+            top = np.sort(lg[b])[-2:]
+            margins.append(float((top[1] - top[0]) / (abs(top[1]) * 2.0 ** -8)))      # in bf16 steps of the winner
+        note(f"token {i}: oracle {nxt.tolist()} GPU {ids_gpu[i].tolist()}; top-1 and top-2 "
+             f"{', '.join('%.1f' % m for m in margins)} bf16 steps apart; {time.time() - t0:.0f} s")
+        assert (nxt == ids_gpu[i]).all(), f"token {i}: the oracle samples {nxt.tolist()}, the GPU {ids_gpu[i].tolist()}"
         bad = int(np.count_nonzero(lg.view(np.uint32) != logits_gpu[i]))
         assert bad == 0, f"token {i}: {bad} of {lg.size} logits differ"
-        cur = nxt
-    assert (om.hidden(1) == hidden_gpu).all(), "final hidden state differs"
+        cur = nxt.copy()
+    assert (om.hidden(batch) == hidden_gpu).all(), "final hidden state differs"
     for layer in range(cfg.n_layers):
-        lat = om.latent(layer)[0, :total]
-        assert (lat == rows_gpu[layer]).all(), f"cache rows of layer {layer} differ"
-    note(f"24 layers: {n_tokens} ids, their logits, the hidden state and {cfg.n_layers} x {total} cache rows identical; "
-         f"{ox.ox_model_experts_produced(om.h)} experts produced by the oracle")
+        lat = om.latent(layer)
+        for b in range(batch):
+            assert (lat[b, :total] == rows_gpu[layer][b]).all(), f"cache rows of layer {layer}, sequence {b} differ"
+    note(f"24 layers: {n_tokens} x {batch} ids, their logits, the hidden states and {cfg.n_layers} x {batch} x {total} cache rows "
+         f"identical; {ox.ox_model_experts_produced(om.h)} experts produced by the oracle")
     om.close()
 
 
