@@ -55,3 +55,15 @@ static inline int kx_guard(const char *who, F &&body) {
 
 static inline hipStream_t kx_stream(void *s) { return (hipStream_t)s; }
 static inline int kx_cdiv(int a, int b) { return (a + b - 1) / b; }
+
+// CUs of the current device (0 when the query fails), remembered per device: the launchers of the resident kernels
+// ask before every launch whether all their workgroups fit on the device at once.
+static inline int kx_device_cus() {
+  static int cus[16];
+  int dev = 0, v = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  if (dev >= 0 && dev < 16 && cus[dev]) return cus[dev];
+  if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) return 0;
+  if (dev >= 0 && dev < 16) cus[dev] = v;
+  return v;
+}

@@ -738,12 +738,7 @@ __global__ void __launch_bounds__(BK_THREADS) attn_back_k(BackArgs a) {
 int kx_attn_front_launch(const KxGemvArgs &g_qkv, const KxGemvArgs &g_qb, const QAbsArgs &q, uint32_t *hand, uint32_t tag, int *err,
                          bool *done, hipStream_t st) {
   *done = false;
-  static int cus = 0;
-  if (!cus) {
-    int dev = 0;
-    KX_HIP(hipGetDevice(&dev));
-    KX_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-  }
+  const int cus = kx_device_cus();  // 0 (query failed): the resident form is declined below
   const int hidden = g_qkv.cols, q_rank = g_qb.cols, qk = q.nope + q.rope, G = 4 * q.heads, kva = q.kv_rank + q.rope;
   if (g_qkv.tokens != 1 || g_qb.tokens != 1 || !hand || !err || !q.cache || !g_qkv.norm_w || !g_qb.norm_w || tag < 1 || tag > 65535) return KX_OK;
   if (G > cus || hidden != 14 * 512 || q_rank % 512 || q_rank / 512 > 4 || q_rank / 8 > 256) return KX_OK;
@@ -780,12 +775,7 @@ int kx_attn_back_launch(const KxGemvArgs &g_uv, const KxGemvArgs &g_o, const KxM
                         bool *done, bool *head_done, hipStream_t st) {
   *done = false;
   *head_done = false;
-  static int cus = 0;
-  if (!cus) {
-    int dev = 0;
-    KX_HIP(hipGetDevice(&dev));
-    KX_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-  }
+  const int cus = kx_device_cus();  // 0 (query failed): the resident form is declined below
   const int heads = g_uv.mla_heads, G = 4 * heads;
   if (g_uv.tokens != 1 || g_o.tokens != 1 || !g_uv.mla_po || !hand || !err || tag < 1 || tag > 65535) return KX_OK;
   if (g_uv.mla_spans < 1 || g_uv.mla_spans > BK_SPANS || G > cus || g_uv.cols != 512 || g_uv.row_block != 128 || g_uv.rows != heads * 128) return KX_OK;

@@ -693,12 +693,7 @@ int kx_i4_routed_shared_launch(const uint32_t *gate_packed, const uint16_t *gate
   *fused = false;
   if (tail.tokens != 1 || shared.tokens != 1 || !tail.counter || !work || shared.rows != hidden || !hand || !err || tag < 1 || tag > 65535)
     return KX_OK;
-  static int cus = 0;
-  if (!cus) {
-    int dev = 0;
-    KX_HIP(hipGetDevice(&dev));
-    KX_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-  }
+  const int cus = kx_device_cus();  // 0 (query failed): the resident form is declined below
   I4Launch pu, pd;
   int rc = plan(hidden, inter, 2, 1, pu);
   if (rc) return rc;

@@ -79,10 +79,10 @@ struct kx_model {
   float *qabs, *partial, *logits, *argmax_scratch;
   uint32_t *ids, *next, *history;  // [max_context][B], [B], [max_context][B]
   int *head_count;                 // [heads] arrival counters of the q_b GEMV that finishes the query; zero between launches
-  int *front_err;                  // error flag of the fused attention front (kx_front.hip): a wait gave up
-  uint32_t *front_hand;            // its tagged words
+  int *hand_err;                   // error flag of the resident launches (kx_front.hip, kx_i4.hip): a wait for another workgroup's values gave up
+  uint32_t *front_hand;            // tagged words of the attention block's front launch (q_a, kv_a, q)
   uint32_t front_tag = 0;          // tag of its last launch
-  uint32_t *back_hand;             // tagged words of the fused back of the attention block (W_UV output)
+  uint32_t *back_hand;             // tagged words of the attention block's back launch (attention output, residual row, router logits)
   uint32_t back_tag = 0;
   int4 *head_work;                 // [heads], [step tokens * heads]: the groups of head_groups_k
   int *head_pairs;
@@ -207,7 +207,7 @@ int layout(const kx_config *c, Plan &p, kx_model *m) {
   auto *next = KX_AT(uint32_t *, B * 4);
   auto *history = KX_AT(uint32_t *, (size_t)c->max_context * B * 4);
   auto *head_count = KX_AT(int *, (size_t)c->heads * 4);
-  auto *front_err = KX_AT(int *, 4);
+  auto *hand_err = KX_AT(int *, 4);
   auto *front_hand = KX_AT(uint32_t *, kx_front_hand_words(c->q_rank, (int)KVA, (int)KD) * 4);
   auto *back_hand = KX_AT(uint32_t *, kx_back_hand_words((int)VD, c->hidden, c->experts) * 4);
   auto *head_work = KX_AT(int4 *, (size_t)c->heads * 16);
@@ -217,7 +217,7 @@ int layout(const kx_config *c, Plan &p, kx_model *m) {
   if (m) {
     m->x = x; m->n = n; m->qkv = qkv; m->qa = qa; m->q = q; m->o_lat = o_lat; m->att = att; m->dmid = dmid;
     m->qabs = qabs; m->partial = partial; m->logits = logits; m->argmax_scratch = argmax_scratch; m->ids = ids; m->next = next; m->history = history;
-    m->head_count = head_count; m->front_err = front_err; m->front_hand = front_hand; m->back_hand = back_hand; m->head_work = head_work; m->head_pairs = head_pairs;
+    m->head_count = head_count; m->hand_err = hand_err; m->front_hand = front_hand; m->back_hand = back_hand; m->head_work = head_work; m->head_pairs = head_pairs;
   }
   return KX_OK;
 }
@@ -335,7 +335,7 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample, int C = 1) {
     bool front = false;
     if (fuse && B == 1 && (m->fusion & KX_FUSE_FRONT)) {
       const uint32_t tag = m->front_tag % 65535u + 1u;
-      KX_TRY(kx_attn_front_launch(g, gb, qa, m->front_hand, tag, m->front_err, &front, st));
+      KX_TRY(kx_attn_front_launch(g, gb, qa, m->front_hand, tag, m->hand_err, &front, st));
       if (front) m->front_tag = tag;
     }
     if (!front) {
@@ -396,7 +396,7 @@ int step(kx_model *m, const uint32_t *d_ids, bool sample, int C = 1) {
         KxMoeHeadArgs hd;
         const bool want_head = l >= c.first_dense && (m->fusion & KX_FUSE_MOE_HEAD);
         if (want_head) kx_moe_head_args(&c, &L.moe, m->moe_ws, m->n, L.post_ln, &hd);
-        KX_TRY(kx_attn_back_launch(g, go, want_head ? &hd : nullptr, m->back_hand, tag, m->front_err, &back, &moe_head_done, st));
+        KX_TRY(kx_attn_back_launch(g, go, want_head ? &hd : nullptr, m->back_hand, tag, m->hand_err, &back, &moe_head_done, st));
         if (back) m->back_tag = tag;
       }
       if (!back) {
@@ -504,9 +504,9 @@ static int model_new(const kx_config *cfg, const char *who, kx_model **out) {
   for (auto &ev : m->ev)
     if (!rc && hipEventCreate(&ev) != hipSuccess) rc = KX_ERR_HIP;
   if (!rc && cfg->first_dense < cfg->n_layers) rc = kx_moe_workspace_create(cfg, step_tokens(cfg), &m->moe_ws);
-  if (!rc && m->moe_ws) kx_moe_workspace_set_err(m->moe_ws, m->front_err);
+  if (!rc && m->moe_ws) kx_moe_workspace_set_err(m->moe_ws, m->hand_err);
   if (!rc && (hipMemsetAsync(m->head_count, 0, (size_t)cfg->heads * 4, m->st) != hipSuccess ||
-              hipMemsetAsync(m->front_err, 0, 4, m->st) != hipSuccess ||
+              hipMemsetAsync(m->hand_err, 0, 4, m->st) != hipSuccess ||
               hipMemsetAsync(m->back_hand, 0, kx_back_hand_words(cfg->heads * cfg->v_head, cfg->hidden, cfg->experts) * 4, m->st) != hipSuccess ||
               hipMemsetAsync(m->front_hand, 0, kx_front_hand_words(cfg->q_rank, cfg->kv_rank + cfg->qk_rope, cfg->heads * (cfg->qk_nope + cfg->qk_rope)) * 4, m->st) != hipSuccess || hipStreamSynchronize(m->st) != hipSuccess))
     rc = KX_ERR_HIP;
@@ -628,7 +628,7 @@ static int check_ids(const kx_model *m, const uint32_t *ids, size_t n) {
 // launch of kx_i4.hip) that was given up: the steps since then computed with values that were not there yet.
 static int check_front(kx_model *m) {
   int flag = 0;
-  KX_HIP(hipMemcpyAsync(&flag, m->front_err, 4, hipMemcpyDeviceToHost, m->st));
+  KX_HIP(hipMemcpyAsync(&flag, m->hand_err, 4, hipMemcpyDeviceToHost, m->st));
   KX_HIP(hipStreamSynchronize(m->st));
   if (flag) {
     kx_set_error("kx_model: a workgroup of a resident launch gave up waiting for values from the others (not all workgroups of the launch "
@@ -774,7 +774,7 @@ extern "C" int kx_model_rewind(kx_model *m, int32_t positions) {
 extern "C" int kx_model_debug_fail_waits(kx_model *m) {
   KX_REQUIRE(m, "kx_model_debug_fail_waits: null model");
   const int one = 1;
-  KX_HIP(hipMemcpyAsync(m->front_err, &one, 4, hipMemcpyHostToDevice, m->st));
+  KX_HIP(hipMemcpyAsync(m->hand_err, &one, 4, hipMemcpyHostToDevice, m->st));
   KX_HIP(hipStreamSynchronize(m->st));
   return KX_OK;
 }
