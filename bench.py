@@ -63,6 +63,35 @@ def _profile_figure(path, key, kind):
     return None
 
 
+# The launches of one MoE layer of a batch-1 decode step: algorithmic bytes from the shapes, kernel time from the
+# committed `rocprofv3 --kernel-trace --stats` summary of the default run's batch-1 leg (a table row per kernel).
+STACK_PROFILE = "profiles/stack_decode.md"
+
+
+def stack_launches(args):
+    from blok_amd.lib import default_config
+    c = default_config()
+    H, qk, VD = c.hidden, c.qk_nope + c.qk_rope, c.heads * c.v_head
+    attn_front = 2 * ((c.q_rank + c.kv_rank + c.qk_rope) * H + c.heads * qk * c.q_rank + c.heads * c.qk_nope * c.kv_rank)
+    attn_back = 2 * (c.heads * c.v_head * c.kv_rank + H * VD)
+    head = 2 * (2 * c.shared_inter * H + c.experts * H)
+    routed = c.topk * 3 * (c.moe_inter * H // 2 + c.moe_inter * (H // 32) * 2) + 2 * H * c.shared_inter
+    rows = {"attn_front_k": attn_front, "attn_back_k<true>": attn_back + head, "i4_routed_shared_k": routed}
+    out = {}
+    try:
+        text = open(os.path.join(ROOT, STACK_PROFILE)).read()
+    except OSError:
+        return None
+    for name, nbytes in rows.items():
+        for line in text.splitlines():
+            cells = [x.strip() for x in line.split("|")]
+            if len(cells) > 3 and cells[1] == f"`{name}`":
+                us = float(cells[3])
+                out[name] = {"algorithmic_bytes": int(nbytes), "profile_avg_us": us,
+                             "frac_of_hbm_peak": round(nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)}
+    return dict(out, profile_from=STACK_PROFILE) if out else None
+
+
 def device_tokens(lib, n, seed, vocab):
     """n uniform-random token ids generated on the device (tensor id 4 of the seed) and copied back: what kx_prefill
     takes is a host array, as the reference's executor takes its prompt from argv."""
@@ -242,6 +271,7 @@ def run_moe_layer(args, emit=True):
                          f"(oracle mode 0), OpenMP over output rows, {dt:.1f} s"}
     check(lib.kx_moe_workspace_destroy(ws))
 
+    launches = stack_launches(args) if args.batch == 1 else None
     out = {
         "metric": "decode tok/s + INT4 expert GEMV HBM GB/s (% of peak), Kimi-K2 shapes, 1 GPU",
         "value": round(T / (ms_per_step * 1e-3), 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
@@ -447,6 +477,8 @@ def run_default(args):
         "stack": {k: stack[k] for k in ("wall_ms_per_step", "prefill_ms_per_token", "model_create_s", "stack_hbm", "last_ids")},
         "cpu_baseline": cpu,
     }
+    if launches:
+        out["stack"]["launches_per_moe_layer"] = launches
     for b, leg in stack["extra"].items():     # config 5 names batch 32 too: the same resident model, same prompt length
         out[f"stack_b{b}"] = {"tok_s": leg["value"], "ms_per_step": leg["ms_per_step"], "steps": args.steps, "warmup": args.warmup,
                               "prompt": args.prompt, "prefill": leg["prefill"], "prefill_ms_per_token": leg["prefill_ms_per_token"],
