@@ -366,6 +366,30 @@ def test_fused_and_separate_launches_agree(kxlib, ox, shape):
         assert (h1 == h0).all() and (l1 == l0).all() and (o1 == o0).all()
 
 
+def test_resident_launches_at_and_past_their_span_limit(kxlib, ox):
+    # The back launch of the attention block holds up to 32 span partials per thread.  With the bit-reproducible
+    # attention kernel kept at every length, positions 1985 .. 2048 are 32 spans -- the last the launch takes -- and from
+    # 2049 on there are 33 and the model goes back to the W_UV GEMV that merges while it loads.  A generation that
+    # crosses that line must equal, to the bit, the same generation with every step a launch of its own.
+    say("kimi shape 2-layer stack across 2048 positions: resident launches against separate ones")
+    cfg = default_config()
+    plen, n_tokens = 2030, 40
+    cfg.n_layers, cfg.first_dense, cfg.max_batch, cfg.max_context, cfg.seed = 2, 1, 1, plen + n_tokens, 13
+    prompt = O.tokens_u32(plen, cfg.seed, 4, cfg.vocab).reshape(1, plen)
+    got = []
+    for mask in (63, 3):
+        km = KxModel(kxlib, cfg)
+        check(kxlib.kx_model_set_fusion(km.h, mask))
+        check(kxlib.kx_model_set_attention_kernel(km.h, 1))     # KX_MLA_VALU at every length
+        rc, out, _ = km.generate(prompt, n_tokens)
+        assert rc == 0, kxlib.kx_last_error()
+        total = plen + n_tokens - 1
+        got.append((out.copy(), km.hidden(1), km.logits(1).view(np.uint32), km.latent(1, 0, total)))
+        km.close()
+    for a, b in zip(*got):
+        assert (a == b).all(), "the resident launches and the separate ones differ"
+
+
 @pytest.mark.parametrize("tokens", [1, 3, 9, 32, 70])
 def test_q_absorb_operator(kxlib, ox, tokens):
     # bf(W_UK^T q_nope): eight fp32 chains over d = j, j+8, ... summed ((0+1)+(2+3))+((4+5)+(6+7)) (bf16 products are
