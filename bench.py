@@ -271,7 +271,6 @@ def run_moe_layer(args, emit=True):
                          f"(oracle mode 0), OpenMP over output rows, {dt:.1f} s"}
     check(lib.kx_moe_workspace_destroy(ws))
 
-    launches = stack_launches(args) if args.batch == 1 else None
     out = {
         "metric": "decode tok/s + INT4 expert GEMV HBM GB/s (% of peak), Kimi-K2 shapes, 1 GPU",
         "value": round(T / (ms_per_step * 1e-3), 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
@@ -477,6 +476,7 @@ def run_default(args):
         "stack": {k: stack[k] for k in ("wall_ms_per_step", "prefill_ms_per_token", "model_create_s", "stack_hbm", "last_ids")},
         "cpu_baseline": cpu,
     }
+    launches = stack_launches(args) if args.batch == 1 else None
     if launches:
         out["stack"]["launches_per_moe_layer"] = launches
     for b, leg in stack["extra"].items():     # config 5 names batch 32 too: the same resident model, same prompt length

@@ -211,15 +211,21 @@ struct MlaArgs {
 // workgroup with coalesced 16-byte loads (row pitch 1168 B, so that both the row-per-lane reads
 // of the score pass and the column-per-lane reads of the PV pass are free of bank conflicts).
 constexpr int MLA_R = 512, MLA_KVA = 576, MLA_PITCH = 584;  // bf16 elements; 1168 B per staged row
+constexpr int MLA_PITCH_F = 580;  // F32: floats per staged row (2320 B: 580 mod 32 = 4, so eight rows' 16-byte reads cover all banks)
 
 // W waves per workgroup, HG heads per wave.  The waves of a workgroup share the staged tile; with W = 6 .. 8 (HG = 1)
 // the last workgroup of a span may hold waves past the last head: they stage and keep the barriers, and compute the
 // last head again without storing it.
-template <int HG, int W = 4>
+// F32 (launches of at most one workgroup per CU, which then has the LDS for it): the tile is staged as floats, the
+// bf16 -> f32 conversion done once by the threads that stage instead of by every wave on every read: half of a
+// wave's VALU work in both passes is that conversion, and the SIMDs that hold two waves are what the launch waits
+// for.  The values and the order of the sums are the same.
+template <int HG, int W = 4, bool F32 = false>
 __global__ void __launch_bounds__(W * 64) mla_partial_k(MlaArgs a) {
-  constexpr int R = MLA_R, KVA = MLA_KVA, PITCH = MLA_PITCH;
-  extern __shared__ __attribute__((aligned(16))) uint16_t tile_lds[];  // [64][PITCH] then p [W][HG][64] floats
-  float(*p_lds)[HG][64] = (float(*)[HG][64])(tile_lds + 64 * PITCH);
+  constexpr int R = MLA_R, KVA = MLA_KVA, PITCH = MLA_PITCH, PITCH_F = MLA_PITCH_F;
+  extern __shared__ __attribute__((aligned(16))) uint16_t tile_lds[];  // [64][PITCH] bf16 or [64][PITCH_F] floats, then p [W][HG][64] floats
+  float *tile_f = (float *)tile_lds;
+  float(*p_lds)[HG][64] = F32 ? (float(*)[HG][64])(tile_f + 64 * PITCH_F) : (float(*)[HG][64])(tile_lds + 64 * PITCH);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: q is then read through the scalar path
   const int span = blockIdx.x, b = blockIdx.z;
@@ -231,6 +237,9 @@ __global__ void __launch_bounds__(W * 64) mla_partial_k(MlaArgs a) {
   const float *q = a.qabs + ((size_t)b * a.heads + h0) * KVA;
   const int tiles = (seq + 63) >> 6;  // a span past them leaves M = -inf, Z = 0, O = 0, which the merge weighs with 0
   const int tile_end = min(tiles, (span + 1) * a.span_tiles);
+  // the lane's 8 latent columns in the PV pass: contiguous over the bf16 tile; two groups of four, 256 apart, over the
+  // float tile, so that a wave's reads of a row are two runs of 1 KB (each column's sum is its own chain either way)
+  const int pv_lo = F32 ? lane * 4 : lane * 8, pv_hi = F32 ? 256 + lane * 4 : lane * 8 + 4;
   float M[HG], Z[HG], O[HG][8];
 #pragma unroll
   for (int h = 0; h < HG; ++h) {
@@ -254,19 +263,37 @@ __global__ void __launch_bounds__(W * 64) mla_partial_k(MlaArgs a) {
 #pragma unroll
       for (int i = 0; i < NP; ++i) {
         const int idx = threadIdx.x + i * (W * 64), row = idx / 72, j = idx - row * 72;
-        if ((64 * 72) % (W * 64) == 0 || idx < 64 * 72) *(uint4 *)(tile_lds + row * PITCH + j * 8) = v[i];
+        if ((64 * 72) % (W * 64) == 0 || idx < 64 * 72) {
+          if (F32) {
+            float cf[8];
+            unpack8(cf, v[i]);
+            float4 *dst = (float4 *)(tile_f + row * PITCH_F + j * 8);
+            dst[0] = make_float4(cf[0], cf[1], cf[2], cf[3]);
+            dst[1] = make_float4(cf[4], cf[5], cf[6], cf[7]);
+          } else {
+            *(uint4 *)(tile_lds + row * PITCH + j * 8) = v[i];
+          }
+        }
       }
     }
     __syncthreads();
+    // 8 values of row r from column c_lo and (F32) c_hi on: a float4 each, so that 64 lanes read 1 KB in a row
+    auto tile8 = [&](float (&cf)[8], int r, int c_lo, int c_hi) {
+      if (F32) {
+        const float4 lo = *(const float4 *)(tile_f + r * PITCH_F + c_lo), hi = *(const float4 *)(tile_f + r * PITCH_F + c_hi);
+        cf[0] = lo.x; cf[1] = lo.y; cf[2] = lo.z; cf[3] = lo.w; cf[4] = hi.x; cf[5] = hi.y; cf[6] = hi.z; cf[7] = hi.w;
+      } else {
+        unpack8(cf, *(const uint4 *)(tile_lds + r * PITCH + c_lo));
+      }
+    };
     // scores: lane = position, one fma chain over the 576 columns per head
-    const uint16_t *row = tile_lds + lane * PITCH;
     float acc[HG];
 #pragma unroll
     for (int h = 0; h < HG; ++h) acc[h] = 0.0f;
 #pragma unroll 4
     for (int j = 0; j < KVA / 8; ++j) {
       float cf[8];
-      unpack8(cf, *(const uint4 *)(row + j * 8));
+      tile8(cf, lane, j * 8, j * 8 + 4);
 #pragma unroll
       for (int h = 0; h < HG; ++h) {
         const float *qh = q + h * KVA + j * 8;
@@ -290,17 +317,17 @@ __global__ void __launch_bounds__(W * 64) mla_partial_k(MlaArgs a) {
       M[h] = Mn;
       p_lds[wave][h][lane] = kx_bfround(p);
     }
-    // PV: lane = 8 latent columns, positions in order (p of this wave was written by this wave)
+    // PV: lane = 8 latent columns (pv_lo .. +3 and pv_hi .. +3 as floats, pv_lo .. +7 as bf16), positions in order (p of
+    // this wave was written by this wave)
 #pragma unroll
     for (int h = 0; h < HG; ++h)
 #pragma unroll
       for (int e = 0; e < 8; ++e) O[h][e] = O[h][e] * alpha[h];
     // all 64 rows: rows past the sequence are staged as zeros and carry p = 0, which leaves O unchanged
-    const uint16_t *col = tile_lds + lane * 8;
 #pragma unroll 8
     for (int t = 0; t < 64; ++t) {
       float cf[8];
-      unpack8(cf, *(const uint4 *)(col + t * PITCH));
+      tile8(cf, t, pv_lo, pv_hi);
 #pragma unroll
       for (int h = 0; h < HG; ++h) {
         const float p = p_lds[wave][h][t];
@@ -315,9 +342,8 @@ __global__ void __launch_bounds__(W * 64) mla_partial_k(MlaArgs a) {
     if (!h_valid) break;
     const size_t idx = ((size_t)b * a.spans + span) * a.heads + h0 + h;
     if (lane == 0) { a.pm[idx] = M[h]; a.pz[idx] = Z[h]; }
-    float4 *o = (float4 *)(a.po + idx * R + lane * 8);
-    o[0] = make_float4(O[h][0], O[h][1], O[h][2], O[h][3]);
-    o[1] = make_float4(O[h][4], O[h][5], O[h][6], O[h][7]);
+    *(float4 *)(a.po + idx * R + pv_lo) = make_float4(O[h][0], O[h][1], O[h][2], O[h][3]);
+    *(float4 *)(a.po + idx * R + pv_hi) = make_float4(O[h][4], O[h][5], O[h][6], O[h][7]);
   }
 }
 
@@ -770,7 +796,10 @@ int kx_mla_partials_launch(const kx_config *c, const uint16_t *cache, size_t seq
       if ((long)batch * a.spans * kx_cdiv(c->heads, w) <= mla_compute_units()) wv = w;
   }
   dim3 g(a.spans, kx_cdiv(c->heads, wv * hg), batch), b(wv * 64);
-  const size_t lds = (size_t)64 * MLA_PITCH * 2 + (size_t)wv * hg * 64 * sizeof(float);
+  // one workgroup per CU at most: the tile as floats (see the kernel)
+  const bool f32 = hg == 1 && !use_mfma && (long)g.x * g.y * g.z <= mla_compute_units();
+  const size_t lds = f32 ? (size_t)64 * MLA_PITCH_F * 4 + (size_t)wv * 64 * sizeof(float)
+                         : (size_t)64 * MLA_PITCH * 2 + (size_t)wv * hg * 64 * sizeof(float);
   static std::atomic<bool> attr_set{false};  // setting it twice from two threads is harmless
   if (!attr_set) {  // more than 64 KB of dynamic LDS has to be allowed per kernel
     KX_HIP(hipFuncSetAttribute((const void *)mla_partial_k<1>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
@@ -780,6 +809,10 @@ int kx_mla_partials_launch(const kx_config *c, const uint16_t *cache, size_t seq
     KX_HIP(hipFuncSetAttribute((const void *)mla_partial_k<2>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
     KX_HIP(hipFuncSetAttribute((const void *)mla_partial_k<4>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
     KX_HIP(hipFuncSetAttribute((const void *)mla_partial_k<8>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
+    KX_HIP(hipFuncSetAttribute((const void *)mla_partial_k<1, 4, true>, hipFuncAttributeMaxDynamicSharedMemorySize, 152 * 1024));
+    KX_HIP(hipFuncSetAttribute((const void *)mla_partial_k<1, 6, true>, hipFuncAttributeMaxDynamicSharedMemorySize, 152 * 1024));
+    KX_HIP(hipFuncSetAttribute((const void *)mla_partial_k<1, 7, true>, hipFuncAttributeMaxDynamicSharedMemorySize, 152 * 1024));
+    KX_HIP(hipFuncSetAttribute((const void *)mla_partial_k<1, 8, true>, hipFuncAttributeMaxDynamicSharedMemorySize, 152 * 1024));
     attr_set = true;
   }
   if (use_mfma) {
@@ -794,7 +827,11 @@ int kx_mla_partials_launch(const kx_config *c, const uint16_t *cache, size_t seq
     out->pm = a.pm; out->pz = a.pz; out->po = a.po; out->spans = a.spans;
     return KX_OK;
   }
-  if (hg == 1 && wv == 6) hipLaunchKernelGGL((mla_partial_k<1, 6>), g, b, lds, st, a);
+  if (f32 && wv == 4) hipLaunchKernelGGL((mla_partial_k<1, 4, true>), g, b, lds, st, a);
+  else if (f32 && wv == 6) hipLaunchKernelGGL((mla_partial_k<1, 6, true>), g, b, lds, st, a);
+  else if (f32 && wv == 7) hipLaunchKernelGGL((mla_partial_k<1, 7, true>), g, b, lds, st, a);
+  else if (f32 && wv == 8) hipLaunchKernelGGL((mla_partial_k<1, 8, true>), g, b, lds, st, a);
+  else if (hg == 1 && wv == 6) hipLaunchKernelGGL((mla_partial_k<1, 6>), g, b, lds, st, a);
   else if (hg == 1 && wv == 7) hipLaunchKernelGGL((mla_partial_k<1, 7>), g, b, lds, st, a);
   else if (hg == 1 && wv == 8) hipLaunchKernelGGL((mla_partial_k<1, 8>), g, b, lds, st, a);
   else if (hg == 1) hipLaunchKernelGGL(mla_partial_k<1>, g, b, lds, st, a);
