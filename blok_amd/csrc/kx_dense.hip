@@ -301,13 +301,32 @@ int kx_gemv_launch(int epi, KxGemvArgs a, hipStream_t st) {
   // 8 tokens and more against a matrix that stays in L2: the token blocks side by side (gemv_tokblk_k), all in one launch
   if (all_tokens >= 8 && all_tokens <= 4 * 65535 && (epi == KX_EPI_BF16 || epi == KX_EPI_F32) && !a.norm_w && !a.mla_po &&
       kx_cdiv(a.rows, CR) <= 4096 && (size_t)a.rows * a.cols * 2 <= (16u << 20)) {
-    // longer chunks, about 512 workgroups in all: a chunk's activations are read once, so rows per chunk divide the
-    // L2 traffic of the activations (one row per chunk: 57 KB of them against 14 KB of weights for the router)
+    // A CU holds one workgroup of this kernel, and a wave spends a load's latency on every tile it goes through: one
+    // round of workgroups (256 over the token blocks) and four rows per wave and tile, so that a chunk is a few steps
+    // with four rows in flight per lane.  Longer chunks also divide the L2 traffic of the activations, which a chunk
+    // reads once (one row per chunk: 57 KB of them against 14 KB of weights for the router).  The router at 32
+    // tokens: 32 chunks of 12 rows in three steps per token block instead of 64 chunks of 6 rows in six steps and two
+    // rounds.
     const int blocks = kx_cdiv(all_tokens, 4);
     KxGemvArgs b = a;
     int ri4;
-    const int CR4 = gemv_plan(epi, b, ri4, 4, 512 / blocks > 32 ? 512 / blocks : 32);
+    int CR4 = gemv_plan(epi, b, ri4, 4, 512 / blocks > 32 ? 512 / blocks : 32);
     if (CR4 < 0) return KX_ERR_ARG;
+    {
+      int r4 = 4;
+      while (r4 > 1 && (r4 * b.rs > a.rows || (a.row_block && a.row_block % (r4 * b.rs)))) r4 >>= 1;
+      const int rt = r4 * b.rs;
+      const int per_block = 256 / blocks > 1 ? 256 / blocks : 1;
+      int nt = kx_cdiv(kx_cdiv(a.rows, per_block), rt);
+      nt = nt < 1 ? 1 : nt > 8 ? 8 : nt;
+      if (a.row_block && a.row_block % rt == 0)
+        while (a.row_block % (rt * nt)) --nt;
+      if (rt * nt <= a.rows && (!a.row_block || a.row_block % rt == 0) && (size_t)rt * nt * 4 * S * sizeof(float) <= 64 * 1024) {
+        ri4 = r4;
+        b.nt = nt;
+        CR4 = rt * nt;
+      }
+    }
     const size_t lds4 = (size_t)CR4 * 4 * S * sizeof(float);
     KX_REQUIRE(lds4 <= 64 * 1024, "kx_gemv: %zu bytes of LDS needed", lds4);
     const dim3 g(kx_cdiv(a.rows, CR4), blocks), blk(b.nw * b.rs * 64);

@@ -222,18 +222,18 @@ extern "C" int kx_bucket(const void *d_ids, int32_t tokens, int32_t experts, int
                           (int *)d_pairs, (int4 *)d_work, (int *)d_n_active, kx_stream(stream), nullptr);
 }
 
-// top-k and bucketing; one launch when the tokens fit one workgroup (16 waves), two otherwise
+// top-k and bucketing; one launch up to 32 tokens (one workgroup of up to 16 waves, each taking tokens in turn), two otherwise
 int kx_route_launch(const float *logits, const float *bias, uint16_t *ids, float *weights, int tokens, int experts,
                     int topk, float routed_scale, int *counts, int *offsets, int *pairs, int4 *work, int *n_active,
                     hipStream_t st, int4 *pair_work) {
-  if (tokens > 16 || experts > 1024) {
+  if (tokens > 32 || experts > 1024 || (long)tokens * topk > 1024) {
     int rc = kx_router_topk_launch(logits, bias, ids, weights, tokens, experts, topk, routed_scale, st);
     if (rc) return rc;
     return kx_bucket_launch(ids, tokens, experts, topk, counts, offsets, pairs, work, n_active, st, pair_work);
   }
   KX_REQUIRE(tokens > 0 && experts > 0 && topk > 0 && topk <= 64 && topk <= experts, "kx_route: tokens=%d experts=%d topk=%d", tokens, experts, topk);
   int threads = kx_cdiv(experts, 64) * 64;
-  if (threads < tokens * 64) threads = tokens * 64;
+  if (threads < tokens * 64) threads = tokens * 64 < 1024 ? tokens * 64 : 1024;
   const size_t lds = (size_t)kx_cdiv(tokens * topk, 8) * 16;
   const int epl = kx_cdiv(experts, 64);
 #define KX_TB(N) hipLaunchKernelGGL(topk_bucket_k<N>, dim3(1), dim3(threads), lds, st, logits, bias, ids, weights, tokens, experts, topk, routed_scale, counts, offsets, pairs, work, n_active, pair_work)

@@ -40,6 +40,8 @@ def test_rmsnorm_parity(kxlib, ox, n, tokens):
     (40, 18432, 2, 0),      # dense down width (three slices per wave)
     (96, 2048, 5, 0),
     (384, 7168, 32, 1),     # 8 tokens and more against a small matrix: token blocks side by side in the grid
+    (384, 7168, 16, 1),
+    (8192, 512, 32, 0),     # 32 chunks of 256 rows per token block
     (1000, 1536, 13, 0),    # the same, ragged rows and a ragged last token block
     (2048, 512, 9, 0),
     (384, 1024, 70, 1),     # more than 32 tokens: still one launch
