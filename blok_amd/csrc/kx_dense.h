@@ -97,6 +97,12 @@ int kx_router_topk_launch(const float *logits, const float *bias, uint16_t *ids,
 int kx_gemv_pair_route_launch(KxGemvArgs shared_gate_up, KxGemvArgs router, const float *bias, uint16_t *ids, float *weights,
                               int experts, int topk, float routed_scale, int *counts, int *offsets, int *pairs, int4 *work,
                               int *n_active, int *counter, bool *fused, hipStream_t st, int4 *pair_work = nullptr);
+// The router's logits GEMV (fp32 epilogue) of any number of tokens.  From 8 to 32 tokens the launch also does the
+// routing -- *routed = true; counters: 1 + ceil(tokens / 4) ints, zero before the call and left at zero --, otherwise
+// kx_route_launch follows.
+int kx_gemv_route_launch(KxGemvArgs router, const float *bias, uint16_t *ids, float *weights, int experts, int topk,
+                         float routed_scale, int *counts, int *offsets, int *pairs, int4 *work, int *n_active, int *counters,
+                         bool *routed, hipStream_t st, int4 *pair_work = nullptr);
 int kx_route_launch(const float *logits, const float *bias, uint16_t *ids, float *weights, int tokens, int experts,
                     int topk, float routed_scale, int *counts, int *offsets, int *pairs, int4 *work, int *n_active,
                     hipStream_t st, int4 *pair_work = nullptr);

@@ -100,6 +100,46 @@ struct KxRouteArgs {
   int *n_active;
   int4 *pair_work;  // optional second work list, one record per pair
 };
+// gemv_tokblk_k for the router's logits of 8 to 32 tokens that also routes them, in two steps of "the last one in
+// finishes the job": the workgroup that completes a block of four tokens does their top-k (a wave per token), and
+// the one of those that comes last buckets all tokens (kxr::bucket_masks).  r.counter: 1 + gridDim.y ints, zero
+// before the launch and left at zero.
+template <int RI>
+__global__ void __launch_bounds__(512) gemv_tokblk_route_k(KxGemvArgs a, KxRouteArgs r) {
+  extern __shared__ float part[];
+  __shared__ int s_last;
+  __shared__ int s_mask[512];
+  __shared__ int s_pos[512];
+  __shared__ uint16_t s_ids[1024];
+  const int tokens = a.tokens, t0 = blockIdx.y * 4, nt = min(4, tokens - t0);
+  const float *logits = (const float *)a.out + (size_t)t0 * a.out_stride;
+  const int stride = a.out_stride;
+  a.x += (size_t)t0 * a.x_stride;
+  a.out = (float *)a.out + (size_t)t0 * a.out_stride;
+  a.tokens = nt;
+  gemv_body<1, RI, 4>(a, blockIdx.x, gridDim.x, part);
+  kx_arrive_writes_done();
+  __syncthreads();
+  if (threadIdx.x == 0) s_last = kx_arrive_is_last(r.counter + 1 + blockIdx.y, gridDim.x);
+  __syncthreads();
+  if (!s_last) return;
+  const int wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+  for (int t = wave; t < nt; t += waves)
+    kxr::topk_token_any<true, true>(logits + (size_t)t * stride, r.bias, r.ids + (size_t)(t0 + t) * r.topk,
+                                    r.weights + (size_t)(t0 + t) * r.topk, r.experts, r.topk, r.routed_scale, threadIdx.x & 63);
+  if (threadIdx.x == 0) kx_arrive_reset(r.counter + 1 + blockIdx.y);
+  kx_arrive_writes_done();
+  __syncthreads();  // also: every thread has read s_last before it is written again
+  if (threadIdx.x == 0) s_last = kx_arrive_is_last(r.counter, gridDim.y);
+  __syncthreads();
+  if (!s_last) return;
+  const int n_pairs = tokens * r.topk;
+  for (int p = threadIdx.x; p < n_pairs; p += blockDim.x) s_ids[p] = kx_arrive_load(r.ids + p);
+  __syncthreads();
+  kxr::bucket_masks(s_ids, tokens, r.topk, r.experts, r.counts, r.offsets, r.pairs, r.work, r.n_active, s_mask, s_pos, r.pair_work);
+  if (threadIdx.x == 0) kx_arrive_reset(r.counter);
+}
+
 template <int RI0, int RI1, int TT>
 __global__ void __launch_bounds__(TT > 1 ? 512 : 1024) gemv_pair_k(KxGemvArgs a0, KxGemvArgs a1, int n0, KxRouteArgs r) {
   extern __shared__ float part[];
@@ -288,7 +328,8 @@ int gemv_plan(int epi, KxGemvArgs &a, int &ri, int ri_max, int target_chunks = 2
 int kx_gemv_plan(int epi, KxGemvArgs &a, int *ri) { return gemv_plan(epi, a, *ri, 4); }
 
 // Tokens are taken in blocks of at most 32 (LDS holds a partial per token and slice).
-int kx_gemv_launch(int epi, KxGemvArgs a, hipStream_t st) {
+// route, routed: the router's logits; *routed says whether the launch has also done the routing (gemv_tokblk_route_k)
+static int gemv_launch_impl(int epi, KxGemvArgs a, hipStream_t st, const KxRouteArgs *route, bool *routed) {
   int ri;
   const int CR = gemv_plan(epi, a, ri, 4);
   if (CR < 0) return KX_ERR_ARG;
@@ -330,6 +371,17 @@ int kx_gemv_launch(int epi, KxGemvArgs a, hipStream_t st) {
     const size_t lds4 = (size_t)CR4 * 4 * S * sizeof(float);
     KX_REQUIRE(lds4 <= 64 * 1024, "kx_gemv: %zu bytes of LDS needed", lds4);
     const dim3 g(kx_cdiv(a.rows, CR4), blocks), blk(b.nw * b.rs * 64);
+    const int threads = b.nw * b.rs * 64;
+    if (route && epi == KX_EPI_F32 && all_tokens <= 32 && route->experts == a.rows && route->experts <= threads && threads <= 512 &&
+        all_tokens * route->topk <= 1024 && route->topk <= 64 && route->topk <= route->experts && a.out_stride >= a.rows) {
+      b.flags |= KX_GEMV_COHERENT_OUT;
+      if (ri4 == 4) hipLaunchKernelGGL(gemv_tokblk_route_k<4>, g, blk, lds4, st, b, *route);
+      else if (ri4 == 2) hipLaunchKernelGGL(gemv_tokblk_route_k<2>, g, blk, lds4, st, b, *route);
+      else hipLaunchKernelGGL(gemv_tokblk_route_k<1>, g, blk, lds4, st, b, *route);
+      KX_LAUNCH_CHECK();
+      *routed = true;
+      return KX_OK;
+    }
     if (ri4 == 4) hipLaunchKernelGGL(gemv_tokblk_k<4>, g, blk, lds4, st, b);
     else if (ri4 == 2) hipLaunchKernelGGL(gemv_tokblk_k<2>, g, blk, lds4, st, b);
     else hipLaunchKernelGGL(gemv_tokblk_k<1>, g, blk, lds4, st, b);
@@ -355,6 +407,19 @@ int kx_gemv_launch(int epi, KxGemvArgs a, hipStream_t st) {
     KX_LAUNCH_CHECK();
   }
   return KX_OK;
+}
+
+int kx_gemv_launch(int epi, KxGemvArgs a, hipStream_t st) { return gemv_launch_impl(epi, a, st, nullptr, nullptr); }
+
+int kx_gemv_route_launch(KxGemvArgs router, const float *bias, uint16_t *ids, float *weights, int experts, int topk,
+                         float routed_scale, int *counts, int *offsets, int *pairs, int4 *work, int *n_active, int *counters,
+                         bool *routed, hipStream_t st, int4 *pair_work) {
+  KxRouteArgs r;
+  r.counter = counters; r.bias = bias; r.ids = ids; r.weights = weights; r.experts = experts; r.topk = topk;
+  r.routed_scale = routed_scale; r.counts = counts; r.offsets = offsets; r.pairs = pairs; r.work = work; r.n_active = n_active;
+  r.pair_work = pair_work;
+  *routed = false;
+  return gemv_launch_impl(KX_EPI_F32, router, st, &r, routed);
 }
 
 // The shared expert's gate/up GEMV (SwiGLU epilogue) and the router's logits GEMV in one launch,

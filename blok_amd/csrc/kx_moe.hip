@@ -35,7 +35,7 @@ struct kx_moe_workspace {
   int4 *work;         // [E] {expert, first, last, first pair}
   int4 *pair_work;    // [T*topk] one record per pair {expert, q, q + 1, pairs[q]}
   int *n_active;      // [1]
-  int *route_counter; // [1] zero between launches: workgroups of the router GEMV count themselves in
+  int *route_counter; // [10] zero between launches: workgroups of the router GEMV count themselves in (one counter, or one and one per block of four tokens)
   int *tail_count;    // [KX_TAIL_BLOCKS] zero between launches: arrivals per block of output rows (routed down + shared down)
   uint16_t *mid;      // [T*topk, moe_inter]
   uint16_t *eout;     // [T*topk, hidden]
@@ -74,7 +74,7 @@ extern "C" int kx_moe_workspace_create(const kx_config *cfg, int32_t max_tokens,
   struct { void **p; size_t bytes; } allocs[] = {
       {(void **)&ws->logits, T * E * 4}, {(void **)&ws->ids, T * K * 2}, {(void **)&ws->weights, T * K * 4},
       {(void **)&ws->counts, E * 4}, {(void **)&ws->offsets, (E + 1) * 4}, {(void **)&ws->pairs, T * K * 4},
-      {(void **)&ws->work, E * 16}, {(void **)&ws->pair_work, T * K * 16}, {(void **)&ws->n_active, 8}, {(void **)&ws->tail_count, KX_TAIL_BLOCKS * 4},
+      {(void **)&ws->work, E * 16}, {(void **)&ws->pair_work, T * K * 16}, {(void **)&ws->n_active, 64}, {(void **)&ws->tail_count, KX_TAIL_BLOCKS * 4},
       {(void **)&ws->mid, T * K * (size_t)cfg->moe_inter * 2}, {(void **)&ws->eout, T * K * (size_t)cfg->hidden * 2},
       {(void **)&ws->smid, T * (size_t)cfg->shared_inter * 2}, {(void **)&ws->sy, T * (size_t)cfg->hidden * 2},
       {(void **)&ws->mid_hand, K * (size_t)cfg->moe_inter * 4}};
@@ -91,7 +91,7 @@ extern "C" int kx_moe_workspace_create(const kx_config *cfg, int32_t max_tokens,
   // tokens than the last one had, then does nothing instead of following uninitialised records
   hipError_t e = hipMemset(ws->work, 0xff, E * 16);
   if (e == hipSuccess) e = hipMemset(ws->pair_work, 0xff, T * K * 16);
-  if (e == hipSuccess) e = hipMemset(ws->n_active, 0, 8);
+  if (e == hipSuccess) e = hipMemset(ws->n_active, 0, 64);
   if (e == hipSuccess) e = hipMemset(ws->tail_count, 0, KX_TAIL_BLOCKS * 4);
   if (e == hipSuccess) e = hipMemset(ws->mid_hand, 0, K * (size_t)cfg->moe_inter * 4);
   for (auto &ev : ws->ev)
@@ -275,8 +275,11 @@ static int moe_layer_body(const kx_config *c, const kx_moe_weights *w, kx_moe_wo
                                       ws->counts, ws->offsets, ws->pairs, ws->work, ws->n_active, ws->route_counter, &paired,
                                       st, routed_per_pair(tokens, K, E) ? ws->pair_work : nullptr))) return rc;
   if (!paired) {
-    if ((rc = kx_gemv_launch(KX_EPI_F32, g, st))) return rc;
-    if ((rc = kx_route_launch(ws->logits, (const float *)w->d_router_bias, ws->ids, ws->weights, tokens, E, K, c->routed_scale,
+    bool routed = false;
+    if ((rc = kx_gemv_route_launch(g, (const float *)w->d_router_bias, ws->ids, ws->weights, E, K, c->routed_scale, ws->counts,
+                                   ws->offsets, ws->pairs, ws->work, ws->n_active, ws->route_counter, &routed, st,
+                                   routed_per_pair(tokens, K, E) ? ws->pair_work : nullptr))) return rc;
+    if (!routed && (rc = kx_route_launch(ws->logits, (const float *)w->d_router_bias, ws->ids, ws->weights, tokens, E, K, c->routed_scale,
                               ws->counts, ws->offsets, ws->pairs, ws->work, ws->n_active, st,
                               routed_per_pair(tokens, K, E) ? ws->pair_work : nullptr))) return rc;
   }

@@ -12,8 +12,9 @@ namespace kxr {
 using kxw::wave_max_f32;
 using kxw::wave_min_i32;
 
-// top-k of one token by one wave; lane owns experts lane, lane+64, ... (EPL of them)
-template <int EPL, bool COHERENT = false>
+// top-k of one token by one wave; lane owns experts lane, lane+64, ... (EPL of them).  COHERENT: the logits were
+// written by other workgroups of the launch; HAND_IDS: the ids are read by another workgroup of the launch
+template <int EPL, bool COHERENT = false, bool HAND_IDS = false>
 __device__ __forceinline__ void topk_token(const float *lg, const float *__restrict__ bias,
                                            uint16_t *__restrict__ ids, float *__restrict__ weights, int E, int topk,
                                            float routed_scale, int lane, uint16_t *s_ids = nullptr) {
@@ -52,11 +53,26 @@ __device__ __forceinline__ void topk_token(const float *lg, const float *__restr
     sum += s_win;
     if (lane == k) my_w = s_win;
     if (lane == 0) {
-      ids[k] = (uint16_t)win;
+      if (HAND_IDS) kx_arrive_store(ids + k, (uint16_t)win);
+      else ids[k] = (uint16_t)win;
       if (s_ids) s_ids[k] = (uint16_t)win;
     }
   }
   if (lane < topk) weights[lane] = my_w / (sum + 1.0e-20f) * routed_scale;
+}
+
+// topk_token with the per-lane expert count chosen at run time (up to 512 experts)
+template <bool COHERENT, bool HAND_IDS>
+__device__ __forceinline__ void topk_token_any(const float *lg, const float *bias, uint16_t *ids, float *weights, int E,
+                                               int topk, float routed_scale, int lane) {
+  const int epl = (E + 63) >> 6;
+#define KX_TK(N) topk_token<N, COHERENT, HAND_IDS>(lg, bias, ids, weights, E, topk, routed_scale, lane)
+  if (epl <= 1) KX_TK(1);
+  else if (epl <= 2) KX_TK(2);
+  else if (epl <= 4) KX_TK(4);
+  else if (epl <= 6) KX_TK(6);
+  else KX_TK(8);
+#undef KX_TK
 }
 
 // one workgroup, thread e owns expert e: count, exclusive scan, stable placement.
@@ -151,9 +167,74 @@ __device__ __forceinline__ void bucket_block(const uint16_t *__restrict__ ids, i
   }
 }
 
+// Bucketing of up to 32 tokens whose ids are distinct within a token (what the top-k gives): one bit per expert and
+// token, so an expert's count and a pair's place among its expert's pairs are population counts, and no thread goes
+// over all pairs (bucket_block at 256 pairs: 15 us of the 384 threads each scanning them twice).  The results are
+// bucket_block's.  A workgroup of at least E threads, a multiple of 64 and at most 1024; s_mask and s_pos: E ints each.
+__device__ __forceinline__ void bucket_masks(const uint16_t *s_ids, int tokens, int topk, int E, int *__restrict__ counts,
+                                             int *__restrict__ offsets, int *__restrict__ pairs, int4 *__restrict__ work,
+                                             int *__restrict__ n_active, int *s_mask, int *s_pos,
+                                             int4 *__restrict__ pair_work) {
+  __shared__ int s_wave[2][16];
+  const int tid = threadIdx.x, n = blockDim.x, n_pairs = tokens * topk;
+  for (int e = tid; e < E; e += n) s_mask[e] = 0;
+  __syncthreads();
+  for (int p = tid; p < n_pairs; p += n) atomicOr((unsigned *)&s_mask[s_ids[p]], 1u << (p / topk));
+  __syncthreads();
+  const unsigned m = tid < E ? (unsigned)s_mask[tid] : 0u;
+  const int cnt = __popc(m), act = cnt > 0 ? 1 : 0;
+  // exclusive scans of counts and of the experts with work: inside the wave by shuffles, across the waves by their totals
+  int sc = cnt, sa = act;
+  const int lane = tid & 63, wave = tid >> 6, waves = n >> 6;
+  for (int d = 1; d < 64; d <<= 1) {
+    const int a = __shfl_up(sc, d), b = __shfl_up(sa, d);
+    if (lane >= d) {
+      sc += a;
+      sa += b;
+    }
+  }
+  if (lane == 63) {
+    s_wave[0][wave] = sc;
+    s_wave[1][wave] = sa;
+  }
+  __syncthreads();
+  int base_c = 0, base_a = 0, total = 0, total_active = 0;
+  for (int w = 0; w < waves; ++w) {
+    const int c = s_wave[0][w], a = s_wave[1][w];
+    if (w < wave) {
+      base_c += c;
+      base_a += a;
+    }
+    total += c;
+    total_active += a;
+  }
+  const int off = base_c + sc - cnt, slot = base_a + sa - act;
+  if (tid < E) {
+    counts[tid] = cnt;
+    offsets[tid] = off;
+    s_pos[tid] = off | (slot << 16);
+    if (tid >= total_active) work[tid] = make_int4(-1, 0, 0, 0);
+  }
+  if (tid == 0) {
+    offsets[E] = total;
+    *n_active = total_active;
+  }
+  __syncthreads();
+  for (int p = tid; p < n_pairs; p += n) {
+    const int id = s_ids[p], t = p / topk;
+    const unsigned mm = (unsigned)s_mask[id];
+    const int rank = __popc(mm & ((1u << t) - 1u));
+    const int po = s_pos[id], o = po & 0xffff, pos = o + rank;
+    pairs[pos] = p;
+    if (pair_work) pair_work[pos] = make_int4(id, pos, pos + 1, p);
+    if (rank == 0) work[po >> 16] = make_int4(id, o, o + __popc(mm), p);
+  }
+}
+
 // top-k of `tokens` tokens (wave w takes tokens w, w + waves, ...), then the bucketing, by one workgroup
 // of at least E threads.  s_ids4 holds ceil(tokens * topk / 8) pieces; s_cnt and s_act blockDim ints each.
-template <int EPL, bool COHERENT = false>
+// MASKS: more than 64 pairs of up to 32 tokens are bucketed by bucket_masks.
+template <int EPL, bool COHERENT = false, bool MASKS = false>
 __device__ __forceinline__ void route_block(const float *__restrict__ logits, const float *__restrict__ bias,
                                             uint16_t *__restrict__ ids, float *__restrict__ weights, int tokens, int E,
                                             int topk, float routed_scale, int *__restrict__ counts,
@@ -168,7 +249,10 @@ __device__ __forceinline__ void route_block(const float *__restrict__ logits, co
     topk_token<EPL, COHERENT>(logits + (size_t)t * E, bias, ids + (size_t)t * topk, weights + (size_t)t * topk, E, topk,
                               routed_scale, threadIdx.x & 63, s_ids + t * topk);
   __syncthreads();
-  bucket_block(ids, n_pairs, E, counts, offsets, pairs, work, n_active, s_ids4, s_cnt, s_act, true, pair_work);
+  if (MASKS && n_pairs > 64 && tokens <= 32 && n_pairs < 65536 && (blockDim.x & 63) == 0)
+    bucket_masks(s_ids, tokens, topk, E, counts, offsets, pairs, work, n_active, s_cnt, s_act, pair_work);
+  else
+    bucket_block(ids, n_pairs, E, counts, offsets, pairs, work, n_active, s_ids4, s_cnt, s_act, true, pair_work);
 }
 
 // route_block with the per-lane expert count chosen at run time; COHERENT: the logits were written by other

@@ -53,7 +53,7 @@ __global__ void __launch_bounds__(1024) topk_bucket_k(const float *__restrict__ 
   extern __shared__ uint4 s_ids4[];
   __shared__ int s_cnt[1024];
   __shared__ int s_act[1024];
-  kxr::route_block<EPL>(logits, bias, ids, weights, tokens, E, topk, routed_scale, counts, offsets, pairs, work, n_active,
+  kxr::route_block<EPL, false, true>(logits, bias, ids, weights, tokens, E, topk, routed_scale, counts, offsets, pairs, work, n_active,
                         s_ids4, s_cnt, s_act, pair_work);
 }
 

@@ -108,6 +108,15 @@ def _run_layer(kxlib, ox, H, I, SI, E, K, T, seed, flags=0, gpu_flags=0, mode0_t
     got["weights"] = grab(views[2], np.float32, (T, K))
     got["mid"] = grab(views[6], np.uint16, (T * K, I))
     got["eout"] = grab(views[7], np.uint16, (T * K, H))
+    # the bucketing the layer's own routing launch did (for up to 32 tokens with more than 64 pairs: by bit masks per
+    # expert), against the oracle's on the same ids
+    counts, offsets, pairs = np.empty(E, np.int32), np.empty(E + 1, np.int32), np.empty(T * K, np.int32)
+    active = np.empty(E, np.int32)
+    ids = np.ascontiguousarray(got["ids"])
+    ox.ox_bucket(ptr(ids), T, E, K, ptr(counts), ptr(offsets), ptr(pairs), ptr(active))
+    assert (grab(views[3], np.int32, (E,)) == counts).all(), "expert counts of the layer's routing differ"
+    assert (grab(views[4], np.int32, (E + 1,)) == offsets).all(), "expert offsets of the layer's routing differ"
+    assert (grab(views[5], np.int32, (T * K,)) == pairs).all(), "sorted pairs of the layer's routing differ"
     tmp.ptr = None
     check(kxlib.kx_moe_workspace_destroy(ws))
     exp = {}
@@ -157,7 +166,7 @@ def _assert_layer(got, exp):
     assert max(errs[0], errs[2]) < 1e-2 and max(errs[1], errs[3]) < 2e-2
 
 
-@pytest.mark.parametrize("T", [1, 8, 64])
+@pytest.mark.parametrize("T", [1, 8, 23, 32, 64])
 def test_moe_layer_small_shape(kxlib, ox, T):
     say(f"moe layer small T={T}")
     got, exp = _run_layer(kxlib, ox, 1024, 1024, 512, 32, 4, T, 7)
