@@ -365,36 +365,44 @@ __global__ void __launch_bounds__(W * 64) mla_partial_k(MlaArgs a) {
 
 // ---- the same partials on the matrix cores, for long contexts -----------------------------------
 // q_abs and p = bf(exp(s - m)) are bf16-representable and the cache is bf16, so q.c and p.c are exact
-// products summed in fp32: v_mfma_f32_16x16x32_bf16 computes what mla_partial_k computes with another
+// products summed in fp32: v_mfma_f32_32x32x16_bf16 computes what mla_partial_k computes with another
 // summation order (held to the 1e-2 bar, not bit-exact; the token-identity runs use mla_partial_k).
-// Workgroup = (sequence, span), 8 waves, 32-position tiles staged in LDS at their natural layout; the two
-// products split the work differently and hand p, the running-maximum factor and the row sums over through LDS:
-//  * scores: wave (hw, pb) computes heads 16 hw .. +15 against positions 16 pb .. +15 of the tile,
-//    S^T[pos, head] = C[pos, 576] Q^T[576, head] with v_mfma_f32_16x16x32_bf16 (A = cache rows from LDS, B = the
-//    lane's head of q in registers, 18 K steps); the two waves of a head group exchange their maxima, then each
-//    writes p = bf(exp(s - m)) of its 16 positions at the K indices the second product reads them from;
-//  * O^T[col, head] += C^T[col, pos] P^T[pos, head]: wave (hb, cq) owns heads 32 hb .. +31 and latent columns
-//    128 cq .. +127 (v_mfma_f32_32x32x16_bf16, two K steps per tile).  The A operand needs 8 positions of one
-//    column; ds_read_b64_tr_b16 delivers them from the row-major tile: within 16 lanes, lane i points at four
-//    consecutive columns of row i / 4, and lane j receives column j of the four rows;
-//  * the loop is software-pipelined: between two barriers a wave issues the second product of tile t-1 and the
-//    scores of tile t (independent MFMA chains, interleaved), then the maxima are exchanged, and after the
-//    second barrier the exponentials and p of tile t are written.  Two barriers per tile;
-//  * the 32 cache rows of tile t+2 are copied global -> LDS (no registers) while tile t is computed, into a ring
-//    of four buffers (tile t-1 is still read by the second product); rows sit at their natural pitch of 1152 B
-//    with the 16-byte pieces xor-swizzled by the row, so the row-per-lane operand reads of the scores are free
-//    of bank conflicts, and a transposing read touches rows that differ in bit 3 of the position in its two
-//    lane halves, which spreads it over all banks.
+// Workgroup = (sequence, span), 8 waves, 32-position tiles staged in LDS at their natural layout.  The two products
+// run on different waves: waves 0-3 compute the scores of tile t, waves 4-7 the second product of tile t-1, and every
+// SIMD holds one wave of each kind, so the matrix cores are fed from one wave while the other exponentiates, reads
+// its operands or waits at a barrier:
+//  * scores: wave (hb, kh) computes S^T[32 positions, heads 32 hb .. +31] over K steps 18 kh .. +17 of the 36 with
+//    v_mfma_f32_32x32x16_bf16 (A = the 32 cache rows of the tile, one row per lane and 16-byte piece 2 ks + half;
+//    B = the lane's head of q).  Every operand row is read by two waves.  Wave kh then takes heads 16 kh .. +15 of
+//    the block: the sums of the other 16 heads go to the other wave through LDS, and the lanes that held them take
+//    over half the positions of the wave's own heads, so all 32 positions of a head sit in four lanes of one wave:
+//    maximum, exponentials, row sum and the running sum Z need no exchange between waves.  The wave writes
+//    p = bf(exp(s - m)) at the K indices the second product reads them from, and exp(M_old - M_new);
+//  * O^T[col, head] += C^T[col, pos] P^T[pos, head]: wave cq owns latent columns 128 cq .. +127 for all 64 heads
+//    (two K steps per tile).  The A operand needs 8 positions of one column; ds_read_b64_tr_b16 delivers them from
+//    the row-major tile: within 16 lanes, lane i points at four consecutive columns of row i / 4, and lane j
+//    receives column j of the four rows.  The transposed reads of a tile are done once per column block and used
+//    for both head blocks;
+//  * two barriers per tile: behind the first, tile t has landed and p and the factors of tile t-1 are complete;
+//    behind the second, the score sums are visible, and p and the operands of tile t-1 are in the registers of the
+//    waves that use them: its ring buffer is free;
+//  * the 32 cache rows of a tile are copied global -> LDS (no registers) by the waves of the second product, which
+//    have the time, three tiles ahead into a ring of four buffers; rows sit at their natural pitch of 1152 B with
+//    the 16-byte pieces xor-swizzled by the row, so the row-per-lane operand reads of the scores are free of bank
+//    conflicts (counted: none), and a transposing read touches rows that differ in bit 3 of the position in its
+//    two lane halves, which spreads it over all banks.
+// An earlier form had all eight waves do both products (scores as 16 x 16 blocks, four waves reading every
+// operand row, the maxima exchanged between waves): 0.54-0.55 ms against 0.52 ms at 16 sequences of 131072
+// positions, 56 against 49 us at 32 sequences of 4096.
 constexpr int MM_T = 32;                      // positions per tile
 constexpr int MM_NAT = MM_T * MLA_KVA * 2;    // bytes of one staged tile
 constexpr int MM_RING = 4;
 constexpr int MM_P_PITCH = 80;                // bytes per head of the staged probabilities: 32 positions + pad
-constexpr int MM_LDS = MM_RING * MM_NAT;  // dynamic part: the tile ring
+constexpr int MM_LDS = MM_RING * MM_NAT;     // dynamic part: the tile ring
 typedef float kx_f32x16v __attribute__((ext_vector_type(16)));
 typedef __bf16 kx_bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 kx_bf16x2v __attribute__((ext_vector_type(2)));
 typedef float kx_f32x2v __attribute__((ext_vector_type(2)));
-typedef float kx_f32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 kx_bf16x4t;
 // two f32 -> packed bf16 pair, round to nearest even (v_cvt_pk_bf16_f32; the same values as kx_bf16_rne for finite inputs)
 __device__ __forceinline__ uint32_t mm_pack_bf16(float lo, float hi) {
@@ -412,25 +420,18 @@ __device__ __forceinline__ void mm_copy16_to_lds(const void *src, uint32_t lds_b
 __device__ __forceinline__ void mm_barrier() { kx_lds_barrier(); }
 
 __global__ void __launch_bounds__(512, 1) mla_partial_mfma_k(MlaArgs a) {
-  // the tile ring is the dynamic LDS; what the waves exchange lives in separate objects, so that the compiler can
-  // tell a store to them from the global -> LDS copies in flight (it would wait for those before the store)
   extern __shared__ __attribute__((aligned(128))) uint8_t mm_lds[];
   uint8_t *nat = mm_lds;                       // [4][32 rows][72 pieces of 16 B]
-  __shared__ __attribute__((aligned(16))) uint8_t p_lds[64 * MM_P_PITCH];  // [64 heads]: bf16 p by position
-  __shared__ float mx_lds[128];                // [2][64] tile maxima of the two position halves
-  __shared__ float ps_lds[128];                // [2][64] row sums of the two position halves
+  __shared__ __attribute__((aligned(16))) uint8_t p_lds[64 * MM_P_PITCH];    // [64 heads]: bf16 p by K index
+  __shared__ __attribute__((aligned(16))) float sp_lds[2 * 2 * 4 * 32 * 4];  // [hb][kh][q][16 half + head % 16]: score sums of wave (hb, kh) for the other wave's heads
   __shared__ float al_lds[64];                 // [64] exp(M_old - M_new)
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int span = blockIdx.x, b = blockIdx.z;
-  // role in the score product
-  const int hw = wave & 3, pb = wave >> 2;
-  const int c16 = lane & 15, g = lane >> 4;
-  const int head = hw * 16 + c16;
-  // role in the PV product
-  const int hb = wave & 1, cq = wave >> 1;
   const int l32 = lane & 31, half = lane >> 5;
-  const int head2 = hb * 32 + l32;
+  const bool scorer = wave < 4;
+  const int hb = wave & 1, kh = (wave >> 1) & 1;  // score waves
+  const int cq = wave & 3;                        // waves of the second product
   const int seq = a.seqs ? a.seq - (int)(gridDim.z / a.seqs) + 1 + b / a.seqs : a.seq;
   const uint16_t *cache = a.cache + (size_t)(a.seqs ? b % a.seqs : b) * a.seq_stride;
   const int pos0 = span * a.span_tiles * 64, pos_end = min(seq, (span + 1) * a.span_tiles * 64);
@@ -443,219 +444,259 @@ __global__ void __launch_bounds__(512, 1) mla_partial_mfma_k(MlaArgs a) {
   const int n_tiles = (pos_end - pos0 + MM_T - 1) / MM_T;
   const float scale = a.rs * a.mscale * a.mscale;
   constexpr float LOG2E = 1.44269504088896341f;
-  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)nat;  // LDS address of the ring
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)nat;
 
-  // q of this lane's head as B operands: K step ks covers columns 32 ks .. +31, lane group g its 8 g .. +7
-  kx_bf16x8 qf[18];
-  {
-    const float *q = a.qabs + ((size_t)b * a.heads + head) * MLA_KVA;
+  // global -> LDS copy of a tile by the four waves of the second product, which have the time: 2304 pieces = 36
+  // instructions, nine per wave; slot (row p, j') holds piece j' ^ ((p >> 1) & 7) (low three bits) of the row; rows past
+  // the sequence repeat its last row.  The lane's places inside a tile do not change from tile to tile: the nine
+  // source offsets are kept, and only a tile that reaches past the sequence goes through the row clamp.
+  const int cw = wave & 3;
+  int c_off[9];   // elements from the tile's first row
+  int c_row[9];
 #pragma unroll
-    for (int ks = 0; ks < 18; ++ks) {
-      const float4 lo = *(const float4 *)(q + ks * 32 + g * 8), hi = *(const float4 *)(q + ks * 32 + g * 8 + 4);
-      const uint4 u = make_uint4((kx_f32_bits(lo.x) >> 16) | (kx_f32_bits(lo.y) & 0xffff0000u),
-                                 (kx_f32_bits(lo.z) >> 16) | (kx_f32_bits(lo.w) & 0xffff0000u),
-                                 (kx_f32_bits(hi.x) >> 16) | (kx_f32_bits(hi.y) & 0xffff0000u),
-                                 (kx_f32_bits(hi.z) >> 16) | (kx_f32_bits(hi.w) & 0xffff0000u));
-      qf[ks] = __builtin_bit_cast(kx_bf16x8, u);
-    }
+  for (int u = 0; u < 9; ++u) {
+    const int slot = (cw + 4 * u) * 64 + lane;
+    const int p = slot / 72, js = slot - p * 72;
+    const int j = (js & ~7) | ((js ^ (p >> 1)) & 7);
+    c_row[u] = p;
+    c_off[u] = p * MLA_KVA + j * 8;
   }
-  // global -> LDS copy of a tile: 2304 pieces = 36 instructions over the 8 waves; slot (row p, j') holds
-  // piece j' ^ ((p >> 1) & 7) (low three bits) of the row; rows past the sequence repeat its last row
   auto copy_tile = [&](int t) {
+    const int row0 = pos0 + t * MM_T;
+    const uint16_t *src = cache + (size_t)row0 * MLA_KVA;
+    const uint32_t dst = lds0 + (t % MM_RING) * MM_NAT + cw * 1024;
+    if (row0 + MM_T <= seq) {
 #pragma unroll
-    for (int u = 0; u < 5; ++u) {
-      const int ii = wave + 8 * u;
-      if (ii < 36) {
-        const int slot = ii * 64 + lane;
-        const int p = slot / 72, js = slot - p * 72;
-        const int j = (js & ~7) | ((js ^ (p >> 1)) & 7);
-        const int row = min(pos0 + t * MM_T + p, seq - 1);
-        mm_copy16_to_lds(cache + (size_t)row * MLA_KVA + j * 8, lds0 + (t % MM_RING) * MM_NAT + ii * 1024);
-      }
-    }
-  };
-  // byte offsets of this lane's A operands of the score product: row 16 pb + c16, piece 4 ks + g = 8 (ks / 2) + (4 (ks % 2) + g)
-  int s_off[2];
-#pragma unroll
-  for (int o = 0; o < 2; ++o) {
-    const int pr = pb * 16 + c16;
-    s_off[o] = pr * (MLA_KVA * 2) + (((4 * o + g) ^ (pr >> 1)) & 7) * 16;
-  }
-  // byte offsets of this lane's transposing reads for the PV product.  Position r (0-15 inside the 16 positions of
-  // MFMA step s) sits at K index kk(r) = 4 ((r & 7) >> 1) + 2 (r >> 3) + (r & 1): the four K slots 4 w .. 4 w + 3 of
-  // lane half `half` are then positions a, a+1, a+8, a+9 with a = 16 s + 4 half + 2 w, four rows that fall into
-  // four different quarters of the banks (a row is 1152 B = 4.5 bank lines, and the xor of the 16-byte pieces moves
-  // with bit 3 of the position), so a transposing read of a half-wave is free of bank conflicts.  Lane i of its
-  // group of 16 points at row a + ((i >> 2) & 1) + 8 (i >> 3), columns 128 cq + 32 cbk + 16 (group & 1) + 4 (i & 3) .. +3,
-  // i.e. piece 16 cq + 4 cbk + 2 (group & 1) + ((i >> 1) & 1), low or high half by i & 1.  cbk odd flips bit 2 of the
-  // piece (xor 64 on the swizzled offset), cbk >> 1 adds 128.
-  int t_off[2][2];
-  {
-    const int i = lane & 15, grp = (lane >> 4) & 1;
-#pragma unroll
-    for (int sidx = 0; sidx < 2; ++sidx)
-#pragma unroll
-      for (int w = 0; w < 2; ++w) {
-        const int p = 16 * sidx + 4 * half + 2 * w + ((i >> 2) & 1) + 8 * (i >> 3);
-        const int low3 = 2 * grp + ((i >> 1) & 1);
-        t_off[sidx][w] = p * (MLA_KVA * 2) + (2 * cq) * 128 + ((low3 ^ (p >> 1)) & 7) * 16 + (i & 1) * 8;
-      }
-  }
-  // where this score lane's p values go: positions 16 pb + 4 g + v, v = 0, 1 at K index kk0, kk0 + 1 and v = 2, 3 at
-  // kk0 + 4, kk0 + 5 (r = 4 g + v in the formula above)
-  const int p_off = head * MM_P_PITCH + (16 * pb + 8 * (g & 1) + 2 * (g >> 1)) * 2;
-  float M = -__builtin_inff(), Z = 0.0f;  // of `head`; the two waves of a head group keep identical copies
-  float alpha_prev = 1.0f;
-  kx_f32x16v O[4];                        // heads 32 hb .. +31 x columns 128 cq + 32 cbk .. +31
-#pragma unroll
-  for (int cbk = 0; cbk < 4; ++cbk)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) O[cbk][i] = 0.0f;
-
-  // tiles are copied two ahead into the ring; loads complete in order, so waiting until only the copies of the
-  // newest tile (5 instructions for waves 0-3, 4 for the others) are outstanding means tile t has landed
-  auto wait_tile = [&](int t) {
-    if (t + 1 < n_tiles) {
-      if (wave < 4) asm volatile("s_waitcnt vmcnt(5)" ::: "memory");
-      else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+      for (int u = 0; u < 9; ++u) mm_copy16_to_lds(src + c_off[u], dst + u * 4096);
     } else {
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    }
-  };
-  // what follows the first barrier of iteration t for the second product of tile t-1: row sums, p, rescale
-  kx_bf16x8 pf[2];
-  auto pv_begin = [&]() {
-    Z = __builtin_fmaf(Z, alpha_prev, ps_lds[head] + ps_lds[64 + head]);
-    pf[0] = *(const kx_bf16x8 *)(p_lds + head2 * MM_P_PITCH + half * 16);
-    pf[1] = *(const kx_bf16x8 *)(p_lds + head2 * MM_P_PITCH + 32 + half * 16);
-    const float alpha2 = al_lds[head2];
-    if (__builtin_amdgcn_ballot_w64(alpha2 != 1.0f) != 0) {  // the running maximum of some head of the wave moved
-      asm volatile("" ::: "memory");                          // keep this a branch: it is rarely taken after the first tiles
 #pragma unroll
-      for (int cbk = 0; cbk < 4; ++cbk) O[cbk] *= alpha2;
-    }
-  };
-  // the A operands of the second product of the tile staged at LDS byte address sp: for block cbk = m / 2 and
-  // step sidx = m % 2 two transposing reads (K slots 0-3 and 4-7 of the lane's eight)
-  kx_bf16x8 pa[8];
-  auto pv_operands = [&](uint32_t sp) {
-#pragma unroll
-    for (int sidx = 0; sidx < 2; ++sidx) {
-      const uint32_t a0 = sp + t_off[sidx][0], a1 = sp + t_off[sidx][1];              // blocks 0 and 2
-      const uint32_t b0 = sp + (t_off[sidx][0] ^ 64), b1 = sp + (t_off[sidx][1] ^ 64);  // blocks 1 and 3
-      const uint2 l0 = mm_read_tr(a0), h0 = mm_read_tr(a1), l1 = mm_read_tr(b0), h1 = mm_read_tr(b1);
-      const uint2 l2 = mm_read_tr(a0 + 128), h2 = mm_read_tr(a1 + 128), l3 = mm_read_tr(b0 + 128), h3 = mm_read_tr(b1 + 128);
-      pa[0 + sidx] = __builtin_bit_cast(kx_bf16x8, make_uint4(l0.x, l0.y, h0.x, h0.y));
-      pa[2 + sidx] = __builtin_bit_cast(kx_bf16x8, make_uint4(l1.x, l1.y, h1.x, h1.y));
-      pa[4 + sidx] = __builtin_bit_cast(kx_bf16x8, make_uint4(l2.x, l2.y, h2.x, h2.y));
-      pa[6 + sidx] = __builtin_bit_cast(kx_bf16x8, make_uint4(l3.x, l3.y, h3.x, h3.y));
-    }
-  };
-  auto pv_frag = [&](int m) { return pa[m]; };
-  // scores of tile t (staged at st) and, with PV, the second product of tile t-1 (staged at sp), interleaved
-  auto products = [&](auto with_pv, const uint8_t *st, uint32_t sp) {
-    constexpr bool PV = decltype(with_pv)::value;
-    constexpr int AH = 3;  // score operands are read three K steps ahead of the MFMAs that consume them
-    kx_f32x4 sacc = kx_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-    kx_bf16x8 av[AH + 1];
-    if (PV) pv_operands(sp);
-#pragma unroll
-    for (int ks = 0; ks < AH; ++ks) av[ks] = *(const kx_bf16x8 *)(st + s_off[ks & 1] + (ks >> 1) * 128);
-#pragma unroll
-    for (int ks = 0; ks < 18; ++ks) {
-      if (ks + AH < 18) av[(ks + AH) % (AH + 1)] = *(const kx_bf16x8 *)(st + s_off[(ks + AH) & 1] + ((ks + AH) >> 1) * 128);
-      sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[ks % (AH + 1)], qf[ks], sacc, 0, 0, 0);
-      if (PV && (ks & 1) && ks < 16) {  // one MFMA of the second product after every other score step
-        const int m = ks >> 1;
-        O[m >> 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pv_frag(m), pf[m & 1], O[m >> 1], 0, 0, 0);
+      for (int u = 0; u < 9; ++u) {
+        const int back = max(row0 + c_row[u] - (seq - 1), 0);  // rows past the last one
+        mm_copy16_to_lds(src + c_off[u] - back * MLA_KVA, dst + u * 4096);
       }
     }
-    return sacc;
   };
-  // maxima, exponentials, p and row sums of tile t from its score accumulators; contains the second barrier
-  auto softmax_tile = [&](int t, kx_f32x4 sacc) {
-    float sv[4];
-    float mloc = -__builtin_inff();
-#pragma unroll
-    for (int v = 0; v < 4; v += 2) {
-      const int pos = pos0 + t * MM_T + pb * 16 + g * 4 + v;
-      const uint32_t r0 = mm_pack_bf16(sacc[v], sacc[v + 1]);                                                  // bf(q.k)
-      const uint32_t r1 = mm_pack_bf16(kx_bits_f32(r0 << 16) * scale, kx_bits_f32(r0 & 0xffff0000u) * scale);  // bf(. * scale), :429
-      float s0 = kx_bits_f32(r1 << 16), s1 = kx_bits_f32(r1 & 0xffff0000u);
-      if (pos >= pos_end) s0 = -__builtin_inff();
-      if (pos + 1 >= pos_end) s1 = -__builtin_inff();
-      sv[v] = s0;
-      sv[v + 1] = s1;
-      mloc = fmaxf(mloc, fmaxf(s0, s1));
-    }
-    {  // maximum over the four lane groups of the head: lanes l ^ 16 and l ^ 32
-      float o = mloc;
-      kxw::swap_rows16(mloc, o);
-      mloc = fmaxf(mloc, o);
-      o = mloc;
-      kxw::swap_halves32(mloc, o);
-      mloc = fmaxf(mloc, o);
-    }
-    if (g == 0) mx_lds[pb * 64 + head] = mloc;
-    mm_barrier();  // the maxima of both position halves are complete; every wave is done reading p of tile t-1
-    const float Mn = fmaxf(M, fmaxf(mloc, mx_lds[(pb ^ 1) * 64 + head]));
-    // exponentials through v_exp_f32: this path is held to a tolerance, not to the bits of kx_expf
-    const float alpha = __builtin_amdgcn_exp2f((M - Mn) * LOG2E);
-    const float e0 = __builtin_amdgcn_exp2f((sv[0] - Mn) * LOG2E), e1 = __builtin_amdgcn_exp2f((sv[1] - Mn) * LOG2E);
-    const float e2 = __builtin_amdgcn_exp2f((sv[2] - Mn) * LOG2E), e3 = __builtin_amdgcn_exp2f((sv[3] - Mn) * LOG2E);
-    float ps = (e0 + e1) + (e2 + e3);
-    {
-      float o = ps;
-      kxw::swap_rows16(ps, o);
-      ps += o;
-      o = ps;
-      kxw::swap_halves32(ps, o);
-      ps += o;
-    }
-    *(uint32_t *)(p_lds + p_off) = mm_pack_bf16(e0, e1);
-    *(uint32_t *)(p_lds + p_off + 8) = mm_pack_bf16(e2, e3);
-    if (g == 0) {
-      ps_lds[pb * 64 + head] = ps;
-      if (pb == 0) al_lds[head] = alpha;
-    }
-    M = Mn;
-    alpha_prev = alpha;
+  // Tile t + 3 is requested behind the second barrier of iteration t, into the ring buffer of tile t - 1 (whose
+  // operands are in registers by then).  At the top of iteration t the copies of tiles t + 1 and t + 2, nine each,
+  // are the wave's newest: tile t has landed when only they are outstanding.
+  auto wait_tile = [&](int t) {
+    if (t + 2 < n_tiles) asm volatile("s_waitcnt vmcnt(18)" ::: "memory");
+    else if (t + 1 < n_tiles) asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   };
 
-  copy_tile(0);
-  if (n_tiles > 1) copy_tile(1);
-  // tile 0: scores only
-  wait_tile(0);
-  mm_barrier();
-  if (2 < n_tiles) copy_tile(2);
-  softmax_tile(0, products(std::false_type{}, nat, lds0));
-  for (int t = 1; t < n_tiles; ++t) {
-    wait_tile(t);
-    mm_barrier();  // everybody's share of tile t has landed; p, row sums and rescale factors of tile t-1 are complete
-    if (t + 2 < n_tiles) copy_tile(t + 2);
-    pv_begin();
-    softmax_tile(t, products(std::true_type{}, nat + (t % MM_RING) * MM_NAT, lds0 + ((t - 1) % MM_RING) * MM_NAT));
+  if (!scorer) {
+    copy_tile(0);
+    if (n_tiles > 1) copy_tile(1);
+    if (n_tiles > 2) copy_tile(2);
   }
-  // the second product of the last tile
-  mm_barrier();
-  pv_begin();
-  pv_operands(lds0 + ((n_tiles - 1) % MM_RING) * MM_NAT);
+  // One loop per kind of wave, with the same barriers in the same order: the registers of one kind (q, 72; the
+  // output blocks, 128) are then not live in the other's loop.
+  if (scorer) {
+    // q of head 32 hb + l32 as B operands; K step 18 kh + i covers columns 16 (18 kh + i) + 8 half .. +7
+    kx_bf16x8 qf[18];
+    {
+      const float *q = a.qabs + ((size_t)b * a.heads + hb * 32 + l32) * MLA_KVA + kh * 288 + half * 8;
 #pragma unroll
-  for (int m = 0; m < 8; ++m) O[m >> 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pv_frag(m), pf[m & 1], O[m >> 1], 0, 0, 0);
-  // partials.  Maxima and sums: the score lanes of the first position half; O: lane = (head, column
-  // 128 cq + 32 cbk + 8 q + 4 half + c) for accumulator register 4 q + c
-  if (pb == 0 && g == 0) {
-    const size_t idx = ((size_t)b * a.spans + span) * a.heads + head;
-    a.pm[idx] = M;
-    a.pz[idx] = Z;
+      for (int i = 0; i < 18; ++i) {
+        const float4 lo = *(const float4 *)(q + i * 16), hi = *(const float4 *)(q + i * 16 + 4);
+        const uint4 u = make_uint4((kx_f32_bits(lo.x) >> 16) | (kx_f32_bits(lo.y) & 0xffff0000u),
+                                   (kx_f32_bits(lo.z) >> 16) | (kx_f32_bits(lo.w) & 0xffff0000u),
+                                   (kx_f32_bits(hi.x) >> 16) | (kx_f32_bits(hi.y) & 0xffff0000u),
+                                   (kx_f32_bits(hi.z) >> 16) | (kx_f32_bits(hi.w) & 0xffff0000u));
+        qf[i] = __builtin_bit_cast(kx_bf16x8, u);
+      }
+    }
+    // A operands: row l32, piece 2 ks + half = 8 (ks / 4) + (2 (ks % 4) + half) with ks = 18 kh + i; s_off[u] is the
+    // swizzled place of piece 2 u + half inside its group of eight
+    int s_off[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) s_off[u] = l32 * (MLA_KVA * 2) + (((2 * u + half) ^ (l32 >> 1)) & 7) * 16;
+    // After the products, wave kh keeps heads 16 kh .. +15 of the block.  Its lanes with the other wave's heads
+    // (row = lane / 16 odd for kh = 0, even for kh = 1) put their sums into LDS for that wave and then take over
+    // positions 16 .. 31 of the head 16 lanes away (v_permlane16_swap), so that every lane has eight positions of a
+    // head of the wave: lane = (head 16 kh + lane % 16, half, qsel), positions 8 q + 4 half + c with q = 2 qsel + j / 4,
+    // c = j % 4 for value j.
+    const int h16 = lane & 15;
+    const int qsel = ((l32 >> 4) != kh) ? 1 : 0;
+    const int headx = hb * 32 + kh * 16 + h16;
+    float M = -__builtin_inff(), Z = 0.0f;  // of headx; the four lanes of a head keep identical copies
+    kx_f32x16v sacc;
+    float v[8];
+    auto scores = [&](auto k_first, const uint8_t *st) {
+      constexpr int K0 = decltype(k_first)::value;
+      constexpr int AH = 3;
+      kx_bf16x8 av[AH + 1];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) sacc[i] = 0.0f;
+#pragma unroll
+      for (int i = 0; i < AH; ++i) av[i] = *(const kx_bf16x8 *)(st + s_off[(K0 + i) & 3] + ((K0 + i) >> 2) * 128);
+#pragma unroll
+      for (int i = 0; i < 18; ++i) {
+        if (i + AH < 18)
+          av[(i + AH) % (AH + 1)] = *(const kx_bf16x8 *)(st + s_off[(K0 + i + AH) & 3] + ((K0 + i + AH) >> 2) * 128);
+        sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[i % (AH + 1)], qf[i], sacc, 0, 0, 0);
+      }
+      // accumulator 4 q + c of lane (head l32, half) is position 8 q + 4 half + c
+      if (qsel) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          *(float4 *)(sp_lds + ((((hb * 2 + kh) * 4 + q) * 32) + 16 * half + h16) * 4) =
+              make_float4(sacc[4 * q], sacc[4 * q + 1], sacc[4 * q + 2], sacc[4 * q + 3]);
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        float x = sacc[j], y = sacc[8 + j];
+        if (K0 == 0) {  // rows 1, 3 of x <- rows 0, 2 of y
+          kxw::swap_rows16(x, y);
+          v[j] = x;
+        } else {        // rows 0, 2 of x <- rows 1, 3 of y
+          kxw::swap_rows16(y, x);
+          v[j] = x;
+        }
+      }
+    };
+    auto softmax_tile = [&](int t) {
+      float sv[8];
+      float mloc = -__builtin_inff();
+#pragma unroll
+      for (int qq = 0; qq < 2; ++qq) {
+        const int q = 2 * qsel + qq;
+        const float4 o = *(const float4 *)(sp_lds + ((((hb * 2 + (kh ^ 1)) * 4 + q) * 32) + 16 * half + h16) * 4);
+        const float sum[4] = {v[4 * qq] + o.x, v[4 * qq + 1] + o.y, v[4 * qq + 2] + o.z, v[4 * qq + 3] + o.w};
+#pragma unroll
+        for (int c = 0; c < 4; c += 2) {
+          const int pos = pos0 + t * MM_T + 8 * q + 4 * half + c;
+          const uint32_t r0 = mm_pack_bf16(sum[c], sum[c + 1]);                                                     // bf(q.k)
+          const uint32_t r1 = mm_pack_bf16(kx_bits_f32(r0 << 16) * scale, kx_bits_f32(r0 & 0xffff0000u) * scale);  // bf(. * scale)
+          float s0 = kx_bits_f32(r1 << 16), s1 = kx_bits_f32(r1 & 0xffff0000u);
+          if (pos >= pos_end) s0 = -__builtin_inff();
+          if (pos + 1 >= pos_end) s1 = -__builtin_inff();
+          sv[4 * qq + c] = s0;
+          sv[4 * qq + c + 1] = s1;
+          mloc = fmaxf(mloc, fmaxf(s0, s1));
+        }
+      }
+      {  // maximum over the four lanes of the head: lanes l ^ 16 and l ^ 32
+        float o = mloc;
+        kxw::swap_rows16(mloc, o);
+        mloc = fmaxf(mloc, o);
+        o = mloc;
+        kxw::swap_halves32(mloc, o);
+        mloc = fmaxf(mloc, o);
+      }
+      const float Mn = fmaxf(M, mloc);
+      const float alpha = __builtin_amdgcn_exp2f((M - Mn) * LOG2E);
+      float e[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) e[i] = __builtin_amdgcn_exp2f((sv[i] - Mn) * LOG2E);
+      float ps = ((e[0] + e[1]) + (e[2] + e[3])) + ((e[4] + e[5]) + (e[6] + e[7]));
+      {
+        float o = ps;
+        kxw::swap_rows16(ps, o);
+        ps += o;
+        o = ps;
+        kxw::swap_halves32(ps, o);
+        ps += o;
+      }
+      // the lane's positions are those of MFMA step qsel; inside the step position 8 (q % 2) + 4 half + c sits at K index
+      // 8 half + 4 (c / 2) + 2 (q % 2) + (c % 2): one 16-byte piece per lane
+      *(uint4 *)(p_lds + headx * MM_P_PITCH + qsel * 32 + half * 16) =
+          make_uint4(mm_pack_bf16(e[0], e[1]), mm_pack_bf16(e[4], e[5]), mm_pack_bf16(e[2], e[3]), mm_pack_bf16(e[6], e[7]));
+      if (half == 0 && qsel == 0) al_lds[headx] = alpha;
+      Z = __builtin_fmaf(Z, alpha, ps);
+      M = Mn;
+    };
+    for (int t = 0; t <= n_tiles; ++t) {
+      mm_barrier();  // tile t has landed (the copying waves have waited for it); p and the factors of tile t-1 are complete
+      if (t < n_tiles) {
+        const uint8_t *st = nat + (t % MM_RING) * MM_NAT;
+        if (kh == 0) scores(std::integral_constant<int, 0>{}, st);
+        else scores(std::integral_constant<int, 18>{}, st);
+      }
+      mm_barrier();  // the score sums are visible; p of tile t-1 is in the registers of the other waves
+      if (t < n_tiles) softmax_tile(t);
+    }
+    if (half == 0 && qsel == 0) {
+      const size_t idx = ((size_t)b * a.spans + span) * a.heads + headx;
+      a.pm[idx] = M;
+      a.pz[idx] = Z;
+    }
+  } else {
+    // transposing reads of the second product: as in mla_partial_mfma_k
+    int t_off[2][2];
+    {
+      const int i = lane & 15, grp = (lane >> 4) & 1;
+#pragma unroll
+      for (int sidx = 0; sidx < 2; ++sidx)
+#pragma unroll
+        for (int w = 0; w < 2; ++w) {
+          const int p = 16 * sidx + 4 * half + 2 * w + ((i >> 2) & 1) + 8 * (i >> 3);
+          const int low3 = 2 * grp + ((i >> 1) & 1);
+          t_off[sidx][w] = p * (MLA_KVA * 2) + (2 * cq) * 128 + ((low3 ^ (p >> 1)) & 7) * 16 + (i & 1) * 8;
+        }
+    }
+    kx_f32x16v O[2][4];  // [head block][cbk]: heads x columns 128 cq + 32 cbk .. +31
+#pragma unroll
+    for (int h2 = 0; h2 < 2; ++h2)
+#pragma unroll
+      for (int cbk = 0; cbk < 4; ++cbk)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) O[h2][cbk][i] = 0.0f;
+    kx_bf16x8 pf[2][2], pa[8];
+    // what the second product of a tile needs from LDS: p of both head blocks, the factors, the transposed operands
+    auto pv_begin = [&](uint32_t sp) {
+#pragma unroll
+      for (int h2 = 0; h2 < 2; ++h2) {
+        pf[h2][0] = *(const kx_bf16x8 *)(p_lds + (h2 * 32 + l32) * MM_P_PITCH + half * 16);
+        pf[h2][1] = *(const kx_bf16x8 *)(p_lds + (h2 * 32 + l32) * MM_P_PITCH + 32 + half * 16);
+        const float alpha2 = al_lds[h2 * 32 + l32];
+        if (__builtin_amdgcn_ballot_w64(alpha2 != 1.0f) != 0) {  // the running maximum of some head of the block moved
+          asm volatile("" ::: "memory");                          // keep this a branch: it is rarely taken after the first tiles
+#pragma unroll
+          for (int cbk = 0; cbk < 4; ++cbk) O[h2][cbk] *= alpha2;
+        }
+      }
+#pragma unroll
+      for (int sidx = 0; sidx < 2; ++sidx) {
+        const uint32_t a0 = sp + t_off[sidx][0], a1 = sp + t_off[sidx][1];
+        const uint32_t b0 = sp + (t_off[sidx][0] ^ 64), b1 = sp + (t_off[sidx][1] ^ 64);
+        const uint2 l0 = mm_read_tr(a0), h0 = mm_read_tr(a1), l1 = mm_read_tr(b0), h1 = mm_read_tr(b1);
+        const uint2 l2 = mm_read_tr(a0 + 128), h2 = mm_read_tr(a1 + 128), l3 = mm_read_tr(b0 + 128), h3 = mm_read_tr(b1 + 128);
+        pa[0 + sidx] = __builtin_bit_cast(kx_bf16x8, make_uint4(l0.x, l0.y, h0.x, h0.y));
+        pa[2 + sidx] = __builtin_bit_cast(kx_bf16x8, make_uint4(l1.x, l1.y, h1.x, h1.y));
+        pa[4 + sidx] = __builtin_bit_cast(kx_bf16x8, make_uint4(l2.x, l2.y, h2.x, h2.y));
+        pa[6 + sidx] = __builtin_bit_cast(kx_bf16x8, make_uint4(l3.x, l3.y, h3.x, h3.y));
+      }
+    };
+    auto pv_mfma = [&](int m0, int m1) {
+#pragma unroll
+      for (int m = 0; m < 8; ++m)
+        if (m >= m0 && m < m1) {
+          O[0][m >> 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pa[m], pf[0][m & 1], O[0][m >> 1], 0, 0, 0);
+          O[1][m >> 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pa[m], pf[1][m & 1], O[1][m >> 1], 0, 0, 0);
+        }
+    };
+    for (int t = 0; t <= n_tiles; ++t) {
+      if (t < n_tiles) wait_tile(t);
+      mm_barrier();
+      if (t > 0) pv_begin(lds0 + ((t - 1) % MM_RING) * MM_NAT);
+      mm_barrier();
+      if (t + 3 < n_tiles) copy_tile(t + 3);
+      if (t > 0) pv_mfma(0, 8);
+    }
+    // O: lane = (head, column 128 cq + 32 cbk + 8 q + 4 half + c) for accumulator register 4 q + c
+#pragma unroll
+    for (int h2 = 0; h2 < 2; ++h2) {
+      const size_t idx2 = ((size_t)b * a.spans + span) * a.heads + h2 * 32 + l32;
+#pragma unroll
+      for (int cbk = 0; cbk < 4; ++cbk)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          *(float4 *)(a.po + idx2 * MLA_R + cq * 128 + cbk * 32 + q * 8 + half * 4) =
+              make_float4(O[h2][cbk][4 * q], O[h2][cbk][4 * q + 1], O[h2][cbk][4 * q + 2], O[h2][cbk][4 * q + 3]);
+    }
   }
-  const size_t idx2 = ((size_t)b * a.spans + span) * a.heads + head2;
-#pragma unroll
-  for (int cbk = 0; cbk < 4; ++cbk)
-#pragma unroll
-    for (int q = 0; q < 4; ++q)
-      *(float4 *)(a.po + idx2 * MLA_R + cq * 128 + cbk * 32 + q * 8 + half * 4) =
-          make_float4(O[cbk][4 * q], O[cbk][4 * q + 1], O[cbk][4 * q + 2], O[cbk][4 * q + 3]);
 }
 
 // merge of the spans; grid (heads, B), one wave, lane = 8 latent columns

@@ -59,8 +59,11 @@ class KxModel:
 EXCUSED_SMALL_STACK = {(16, 1): [], (16, 0): [], (8, 1): [], (8, 0): [], (5, 1): [], (5, 0): [],
                        (40, 1): [("sequence 16", "argmax", None)], (40, 0): [("sequence 16", "argmax", None)]}
 EXCUSED_ATTENTION_PATHS = []
-EXCUSED_AGAINST_SINGLE = {16: [("sequence 0", "router", 1)],
-                          32: [("sequence 0", "router", 1), ("sequence 20", "router", 1), ("sequence 29", "argmax", None)]}
+# (sequence 7: the reference run's two largest logits are equal to the bit; it joined the sets with the matrix-core
+# attention kernel that splits the two products between the waves, whose sums run in another order)
+EXCUSED_AGAINST_SINGLE = {16: [("sequence 0", "router", 1), ("sequence 7", "argmax", None)],
+                          32: [("sequence 0", "router", 1), ("sequence 20", "router", 1), ("sequence 29", "argmax", None),
+                               ("sequence 7", "argmax", None)]}
 
 
 def test_rope_table_matches_oracle(kxlib, ox):
