@@ -116,6 +116,13 @@ int kx_grouped_gemm_launch(bool dual, bool i4, const void *w0, const uint16_t *s
                            const uint16_t *x, void *out, int out_mode, const int4 *work, const int *pairs, int n_pairs,
                            int n_slots, int N, int K, int x_div, size_t expert_w, size_t expert_s, int n_pairs_max,
                            hipStream_t st, int cnt_lo = 0);
+// kx_i4mm.hip: the experts of the work list with cnt_lo .. cnt_hi pairs as W4A16 products on the matrix cores with the
+// weights streamed into registers, up to 32 tokens of an expert per pass (passes: grid depth; an expert's pairs beyond
+// 32 * passes are not computed).  out[pair][N] = W[expert] x[pair / x_div], or swiglu(W0 x, W1 x) with two matrices.
+// *done = false (nothing launched) when the shape is not the kernel's.
+int kx_i4mm_launch(bool dual, const uint32_t *w0, const uint16_t *s0, const uint32_t *w1, const uint16_t *s1, const uint16_t *x,
+                   uint16_t *out, const int4 *work, const int *pairs, int n_slots, int N, int K, int x_div, size_t expert_w,
+                   size_t expert_s, int cnt_lo, int cnt_hi, int passes, bool *done, hipStream_t st);
 // kx_skinny.hip: one tile of up to 32 tokens against a bf16 matrix (two for SwiGLU) on the matrix cores, out_mode as
 // above.  *done = false (nothing launched) when the shape is not the kernel's.
 int kx_skinny_gemm_launch(bool dual, const uint16_t *w0, const uint16_t *w1, const uint16_t *x, int x_stride, void *out,
@@ -132,7 +139,8 @@ struct kx_moe_workspace;
 #define KX_MOE_SHARED_MATRIX_CORES 0x200u
 // 5 tokens and more: the routed experts with three or more pairs as W4A16 grouped GEMMs on the matrix cores
 // (kx_prefill.hip) instead of the GEMV kernels: such an expert's weights are streamed and dequantised once for all its
-// tokens (tolerance instead of bit parity); the experts with one or two pairs keep the GEMV kernel
+// tokens (tolerance instead of bit parity); the experts with one or two pairs keep the GEMV kernel.  From 32 to 64
+// tokens: the experts with two or more pairs through kx_i4mm.hip (weights dequantized in registers, f16 products)
 #define KX_MOE_ROUTED_MATRIX_CORES 0x400u
 // internal (not among the public flags): the layer's first launch -- normed row in d_n, router logits, routing, shared
 // gate/up -- has been done by the caller's own launch (kx_front.hip's back launch with kx_moe_head_args): one token

@@ -258,7 +258,13 @@ static int moe_layer_body(const kx_config *c, const kx_moe_weights *w, kx_moe_wo
   // workgroup holds a CU for the whole of its 112 K steps whatever its tokens, and at 32 sequences the experts with
   // two pairs made the GEMMs a round of 256 workgroups and a twelfth (measured, batch 32: 1897 tok/s with the line
   // at two pairs, 1983 at three, 1941 at four, 1812 at six; batch 16: 1313 -> 1325; batch 12: level)
-  constexpr int rmm_min = 3;
+  // From 32 to 64 tokens the matrix-core class is run by the kernel that dequantizes in registers (kx_i4mm.hip),
+  // which costs about as much as a GEMV pass over the expert whatever its tokens: it takes the experts from two
+  // pairs on (batch 32: 2514 tok/s against 2497 with the grouped GEMMs from three pairs and 2435 / 2296 with this
+  // kernel from three / one; 64 tokens of the one-layer bench: 1.87 ms against 2.00 ms on the GEMV kernels alone and
+  // 2.10 ms with the grouped GEMMs; batch 16: 1526 against 1570, so smaller batches keep the grouped GEMMs).
+  const bool i4mm = rmm && tokens >= 32 && tokens <= 64;
+  const int rmm_min = i4mm ? 2 : 3;
   bool shared_up_done = false, shared_down_done = false;
   if (mm && !norm_w) {
     KX_HIP(hipEventRecord(ws->fork, st));
@@ -320,7 +326,13 @@ static int moe_layer_body(const kx_config *c, const kx_moe_weights *w, kx_moe_wo
     KX_HIP(hipEventRecord(ws->fork, st));  // the routing is in
     KX_HIP(hipStreamWaitEvent(ws->side, ws->fork, 0));
     forked = true;
-    if ((rc = kx_grouped_gemm_launch(true, true, w->d_gate_packed, (const uint16_t *)w->d_gate_scale, w->d_up_packed,
+    bool mm_done = false;
+    if (i4mm &&
+        (rc = kx_i4mm_launch(true, (const uint32_t *)w->d_gate_packed, (const uint16_t *)w->d_gate_scale, (const uint32_t *)w->d_up_packed,
+                             (const uint16_t *)w->d_up_scale, n, ws->mid, ws->work, ws->pairs, n_slots, I, H, K, (size_t)I * (H / 8),
+                             (size_t)I * (H / 32), rmm_min, 1 << 30, kx_cdiv(tokens, 32), &mm_done, st))) return rc;
+    if (!mm_done &&
+        (rc = kx_grouped_gemm_launch(true, true, w->d_gate_packed, (const uint16_t *)w->d_gate_scale, w->d_up_packed,
                                      (const uint16_t *)w->d_up_scale, n, ws->mid, KX_GG_BF16, ws->work, ws->pairs, 0, n_slots, I, H,
                                      K, (size_t)I * (H / 8), (size_t)I * (H / 32), tokens, st, rmm_min))) return rc;
     if ((rc = kx_i4_launch(true, (const uint32_t *)w->d_gate_packed, (const uint16_t *)w->d_gate_scale,
@@ -347,7 +359,13 @@ static int moe_layer_body(const kx_config *c, const kx_moe_weights *w, kx_moe_wo
   // routed down
   if (rmm) {
     const int I = c->moe_inter;
-    if ((rc = kx_grouped_gemm_launch(false, true, w->d_down_packed, (const uint16_t *)w->d_down_scale, nullptr, nullptr,
+    bool mm_done = false;
+    if (i4mm &&
+        (rc = kx_i4mm_launch(false, (const uint32_t *)w->d_down_packed, (const uint16_t *)w->d_down_scale, nullptr, nullptr, ws->mid,
+                             ws->eout, ws->work, ws->pairs, n_slots, H, I, 1, (size_t)H * (I / 8), (size_t)H * (I / 32), rmm_min,
+                             1 << 30, kx_cdiv(tokens, 32), &mm_done, st))) return rc;
+    if (!mm_done &&
+        (rc = kx_grouped_gemm_launch(false, true, w->d_down_packed, (const uint16_t *)w->d_down_scale, nullptr, nullptr,
                                      ws->mid, ws->eout, KX_GG_BF16, ws->work, ws->pairs, 0, n_slots, H, I, 1, (size_t)H * (I / 8),
                                      (size_t)H * (I / 32), tokens, st, rmm_min))) return rc;
     if ((rc = kx_i4_launch(false, (const uint32_t *)w->d_down_packed, (const uint16_t *)w->d_down_scale, nullptr, nullptr,

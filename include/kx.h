@@ -190,7 +190,8 @@ int kx_moe_workspace_views(kx_moe_workspace *ws, void **d_logits, void **d_ids, 
  *             summation order: within max-rel 1e-2 of the default instead of equal to the bit).
  *       bit10: 5 tokens and more: the routed experts that have three or more (token, slot) pairs as W4A16
  *             grouped GEMMs on the matrix cores, the experts with one or two pairs through the GEMV kernel (same
- *             tolerance).  The router is not affected by either bit, so the routing stays the default's.
+ *             tolerance); from 32 to 64 tokens the experts with two or more pairs, by a kernel that dequantizes
+ *             to f16 in registers.  The router is not affected by either bit, so the routing stays the default's.
  *             The decoder stack sets bit9 from 5 sequences on and bit10 from 12. */
 int kx_moe_decode_layer(const kx_config *cfg, const kx_moe_weights *w, kx_moe_workspace *ws,
                         const void *d_n, void *d_x, int32_t tokens, uint32_t flags, void *stream);

@@ -112,10 +112,16 @@ def judge_sequences(names, errs, bar, routes_a, routes_ref, ids_a, ids_ref, logi
 
 def assert_excused(excused, expected, what):
     """The excused sequences of a fixed seed are a fixed set: anything else excused, or a sequence no longer excused,
-    is a change of the kernels' arithmetic and has to be looked at, not absorbed by a budget."""
+    is a change of the kernels' arithmetic and has to be looked at, not absorbed by a budget.  An entry with a fourth
+    element, (sequence, "argmax", None, "either way"), names a sequence whose two largest reference logits are so close
+    (equal to the bit, in the cases recorded) that every change of a summation order may break the tie the other way:
+    it may be excused or not; judge_sequences has checked the gap when it is."""
     got = sorted(e.key for e in excused)
     print(f"{what}: excused keys {got}", flush=True)
-    assert got == sorted(expected), f"{what}: excused {got}, expected {sorted(expected)}"
+    required = sorted(e[:3] for e in expected if len(e) == 3)
+    optional = [e[:3] for e in expected if len(e) == 4]
+    left = sorted(k for k in got if k not in optional)
+    assert left == required, f"{what}: excused {got}, expected {required} (and possibly {optional})"
 
 
 def moe_device_weights(host):

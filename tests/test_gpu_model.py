@@ -56,14 +56,15 @@ class KxModel:
 # "argmax", first MoE layer whose expert set differs).  Every entry was checked when it was recorded -- the reference
 # run's selection gap in that layer is below kxt.NEAR_TIE, or its two largest logits lie closer than the bar -- and
 # judge_sequences checks it again on every run.  A set that changes means the arithmetic of a kernel changed.
+EITHER = "either way"  # a tie of the reference's two largest logits: see kxt.assert_excused
 EXCUSED_SMALL_STACK = {(16, 1): [], (16, 0): [], (8, 1): [], (8, 0): [], (5, 1): [], (5, 0): [],
-                       (40, 1): [("sequence 16", "argmax", None)], (40, 0): [("sequence 16", "argmax", None)]}
+                       (40, 1): [("sequence 16", "argmax", None, EITHER)], (40, 0): [("sequence 16", "argmax", None, EITHER)]}
 EXCUSED_ATTENTION_PATHS = []
-# (sequence 7: the reference run's two largest logits are equal to the bit; it joined the sets with the matrix-core
-# attention kernel that splits the two products between the waves, whose sums run in another order)
-EXCUSED_AGAINST_SINGLE = {16: [("sequence 0", "router", 1), ("sequence 7", "argmax", None)],
+# sequence 7: the reference run's two largest logits are equal to the bit; the matrix-core attention kernel with the
+# two products on different waves broke the tie one way, the f16 routed kernel of 32 sequences the other
+EXCUSED_AGAINST_SINGLE = {16: [("sequence 0", "router", 1), ("sequence 7", "argmax", None, EITHER)],
                           32: [("sequence 0", "router", 1), ("sequence 20", "router", 1), ("sequence 29", "argmax", None),
-                               ("sequence 7", "argmax", None)]}
+                               ("sequence 7", "argmax", None, EITHER)]}
 
 
 def test_rope_table_matches_oracle(kxlib, ox):

@@ -189,10 +189,11 @@ def test_moe_layer_kimi_shape(kxlib, ox, T):
     _assert_layer(got, exp)
 
 
-@pytest.mark.parametrize("T,bits", [(16, 0x600), (32, 0x600), (32, 0x200), (32, 0x400), (7, 0x600)])
+@pytest.mark.parametrize("T,bits", [(16, 0x600), (32, 0x600), (32, 0x200), (32, 0x400), (7, 0x600), (48, 0x400), (64, 0x600)])
 def test_moe_layer_kimi_shape_matrix_core_forms(kxlib, ox, T, bits):
     # What the stack runs from 5 (bit 9: shared expert as bf16 matrix-core products) and 12 sequences on (bit 10:
-    # routed experts with several pairs as W4A16 grouped GEMMs, the others through the one-token GEMV kernel), reached
+    # routed experts with several pairs as W4A16 grouped GEMMs -- from 32 tokens on through the kernel that dequantizes
+    # in registers and multiplies in f16 --, the others through the one-token GEMV kernel), reached
     # through the C ABI.  The layer output `down` (flag bit 0: no residual, so the bar is on the layer's own result):
     # within 1e-2 as normalised maximum (2e-2 element-wise: see _assert_layer) of the default GEMV form for every token, and of the
     # oracle's reference schedule given the GPU's routing on a sample of tokens; the routing itself must be the
