@@ -191,6 +191,16 @@ def test_moe_layer_kimi_shape(kxlib, ox, T):
 
 @pytest.mark.parametrize("T,bits", [(16, 0x600), (32, 0x600), (32, 0x200), (32, 0x400), (7, 0x600), (48, 0x400), (64, 0x600)])
 def test_moe_layer_kimi_shape_matrix_core_forms(kxlib, ox, T, bits):
+    _matrix_core_forms(kxlib, ox, T, bits, ())
+
+
+def test_moe_layer_kimi_shape_matrix_core_forms_with_every_token_on_two_experts(kxlib, ox):
+    # 48 tokens that all select experts 5 and 200 (a large router bias): 48 pairs on each, more than the 32 tokens of
+    # one pass of the kernel that takes the experts of several pairs from 32 tokens on -- two passes, the second with 16
+    _matrix_core_forms(kxlib, ox, 48, 0x400, (5, 200))
+
+
+def _matrix_core_forms(kxlib, ox, T, bits, hot):
     # What the stack runs from 5 (bit 9: shared expert as bf16 matrix-core products) and 12 sequences on (bit 10:
     # routed experts with several pairs as W4A16 grouped GEMMs -- from 32 tokens on through the kernel that dequantizes
     # in registers and multiplies in f16 --, the others through the one-token GEMV kernel), reached
@@ -201,6 +211,10 @@ def test_moe_layer_kimi_shape_matrix_core_forms(kxlib, ox, T, bits):
     say(f"moe layer kimi shape T={T} flags={bits:#x}")
     H, I, SI, E, K = 7168, 2048, 2048, 384, 8
     host, n, x = moe_case(kxlib, H, I, SI, E, K, T, 9)
+    if hot:
+        host = dict(host)   # the cached case stays as it is
+        host["router_bias"] = host["router_bias"].copy()
+        host["router_bias"][list(hot)] += 10.0
     cfg = moe_cfg(H, I, SI, E, K)
     w, bufs = moe_device_weights(host)
     ws = C.c_void_p()
@@ -224,6 +238,8 @@ def test_moe_layer_kimi_shape_matrix_core_forms(kxlib, ox, T, bits):
     (d0, ids0, w0), (d1, ids1, w1) = res[1], res[1 | bits]
     assert (ids0 == ids1).all() and (w0.view(np.uint32) == w1.view(np.uint32)).all()
     pairs = np.bincount(ids0.ravel(), minlength=E)
+    for e in hot:
+        assert pairs[e] == T, f"expert {e} was meant to be selected by every token, has {pairs[e]} pairs"
     e_max, e_el = O.max_rel(d1, d0), O.elem_err(d1, d0)
     print(f"{(pairs > 0).sum()} experts, {(pairs > 1).sum()} with several pairs (most: {pairs.max()}); "
           f"vs the GEMV form: max-rel {e_max:.2e}, element-wise {e_el:.2e}", flush=True)
