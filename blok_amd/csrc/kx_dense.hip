@@ -288,6 +288,10 @@ int gemv_plan(int epi, KxGemvArgs &a, int &ri, int ri_max, int target_chunks = 2
   while (a.rs > 1 && a.rs > a.rows) a.rs >>= 1;
   // rows per wave and tile, tiles per chunk: a few hundred chunks when the matrix allows
   ri = a.rows >= 2048 * a.rs ? 4 : a.rows >= 768 * a.rs ? 2 : 1;
+  // From two tokens on the chunks are made for one round of workgroups anyway (below), and a wave spends a load's
+  // latency on every tile: four rows per tile whatever the matrix (q_a|kv_a at four tokens: 10 steps of two rows per
+  // wave, 23 us; W_UV the same).
+  if (a.tokens >= 2 && !(a.row_block && a.row_block % (4 * a.rs))) ri = 4;
   while (ri > 1 && ri * a.rs > a.rows) ri >>= 1;
   if (ri * mats > 4) ri = 4 / mats;
   if (ri > ri_max) ri = ri_max;
